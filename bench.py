@@ -1,0 +1,214 @@
+"""Benchmark of the tile-kernel hot path on one MI355X.
+
+One "step" is one launch of the headline workload: the fp16 GEMM M=N=K=4096 (A row-major,
+B column-major, f32 accumulate, f16 output), inputs resident in HBM. The other BASELINE
+configurations (GEMM 128x64x256, back-to-back GEMM, FlashAttention-2 forward, fused LSTM)
+are timed in the same run and reported under "configs".
+
+Prints ONE JSON line: the driver's contract fields plus
+  roofline     -- dominant kernel vs the MFMA fp16 dense peak (2.5 PFLOP/s) / HBM (8 TB/s)
+  cpu_baseline -- the CPU oracle (OpenMP, f32) timed on this host for the same workload
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
+HBM_PEAK_GBS = 8000.0
+
+
+def time_kernel(fn, steps, warmup):
+    """Average milliseconds per call of fn(), HIP events on the stream fn launches on
+    (torch's current stream, which is the stream handed to the C-ABI)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--only", default="", help="comma-separated subset of gemm,c1,b2b,attn,lstm (gemm always runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import tiledcuda_amd as tcu
+    from oracle import oracle  # checker + cpu_baseline leg only
+
+    tcu.lib()
+    dev = torch.device("cuda:0")
+    only = set(filter(None, args.only.split(",")))
+
+    def want(name):
+        return not only or name in only
+
+    def to_dev(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    configs = []
+
+    # ---------------------------------------------------------------- C2: GEMM 4096^3 (headline)
+    n = 4096
+    A = oracle.fill_uniform(n * n, 1236).reshape(n, n)
+    Bt = oracle.fill_uniform(n * n, 2236).reshape(n, n)
+    dA, dB = to_dev(A), to_dev(Bt)
+    dC = torch.empty(n, n, dtype=torch.float16, device=dev)
+    gemm_flops = 2.0 * n * n * n
+
+    def gemm_step():
+        tcu.gemm(dA, dB, out=dC)
+
+    for _ in range(args.warmup):
+        gemm_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(args.steps):
+        gemm_step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    gemm_ms = start.elapsed_time(stop) / args.steps
+    gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
+
+    rows = (1920, 2048)
+    ref = oracle.gemm(A, Bt, rows=rows)
+    gemm_err = oracle.max_rel_err(dC[rows[0]:rows[1]].float().cpu().numpy(), ref[rows[0]:rows[1]])
+    configs.append({"name": "gemm_4096", "ms": gemm_ms, "tflops": gemm_tflops,
+                    "frac_mfma_peak": gemm_tflops / MFMA_F16_PEAK_TFLOPS, "max_rel_err": gemm_err})
+
+    # ---------------------------------------------------------------- C1: GEMM 128x64x256
+    if want("c1"):
+        A1 = oracle.fill_uniform(128 * 256, 1235).reshape(128, 256)
+        B1 = oracle.fill_uniform(64 * 256, 2235).reshape(64, 256)
+        d1a, d1b = to_dev(A1), to_dev(B1)
+        d1c = torch.empty(128, 64, dtype=torch.float32, device=dev)
+        for algo in ("global_reg", "pipelined"):
+            ms = time_kernel(lambda: tcu.gemm(d1a, d1b, out=d1c, algo=algo), args.steps, args.warmup)
+            err = oracle.max_rel_err(d1c.cpu().numpy(), oracle.gemm(A1, B1))
+            configs.append({"name": f"gemm_128x64x256_{algo}", "ms": ms, "us": ms * 1e3,
+                            "tflops": 2.0 * 128 * 64 * 256 / (ms * 1e-3) / 1e12, "max_rel_err": err})
+
+    # ---------------------------------------------------------------- C3: back-to-back GEMM
+    if want("b2b"):
+        M, N, K, P = 8192, 256, 128, 128
+        A3 = oracle.fill_normal(M * K, 1237, 0, 0.1).reshape(M, K)
+        B3 = oracle.fill_normal(N * K, 2237, 0, 0.1).reshape(N, K)
+        C3 = oracle.fill_normal(P * N, 3237, 0, 0.1).reshape(P, N)
+        d3a, d3b, d3c = to_dev(A3), to_dev(B3), to_dev(C3)
+        d3d = torch.empty(1, M, P, dtype=torch.float16, device=dev)
+        ms = time_kernel(lambda: tcu.b2b_gemm(d3a, d3b, d3c, out=d3d), args.steps, args.warmup)
+        err = oracle.max_rel_err(d3d[0].float().cpu().numpy(), oracle.b2b_gemm(A3, B3, C3))
+        flops = 2.0 * M * K * N + 2.0 * M * N * P
+        nbytes = 2.0 * (M * K + N * K + P * N + M * P)
+        configs.append({"name": "b2b_8192x256x128x128", "ms": ms, "us": ms * 1e3, "tflops": flops / (ms * 1e-3) / 1e12,
+                        "gbs": nbytes / (ms * 1e-3) / 1e9, "frac_mfma_peak": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                        "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "max_rel_err": err})
+
+    # ---------------------------------------------------------------- C4: FlashAttention-2 forward
+    if want("attn"):
+        B, H, S, D = 4, 16, 2048, 128
+        cnt = B * H * S * D
+        q = oracle.fill_normal(cnt, 1238).reshape(B * H, S, D)
+        k = oracle.fill_normal(cnt, 2238).reshape(B * H, S, D)
+        v = oracle.fill_normal(cnt, 3238).reshape(B * H, S, D)
+        dq, dk, dv = (to_dev(t.reshape(B, H, S, D)) for t in (q, k, v))
+        do = torch.empty(B, H, S, D, dtype=torch.float16, device=dev)
+        ms = time_kernel(lambda: tcu.flash_attention(dq, dk, dv, out=do), max(5, args.steps // 2), max(2, args.warmup // 2))
+        ref = oracle.attention(q[5], k[5], v[5], 1.0 / math.sqrt(D), rows=(1024, 1088))
+        err = oracle.max_abs_err(do.reshape(B * H, S, D)[5, 1024:1088].float().cpu().numpy(), ref[1024:1088])
+        flops = 4.0 * B * H * S * S * D
+        configs.append({"name": "flash_attn_fwd_b4_h16_s2048_d128", "ms": ms, "tflops": flops / (ms * 1e-3) / 1e12,
+                        "frac_mfma_peak": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, "max_abs_err": err})
+
+    # ---------------------------------------------------------------- C5: fused LSTM layer
+    if want("lstm"):
+        T, Bb, I, Hh = 16, 256, 1024, 1024
+        x = oracle.fill_normal(T * Bb * I, 1239, 0, 0.05).reshape(T, Bb, I)
+        W = oracle.fill_normal(4 * Hh * (I + Hh), 2239, 0, 0.05).reshape(4 * Hh, I + Hh)
+        b = oracle.fill_normal(4 * Hh, 3239, 0, 0.05)
+        dx, dW, db = to_dev(x), to_dev(W), to_dev(b)
+        out = {}
+
+        def lstm_step():
+            out["h"], out["c"] = tcu.lstm(dx, dW, db)
+
+        ms = time_kernel(lstm_step, max(5, args.steps // 2), max(2, args.warmup // 2))
+        h_ref, c_ref = oracle.lstm(x, W, b, rows=(0, 2))
+        err = max(oracle.max_abs_err(out["h"][:, 0:2].float().cpu().numpy(), h_ref[:, 0:2]),
+                  oracle.max_abs_err(out["c"][0:2].cpu().numpy(), c_ref[0:2]))
+        step_bytes = 2.0 * (4 * Hh * (I + Hh) + 4 * Hh + Bb * I + 2 * Bb * Hh) + 4.0 * 2 * Bb * Hh
+        flops = 2.0 * Bb * (I + Hh) * 4 * Hh * T
+        configs.append({"name": "lstm_b256_i1024_h1024_t16", "ms": ms, "us_per_step": ms * 1e3 / T,
+                        "gbs": step_bytes * T / (ms * 1e-3) / 1e9,
+                        "frac_hbm_peak": step_bytes * T / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        "tflops": flops / (ms * 1e-3) / 1e12, "max_abs_err": err})
+
+    # ---------------------------------------------------------------- CPU baseline (oracle, bounded)
+    cpu = None
+    if not args.no_cpu_baseline:
+        sample_rows = 2048  # half of the 4096 rows of C: 68.7 GFLOP
+        oracle.gemm(A, Bt, rows=(0, 64))  # warm the thread pool
+        t0 = time.perf_counter()
+        oracle.gemm(A, Bt, rows=(0, sample_rows))
+        dt = time.perf_counter() - t0
+        cpu = {"value": 2.0 * sample_rows * n * n / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(),
+               "kind": "port", "sample": f"rows 0..{sample_rows} of the 4096^3 GEMM ({dt:.1f} s, OpenMP f32 oracle)"}
+
+    result = {
+        "metric": "fp16 GEMM & FA2-fwd TFLOP/s + % MFMA peak on 1 MI355X",
+        "value": gemm_tflops,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": gemm_ms,
+        "wall_ms_per_step": wall_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "fp16 GEMM M=N=K=4096, A row-major, B column-major, f32 accumulate, f16 out "
+                               "(BASELINE configs[1])"},
+        "roofline": {"bound": "mfma", "achieved": gemm_tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": gemm_tflops / MFMA_F16_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "gemm_pipelined<256x256x64>", "flops_per_launch": gemm_flops,
+                     "avg_launch_us": gemm_ms * 1e3},
+        "cpu_baseline": cpu,
+        "max_rel_err": gemm_err,
+        "configs": configs,
+        "device": torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

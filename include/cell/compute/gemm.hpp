@@ -1,0 +1,99 @@
+// Tile-level gemm(a, b, c): c(i, j) += sum_k a(i, k) * b(k, j) over 16x16 BaseTiles,
+// f16 x f16 -> f32. Same entry point and operand types as the reference's
+// include/cell/compute/gemm.hpp:18-88, where each 16x16x16 step is two
+// mma.sync.m16n8k16; here two K-adjacent BaseTiles of A and of B form the operands of one
+// v_mfma_f32_16x16x32_f16 (an odd trailing K tile uses v_mfma_f32_16x16x16_f16).
+//
+// The operands are passed to the instruction swapped (B's share as the first operand):
+// the instruction then produces C^T in its native accumulator distribution, which is C in
+// the row-major BaseTile distribution (lane l: row l % 16, columns 4 * (l / 16) .. +3).
+#pragma once
+
+#include "cell/traits/base.hpp"
+#include "types/layout.hpp"
+#include "types/tile_shape.hpp"
+
+namespace tiledcuda::cell::compute {
+namespace tl = tile_layout;
+
+namespace detail {
+
+template <typename RegTileA, typename RegTileB, typename RegTileC>
+struct Gemm {
+    using InTypeA = typename RegTileA::DType::DType;
+    using InTypeB = typename RegTileB::DType::DType;
+    using OutType = typename RegTileC::DType::DType;
+
+    using BaseShape = traits::BaseTileShape<InTypeA>;
+
+    static_assert(traits::HalfType<InTypeA>, "This GEMM supports only half-precision input elements.");
+    static_assert(std::is_same_v<OutType, float>, "The output type must be float.");
+    static_assert(std::is_same_v<InTypeA, InTypeB>, "Mismatched data type for operand A and B.");
+    static_assert(RegTileB::kRows == RegTileA::kCols, "Mismatched k-dimension for operand A and B.");
+    static_assert(RegTileA::kType == tl::Layout::kRowMajor, "Operand A must be made of row-major BaseTiles.");
+    static_assert(RegTileB::kType == tl::Layout::kColMajor, "Operand B must be made of column-major BaseTiles.");
+    static_assert(RegTileC::kType == tl::Layout::kRowMajor, "The accumulator must be made of row-major BaseTiles.");
+
+    static constexpr int kMs = RegTileA::kRows;
+    static constexpr int kNs = RegTileB::kCols;
+    static constexpr int kKs = RegTileA::kCols;
+    static_assert(kMs && kNs && kKs, "Invalid tile shapes for GEMM.");
+    static_assert(RegTileC::kRows == kMs && RegTileC::kCols == kNs, "Mismatched accumulator shape.");
+
+    DEVICE void operator()(const RegTileA& a, const RegTileB& b, RegTileC& c) {
+#pragma unroll
+        for (int k = 0; k + 1 < kKs; k += 2) {
+#pragma unroll
+            for (int i = 0; i < kMs; ++i) {
+#pragma unroll
+                for (int j = 0; j < kNs; ++j)
+                    mfma_k32(a(i, k).data(), a(i, k + 1).data(), b(k, j).data(), b(k + 1, j).data(),
+                             c(i, j).mutable_data());
+            }
+        }
+        if constexpr (kKs % 2 == 1) {
+#pragma unroll
+            for (int i = 0; i < kMs; ++i) {
+#pragma unroll
+                for (int j = 0; j < kNs; ++j)
+                    mfma_k16(a(i, kKs - 1).data(), b(kKs - 1, j).data(), c(i, j).mutable_data());
+            }
+        }
+    }
+
+  private:
+    DEVICE static f16x4 load4(const InTypeA* p) {
+        f16x4 v;
+        __builtin_memcpy(&v, p, sizeof(v));
+        return v;
+    }
+
+    DEVICE static void mfma_k32(const InTypeA* a0, const InTypeA* a1, const InTypeB* b0, const InTypeB* b1,
+                                OutType* c) {
+        const f16x4 al = load4(a0), ah = load4(a1), bl = load4(b0), bh = load4(b1);
+        const f16x8 av = __builtin_shufflevector(al, ah, 0, 1, 2, 3, 4, 5, 6, 7);
+        const f16x8 bv = __builtin_shufflevector(bl, bh, 0, 1, 2, 3, 4, 5, 6, 7);
+        f32x4 acc;
+        __builtin_memcpy(&acc, c, sizeof(acc));
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bv, av, acc, 0, 0, 0);
+        __builtin_memcpy(c, &acc, sizeof(acc));
+    }
+
+    DEVICE static void mfma_k16(const InTypeA* a, const InTypeB* b, OutType* c) {
+        const f16x4 av = load4(a), bv = load4(b);
+        f32x4 acc;
+        __builtin_memcpy(&acc, c, sizeof(acc));
+        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(bv, av, acc, 0, 0, 0);
+        __builtin_memcpy(c, &acc, sizeof(acc));
+    }
+};
+
+}  // namespace detail
+
+template <typename RegTileA, typename RegTileB, typename RegTileC>
+DEVICE void gemm(const RegTileA& a, const RegTileB& b, RegTileC& c) {
+    detail::Gemm<RegTileA, RegTileB, RegTileC> gemm;
+    gemm(a, b, c);
+}
+
+}  // namespace tiledcuda::cell::compute

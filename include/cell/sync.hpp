@@ -1,0 +1,28 @@
+// Copy-completion fences. Same names as the reference's include/cell/sync.hpp:8-23
+// (wait_group<N>, commit_copy_group, __copy_async). On gfx950 a global->LDS copy is a
+// vector-memory load followed by an LDS write (or a direct-to-LDS load), both tracked by
+// the wavefront's vmcnt / lgkmcnt counters, so "wait for my copies" is s_waitcnt; making
+// the data visible to the other wavefronts still takes the __syncthreads() that follows in
+// user code, exactly as with cp.async.
+#pragma once
+
+#include "config.hpp"
+
+namespace tiledcuda::cell {
+
+/// Wait until at most N of this wavefront's vector-memory loads are outstanding.
+template <int N>
+DEVICE void wait_group() {
+    __builtin_amdgcn_s_waitcnt(/*vmcnt(N) lgkmcnt(0)*/ 0x0070 | (N & 0xF) | ((N >> 4) << 14));
+}
+
+/// Copies are issued in program order; nothing to commit explicitly.
+DEVICE void commit_copy_group() { __builtin_amdgcn_sched_barrier(0); }
+
+/// Wait for every outstanding copy of this wavefront.
+DEVICE void __copy_async() {
+    commit_copy_group();
+    __builtin_amdgcn_s_waitcnt(0);
+}
+
+}  // namespace tiledcuda::cell

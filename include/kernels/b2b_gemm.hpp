@@ -1,0 +1,171 @@
+// Back-to-back GEMM D = (A·B)·C with the [kTM x kTN] intermediate kept in registers.
+// Follows the structure of the reference's examples/cpp/02_fused_two_gemms/fused_gemm.hpp:12-181
+// (FusedGemmTraits / KeFusedGemm): A, D row-major; B, C column-major; the f32 accumulator of
+// the first product is rounded to f16 and used as the A operand of the second one.
+// Differences: M and the batch count are run-time values (every stride depends only on
+// N, K, P), D may be f16 or f32, and A is read from global memory once, before the n-loop
+// (the reference re-reads it on every iteration, fused_gemm.hpp:156).
+#pragma once
+
+#include "cell/mod.hpp"
+#include "types/mod.hpp"
+
+namespace tiledcuda::kernels {
+
+using namespace tiledcuda::cell;
+using namespace tiledcuda::cell::copy;
+namespace tl = tile_layout;
+
+template <const int kM, const int kN, const int kK, const int kP>
+using FusedGemmShape = TileShape<kM, kN, kK, kP>;
+
+/// WholeShape carries N, K, P (M is a run-time argument of the kernel; its entry in the
+/// shape is only used for documentation).
+template <typename InType, typename AccType, typename OutType, typename WholeShape, typename CtaTileShape,
+          typename WarpLayout_ = tl::RowMajor<2, 1>>
+struct FusedGemmTraits {
+    using BaseShape = traits::BaseTileShape<InType>;
+    using WarpLayout = WarpLayout_;
+
+    static constexpr int kWarpPerRow = tl::num_rows<WarpLayout>;
+    static constexpr int kWarpPerCol = tl::num_cols<WarpLayout>;
+    static_assert(kWarpPerCol == 1, "WarpPerCol must be 1");
+
+    static constexpr int kThreads = tl::get_numel<WarpLayout> * kWaveSize;
+
+    static constexpr int kN = dim_size<1, WholeShape>;
+    static constexpr int kK = dim_size<2, WholeShape>;
+    static constexpr int kP = dim_size<3, WholeShape>;
+
+    static constexpr int kTM = dim_size<0, CtaTileShape>;
+    static constexpr int kTN = dim_size<1, CtaTileShape>;
+    static constexpr int kTK = dim_size<2, CtaTileShape>;
+    static constexpr int kTP = dim_size<3, CtaTileShape>;
+    static_assert(kTK == kK, "The current implementation requires kTK == K.");
+    static_assert(kTP == kP, "The current implementation requires kTP == P.");
+
+    // operand A [M, K] row-major
+    using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK, kK>>;
+    using GIteratorA = GTileIterator<GlobalA, TileShape<kTM, kTK>>;
+    using SharedA = SharedTile<InType, tl::RowMajor<kTM, kTK>, true>;
+
+    static constexpr int kAMs = kTM / kWarpPerRow / BaseShape::kTileSize;
+    static constexpr int kAKs = kTK / BaseShape::kTileSize;
+    using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kAMs, kAKs>>;
+    using SharedALoader = GlobalToSharedLoader<SharedA, WarpLayout>;
+    using RegALoader = SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
+
+    // operand B [K, N] column-major
+    using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kN, kK>>;
+    using GIteratorB = GTileIterator<GlobalB, TileShape<kTK, kTN>>;
+    using SharedB = SharedTile<InType, tl::ColMajor<kTK, kTN>, true>;
+
+    static constexpr int kBKs = kTK / BaseShape::kTileSize;
+    static constexpr int kBNs = kTN / kWarpPerCol / BaseShape::kTileSize;
+    using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kBKs, kBNs>>;
+    using SharedBLoader = GlobalToSharedLoader<SharedB, WarpLayout>;
+    using RegBLoader = SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
+
+    // operand C [N, P] column-major
+    using GlobalC = GlobalTile<InType, tl::ColMajor<kN, kTP, kN>>;
+    using GIteratorC = GTileIterator<GlobalC, TileShape<kTN, kTP>>;
+    using SharedC = SharedTile<InType, tl::ColMajor<kTN, kTP>, true>;
+
+    static constexpr int kCNs = kTN / BaseShape::kTileSize;
+    static constexpr int kCPs = kTP / kWarpPerCol / BaseShape::kTileSize;
+    using RegC = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kCNs, kCPs>>;
+    using SharedCLoader = GlobalToSharedLoader<SharedC, WarpLayout>;
+    using RegCLoader = SharedToRegLoader<RegC, WarpLayout, WarpReuse::kColReuseCont>;
+
+    // output D [M, P] row-major
+    using GlobalD = GlobalTile<OutType, tl::RowMajor<kTM, kTP, kP>>;
+
+    static constexpr int kDMs = kTM / kWarpPerRow / BaseShape::kTileSize;
+    static constexpr int kDPs = kTP / kWarpPerCol / BaseShape::kTileSize;
+    using RegD = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kDMs, kDPs>>;
+    using RegDCast = RegTile<BaseTileRowMajor<OutType>, tl::RowMajor<kDMs, kDPs>>;
+    using DStorer = RegToGlobalStorer<GlobalD, RegDCast, WarpLayout>;
+    using ConvertD = compute::RegTileConvert<RegD, RegDCast>;
+
+    static constexpr int kAccMs = kTM / kWarpPerRow / BaseShape::kTileSize;
+    static constexpr int kAccNs = kTN / kWarpPerCol / BaseShape::kTileSize;
+    using RegAcc = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kAccMs, kAccNs>>;
+    using RegAccCast = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kAccMs, kAccNs>>;
+    using ConvertAcc = compute::RegTileConvert<RegAcc, RegAccCast>;
+
+    static constexpr int kShmBytes = (kTM * kTK + kTK * kTN + kTN * kTP) * sizeof(InType);
+};
+
+/// grid = (M / kTM, 1, batch), block = Traits::kThreads, dynamic LDS = Traits::kShmBytes.
+template <typename InType, typename OutType, typename Traits>
+__global__ void __launch_bounds__(Traits::kThreads) KeFusedGemm(const InType* dA, const InType* dB, const InType* dC,
+                                                                OutType* dD, int kM) {
+    constexpr int kN = Traits::kN, kK = Traits::kK, kP = Traits::kP;
+    constexpr int kTM = Traits::kTM;
+
+    const InType* A = dA + blockIdx.z * (size_t(kM) * kK) + blockIdx.x * (kTM * kK);
+    const InType* B = dB + blockIdx.z * (kK * kN);
+    const InType* gC_ptr = dC + blockIdx.z * (kN * kP);
+    OutType* gD_ptr = dD + blockIdx.z * (size_t(kM) * kP) + blockIdx.x * (kTM * kP);
+
+    extern __shared__ __align__(16) unsigned char shared_buf[];
+    auto* shm = reinterpret_cast<InType*>(shared_buf);
+    InType* sA_ptr = shm;
+    InType* sB_ptr = shm + Traits::SharedA::kNumel;
+    InType* sC_ptr = sB_ptr + Traits::SharedB::kNumel;
+
+    typename Traits::GIteratorA gAs(A);
+    typename Traits::SharedA sA(sA_ptr);
+    typename Traits::RegA rA;
+    typename Traits::SharedALoader load_sa;
+    typename Traits::RegALoader load_ra;
+
+    typename Traits::GIteratorB gBs(B);
+    typename Traits::SharedB sB(sB_ptr);
+    typename Traits::RegB rB;
+    typename Traits::SharedBLoader load_sb;
+    typename Traits::RegBLoader load_rb;
+
+    typename Traits::GIteratorC gCs(gC_ptr);
+    typename Traits::SharedC sC(sC_ptr);
+    typename Traits::RegC rC;
+    typename Traits::SharedCLoader load_sc;
+    typename Traits::RegCLoader load_rc;
+
+    typename Traits::RegD rD;
+    typename Traits::RegAcc acc;
+    typename Traits::RegAccCast acc_half;
+    typename Traits::ConvertAcc cast_acc;
+
+    // A is needed by every n-iteration: stage it once and keep it in registers.
+    load_sa(gAs(0), sA);
+    __copy_async();
+    __syncthreads();
+    load_ra(sA, rA);
+
+    for (int n = 0; n < Traits::GIteratorC::sc0; ++n) {
+        load_sb(gBs(0, n), sB);
+        load_sc(gCs(n), sC);
+        __copy_async();
+        __syncthreads();
+
+        load_rb(sB, rB);
+        load_rc(sC, rC);
+        __syncthreads();
+
+        compute::gemm(rA, rB, acc);
+        cast_acc(acc, acc_half);
+        compute::gemm(acc_half, rC, rD);
+        acc.clear();
+    }
+
+    typename Traits::RegDCast rD_out;
+    typename Traits::ConvertD cast_d;
+    cast_d(rD, rD_out);
+
+    typename Traits::GlobalD gD(gD_ptr);
+    typename Traits::DStorer storer_d;
+    storer_d(rD_out, gD);
+}
+
+}  // namespace tiledcuda::kernels

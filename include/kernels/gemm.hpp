@@ -1,0 +1,226 @@
+// GEMM kernels composed from the tile primitives.
+//   * GemmTraits / simple_gemm: global -> register -> MFMA; the kernel of the reference's
+//     README and examples/cpp/01_gemm/01_gemm_global_reg/gemm.hpp:13-92.
+//   * KeGemmTraits / gemm: global -> LDS -> register -> MFMA, C staged through LDS; the
+//     kernel of examples/cpp/01_gemm/02_gemm_all_mem/gemm.hpp:15-155. A barrier is added
+//     at the end of each k-step: the reference overwrites the shared tiles of the next
+//     step while other warps may still be reading them.
+// A is row-major [M, K], B is column-major [K, N] (stored [N, K]), C is row-major [M, N].
+#pragma once
+
+#include "cell/mod.hpp"
+#include "types/mod.hpp"
+
+namespace tiledcuda::kernels {
+
+using namespace tiledcuda::cell;
+using namespace tiledcuda::cell::copy;
+namespace tl = tile_layout;
+
+template <const int kM, const int kN, const int kK>
+using GemmShape = TileShape<kM, kN, kK>;
+
+template <typename InType, typename AccType, typename WholeShape, const int kTM, const int kTN, typename WarpLayout,
+          const int kChunkK_ = 64>
+struct GemmTraits {
+    using BaseShape = traits::BaseTileShape<InType>;
+    static constexpr int kChunkK = kChunkK_;
+
+    static constexpr int kThreads = tl::get_numel<WarpLayout> * kWaveSize;
+    static constexpr int kWarpPerRow = tl::num_rows<WarpLayout>;
+    static constexpr int kWarpPerCol = tl::num_cols<WarpLayout>;
+
+    static constexpr int kM = dim_size<0, WholeShape>;
+    static constexpr int kN = dim_size<1, WholeShape>;
+    static constexpr int kK = dim_size<2, WholeShape>;
+
+    // operand A
+    using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK, kK>>;
+    using IteratorA = GTileIterator<GlobalA, TileShape<kTM, kChunkK>>;
+
+    static constexpr int kAMs = kTM / kWarpPerRow / BaseShape::kTileSize;
+    static constexpr int kAKs = kChunkK / BaseShape::kTileSize;
+    using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kAMs, kAKs>>;
+    using ALoader = GlobalToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
+
+    // operand B
+    using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kTN, kK>>;
+    using IteratorB = GTileIterator<GlobalB, TileShape<kChunkK, kTN>>;
+
+    static constexpr int kBKs = kChunkK / BaseShape::kTileSize;
+    static constexpr int kBNs = kTN / kWarpPerCol / BaseShape::kTileSize;
+    using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kBKs, kBNs>>;
+    using BLoader = GlobalToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
+
+    // output C
+    using GlobalC = GlobalTile<AccType, tl::RowMajor<kTM, kTN, kN>>;
+
+    static constexpr int kCMs = kTM / kWarpPerRow / BaseShape::kTileSize;
+    static constexpr int kCNs = kTN / kWarpPerCol / BaseShape::kTileSize;
+    using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kCMs, kCNs>>;
+    using CStorer = RegToGlobalStorer<GlobalC, RegC, WarpLayout>;
+};
+
+template <typename InType, typename AccType,                    //
+          const int kM, const int kN, const int kK,             //
+          const int kTM, const int kTN,                         //
+          typename IteratorA, typename RegA, typename ALoader,  //
+          typename IteratorB, typename RegB, typename BLoader,  //
+          typename GlobalC, typename RegC, typename CStorer>
+__global__ void __launch_bounds__(512) simple_gemm(const InType* dA, const InType* dB, AccType* dC) {
+    const int offset_a = blockIdx.x * kTM * kK;
+    const int offset_b = blockIdx.y * kTN * kK;
+    const int offset_c = blockIdx.x * kTM * kN + blockIdx.y * kTN;
+
+    IteratorA gAs(dA + offset_a);
+    RegA rA;
+    ALoader loader_a;
+
+    IteratorB gBs(dB + offset_b);
+    RegB rB;
+    BLoader loader_b;
+
+    RegC acc;
+    GlobalC gC(dC + offset_c);
+    CStorer storer_c;
+
+    for (int k = 0; k < IteratorA::sc1; ++k) {
+        loader_a(gAs(k), rA);
+        loader_b(gBs(k), rB);
+        compute::gemm(rA, rB, acc);
+    }
+
+    storer_c(acc, gC);
+}
+
+template <typename InType, typename AccType, typename WholeShape, typename CtaTileShape, const int kRK,
+          typename WarpLayout>
+struct KeGemmTraits {
+    using BaseShape = traits::BaseTileShape<InType>;
+
+    static constexpr int kThreads = tl::get_numel<WarpLayout> * kWaveSize;
+    static constexpr int kWarpPerRow = tl::num_rows<WarpLayout>;
+    static constexpr int kWarpPerCol = tl::num_cols<WarpLayout>;
+
+    static constexpr int kM = dim_size<0, WholeShape>;
+    static constexpr int kN = dim_size<1, WholeShape>;
+    static constexpr int kK = dim_size<2, WholeShape>;
+
+    static constexpr int kTM = dim_size<0, CtaTileShape>;
+    static constexpr int kTN = dim_size<1, CtaTileShape>;
+    static constexpr int kTK = dim_size<2, CtaTileShape>;
+
+    static const bool kSwizzled = true;
+
+    // operand A
+    using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK, kK>>;
+    using GIteratorA = GTileIterator<GlobalA, TileShape<kTM, kTK>>;
+    using SharedA = SharedTile<InType, tl::RowMajor<kTM, kTK>, kSwizzled>;
+    using SIteratorA = STileIterator<SharedA, TileShape<kTM, kRK>>;
+
+    static constexpr int kAMs = kTM / kWarpPerRow / BaseShape::kTileSize;
+    static constexpr int kAKs = kRK / BaseShape::kTileSize;
+    using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kAMs, kAKs>>;
+
+    using G2SLoaderA = GlobalToSharedLoader<SharedA, WarpLayout>;
+    using S2RLoaderA = SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
+
+    // operand B
+    using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kTN, kK>>;
+    using GIteratorB = GTileIterator<GlobalB, TileShape<kTK, kTN>>;
+    using SharedB = SharedTile<InType, tl::ColMajor<kTK, kTN>, kSwizzled>;
+    using SIteratorB = STileIterator<SharedB, TileShape<kRK, kTN>>;
+
+    static_assert(GIteratorA::sc1 == GIteratorB::sc0, "mismatched K dimension!");
+    static_assert(SIteratorA::sc1 == SIteratorB::sc0, "mismatched K dimension!");
+
+    static constexpr int kBKs = kRK / BaseShape::kTileSize;
+    static constexpr int kBNs = kTN / kWarpPerCol / BaseShape::kTileSize;
+    using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kBKs, kBNs>>;
+
+    using G2SLoaderB = GlobalToSharedLoader<SharedB, WarpLayout>;
+    using S2RLoaderB = SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
+
+    // output C
+    using GlobalC = GlobalTile<AccType, tl::RowMajor<kTM, kTN, kN>>;
+    using SharedC = SharedTile<AccType, tl::RowMajor<kTM, kTN>, kSwizzled>;
+
+    static constexpr int kCMs = kTM / kWarpPerRow / BaseShape::kTileSize;
+    static constexpr int kCNs = kTN / kWarpPerCol / BaseShape::kTileSize;
+    using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kCMs, kCNs>>;
+
+    using R2SStorerC = RegToSharedStorer<RegC, WarpLayout>;
+    using S2GStorerC = SharedToGlobalStorer<SharedC, WarpLayout>;
+
+    static constexpr int kShmInput = (kTM + kTN) * kTK * sizeof(InType);
+    static constexpr int kShmOutput = kTM * kTN * sizeof(AccType);
+    static constexpr int kShmBytes = kShmInput > kShmOutput ? kShmInput : kShmOutput;
+};
+
+template <typename InType, typename AccType,                  //
+          const int kM, const int kN, const int kK,           //
+          const int kTM, const int kTN, const int kTK,        //
+          typename GIteratorA, typename SIteratorA,           //
+          typename SharedA, typename RegA,                    //
+          typename G2SLoaderA, typename S2RLoaderA,           //
+          typename GIteratorB, typename SIteratorB,           //
+          typename SharedB, typename RegB,                    //
+          typename G2SLoaderB, typename S2RLoaderB,           //
+          typename GlobalC, typename SharedC, typename RegC,  //
+          typename R2SStorerC, typename S2GStorerC>
+__global__ void __launch_bounds__(512) gemm(const InType* dA, const InType* dB, AccType* dC) {
+    const int offset_a = blockIdx.x * kTM * kK;
+    const int offset_b = blockIdx.y * kTN * kK;
+    const int offset_c = blockIdx.x * kTM * kN + blockIdx.y * kTN;
+
+    extern __shared__ __align__(16) unsigned char buf[];
+    InType* sA_ptr = reinterpret_cast<InType*>(buf);
+    InType* sB_ptr = sA_ptr + SIteratorA::Tile::kNumel;
+    AccType* sC_ptr = reinterpret_cast<AccType*>(buf);
+
+    GIteratorA gAs(dA + offset_a);
+    SIteratorA sAs(sA_ptr);
+
+    GIteratorB gBs(dB + offset_b);
+    SIteratorB sBs(sB_ptr);
+
+    SharedA sA(sA_ptr);
+    RegA rA;
+
+    SharedB sB(sB_ptr);
+    RegB rB;
+
+    RegC acc;
+    SharedC sC(sC_ptr);
+    GlobalC gC(dC + offset_c);
+
+    G2SLoaderA g2s_a;
+    S2RLoaderA s2r_a;
+
+    G2SLoaderB g2s_b;
+    S2RLoaderB s2r_b;
+
+    R2SStorerC r2s_c;
+    S2GStorerC s2g_c;
+
+    for (int k1 = 0; k1 < GIteratorA::sc1; ++k1) {
+        g2s_a(gAs(k1), sA);
+        g2s_b(gBs(k1), sB);
+        __copy_async();
+        __syncthreads();
+
+#pragma unroll
+        for (int k2 = 0; k2 < SIteratorA::sc1; ++k2) {
+            s2r_a(sAs(k2), rA);
+            s2r_b(sBs(k2), rB);
+
+            compute::gemm(rA, rB, acc);
+        }
+        __syncthreads();  // everyone is done reading sA / sB before the next step overwrites them
+    }
+    r2s_c(acc, sC);
+    __syncthreads();
+    s2g_c(sC, gC);
+}
+
+}  // namespace tiledcuda::kernels

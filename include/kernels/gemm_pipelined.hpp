@@ -1,0 +1,288 @@
+// Pipelined fp16 GEMM for gfx950: C[M, N] = A[M, K] · B, A row-major, B column-major (stored
+// [N, K]), f32 accumulate, C row-major in f16 or f32. This is the multi-stage kernel the
+// reference's examples/cpp/01_gemm/02_gemm_all_mem/gemm.hpp:103-155 lacks (it has one LDS
+// stage and waits for every load), built for the CDNA4 execution model:
+//   * one workgroup of kWM x kWN wavefronts per kBM x kBN tile of C, v_mfma_f32_32x32x16_f16,
+//     accumulators resident in registers for the whole K loop;
+//   * A and B tiles go global -> LDS directly (global_load_lds_dwordx4, 16 B per lane, no
+//     VGPR staging), kStages LDS buffers; the loads of tile k+1 are in flight while tile k
+//     is multiplied;
+//   * LDS rows are kBK halves (128 B for kBK = 64); the 16-byte chunks of a row are
+//     XOR-permuted with (row / 2) % 8 so that the ds_read_b128 of 32 consecutive rows at one
+//     k-offset is bank-conflict free; the permutation is applied on the global-address side
+//     because a direct-to-LDS load writes 64 lanes x 16 B contiguously;
+//   * register double-buffering of the MFMA operands: the ds_reads of k-substep kk+1 are
+//     issued before the MFMAs of substep kk; the barrier that hands over an LDS stage sits
+//     before the last substep so its latency hides under 16 MFMAs;
+//   * the result is staged through LDS so that global stores are full 16-byte, row-contiguous;
+//   * workgroup ids are remapped so that the 32 workgroups an XCD receives (ids congruent
+//     modulo 8) form a compact block of tiles and share A / B panels in that XCD's L2.
+// M % kBM == 0, N % kBN == 0, K % kBK == 0 are required (checked by the host launcher).
+#pragma once
+
+#include "config.hpp"
+#include "hip_utils.hpp"
+
+namespace tiledcuda::kernels {
+
+template <const int kBM_, const int kBN_, const int kBK_, const int kWM_, const int kWN_, const int kStages_ = 2>
+struct PipelinedGemmTraits {
+    static constexpr int kBM = kBM_, kBN = kBN_, kBK = kBK_, kWM = kWM_, kWN = kWN_, kStages = kStages_;
+    static constexpr int kWaves = kWM * kWN;
+    static constexpr int kThreads = kWaves * kWaveSize;
+
+    static constexpr int kWaveM = kBM / kWM;  // rows of C per wavefront
+    static constexpr int kWaveN = kBN / kWN;
+    static constexpr int kMT = kWaveM / 32;  // 32x32 MFMA tiles per wavefront along M
+    static constexpr int kNT = kWaveN / 32;
+    static constexpr int kKS = kBK / 16;  // MFMA k-substeps per LDS tile
+
+    static_assert(kBK == 64, "LDS rows are 128 bytes: kBK must be 64 halves");
+    static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0, "a wavefront owns whole 32x32 MFMA tiles");
+
+    static constexpr int kRowBytes = kBK * 2;                    // 128
+    static constexpr int kABytes = kBM * kRowBytes;              // one stage of A
+    static constexpr int kBBytes = kBN * kRowBytes;              // one stage of B
+    static constexpr int kStageBytes = kABytes + kBBytes;
+    static constexpr int kRowsPerLoad = 1024 / kRowBytes;        // 8 rows per direct-to-LDS instruction
+    static constexpr int kALoads = kBM / kRowsPerLoad / kWaves;  // instructions per wavefront per stage
+    static constexpr int kBLoads = kBN / kRowsPerLoad / kWaves;
+    static_assert(kBM % (kRowsPerLoad * kWaves) == 0 && kBN % (kRowsPerLoad * kWaves) == 0,
+                  "the tile rows must divide evenly over the wavefronts' 8-row loads");
+
+    // epilogue staging: every wavefront stages its kWaveM x kWaveN block, kEpiBytes per element
+    static constexpr int kLdsBytesMain = kStages * kStageBytes;
+    template <typename OutType>
+    static constexpr int epilogue_bytes() {
+        return kWaves * kWaveM * kWaveN * int(sizeof(OutType));
+    }
+    template <typename OutType>
+    static constexpr int lds_bytes() {
+        // f32 output is stored directly from registers (no staging), so only f16 needs the space
+        return sizeof(OutType) == 2 && epilogue_bytes<OutType>() > kLdsBytesMain ? epilogue_bytes<OutType>()
+                                                                                 : kLdsBytesMain;
+    }
+};
+
+namespace detail {
+
+using lds_ptr_t = __attribute__((address_space(3))) void*;
+using glb_ptr_t = const __attribute__((address_space(1))) void*;
+
+/// 16 bytes per lane, global -> LDS, no register staging. `lds_wave_base` must be wave-uniform;
+/// lane i's data lands at lds_wave_base + 16 * i.
+DEVICE void load_lds_16B(const void* gptr, void* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((glb_ptr_t)gptr, (lds_ptr_t)lds_wave_base, 16, 0, 0);
+}
+
+/// Tile coordinates for workgroup `bid` of a grid of tiles_m x tiles_n tiles: ids that are
+/// congruent modulo 8 (same XCD) are gathered into compact blocks of tiles.
+HOST_DEVICE void xcd_tile_coords(int bid, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+    const int total = tiles_m * tiles_n;
+    constexpr int kXcds = 8;
+    if (total % kXcds == 0 && tiles_m % 4 == 0) {
+        const int per_xcd = total / kXcds;
+        const int xcd = bid % kXcds;
+        const int local = bid / kXcds;
+        const int lin = xcd * per_xcd + local;  // consecutive `lin` = same XCD
+        // walk the grid in column panels 4 tiles tall so that an XCD's run of per_xcd tiles is compact
+        const int panel = lin / (4 * tiles_n);
+        const int in_panel = lin % (4 * tiles_n);
+        tile_m = panel * 4 + in_panel % 4;
+        tile_n = in_panel / 4;
+    } else {
+        tile_m = bid % tiles_m;
+        tile_n = bid / tiles_m;
+    }
+}
+
+}  // namespace detail
+
+template <typename Traits, typename OutType>
+__global__ void __launch_bounds__(Traits::kThreads)
+    gemm_pipelined(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N,
+                   int K) {
+    constexpr int kBM = Traits::kBM, kBN = Traits::kBN, kBK = Traits::kBK;
+    constexpr int kMT = Traits::kMT, kNT = Traits::kNT, kKS = Traits::kKS;
+    constexpr int kStages = Traits::kStages;
+
+    extern __shared__ __align__(1024) unsigned char lds[];
+
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+    const int wave_m = wave / Traits::kWN;
+    const int wave_n = wave % Traits::kWN;
+
+    int tile_m, tile_n;
+    detail::xcd_tile_coords(blockIdx.x, M / kBM, N / kBN, tile_m, tile_n);
+    const int m0 = tile_m * kBM;
+    const int n0 = tile_n * kBN;
+
+    // ---- global -> LDS addressing -------------------------------------------------------
+    // Load instruction j of this wavefront fills LDS rows [8 * g, 8 * g + 8), g = wave * kLoads + j.
+    // Lane i writes physical chunk p = i % 8 of row 8 * g + i / 8, which must hold logical chunk
+    // p ^ ((row / 2) % 8).
+    const int lrow = lane >> 3;  // row within the 8-row group
+    const int lchk = lane & 7;   // physical 16-byte chunk
+    auto a_src = [&](int j, int k0) -> const __half* {
+        const int row = (wave * Traits::kALoads + j) * Traits::kRowsPerLoad + lrow;
+        const int chunk = lchk ^ ((row >> 1) & 7);
+        return A + size_t(m0 + row) * K + k0 + chunk * 8;
+    };
+    auto b_src = [&](int j, int k0) -> const __half* {
+        const int row = (wave * Traits::kBLoads + j) * Traits::kRowsPerLoad + lrow;
+        const int chunk = lchk ^ ((row >> 1) & 7);
+        return Bt + size_t(n0 + row) * K + k0 + chunk * 8;
+    };
+    auto issue_stage = [&](int stage, int k0) {
+        unsigned char* sa = lds + stage * Traits::kStageBytes;
+        unsigned char* sb = sa + Traits::kABytes;
+#pragma unroll
+        for (int j = 0; j < Traits::kALoads; ++j)
+            detail::load_lds_16B(a_src(j, k0), sa + (wave * Traits::kALoads + j) * 1024);
+#pragma unroll
+        for (int j = 0; j < Traits::kBLoads; ++j)
+            detail::load_lds_16B(b_src(j, k0), sb + (wave * Traits::kBLoads + j) * 1024);
+    };
+
+    // ---- LDS -> register addressing -----------------------------------------------------
+    // 32x32x16 operand: lane l holds row l % 32, k = 8 * (l / 32) .. +7 of the 16-wide substep,
+    // i.e. logical chunk 2 * kk + l / 32 of its row.
+    const int frow = lane & 31;
+    const int fhalf = lane >> 5;
+    auto read_frag = [&](const unsigned char* base, int row, int kk) -> f16x8 {
+        const int chunk = (2 * kk + fhalf) ^ ((row >> 1) & 7);
+        return *reinterpret_cast<const f16x8*>(base + row * Traits::kRowBytes + chunk * 16);
+    };
+
+    f32x16 acc[kMT][kNT];
+#pragma unroll
+    for (int i = 0; i < kMT; ++i)
+#pragma unroll
+        for (int j = 0; j < kNT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    f16x8 fa[2][kMT], fb[2][kNT];
+
+    auto load_frags = [&](int buf, int stage, int kk) {
+        const unsigned char* sa = lds + stage * Traits::kStageBytes;
+        const unsigned char* sb = sa + Traits::kABytes;
+#pragma unroll
+        for (int i = 0; i < kMT; ++i) fa[buf][i] = read_frag(sa, wave_m * Traits::kWaveM + i * 32 + frow, kk);
+#pragma unroll
+        for (int j = 0; j < kNT; ++j) fb[buf][j] = read_frag(sb, wave_n * Traits::kWaveN + j * 32 + frow, kk);
+    };
+    auto mma = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < kMT; ++i)
+#pragma unroll
+            for (int j = 0; j < kNT; ++j)
+                // operands swapped: the accumulator then holds C (not C^T) with 4 consecutive
+                // columns per register quad
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+    };
+
+    const int ktiles = K / kBK;
+
+    // prologue: tile 0 -> stage 0 (and tile 1 -> stage 1 when 3 stages are used)
+    issue_stage(0, 0);
+    if constexpr (kStages > 2) {
+        if (ktiles > 1) issue_stage(1, kBK);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070 | (kStages > 2 ? (Traits::kALoads + Traits::kBLoads) & 0xF : 0));
+    __syncthreads();
+    if constexpr (kStages == 2) {
+        if (ktiles > 1) issue_stage(1, kBK);
+    }
+    load_frags(0, 0, 0);
+
+    int stage = 0;
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const int next_stage = stage + 1 == kStages ? 0 : stage + 1;
+#pragma unroll
+        for (int kk = 0; kk < kKS - 1; ++kk) {
+            load_frags((kk + 1) & 1, stage, kk + 1);
+            mma(kk & 1);
+        }
+        // Every LDS read of `stage` has been issued; once they return and all wavefronts agree,
+        // the stage can be refilled and the next one (whose loads were issued one tile ago) read.
+        if (kt + 1 < ktiles) {
+            if constexpr (kStages == 2) {
+                __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): tile kt+1 landed, my reads returned
+                __syncthreads();
+                if (kt + 2 < ktiles) issue_stage(stage, (kt + 2) * kBK);
+            } else {
+                // tile kt+1 landed if at most one stage's worth of loads (tile kt+2) is still in flight
+                if (kt + 2 < ktiles)
+                    __builtin_amdgcn_s_waitcnt(0x0070 | ((Traits::kALoads + Traits::kBLoads) & 0xF));
+                else
+                    __builtin_amdgcn_s_waitcnt(0x0070);
+                __syncthreads();
+                // stage (kt+3) % 3 == stage kt % 3 ... only with kStages == 3: refill the stage just drained
+                if (kt + kStages < ktiles + 0 && kStages == 3) issue_stage(stage, (kt + 3) * kBK);
+            }
+            load_frags(kKS & 1, next_stage, 0);
+        }
+        mma((kKS - 1) & 1);
+        stage = next_stage;
+    }
+
+    // ---- epilogue -----------------------------------------------------------------------
+    // acc[i][j][r]: row = lane % 32, col = 8 * (r / 4) + 4 * (lane / 32) + r % 4 of the 32x32 tile.
+    if constexpr (sizeof(OutType) == 2) {
+        __syncthreads();  // everyone is done with the operand stages
+        constexpr int kWaveN = Traits::kWaveN, kWaveM = Traits::kWaveM;
+        constexpr int kPitch = kWaveN * 2;  // bytes per staged row
+        unsigned char* stg = lds + wave * (kWaveM * kPitch);
+        // write: lane owns row (i*32 + frow); 4 halves (8 B) at column j*32 + 8*q + 4*fhalf.
+        // 8-byte slots of a row are XOR-ed with (row % 16) * 2 (bit 0 untouched) to spread banks.
+#pragma unroll
+        for (int i = 0; i < kMT; ++i) {
+            const int row = i * 32 + frow;
+#pragma unroll
+            for (int j = 0; j < kNT; ++j) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int slot = (j * 32 + 8 * q + 4 * fhalf) >> 2;  // 8-byte slot index in the row
+                    const int pslot = slot ^ ((row & 15) << 1);
+                    f16x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc[i][j][4 * q + e]);
+                    *reinterpret_cast<f16x4*>(stg + row * kPitch + pslot * 8) = v;
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's staging writes are done
+        // read back 16 B per lane, row-contiguous: kWaveN / 8 lanes per row
+        constexpr int kLanesPerRow = kWaveN / 8;
+        constexpr int kRowsPerIter = kWaveSize / kLanesPerRow;
+        const int rr = lane / kLanesPerRow;
+        const int cc = lane % kLanesPerRow;  // 16-byte chunk = 8-byte slots 2cc, 2cc+1
+        OutType* cbase = C + size_t(m0 + wave_m * kWaveM) * N + n0 + wave_n * kWaveN;
+#pragma unroll
+        for (int it = 0; it < kWaveM / kRowsPerIter; ++it) {
+            const int row = it * kRowsPerIter + rr;
+            const int pslot = (2 * cc) ^ ((row & 15) << 1);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kPitch + pslot * 8);
+            *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(cbase + size_t(row) * N) + cc * 16) = v;
+        }
+    } else {
+        OutType* cbase = C + size_t(m0 + wave_m * Traits::kWaveM) * N + n0 + wave_n * Traits::kWaveN;
+#pragma unroll
+        for (int i = 0; i < kMT; ++i) {
+#pragma unroll
+            for (int j = 0; j < kNT; ++j) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    f32x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
+                    *reinterpret_cast<f32x4*>(cbase + size_t(i * 32 + frow) * N + j * 32 + 8 * q + 4 * fhalf) = v;
+                }
+            }
+        }
+    }
+}
+
+}  // namespace tiledcuda::kernels

@@ -1,0 +1,96 @@
+/*
+ * C-ABI of the MI355X tile-kernel library: the boundary a host program (C, C++, Python
+ * ctypes, a torch op) binds to. Plain pointers and sizes only; every pointer is a device
+ * pointer owned by the caller; nothing is allocated, freed or synchronised by the library;
+ * work is enqueued on the hipStream_t passed as `stream` (NULL = the default stream).
+ * Every function returns 0 on success or a negative tcu_status; tcu_last_error() gives the
+ * message of the last failure on the calling thread. No function ever calls exit().
+ *
+ * Precedent in the reference: `extern "C" int kernel_entry(__half*, __half*, float*)` loaded
+ * with ctypes (examples/python/gemm/entry.py:56-67, compile.py:129-137).
+ */
+#ifndef TCU_C_API_H_
+#define TCU_C_API_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    TCU_OK = 0,
+    TCU_ERR_INVALID_ARGUMENT = -1,  /* null pointer, non-positive size, bad enum value */
+    TCU_ERR_UNSUPPORTED_SHAPE = -2, /* shape not divisible by the tile / not instantiated */
+    TCU_ERR_HIP = -3,               /* a HIP runtime call failed (message has the HIP error) */
+    TCU_ERR_NO_DEVICE = -4          /* no HIP device is available to this process */
+} tcu_status;
+
+typedef enum { TCU_DTYPE_F32 = 0, TCU_DTYPE_F16 = 1 } tcu_dtype;
+
+/* Which GEMM kernel to run. AUTO picks the pipelined kernel when the shape allows. */
+typedef enum {
+    TCU_GEMM_AUTO = 0,
+    TCU_GEMM_GLOBAL_REG = 1, /* global -> register -> MFMA (README kernel of the reference) */
+    TCU_GEMM_ALL_MEM = 2,    /* global -> LDS -> register -> MFMA, single stage */
+    TCU_GEMM_PIPELINED = 3   /* direct-to-LDS, multi-stage, 32x32x16 MFMA */
+} tcu_gemm_algo;
+
+/* Layout of V in tcu_flash_attn_fwd_f16. */
+typedef enum {
+    TCU_V_COL_MAJOR = 0, /* V stored [P, N] per batch item: the reference op's convention */
+    TCU_V_ROW_MAJOR = 1  /* V stored [N, P] per batch item: the usual [seq, head_dim] */
+} tcu_v_layout;
+
+/* Library version (major * 10000 + minor * 100 + patch). */
+int tcu_version(void);
+
+/* Message of the last error raised on the calling thread ("" if none). */
+const char* tcu_last_error(void);
+
+/* Number of HIP devices visible, or a negative tcu_status. */
+int tcu_device_count(void);
+
+/*
+ * C[M, N] = A[M, K] · B.  A row-major f16; B column-major f16 (stored as [N, K]); C row-major,
+ * out_dtype f32 or f16; f32 accumulation.
+ * Replaces the launches in the reference's examples/cpp/01_gemm/01_gemm_global_reg/main.cu:59-63
+ * and examples/cpp/01_gemm/02_gemm_all_mem/main.cu:54-72 (kernels gemm.hpp:65-92 / :103-155), and
+ * the ctypes entry examples/python/gemm/entry.py:56-67.
+ */
+int tcu_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K, int out_dtype, int algo, void* stream);
+
+/*
+ * D[b, M, P] = f16(A[b, M, K] · B[b]) · C[b].  A row-major; B column-major [K, N] (stored [N, K]);
+ * C column-major [N, P] (stored [P, N]); D row-major, f32 or f16. The [M, N] intermediate
+ * never leaves the chip.
+ * Replaces run_fused_gemm / KeFusedGemm of the reference's
+ * examples/cpp/02_fused_two_gemms/fused_gemm.cu:86-113 and fused_gemm.hpp:107-181.
+ */
+int tcu_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D, int M, int N, int K, int P, int batch,
+                     int out_dtype, void* stream);
+
+/*
+ * O[b, M, P] = softmax(scale · Q[b, M, K] · K[b]) · V[b], f16 in / f16 out, f32 softmax
+ * statistics. Q row-major; keys column-major [K, N] (stored [N, K]); V per v_layout.
+ * Replaces run_flash_attention / custom_flash_attention_op of the reference's
+ * src/kernels/flash_attn.cu:314-456 (the body of torch.ops.tiledcuda.flash_attention_fwd).
+ * The reference computes with scale = 1; pass 1.0f for that behaviour.
+ */
+int tcu_flash_attn_fwd_f16(const void* Q, const void* K, const void* V, void* O, int batch, int M, int N, int Kdim,
+                           int P, float scale, int v_layout, void* stream);
+
+/*
+ * Fused LSTM layer over T steps. x [T, B, I] f16; W [4H, I+H] f16 row-major, gate rows in the
+ * order i, f, g, o, columns concat(x_t, h_{t-1}); bias [4H] f16; h0 [B, H] f16 or NULL (zeros);
+ * c0 [B, H] f32 or NULL (zeros); h_all [T, B, H] f16 receives every h_t; c_out [B, H] f32
+ * receives c_T (it is also the running cell state, so it must not alias c0 unless c0 == c_out).
+ * One kernel per step (gate GEMM fused with the cell update).
+ * The reference snapshot has no LSTM entry (Makefile:3 names a test only).
+ */
+int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                 void* c_out, int T, int B, int I, int H, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TCU_C_API_H_ */

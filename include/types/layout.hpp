@@ -1,0 +1,123 @@
+// Compile-time 2-D layouts and the LDS swizzle.
+//
+// MatrixLayout / RowMajor / ColMajor and the free-standing queries keep the names and
+// meaning of the reference's include/types/layout.hpp:26-53,275-296. The shared-memory
+// layout is new: the reference stores every 16x16 BaseTile contiguously and applies
+// CuTe Swizzle<2,3,3> inside it (layout.hpp:58-206) to serve ldmatrix; here a shared tile
+// is a plain pitched 2-D array whose 4-element chunks are XOR-permuted within each line so
+// that the per-lane 64-bit (f16) / 128-bit (f32) LDS accesses of a wavefront fall on
+// distinct banks (64 banks x 4 B on gfx950).
+#pragma once
+
+#include "cell/traits/base.hpp"
+#include "config.hpp"
+
+#include <cstddef>
+
+namespace tiledcuda::cell {
+
+namespace tile_layout {
+
+enum class Layout {
+    kRowMajor = 0,
+    kColMajor = 1,
+    kSwizzledRowMajor = 2,
+    kSwizzledColMajor = 3
+};
+
+HOST_DEVICE constexpr const char* layout_type_to_str(Layout type) {
+    switch (type) {
+        case Layout::kRowMajor: return "RowMajor";
+        case Layout::kColMajor: return "ColMajor";
+        case Layout::kSwizzledRowMajor: return "SwizzledRowMajor";
+        case Layout::kSwizzledColMajor: return "SwizzledColMajor";
+    }
+    return "Unknown";
+}
+
+template <const int kRows_, const int kCols_, const int kRowStride_, const int kColStride_>
+struct MatrixLayout {
+    static constexpr int kRows = kRows_;
+    static constexpr int kCols = kCols_;
+
+    static constexpr int kRowStride = kRowStride_;
+    static constexpr int kColStride = kColStride_;
+
+    static constexpr int kNumel = kRows * kCols;
+
+    // A layout whose column stride is 1 counts as row-major (so ColMajor<1, 1> does too).
+    static constexpr Layout kType = kColStride == 1 ? Layout::kRowMajor : Layout::kColMajor;
+
+    HOST_DEVICE constexpr int operator()(int i, int j) const { return i * kRowStride + j * kColStride; }
+};
+
+// The last dimension is contiguous.
+template <const int kRow, const int kCol, const int kStride = kCol>
+using RowMajor = MatrixLayout<kRow, kCol, kStride, 1>;
+
+// The first dimension is contiguous.
+template <const int kRow, const int kCol, const int kStride = kRow>
+using ColMajor = MatrixLayout<kRow, kCol, 1, kStride>;
+
+template <typename Layout>
+static constexpr size_t num_rows = Layout::kRows;
+
+template <typename Layout>
+static constexpr size_t num_cols = Layout::kCols;
+
+template <typename Layout>
+static constexpr size_t row_stride = Layout::kRowStride;
+
+template <typename Layout>
+static constexpr size_t col_stride = Layout::kColStride;
+
+template <typename Layout>
+static constexpr size_t get_numel = Layout::kNumel;
+
+template <typename Layout_>
+static constexpr Layout layout_type = Layout_::kType;
+
+template <const int kShape1, const int kShape2, const int kStride1, const int kStride2>
+HOST_DEVICE constexpr auto make_tile_layout() {
+    return MatrixLayout<kShape1, kShape2, kStride1, kStride2>{};
+}
+
+namespace detail {
+HOST_DEVICE constexpr int cmax(int a, int b) { return a > b ? a : b; }
+HOST_DEVICE constexpr int cmin(int a, int b) { return a < b ? a : b; }
+// largest power of two dividing x (x > 0)
+HOST_DEVICE constexpr int pow2_divisor(int x) { return x & (-x); }
+}  // namespace detail
+
+/// XOR permutation of the 4-element chunks of one line (row of a row-major tile, column of a
+/// column-major one) of a pitched LDS tile.
+///
+/// One wavefront access touches 16 consecutive lines at one or two chunk positions per
+/// pass (a 64-bit access is served 32 lanes at a time, a 128-bit access 16 lanes at a time,
+/// 256 B = all 64 banks per pass). Lines whose start addresses coincide modulo 256 B would
+/// collide, so their chunk index is XOR-ed with a per-line value. The XOR leaves bit 0 of
+/// the chunk index of 2-byte elements alone, so a 16-byte global->LDS store of 8 halves
+/// stays contiguous.
+template <const int kPitch, const int kElemBytes>
+struct LdsSwizzle {
+    static constexpr int kChunk = 4;
+    static constexpr int kChunkBytes = kChunk * kElemBytes;
+    static constexpr int kChunksPerLine = kPitch / kChunk;
+    static constexpr int kWindowChunks = 256 / kChunkBytes;
+    static constexpr int kShift = kWindowChunks >= 32 ? 1 : 0;
+    static constexpr int kLinesPerWindow = detail::cmin(16, detail::cmax(1, kWindowChunks / kChunksPerLine));
+    static constexpr int kNumSwz =
+        detail::cmax(1, detail::cmin(16 / kLinesPerWindow, detail::pow2_divisor(kChunksPerLine) >> kShift));
+
+    static_assert(kPitch % kChunk == 0, "the pitch of a shared tile must be a multiple of 4 elements");
+
+    /// Position, within its line, of logical element `elem` of line `line`.
+    HOST_DEVICE static constexpr int apply(int line, int elem) {
+        const int chunk = elem >> 2;
+        const int s = ((line / kLinesPerWindow) & (kNumSwz - 1)) << kShift;
+        return ((chunk ^ s) << 2) | (elem & 3);
+    }
+};
+
+}  // namespace tile_layout
+}  // namespace tiledcuda::cell

@@ -1,0 +1,588 @@
+// Device-side unit tests of the tile primitives, exported through a small C table so that
+// pytest can drive them (one process, torch-owned device buffers).
+//
+// The cases restate the reference's C++ unit tests with the same shapes and warp layouts:
+//   g2s round trip          tests/cpp/cell/test_g2s_load.cu:118-144
+//   swizzled vs plain load  tests/cpp/cell/test_swizzled_copy.cu:399-450 (strengthened: the
+//                           register tiles are written back and must equal the source)
+//   store round trip        tests/cpp/cell/test_swizzled_copy.cu:452-499
+//   g2r / r2g               tests/cpp/cell/test_g2r_copy.cu (which only prints)
+//   tile gemm               tests/cpp/cell/test_gemm.cu:306-351
+//   reduce / broadcast      tests/cpp/cell/test_reduce.cu, test_broadcast.cu (which only print)
+//   softmax                 tests/cpp/cell/test_softmax.cu:117-163
+// Every kernel is launched with one workgroup; the host side checks results against the
+// CPU oracle or against the identity.
+#include "cell/mod.hpp"
+#include "types/mod.hpp"
+
+#include <string>
+#include <vector>
+
+using namespace tiledcuda;
+using namespace tiledcuda::cell;
+using namespace tiledcuda::cell::copy;
+namespace tl = tiledcuda::cell::tile_layout;
+
+namespace {
+
+template <bool kRowMajor, int kRows, int kCols>
+using LayoutOf = std::conditional_t<kRowMajor, tl::RowMajor<kRows, kCols>, tl::ColMajor<kRows, kCols>>;
+
+// ------------------------------------------------------------------ global -> shared -> global
+template <typename Element, bool kRowMajor, int kRows, int kCols, typename WarpLayout, bool kSwizzled>
+__global__ void __launch_bounds__(512) k_g2s_roundtrip(const Element* src, Element* dst) {
+    extern __shared__ __align__(16) unsigned char buf[];
+    auto* smem = reinterpret_cast<Element*>(buf);
+    using Layout = LayoutOf<kRowMajor, kRows, kCols>;
+    using Global = GlobalTile<Element, Layout>;
+    using Shared = SharedTile<Element, Layout, kSwizzled>;
+
+    Global g_src(src);
+    Global g_dst(dst);
+    Shared s(smem);
+    GlobalToSharedLoader<Shared, WarpLayout> loader;
+    SharedToGlobalStorer<Shared, WarpLayout> storer;
+    loader(g_src, s);
+    __copy_async();
+    __syncthreads();
+    storer(s, g_dst);
+}
+
+// ------------------------------------------------------------------ global -> shared -> (iterator) -> reg -> global
+// Operand-A style: row-major tile, chunks along the columns, RowReuseCont; every wavefront
+// row's register tile is written back (wavefront columns hold copies, so only column 0 writes).
+template <typename Element, int kRows, int kCols, int kChunk, typename WarpLayout, bool kSwizzled>
+__global__ void __launch_bounds__(512) k_s2r_row_major(const Element* src, Element* dst) {
+    extern __shared__ __align__(16) unsigned char buf[];
+    auto* smem = reinterpret_cast<Element*>(buf);
+    using Global = GlobalTile<Element, tl::RowMajor<kRows, kCols>>;
+    using Shared = SharedTile<Element, tl::RowMajor<kRows, kCols>, kSwizzled>;
+    using SIter = STileIterator<Shared, TileShape<kRows, kChunk>>;
+    constexpr int kWR = tl::num_rows<WarpLayout>;
+    constexpr int kMs = kRows / kWR / 16, kKs = kChunk / 16;
+    using Reg = RegTile<BaseTileRowMajor<Element>, tl::RowMajor<kMs, kKs>>;
+    using OutGlobal = GlobalTile<Element, tl::RowMajor<kRows, kChunk, kCols>>;
+
+    Global g_src(src);
+    Shared s(smem);
+    GlobalToSharedLoader<Shared, WarpLayout> g2s;
+    g2s(g_src, s);
+    __copy_async();
+    __syncthreads();
+
+    SIter iter(smem);
+    SharedToRegLoader<Reg, WarpLayout, WarpReuse::kRowReuseCont> s2r;
+    using Base = warp::CopyBase<WarpLayout, WarpReuse::kRowReuseCont>;
+    for (int k = 0; k < SIter::sc1; ++k) {
+        Reg r;
+        s2r(iter(k), r);
+        if (Base::warp_col_id() == 0) {
+            // write this wavefront-row's block back with a single-column wavefront layout
+            using OutWarps = tl::RowMajor<kWR, 1>;
+            OutGlobal g_out(dst + k * kChunk);
+            // emulate a kWR x 1 layout: wavefront row = warp_row_id()
+            Element* p = g_out.mutable_data() + Base::warp_row_id() * (kRows / kWR) * kCols;
+            using Sub = GlobalTile<Element, tl::RowMajor<kRows / kWR, kChunk, kCols>>;
+            Sub sub(p);
+            RegToGlobalStorer<Sub, Reg, tl::RowMajor<1, 1>> r2g;
+            (void)sizeof(OutWarps);
+            r2g(r, sub);
+        }
+    }
+}
+
+// Operand-B style: column-major tile, chunks along the rows, ColReuseCont.
+template <typename Element, int kRows, int kCols, int kChunk, typename WarpLayout, bool kSwizzled>
+__global__ void __launch_bounds__(512) k_s2r_col_major(const Element* src, Element* dst) {
+    extern __shared__ __align__(16) unsigned char buf[];
+    auto* smem = reinterpret_cast<Element*>(buf);
+    using Global = GlobalTile<Element, tl::ColMajor<kRows, kCols>>;
+    using Shared = SharedTile<Element, tl::ColMajor<kRows, kCols>, kSwizzled>;
+    using SIter = STileIterator<Shared, TileShape<kChunk, kCols>>;
+    constexpr int kWC = tl::num_cols<WarpLayout>;
+    constexpr int kKs = kChunk / 16, kNs = kCols / kWC / 16;
+    using Reg = RegTile<BaseTileColMajor<Element>, tl::ColMajor<kKs, kNs>>;
+
+    Global g_src(src);
+    Shared s(smem);
+    GlobalToSharedLoader<Shared, WarpLayout> g2s;
+    g2s(g_src, s);
+    __copy_async();
+    __syncthreads();
+
+    SIter iter(smem);
+    SharedToRegLoader<Reg, WarpLayout, WarpReuse::kColReuseCont> s2r;
+    using Base = warp::CopyBase<WarpLayout, WarpReuse::kColReuseCont>;
+    for (int k = 0; k < SIter::sc0; ++k) {
+        Reg r;
+        s2r(iter(k), r);
+        if (Base::warp_row_id() == 0) {
+            using Sub = GlobalTile<Element, tl::ColMajor<kChunk, kCols / kWC, kRows>>;
+            Sub sub(dst + k * kChunk + Base::warp_col_id() * (kCols / kWC) * kRows);
+            RegToGlobalStorer<Sub, Reg, tl::RowMajor<1, 1>> r2g;
+            r2g(r, sub);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ global -> reg -> shared -> global
+template <typename Element, bool kRowMajor, int kRows, int kCols, typename WarpLayout, bool kSwizzled>
+__global__ void __launch_bounds__(512) k_store_roundtrip(const Element* src, Element* dst) {
+    extern __shared__ __align__(16) unsigned char buf[];
+    auto* smem = reinterpret_cast<Element*>(buf);
+    using Layout = LayoutOf<kRowMajor, kRows, kCols>;
+    using Global = GlobalTile<Element, Layout>;
+    using Shared = SharedTile<Element, Layout, kSwizzled>;
+    constexpr int kRs = kRows / tl::num_rows<WarpLayout> / 16, kCs = kCols / tl::num_cols<WarpLayout> / 16;
+    using Base = std::conditional_t<kRowMajor, BaseTileRowMajor<Element>, BaseTileColMajor<Element>>;
+    using Reg = RegTile<Base, LayoutOf<kRowMajor, kRs, kCs>>;
+
+    Global g_src(src);
+    Global g_dst(dst);
+    Shared s(smem);
+    Reg r;
+    GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
+    RegToSharedStorer<Reg, WarpLayout> r2s;
+    SharedToGlobalStorer<Shared, WarpLayout> s2g;
+    g2r(g_src, r);
+    r2s(r, s);
+    __syncthreads();
+    s2g(s, g_dst);
+}
+
+// ------------------------------------------------------------------ global -> reg -> global
+template <typename Element, bool kGlobalRowMajor, bool kRegRowMajor, int kRows, int kCols, typename WarpLayout>
+__global__ void __launch_bounds__(512) k_g2r_roundtrip(const Element* src, Element* dst) {
+    using Layout = LayoutOf<kGlobalRowMajor, kRows, kCols>;
+    using Global = GlobalTile<Element, Layout>;
+    constexpr int kRs = kRows / tl::num_rows<WarpLayout> / 16, kCs = kCols / tl::num_cols<WarpLayout> / 16;
+    using Base = std::conditional_t<kRegRowMajor, BaseTileRowMajor<Element>, BaseTileColMajor<Element>>;
+    using Reg = RegTile<Base, LayoutOf<kRegRowMajor, kRs, kCs>>;
+    Global g_src(src);
+    Global g_dst(dst);
+    Reg r;
+    GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
+    RegToGlobalStorer<Global, Reg, WarpLayout> r2g;
+    g2r(g_src, r);
+    r2g(r, g_dst);
+}
+
+// ------------------------------------------------------------------ tile gemm through LDS
+// C[kM, kN] f32 = A[kM, kK] (row-major) · B[kK, kN] (column-major), one workgroup.
+template <int kM, int kN, int kK, typename WarpLayout, int kChunkK, bool kSwizzled>
+__global__ void __launch_bounds__(512) k_tile_gemm(const __half* dA, const __half* dB, float* dC) {
+    extern __shared__ __align__(16) unsigned char buf[];
+    auto* sA_ptr = reinterpret_cast<__half*>(buf);
+    auto* sB_ptr = sA_ptr + kM * kK;
+    constexpr int kWR = tl::num_rows<WarpLayout>, kWC = tl::num_cols<WarpLayout>;
+
+    using GlobalA = GlobalTile<__half, tl::RowMajor<kM, kK>>;
+    using SharedA = SharedTile<__half, tl::RowMajor<kM, kK>, kSwizzled>;
+    using SIterA = STileIterator<SharedA, TileShape<kM, kChunkK>>;
+    using RegA = RegTile<BaseTileRowMajor<__half>, tl::RowMajor<kM / kWR / 16, kChunkK / 16>>;
+
+    using GlobalB = GlobalTile<__half, tl::ColMajor<kK, kN>>;
+    using SharedB = SharedTile<__half, tl::ColMajor<kK, kN>, kSwizzled>;
+    using SIterB = STileIterator<SharedB, TileShape<kChunkK, kN>>;
+    using RegB = RegTile<BaseTileColMajor<__half>, tl::ColMajor<kChunkK / 16, kN / kWC / 16>>;
+
+    using GlobalC = GlobalTile<float, tl::RowMajor<kM, kN>>;
+    using RegC = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kM / kWR / 16, kN / kWC / 16>>;
+
+    GlobalA gA(dA);
+    GlobalB gB(dB);
+    SharedA sA(sA_ptr);
+    SharedB sB(sB_ptr);
+    GlobalToSharedLoader<SharedA, WarpLayout> g2s_a;
+    GlobalToSharedLoader<SharedB, WarpLayout> g2s_b;
+    g2s_a(gA, sA);
+    g2s_b(gB, sB);
+    __copy_async();
+    __syncthreads();
+
+    SIterA sAs(sA_ptr);
+    SIterB sBs(sB_ptr);
+    SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont> s2r_a;
+    SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont> s2r_b;
+    RegA rA;
+    RegB rB;
+    RegC acc;
+    for (int k = 0; k < SIterA::sc1; ++k) {
+        s2r_a(sAs(k), rA);
+        s2r_b(sBs(k), rB);
+        compute::gemm(rA, rB, acc);
+    }
+    GlobalC gC(dC);
+    RegToGlobalStorer<GlobalC, RegC, WarpLayout> r2g;
+    r2g(acc, gC);
+}
+
+// ------------------------------------------------------------------ reduce / broadcast / softmax
+// src [kRows, kCols] f32 row-major, one wavefront per 16... rows split over kW wavefronts.
+// out_vec[kRows]: op 0 = row sum, 1 = row max; out_tile: op 2 = broadcast of row sums,
+// 3 = tile minus row max (fused), 4 = softmax.
+template <typename Element, int kRows, int kCols, int kW, int kOp>
+__global__ void __launch_bounds__(512) k_row_ops(const Element* src, Element* out_vec, Element* out_tile) {
+    using WarpLayout = tl::RowMajor<kW, 1>;
+    using Global = GlobalTile<Element, tl::RowMajor<kRows, kCols>>;
+    constexpr int kRs = kRows / kW / 16, kCs = kCols / 16;
+    using Reg = RegTile<BaseTileRowMajor<Element>, tl::RowMajor<kRs, kCs>>;
+    using Vec = RegTile<Element, tl::RowMajor<kRs, 1>>;
+    Global g_src(src);
+    Reg r;
+    Vec v;
+    GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
+    g2r(g_src, r);
+
+    if constexpr (kOp == 0) {
+        compute::SumReduce<Reg, tl::Layout::kRowMajor> op;
+        op(r, v);
+    } else if constexpr (kOp == 1) {
+        compute::MaxReduce<Reg, tl::Layout::kRowMajor> op;
+        op(r, v);
+    } else if constexpr (kOp == 2) {
+        compute::SumReduce<Reg, tl::Layout::kRowMajor> op;
+        op(r, v);
+        compute::Broadcast<Vec, Reg, tl::Layout::kRowMajor> bc;
+        bc(v, r);
+    } else if constexpr (kOp == 3) {
+        compute::MaxReduce<Reg, tl::Layout::kRowMajor> op;
+        op(r, v);
+        compute::BroadcastSub<Vec, Reg, tl::Layout::kRowMajor> bs;
+        bs(v, r);
+    } else {
+        compute::Softmax<Reg, tl::Layout::kRowMajor> sm;
+        sm(r, v);
+    }
+    // every lane of a row group holds the row value; lanes 0..15 of each wavefront write it
+    const int lane = lane_id();
+    if (lane < 16) {
+#pragma unroll
+        for (int i = 0; i < kRs; ++i) out_vec[wave_id() * (kRows / kW) + i * 16 + lane] = v(i, 0);
+    }
+    Global g_out(out_tile);
+    RegToGlobalStorer<Global, Reg, WarpLayout> r2g;
+    r2g(r, g_out);
+}
+
+// column-wise reductions on column-major tiles: src [kRows, kCols] column-major, kW wavefronts along the columns
+template <typename Element, int kRows, int kCols, int kW, int kOp>
+__global__ void __launch_bounds__(512) k_col_ops(const Element* src, Element* out_vec, Element* out_tile) {
+    using WarpLayout = tl::RowMajor<1, kW>;
+    using Global = GlobalTile<Element, tl::ColMajor<kRows, kCols>>;
+    constexpr int kRs = kRows / 16, kCs = kCols / kW / 16;
+    using Reg = RegTile<BaseTileColMajor<Element>, tl::ColMajor<kRs, kCs>>;
+    using Vec = RegTile<Element, tl::RowMajor<1, kCs>>;
+    Global g_src(src);
+    Reg r;
+    Vec v;
+    GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
+    g2r(g_src, r);
+    if constexpr (kOp == 0) {
+        compute::SumReduce<Reg, tl::Layout::kColMajor> op;
+        op(r, v);
+    } else if constexpr (kOp == 1) {
+        compute::MaxReduce<Reg, tl::Layout::kColMajor> op;
+        op(r, v);
+    } else {
+        compute::MaxReduce<Reg, tl::Layout::kColMajor> op;
+        op(r, v);
+        compute::BroadcastSub<Vec, Reg, tl::Layout::kColMajor> bs;
+        bs(v, r);
+    }
+    const int lane = lane_id();
+    if (lane < 16) {
+#pragma unroll
+        for (int j = 0; j < kCs; ++j) out_vec[wave_id() * (kCols / kW) + j * 16 + lane] = v(0, j);
+    }
+    Global g_out(out_tile);
+    RegToGlobalStorer<Global, Reg, WarpLayout> r2g;
+    r2g(r, g_out);
+}
+
+// ------------------------------------------------------------------ registry
+struct Case {
+    std::string kind;   // which family
+    std::string name;   // human-readable id
+    int dims[8];        // family-specific: rows, cols, (k), elem bytes, row_major, ...
+    int threads;
+    int lds_bytes;
+    void (*launch)(const void* a, const void* b, void* c, void* d, int threads, int lds, hipStream_t s);
+};
+
+std::vector<Case>& registry() {
+    static std::vector<Case> r;
+    return r;
+}
+
+template <auto Kernel, typename E>
+void launch2(const void* a, const void*, void* c, void*, int threads, int lds, hipStream_t s) {
+    hipLaunchKernelGGL(Kernel, dim3(1), dim3(threads), lds, s, static_cast<const E*>(a), static_cast<E*>(c));
+}
+template <auto Kernel>
+void launch_gemm(const void* a, const void* b, void* c, void*, int threads, int lds, hipStream_t s) {
+    hipLaunchKernelGGL(Kernel, dim3(1), dim3(threads), lds, s, static_cast<const __half*>(a),
+                       static_cast<const __half*>(b), static_cast<float*>(c));
+}
+template <auto Kernel, typename E>
+void launch_ops(const void* a, const void*, void* c, void* d, int threads, int lds, hipStream_t s) {
+    hipLaunchKernelGGL(Kernel, dim3(1), dim3(threads), lds, s, static_cast<const E*>(a), static_cast<E*>(c),
+                       static_cast<E*>(d));
+}
+
+template <typename E>
+constexpr const char* ename() {
+    return sizeof(E) == 2 ? "f16" : "f32";
+}
+
+template <typename E, bool kRowMajor, int kRows, int kCols, int kWR, int kWC, bool kSwz>
+void reg_g2s() {
+    using W = tl::RowMajor<kWR, kWC>;
+    registry().push_back({"g2s_roundtrip",
+                          std::string(ename<E>()) + (kRowMajor ? "_row_" : "_col_") + std::to_string(kRows) + "x" +
+                              std::to_string(kCols) + "_w" + std::to_string(kWR) + "x" + std::to_string(kWC) +
+                              (kSwz ? "_swz" : "_plain"),
+                          {kRows, kCols, 0, int(sizeof(E)), kRowMajor, 0, 0, 0},
+                          kWR * kWC * 64,
+                          int(kRows * kCols * sizeof(E)),
+                          &launch2<k_g2s_roundtrip<E, kRowMajor, kRows, kCols, W, kSwz>, E>});
+}
+
+template <typename E, bool kRowMajor, int kRows, int kCols, int kChunk, int kWR, int kWC, bool kSwz>
+void reg_s2r() {
+    using W = tl::RowMajor<kWR, kWC>;
+    Case c{"s2r_identity",
+           std::string(ename<E>()) + (kRowMajor ? "_row_" : "_col_") + std::to_string(kRows) + "x" +
+               std::to_string(kCols) + "_c" + std::to_string(kChunk) + "_w" + std::to_string(kWR) + "x" +
+               std::to_string(kWC) + (kSwz ? "_swz" : "_plain"),
+           {kRows, kCols, kChunk, int(sizeof(E)), kRowMajor, 0, 0, 0},
+           kWR * kWC * 64,
+           int(kRows * kCols * sizeof(E)),
+           nullptr};
+    if constexpr (kRowMajor)
+        c.launch = &launch2<k_s2r_row_major<E, kRows, kCols, kChunk, W, kSwz>, E>;
+    else
+        c.launch = &launch2<k_s2r_col_major<E, kRows, kCols, kChunk, W, kSwz>, E>;
+    registry().push_back(c);
+}
+
+template <typename E, bool kRowMajor, int kRows, int kCols, int kWR, int kWC, bool kSwz>
+void reg_store() {
+    using W = tl::RowMajor<kWR, kWC>;
+    registry().push_back({"store_roundtrip",
+                          std::string(ename<E>()) + (kRowMajor ? "_row_" : "_col_") + std::to_string(kRows) + "x" +
+                              std::to_string(kCols) + "_w" + std::to_string(kWR) + "x" + std::to_string(kWC) +
+                              (kSwz ? "_swz" : "_plain"),
+                          {kRows, kCols, 0, int(sizeof(E)), kRowMajor, 0, 0, 0},
+                          kWR * kWC * 64,
+                          int(kRows * kCols * sizeof(E)),
+                          &launch2<k_store_roundtrip<E, kRowMajor, kRows, kCols, W, kSwz>, E>});
+}
+
+template <typename E, bool kGRow, bool kRRow, int kRows, int kCols, int kWR, int kWC>
+void reg_g2r() {
+    using W = tl::RowMajor<kWR, kWC>;
+    registry().push_back({"g2r_roundtrip",
+                          std::string(ename<E>()) + (kGRow ? "_grow" : "_gcol") + (kRRow ? "_rrow_" : "_rcol_") +
+                              std::to_string(kRows) + "x" + std::to_string(kCols) + "_w" + std::to_string(kWR) + "x" +
+                              std::to_string(kWC),
+                          {kRows, kCols, 0, int(sizeof(E)), kGRow, kRRow, 0, 0},
+                          kWR * kWC * 64,
+                          0,
+                          &launch2<k_g2r_roundtrip<E, kGRow, kRRow, kRows, kCols, W>, E>});
+}
+
+template <int kM, int kN, int kK, int kWR, int kWC, int kChunkK, bool kSwz = true>
+void reg_gemm() {
+    using W = tl::RowMajor<kWR, kWC>;
+    registry().push_back({"tile_gemm",
+                          std::to_string(kM) + "x" + std::to_string(kN) + "x" + std::to_string(kK) + "_w" +
+                              std::to_string(kWR) + "x" + std::to_string(kWC) + "_c" + std::to_string(kChunkK) +
+                              (kSwz ? "_swz" : "_plain"),
+                          {kM, kN, kK, kChunkK, 0, 0, 0, 0},
+                          kWR * kWC * 64,
+                          int((kM * kK + kK * kN) * sizeof(__half)),
+                          &launch_gemm<k_tile_gemm<kM, kN, kK, W, kChunkK, kSwz>>});
+}
+
+template <typename E, int kRows, int kCols, int kW, int kOp>
+void reg_row_op() {
+    static const char* names[] = {"sum", "max", "bcast_sum", "sub_max", "softmax"};
+    registry().push_back({"row_ops",
+                          std::string(ename<E>()) + "_" + names[kOp] + "_" + std::to_string(kRows) + "x" +
+                              std::to_string(kCols) + "_w" + std::to_string(kW),
+                          {kRows, kCols, kOp, int(sizeof(E)), 1, 0, 0, 0},
+                          kW * 64,
+                          0,
+                          &launch_ops<k_row_ops<E, kRows, kCols, kW, kOp>, E>});
+}
+
+template <typename E, int kRows, int kCols, int kW, int kOp>
+void reg_col_op() {
+    static const char* names[] = {"sum", "max", "sub_max"};
+    registry().push_back({"col_ops",
+                          std::string(ename<E>()) + "_" + names[kOp] + "_" + std::to_string(kRows) + "x" +
+                              std::to_string(kCols) + "_w" + std::to_string(kW),
+                          {kRows, kCols, kOp, int(sizeof(E)), 0, 0, 0, 0},
+                          kW * 64,
+                          0,
+                          &launch_ops<k_col_ops<E, kRows, kCols, kW, kOp>, E>});
+}
+
+template <typename E, bool kSwz>
+void reg_g2s_family() {
+    // shapes and warp layouts of the reference's test_g2s_load.cu:118-144
+    reg_g2s<E, true, 16, 16, 1, 1, kSwz>();
+    reg_g2s<E, true, 16, 64, 1, 4, kSwz>();
+    reg_g2s<E, true, 64, 16, 4, 1, kSwz>();
+    reg_g2s<E, true, 32, 32, 2, 2, kSwz>();
+    reg_g2s<E, true, 64, 64, 2, 2, kSwz>();
+    reg_g2s<E, true, 96, 128, 2, 4, kSwz>();
+    reg_g2s<E, true, 192, 32, 2, 2, kSwz>();
+    reg_g2s<E, false, 16, 16, 1, 1, kSwz>();
+    reg_g2s<E, false, 64, 16, 4, 1, kSwz>();
+    reg_g2s<E, false, 16, 64, 1, 4, kSwz>();
+    reg_g2s<E, false, 64, 64, 2, 2, kSwz>();
+    reg_g2s<E, false, 128, 96, 2, 2, kSwz>();
+}
+
+void build_registry() {
+    if (!registry().empty()) return;
+    reg_g2s_family<__half, false>();
+    reg_g2s_family<__half, true>();
+    reg_g2s_family<float, false>();
+    reg_g2s_family<float, true>();
+
+    // swizzled and plain loads must both reproduce the source (test_swizzled_copy.cu:399-450 shapes)
+    reg_s2r<__half, true, 16, 16, 16, 1, 1, false>();
+    reg_s2r<__half, true, 16, 16, 16, 1, 1, true>();
+    reg_s2r<__half, true, 16, 32, 16, 1, 1, true>();
+    reg_s2r<__half, true, 16, 32, 32, 1, 1, true>();
+    reg_s2r<__half, true, 32, 64, 16, 1, 1, true>();
+    reg_s2r<__half, true, 32, 64, 32, 2, 1, true>();
+    reg_s2r<__half, true, 64, 64, 64, 2, 2, true>();
+    reg_s2r<__half, true, 64, 64, 32, 2, 2, false>();
+    reg_s2r<__half, true, 64, 128, 32, 2, 2, true>();
+    reg_s2r<__half, true, 64, 128, 128, 4, 1, true>();
+    reg_s2r<__half, true, 128, 128, 64, 2, 4, true>();
+    reg_s2r<__half, true, 64, 256, 32, 2, 2, true>();
+    reg_s2r<__half, true, 32, 48, 16, 2, 1, true>();
+    reg_s2r<float, true, 32, 64, 32, 2, 1, true>();
+    reg_s2r<__half, false, 16, 16, 16, 1, 1, true>();
+    reg_s2r<__half, false, 32, 16, 16, 1, 1, true>();
+    reg_s2r<__half, false, 64, 32, 32, 1, 2, true>();
+    reg_s2r<__half, false, 64, 64, 64, 2, 2, true>();
+    reg_s2r<__half, false, 64, 64, 32, 2, 2, false>();
+    reg_s2r<__half, false, 128, 64, 32, 2, 2, true>();
+    reg_s2r<__half, false, 128, 128, 64, 4, 2, true>();
+    reg_s2r<__half, false, 32, 256, 32, 2, 2, true>();
+
+    // store round trips (test_swizzled_copy.cu:452-499)
+    reg_store<float, true, 16, 16, 1, 1, true>();
+    reg_store<float, true, 64, 64, 2, 2, true>();
+    reg_store<float, true, 64, 256, 2, 2, true>();
+    reg_store<float, true, 64, 64, 2, 2, false>();
+    reg_store<__half, true, 16, 16, 1, 1, false>();
+    reg_store<__half, true, 64, 128, 2, 2, false>();
+    reg_store<__half, true, 64, 128, 2, 2, true>();
+    reg_store<float, false, 64, 64, 2, 2, true>();
+    reg_store<__half, false, 64, 32, 2, 1, true>();
+
+    // global <-> register, all four orientation combinations
+    reg_g2r<__half, true, true, 16, 16, 1, 1>();
+    reg_g2r<__half, true, true, 64, 64, 2, 2>();
+    reg_g2r<__half, false, false, 64, 64, 2, 2>();
+    reg_g2r<__half, true, false, 32, 32, 1, 1>();
+    reg_g2r<__half, false, true, 32, 32, 2, 1>();
+    reg_g2r<float, true, true, 64, 32, 2, 2>();
+    reg_g2r<float, false, false, 32, 64, 1, 2>();
+
+    // tile gemm: the (M, N, K, warps, chunkK) combinations of the reference's test_gemm.cu:312-350
+    reg_gemm<16, 16, 16, 1, 1, 16>();
+    reg_gemm<16, 16, 32, 1, 1, 16>();
+    reg_gemm<16, 16, 32, 1, 1, 32>();
+    reg_gemm<32, 32, 32, 1, 1, 16>();
+    reg_gemm<32, 32, 32, 1, 1, 32>();
+    reg_gemm<32, 32, 64, 1, 1, 32>();
+    reg_gemm<64, 64, 64, 1, 1, 16>();
+    reg_gemm<64, 64, 64, 1, 1, 64>();
+    reg_gemm<128, 64, 64, 1, 1, 32>();
+    reg_gemm<96, 48, 80, 1, 1, 16>();
+    reg_gemm<96, 48, 80, 1, 1, 80>();
+    reg_gemm<32, 64, 128, 2, 1, 32>();
+    reg_gemm<64, 32, 128, 1, 2, 64>();
+    reg_gemm<32, 32, 64, 2, 2, 32>();
+    reg_gemm<64, 64, 64, 2, 2, 32>();
+    reg_gemm<64, 64, 64, 2, 2, 64>();
+    reg_gemm<64, 32, 128, 4, 1, 64>();
+    reg_gemm<32, 64, 128, 1, 4, 64>();
+    reg_gemm<128, 128, 128, 2, 2, 64>();
+    reg_gemm<64, 128, 128, 2, 4, 32>();
+    reg_gemm<64, 128, 128, 2, 4, 128>();
+    reg_gemm<64, 64, 64, 2, 2, 32, false>();
+    reg_gemm<32, 32, 48, 1, 1, 48>();
+
+    // reductions, broadcasts, softmax (test_reduce.cu / test_broadcast.cu / test_softmax.cu shapes)
+    reg_row_op<float, 16, 16, 1, 0>();
+    reg_row_op<float, 16, 16, 1, 1>();
+    reg_row_op<float, 32, 64, 1, 0>();
+    reg_row_op<float, 32, 64, 2, 1>();
+    reg_row_op<float, 64, 128, 4, 0>();
+    reg_row_op<__half, 32, 32, 1, 0>();
+    reg_row_op<__half, 32, 32, 1, 1>();
+    reg_row_op<float, 32, 64, 1, 2>();
+    reg_row_op<float, 32, 64, 2, 3>();
+    reg_row_op<float, 16, 16, 1, 4>();
+    reg_row_op<float, 32, 32, 1, 4>();
+    reg_row_op<float, 64, 16, 4, 4>();
+    reg_row_op<__half, 32, 32, 1, 4>();
+    reg_col_op<float, 16, 16, 1, 0>();
+    reg_col_op<float, 64, 32, 2, 1>();
+    reg_col_op<float, 64, 32, 1, 2>();
+    reg_col_op<__half, 32, 32, 1, 0>();
+}
+
+thread_local std::string g_err;
+
+}  // namespace
+
+extern "C" {
+
+int tt_num_cases(void) {
+    build_registry();
+    return static_cast<int>(registry().size());
+}
+
+/// kind / name are NUL-terminated strings owned by the library; dims has 8 ints.
+int tt_case_info(int id, const char** kind, const char** name, int* dims, int* threads, int* lds_bytes) {
+    build_registry();
+    if (id < 0 || id >= (int)registry().size()) return -1;
+    const Case& c = registry()[id];
+    *kind = c.kind.c_str();
+    *name = c.name.c_str();
+    for (int i = 0; i < 8; ++i) dims[i] = c.dims[i];
+    *threads = c.threads;
+    *lds_bytes = c.lds_bytes;
+    return 0;
+}
+
+/// Run case `id` on `stream`. Buffers are device pointers; their meaning depends on the family:
+///   copies:    a = src, c = dst
+///   tile_gemm: a = A, b = B, c = C
+///   row/col ops: a = src, c = per-line vector, d = tile output
+int tt_run_case(int id, const void* a, const void* b, void* c, void* d, void* stream) {
+    build_registry();
+    if (id < 0 || id >= (int)registry().size()) return -1;
+    const Case& cs = registry()[id];
+    cs.launch(a, b, c, d, cs.threads, cs.lds_bytes, static_cast<hipStream_t>(stream));
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        g_err = hipGetErrorString(e);
+        return -3;
+    }
+    return 0;
+}
+
+const char* tt_last_error(void) { return g_err.c_str(); }
+
+}  // extern "C"

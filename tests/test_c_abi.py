@@ -1,0 +1,98 @@
+"""The C-ABI boundary without a GPU: the library loads, exports every symbol declared in
+include/tcu_c_api.h, and rejects bad arguments with a status code and a message instead of
+touching the device (the reference's launcher calls exit() on errors, cuda_utils.hpp:20-27;
+its op throws on unsupported shapes, src/kernels/flash_attn.cu:453-455)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tcu_c_api.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tcu_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_entry_points():
+    syms = declared_symbols()
+    for name in ("tcu_gemm_f16", "tcu_b2b_gemm_f16", "tcu_flash_attn_fwd_f16", "tcu_lstm_f16", "tcu_last_error",
+                 "tcu_version", "tcu_device_count"):
+        assert name in syms
+
+
+def test_library_exports_every_declared_symbol(tcu):
+    handle = ctypes.CDLL(tcu.library_path())
+    for name in declared_symbols():
+        assert hasattr(handle, name), f"{name} declared in tcu_c_api.h but not exported"
+    # and the Python binding table covers the same set
+    assert sorted(tcu._SIGNATURES) == declared_symbols()
+
+
+def test_version_and_error_string(tcu):
+    assert tcu.lib().tcu_version() >= 100
+    assert isinstance(tcu.last_error(), str)
+
+
+@pytest.mark.parametrize("call", [
+    lambda l: l.tcu_gemm_f16(0, 0, 0, 128, 64, 256, 0, 0, 0),
+    lambda l: l.tcu_b2b_gemm_f16(0, 0, 0, 0, 64, 64, 64, 64, 1, 0, 0),
+    lambda l: l.tcu_flash_attn_fwd_f16(0, 0, 0, 0, 1, 64, 64, 128, 128, 1.0, 0, 0),
+    lambda l: l.tcu_lstm_f16(0, 0, 0, 0, 0, 0, 0, 1, 64, 128, 128, 0),
+])
+def test_null_pointers_are_rejected(tcu, call):
+    assert call(tcu.lib()) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert "null pointer" in tcu.last_error()
+
+
+def test_bad_sizes_and_enums_are_rejected(tcu):
+    l = tcu.lib()
+    p = 0x1000  # never dereferenced: argument checks come first
+    assert l.tcu_gemm_f16(p, p, p, 0, 64, 64, 0, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_gemm_f16(p, p, p, 64, 64, 64, 7, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert "out_dtype" in tcu.last_error()
+    assert l.tcu_gemm_f16(p, p, p, 64, 64, 64, 0, 9, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_b2b_gemm_f16(p, p, p, p, 64, 64, 64, 64, -1, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 64, 128, 128, 1.0, 5, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_lstm_f16(p, p, p, 0, 0, p, p, 0, 64, 128, 128, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+
+
+def test_unsupported_shapes_are_reported_not_launched(tcu):
+    l = tcu.lib()
+    p = 0x1000
+    assert l.tcu_gemm_f16(p, p, p, 100, 64, 64, 0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_gemm_f16(p, p, p, 64, 64, 48, 0, 3, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_gemm_f16(p, p, p, 256, 256, 256, 0, 1, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_b2b_gemm_f16(p, p, p, p, 64, 96, 64, 64, 1, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 64, 128, 64, 1.0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 100, 128, 128, 1.0, 1, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 192, 128, 128, 1.0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_lstm_f16(p, p, p, 0, 0, p, p, 1, 64, 100, 128, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_lstm_f16(p, p, p, 0, 0, p, p, 1, 10, 128, 128, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+
+
+def test_python_wrappers_validate_before_calling(tcu):
+    import torch
+
+    a = torch.zeros(64, 64, dtype=torch.float16)
+    with pytest.raises(ValueError, match="device memory"):
+        tcu.gemm(a, a)
+    with pytest.raises(ValueError, match="mismatched K"):
+        tcu.gemm(a, torch.zeros(64, 32, dtype=torch.float16))
+    with pytest.raises(ValueError, match="W must be"):
+        tcu.lstm(torch.zeros(1, 64, 128, dtype=torch.float16), torch.zeros(512, 100, dtype=torch.float16),
+                 torch.zeros(512, dtype=torch.float16))
+    err = tcu.TcuError(-2, "x")
+    assert isinstance(err, RuntimeError) and err.status == -2
+
+
+def test_tile_test_library_loads():
+    path = os.path.join(ROOT, "tests", "device", "_build", "libtcu_tile_tests.so")
+    if not os.path.exists(path):
+        pytest.skip("device test library not built")
+    handle = ctypes.CDLL(path)
+    assert handle.tt_num_cases() > 50

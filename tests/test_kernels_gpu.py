@@ -1,0 +1,329 @@
+"""Parity tests of the kernel entries, through the C-ABI (ctypes), against the CPU oracle on
+the same seeded inputs.
+
+Tolerances (BASELINE): GEMM / back-to-back GEMM max relative error <= 1e-3 against the
+f32-accumulated oracle, where "relative" is |x - ref| / max(|ref|, 0.01 * rms(ref)) (outputs
+of a K-long dot product land arbitrarily close to zero, so a plain elementwise ratio is
+meaningless); attention and LSTM max absolute error <= 1e-2.
+Seeds: 1234 + configuration index, as the CPU-baseline plan fixes them.
+"""
+import math
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-3
+ABS_TOL = 1e-2
+
+
+def dev(a, device):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def host(t):
+    return t.float().cpu().numpy() if t.dtype != __import__("torch").float32 else t.cpu().numpy()
+
+
+# ------------------------------------------------------------------------------ GEMM
+@pytest.mark.parametrize("algo", ["global_reg", "all_mem", "pipelined", "auto"])
+def test_gemm_config1_readme_shape(tcu, oracle, device, algo):
+    """C1: M=128 N=64 K=256, U[-1,1], f32 out, every GEMM kernel."""
+    import torch
+
+    print(f"gemm C1 algo={algo}", flush=True)
+    A = oracle.fill_uniform(128 * 256, 1235).reshape(128, 256)
+    Bt = oracle.fill_uniform(64 * 256, 1235 + 1000).reshape(64, 256)
+    C = tcu.gemm(dev(A, device), dev(Bt, device), out_dtype=torch.float32, algo=algo)
+    torch.cuda.synchronize()
+    assert oracle.max_rel_err(host(C), oracle.gemm(A, Bt)) <= REL_TOL
+
+
+def test_gemm_golden_ramp(tcu, oracle, device):
+    import os
+
+    import torch
+
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "golden_small.npz"))
+    A, Bt, C = gold["gemm_128x64x256_A"], gold["gemm_128x64x256_Bt"], gold["gemm_128x64x256_C"]
+    for algo in ("global_reg", "all_mem", "pipelined"):
+        got = tcu.gemm(dev(A, device), dev(Bt, device), out_dtype=torch.float32, algo=algo)
+        assert oracle.max_rel_err(host(got), C) <= REL_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (64, 128, 192), (128, 128, 64), (256, 128, 512), (256, 256, 128),
+                                   (512, 1024, 256), (1024, 768, 320), (2048, 2048, 1024)])
+@pytest.mark.parametrize("out_dtype", ["f32", "f16"])
+def test_gemm_pipelined_shapes(tcu, oracle, device, M, N, K, out_dtype):
+    """Run-time shapes across all three tile configurations, one- and many-k-tile loops."""
+    import torch
+
+    print(f"gemm pipelined {M}x{N}x{K} {out_dtype}", flush=True)
+    A = oracle.fill_uniform(M * K, 7 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 9 + N).reshape(N, K)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    C = tcu.gemm(dev(A, device), dev(Bt, device), out_dtype=dt, algo="pipelined")
+    torch.cuda.synchronize()
+    assert oracle.max_rel_err(host(C), oracle.gemm(A, Bt)) <= REL_TOL
+
+
+def test_gemm_one_hot_index_probe(tcu, device):
+    """C[m, n] = A[m, k] * Bt[n, k] for one-hot operands: pins rows/cols/transposition exactly."""
+    import torch
+
+    M = N = K = 256
+    A = torch.zeros(M, K, dtype=torch.float16, device=device)
+    Bt = torch.zeros(N, K, dtype=torch.float16, device=device)
+    picks = [(0, 0, 0), (37, 201, 99), (255, 3, 255), (128, 64, 32), (200, 255, 1)]
+    for i, (m, n, k) in enumerate(picks):
+        A[m, k] = 1.0 + i
+        Bt[n, k] = 2.0
+    C = tcu.gemm(A, Bt, out_dtype=torch.float32, algo="pipelined").cpu().numpy()
+    want = A.float().cpu().numpy() @ Bt.float().cpu().numpy().T
+    assert np.array_equal(C, want)
+
+
+def test_gemm_reference_driver_shapes(tcu, oracle, device):
+    """The driver shapes of the reference's two GEMM examples (1024x1024x2048 global->register,
+    4096^3 single-stage LDS): checked on a window of rows."""
+    import torch
+
+    for (M, N, K, algo) in [(1024, 1024, 2048, "global_reg"), (4096, 4096, 4096, "all_mem")]:
+        print(f"gemm reference driver {M}x{N}x{K} {algo}", flush=True)
+        A = oracle.fill_uniform(M * K, 1236).reshape(M, K)
+        Bt = oracle.fill_uniform(N * K, 2236).reshape(N, K)
+        C = host(tcu.gemm(dev(A, device), dev(Bt, device), out_dtype=torch.float32, algo=algo))
+        rows = (M // 2 - 32, M // 2 + 32)
+        ref = oracle.gemm(A, Bt, rows=rows)
+        assert oracle.max_rel_err(C[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
+        first = oracle.gemm(A, Bt, rows=(0, 16))
+        assert oracle.max_rel_err(C[:16], first[:16]) <= REL_TOL
+
+
+def test_gemm_config2_4096_cubed(tcu, oracle, device):
+    """C2: M=N=K=4096, U[-1,1], f16 out. Oracle on 768 sampled rows (first/middle/last tiles)
+    plus size-independent properties over the full output."""
+    import torch
+
+    print("gemm C2 4096^3", flush=True)
+    n = 4096
+    A = oracle.fill_uniform(n * n, 1236).reshape(n, n)
+    Bt = oracle.fill_uniform(n * n, 2236).reshape(n, n)
+    dA, dB = dev(A, device), dev(Bt, device)
+    C = tcu.gemm(dA, dB, out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    Ch = host(C)
+    assert np.isfinite(Ch).all()
+    for rows in [(0, 256), (1920, 2176), (3840, 4096)]:
+        ref = oracle.gemm(A, Bt, rows=rows)
+        assert oracle.max_rel_err(Ch[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
+    # column sums: ones^T (A B) = (ones^T A) B, computed in float64 on the host
+    colsum = A.astype(np.float64).sum(0) @ Bt.astype(np.float64).T
+    got = Ch.astype(np.float64).sum(0)
+    assert np.max(np.abs(got - colsum)) <= 1e-3 * np.sqrt(np.mean(colsum ** 2)) * 4 + 4096 * 21 * 2 ** -11 * 0.05
+    # linearity in A: gemm(2A) == 2 gemm(A) exactly (power-of-two scaling commutes with rounding)
+    C2 = tcu.gemm((dA * 2).contiguous(), dB, out_dtype=torch.float16)
+    assert torch.equal(C2, C * 2)
+    # f32 output agrees with the f16 output to f16 rounding
+    C32 = tcu.gemm(dA, dB, out_dtype=torch.float32)
+    assert torch.equal(C32.half(), C)
+
+
+# ------------------------------------------------------------------------------ back-to-back GEMM
+@pytest.mark.parametrize("M,N,K,P,batch", [(64, 64, 64, 64, 1), (48, 64, 64, 64, 3), (128, 128, 64, 64, 2),
+                                           (256, 256, 128, 128, 1), (1024, 256, 128, 128, 2)])
+@pytest.mark.parametrize("out_dtype", ["f32", "f16"])
+def test_b2b_gemm_shapes(tcu, oracle, device, M, N, K, P, batch, out_dtype):
+    import torch
+
+    print(f"b2b {M}x{N}x{K}x{P} b{batch} {out_dtype}", flush=True)
+    A = oracle.fill_normal(batch * M * K, 11, 0, 0.1).reshape(batch, M, K)
+    Bt = oracle.fill_normal(batch * N * K, 12, 0, 0.1).reshape(batch, N, K)
+    Ct = oracle.fill_normal(batch * P * N, 13, 0, 0.1).reshape(batch, P, N)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    D = tcu.b2b_gemm(dev(A, device), dev(Bt, device), dev(Ct, device), out_dtype=dt)
+    torch.cuda.synchronize()
+    ref = oracle.b2b_gemm(A, Bt, Ct)
+    # the f16-rounded intermediate may round differently where the f32 sums differ in the last
+    # bit (different accumulation order); that moves an output by at most 2^-11 * |acc| * |C|
+    assert oracle.max_rel_err(host(D), ref) <= REL_TOL
+
+
+def test_b2b_gemm_config3(tcu, oracle, device):
+    """C3: A [8192x128], B [128x256], C [256x128], N(0, 0.1), f16 D."""
+    import torch
+
+    print("b2b C3", flush=True)
+    M, N, K, P = 8192, 256, 128, 128
+    A = oracle.fill_normal(M * K, 1237, 0, 0.1).reshape(M, K)
+    Bt = oracle.fill_normal(N * K, 2237, 0, 0.1).reshape(N, K)
+    Ct = oracle.fill_normal(P * N, 3237, 0, 0.1).reshape(P, N)
+    D = tcu.b2b_gemm(dev(A, device), dev(Bt, device), dev(Ct, device), out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    assert oracle.max_rel_err(host(D), oracle.b2b_gemm(A, Bt, Ct)) <= REL_TOL
+    # identity second operand: D = f16(A B)
+    eye = np.eye(N, dtype=np.float16)[:P].copy()  # C[n, p] = delta(n, p), stored [P, N]
+    D2 = tcu.b2b_gemm(dev(A, device), dev(Bt, device), dev(eye, device), out_dtype=torch.float32)
+    want = oracle.gemm(A, Bt)[:, :P]
+    assert oracle.max_rel_err(host(D2), want.astype(np.float16).astype(np.float32)) <= REL_TOL
+
+
+# ------------------------------------------------------------------------------ attention
+@pytest.mark.parametrize("n", [64, 128, 256])
+def test_flash_attention_reference_shapes(tcu, oracle, device, n):
+    """The three shapes of the reference's tests/python/test_flash_attn.py (m=64, k=p=128), driven
+    through the mirror of its TiledFlashAttention wrapper (K as [k, n], V as [n, p], scale 1).
+    The reference accepts 8e-2; the bar here is 1e-2."""
+    import torch
+
+    print(f"attention reference shape n={n}", flush=True)
+    m, k, p = 64, 128, 128
+    Q = oracle.fill_normal(m * k, 1234).reshape(m, k)
+    Kmat = oracle.fill_normal(k * n, 1235).reshape(k, n)
+    V = oracle.fill_normal(n * p, 1236).reshape(n, p)
+    op = tcu.TiledFlashAttention(dev(Q, device), dev(Kmat, device), dev(V, device))
+    O = op.forward()
+    torch.cuda.synchronize()
+    assert tuple(O.shape) == (m, p) and O.dtype == torch.float16
+    ref = oracle.attention(Q, np.ascontiguousarray(Kmat.T), V, 1.0)
+    assert oracle.max_abs_err(host(O), ref) <= ABS_TOL
+
+
+@pytest.mark.parametrize("batch,M,N,D", [(1, 64, 64, 128), (3, 128, 192, 128), (2, 256, 512, 128), (2, 128, 256, 64)])
+def test_flash_attention_row_major_v(tcu, oracle, device, batch, M, N, D):
+    import torch
+
+    print(f"attention b{batch} {M}x{N}x{D}", flush=True)
+    q = oracle.fill_normal(batch * M * D, 21).reshape(batch, M, D)
+    k = oracle.fill_normal(batch * N * D, 22).reshape(batch, N, D)
+    v = oracle.fill_normal(batch * N * D, 23).reshape(batch, N, D)
+    O = tcu.flash_attention(dev(q, device), dev(k, device), dev(v, device))
+    torch.cuda.synchronize()
+    ref = oracle.attention(q, k, v, 1.0 / math.sqrt(D))
+    assert oracle.max_abs_err(host(O), ref) <= ABS_TOL
+
+
+def test_flash_attention_properties(tcu, oracle, device):
+    """Size-independent properties: constant V, zero scale, joint permutation of keys/values."""
+    import torch
+
+    B, S, D = 2, 256, 128
+    q = dev(oracle.fill_normal(B * S * D, 31).reshape(B, S, D), device)
+    k = dev(oracle.fill_normal(B * S * D, 32).reshape(B, S, D), device)
+    v = dev(oracle.fill_normal(B * S * D, 33).reshape(B, S, D), device)
+    vconst = v[:, :1, :].expand(B, S, D).contiguous()
+    O = tcu.flash_attention(q, k, vconst)
+    assert torch.allclose(O.float(), vconst.float(), atol=2e-3)
+    O0 = tcu.flash_attention(q, k, v, scale=0.0)
+    assert torch.allclose(O0.float(), v.float().mean(1, keepdim=True).expand(B, S, D), atol=2e-3)
+    perm = torch.randperm(S, device=device, generator=torch.Generator(device=device).manual_seed(1))
+    O1 = tcu.flash_attention(q, k, v)
+    O2 = tcu.flash_attention(q, k[:, perm].contiguous(), v[:, perm].contiguous())
+    assert torch.allclose(O1.float(), O2.float(), atol=4e-3)
+
+
+def test_flash_attention_config4(tcu, oracle, device):
+    """C4: [4, 16, 2048, 128], N(0, 1), scale 1/sqrt(128). Oracle on sampled (batch, head, row
+    window) slices plus the constant-V property on the full shape."""
+    import torch
+
+    print("attention C4", flush=True)
+    B, H, S, D = 4, 16, 2048, 128
+    n = B * H * S * D
+    q = oracle.fill_normal(n, 1238).reshape(B * H, S, D)
+    k = oracle.fill_normal(n, 2238).reshape(B * H, S, D)
+    v = oracle.fill_normal(n, 3238).reshape(B * H, S, D)
+    dq, dk, dv = (dev(t.reshape(B, H, S, D), device) for t in (q, k, v))
+    O = tcu.flash_attention(dq, dk, dv)
+    torch.cuda.synchronize()
+    assert tuple(O.shape) == (B, H, S, D)
+    Oh = host(O).reshape(B * H, S, D)
+    assert np.isfinite(Oh).all()
+    scale = 1.0 / math.sqrt(D)
+    for head, rows in [(0, (0, 128)), (17, (960, 1088)), (63, (1920, 2048))]:
+        ref = oracle.attention(q[head], k[head], v[head], scale, rows=rows)
+        assert oracle.max_abs_err(Oh[head, rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= ABS_TOL
+    vconst = dv[:, :, :1, :].expand(B, H, S, D).contiguous()
+    Oc = tcu.flash_attention(dq, dk, vconst)
+    assert torch.allclose(Oc.float(), vconst.float(), atol=2e-3)
+
+
+def test_unsupported_shape_raises_runtime_error(tcu, device):
+    """The reference op throws std::runtime_error("Unsupported shape") -> Python RuntimeError."""
+    import torch
+
+    q = torch.zeros(64 * 128, dtype=torch.float16, device=device)
+    kk = torch.zeros(192 * 128, dtype=torch.float16, device=device)
+    o = torch.zeros(64 * 128, dtype=torch.float16, device=device)
+    with pytest.raises(RuntimeError):
+        tcu.flash_attention_fwd(q, kk, kk, o, 64, 192, 128, 128)
+    with pytest.raises(RuntimeError):
+        tcu.gemm(torch.zeros(100, 64, dtype=torch.float16, device=device),
+                 torch.zeros(64, 64, dtype=torch.float16, device=device))
+
+
+# ------------------------------------------------------------------------------ LSTM
+@pytest.mark.parametrize("T,B,I,H,with_state", [(1, 64, 128, 128, False), (4, 64, 128, 128, True),
+                                                (3, 128, 64, 128, True)])
+def test_lstm_small(tcu, oracle, device, T, B, I, H, with_state):
+    import torch
+
+    print(f"lstm T{T} B{B} I{I} H{H} state={with_state}", flush=True)
+    x = oracle.fill_normal(T * B * I, 41, 0, 0.5).reshape(T, B, I)
+    W = oracle.fill_normal(4 * H * (I + H), 42, 0, 0.1).reshape(4 * H, I + H)
+    b = oracle.fill_normal(4 * H, 43, 0, 0.1)
+    h0 = oracle.fill_normal(B * H, 44, 0, 0.5).reshape(B, H) if with_state else None
+    c0 = oracle.fill_normal(B * H, 45, 0, 0.5).reshape(B, H).astype(np.float32) if with_state else None
+    h_all, c_T = tcu.lstm(dev(x, device), dev(W, device), dev(b, device),
+                          dev(h0, device) if with_state else None, dev(c0, device) if with_state else None)
+    torch.cuda.synchronize()
+    h_ref, c_ref = oracle.lstm(x, W, b, h0, c0)
+    assert oracle.max_abs_err(host(h_all), h_ref) <= ABS_TOL
+    assert oracle.max_abs_err(host(c_T), c_ref) <= ABS_TOL
+
+
+def test_lstm_zero_weights_closed_form(tcu, device):
+    """W = 0: c_t = sigmoid(b_f) c_{t-1} + sigmoid(b_i) tanh(b_g), h_t = sigmoid(b_o) tanh(c_t)."""
+    import torch
+
+    T, B, I, H = 5, 64, 128, 128
+    x = torch.randn(T, B, I, device=device, generator=torch.Generator(device=device).manual_seed(3)).half()
+    W = torch.zeros(4 * H, I + H, dtype=torch.float16, device=device)
+    b = (torch.arange(4 * H, device=device).float() / (4 * H) - 0.5).half()
+    h_all, c_T = tcu.lstm(x, W, b)
+    bi, bf, bg, bo = (b.double()[j * H:(j + 1) * H] for j in range(4))
+    c = torch.zeros(H, dtype=torch.float64, device=device)
+    for t in range(T):
+        c = torch.sigmoid(bf) * c + torch.sigmoid(bi) * torch.tanh(bg)
+        h = torch.sigmoid(bo) * torch.tanh(c)
+        assert torch.allclose(h_all[t].double(), h.expand(B, H), atol=2e-3)
+    assert torch.allclose(c_T.double(), c.expand(B, H), atol=1e-5)
+
+
+def test_lstm_config5(tcu, oracle, device):
+    """C5: batch 256, input 1024, hidden 1024, 16 steps; x, W ~ N(0, 0.05), bias ~ N(0, 0.05), h0=c0=0.
+    Oracle on 8 sampled batch rows (rows are independent)."""
+    import torch
+
+    print("lstm C5", flush=True)
+    T, B, I, H = 16, 256, 1024, 1024
+    x = oracle.fill_normal(T * B * I, 1239, 0, 0.05).reshape(T, B, I)
+    W = oracle.fill_normal(4 * H * (I + H), 2239, 0, 0.05).reshape(4 * H, I + H)
+    b = oracle.fill_normal(4 * H, 3239, 0, 0.05)
+    h_all, c_T = tcu.lstm(dev(x, device), dev(W, device), dev(b, device))
+    torch.cuda.synchronize()
+    hh, cc = host(h_all), host(c_T)
+    assert np.isfinite(hh).all() and np.isfinite(cc).all()
+    for rows in [(0, 4), (252, 256)]:
+        h_ref, c_ref = oracle.lstm(x, W, b, rows=rows)
+        assert oracle.max_abs_err(hh[:, rows[0]:rows[1]], h_ref[:, rows[0]:rows[1]]) <= ABS_TOL
+        assert oracle.max_abs_err(cc[rows[0]:rows[1]], c_ref[rows[0]:rows[1]]) <= ABS_TOL
+
+
+def test_smoke_entry(device):
+    import __graft_entry__ as g
+
+    g.smoke()

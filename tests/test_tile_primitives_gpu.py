@@ -1,0 +1,124 @@
+"""Device unit tests of the tile primitives (tests/device/tile_tests.hip): every case of the
+registry is run on the GPU and checked on the host against the identity or the CPU oracle.
+Shapes and warp layouts are those of the reference's tests/cpp/cell/*.cu."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "tests", "device", "_build", "libtcu_tile_tests.so")
+
+pytestmark = pytest.mark.gpu
+
+
+def _load():
+    handle = ctypes.CDLL(LIB)
+    handle.tt_num_cases.restype = ctypes.c_int
+    handle.tt_case_info.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(ctypes.c_char_p),
+                                    ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                                    ctypes.POINTER(ctypes.c_int)]
+    handle.tt_run_case.argtypes = [ctypes.c_int] + [ctypes.c_void_p] * 5
+    handle.tt_last_error.restype = ctypes.c_char_p
+    return handle
+
+
+def _cases():
+    if not os.path.exists(LIB):
+        return []
+    handle = _load()
+    out = []
+    for i in range(handle.tt_num_cases()):
+        kind, name = ctypes.c_char_p(), ctypes.c_char_p()
+        dims = (ctypes.c_int * 8)()
+        threads, lds = ctypes.c_int(), ctypes.c_int()
+        assert handle.tt_case_info(i, ctypes.byref(kind), ctypes.byref(name), dims, ctypes.byref(threads),
+                                   ctypes.byref(lds)) == 0
+        out.append((i, kind.value.decode(), name.value.decode(), list(dims)))
+    return out
+
+
+CASES = _cases()
+
+
+def test_registry_is_populated():
+    assert os.path.exists(LIB), "device test library missing: run __graft_entry__.build()"
+    kinds = {c[1] for c in CASES}
+    assert kinds == {"g2s_roundtrip", "s2r_identity", "store_roundtrip", "g2r_roundtrip", "tile_gemm", "row_ops",
+                     "col_ops"}
+
+
+def _np_dtype(nbytes):
+    return np.float16 if nbytes == 2 else np.float32
+
+
+@pytest.mark.parametrize("case", CASES, ids=[f"{c[1]}-{c[2]}" for c in CASES])
+def test_tile_case(case, device, oracle):
+    import torch
+
+    idx, kind, name, dims = case
+    print(f"tile case {idx} {kind} {name}", flush=True)
+    handle = _load()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run(a, b, c, d):
+        rc = handle.tt_run_case(idx, a.data_ptr() if a is not None else 0, b.data_ptr() if b is not None else 0,
+                                c.data_ptr() if c is not None else 0, d.data_ptr() if d is not None else 0, stream)
+        assert rc == 0, handle.tt_last_error()
+        torch.cuda.synchronize()
+
+    if kind in ("g2s_roundtrip", "s2r_identity", "store_roundtrip", "g2r_roundtrip"):
+        rows, cols, _, nbytes = dims[:4]
+        dt = _np_dtype(nbytes)
+        # the reference's ramp (i % 2048), distinct per element for these sizes, exact in f16 up to 2048
+        src = (np.arange(rows * cols) % 2048).astype(dt)
+        a = torch.from_numpy(src).to(device)
+        c = torch.full((rows * cols,), -1.0, dtype=a.dtype, device=device)
+        run(a, None, c, None)
+        assert np.array_equal(c.cpu().numpy(), src)
+    elif kind == "tile_gemm":
+        M, N, K = dims[:3]
+        A = oracle.fill_uniform(M * K, 100 + idx).reshape(M, K)
+        Bt = oracle.fill_uniform(N * K, 200 + idx).reshape(N, K)
+        a, b = torch.from_numpy(A).to(device), torch.from_numpy(Bt).to(device)
+        c = torch.full((M, N), float("nan"), dtype=torch.float32, device=device)
+        run(a, b, c, None)
+        err = oracle.max_rel_err(c.cpu().numpy(), oracle.gemm(A, Bt))
+        assert err <= 1e-3, f"max rel err {err}"
+    elif kind in ("row_ops", "col_ops"):
+        rows, cols, op, nbytes = dims[:4]
+        dt = _np_dtype(nbytes)
+        rng = np.random.default_rng(42 + idx)  # the reference's softmax test seeds with 42, U[-5, 5]
+        x = rng.uniform(-5, 5, (rows, cols)).astype(dt)
+        row_major = kind == "row_ops"
+        mem = x if row_major else np.ascontiguousarray(x.T)  # column-major storage
+        a = torch.from_numpy(mem.copy()).to(device)
+        nvec = rows if row_major else cols
+        vec = torch.full((nvec,), float("nan"), dtype=a.dtype, device=device)
+        tile = torch.full(mem.shape, float("nan"), dtype=a.dtype, device=device)
+        run(a, None, vec, tile)
+        v = vec.cpu().numpy().astype(np.float64)
+        t = tile.cpu().numpy().astype(np.float64)
+        if not row_major:
+            t = t.T
+        x64 = x.astype(np.float64)
+        axis = 1 if row_major else 0
+        tol = 1e-3 if dt == np.float32 else 0.15  # f16 sums of up to 64 values of magnitude 5
+        names = ["sum", "max", "bcast_sum", "sub_max", "softmax"] if row_major else ["sum", "max", "sub_max"]
+        opname = names[op]
+        if opname == "sum":
+            assert np.allclose(v, x64.sum(axis), atol=tol)
+            assert np.array_equal(t, x64)
+        elif opname == "max":
+            assert np.array_equal(v, x64.max(axis))
+        elif opname == "bcast_sum":
+            assert np.allclose(v, x64.sum(axis), atol=tol)
+            assert np.allclose(t, np.repeat(x64.sum(1, keepdims=True), cols, 1), atol=tol)
+        elif opname == "sub_max":
+            assert np.allclose(t, x64 - x64.max(axis, keepdims=True), atol=1e-6 if dt == np.float32 else 1e-2)
+        elif opname == "softmax":
+            e = np.exp(x64 - x64.max(1, keepdims=True))
+            assert np.allclose(t, e / e.sum(1, keepdims=True), atol=1e-3)  # the reference's tolerance
+    else:
+        raise AssertionError(kind)

@@ -1,0 +1,224 @@
+"""MI355X-native tile kernels behind the reference's Python surface.
+
+Mirrors ``pytiledcuda/__init__.py`` of the reference (``flash_attention_fwd``,
+``TiledFlashAttention``) and adds the other kernel entries (``gemm``, ``b2b_gemm``,
+``lstm``, ``flash_attention``).  Everything runs through the C-ABI shared library
+``lib/libtiledcuda_amd.so`` (declared in ``include/tcu_c_api.h``); there is no CPU or
+PyTorch fallback: if the library is missing, importing any op raises.
+
+PyTorch is used only for device memory and the current HIP stream.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import os
+
+import torch
+
+__all__ = [
+    "TcuError", "library_path", "lib", "last_error", "gemm", "b2b_gemm", "flash_attention_fwd",
+    "flash_attention", "TiledFlashAttention", "lstm", "GEMM_ALGOS",
+]
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "lib", "libtiledcuda_amd.so")
+_lib = None
+
+TCU_OK = 0
+TCU_ERR_INVALID_ARGUMENT = -1
+TCU_ERR_UNSUPPORTED_SHAPE = -2
+TCU_ERR_HIP = -3
+TCU_ERR_NO_DEVICE = -4
+
+TCU_DTYPE_F32 = 0
+TCU_DTYPE_F16 = 1
+
+GEMM_ALGOS = {"auto": 0, "global_reg": 1, "all_mem": 2, "pipelined": 3}
+
+TCU_V_COL_MAJOR = 0
+TCU_V_ROW_MAJOR = 1
+
+# every exported symbol with its ctypes signature (also what the symbol test checks)
+_SIGNATURES = {
+    "tcu_version": (ctypes.c_int, []),
+    "tcu_last_error": (ctypes.c_char_p, []),
+    "tcu_device_count": (ctypes.c_int, []),
+    "tcu_gemm_f16": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int] * 5 + [ctypes.c_void_p]),
+    "tcu_b2b_gemm_f16": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 6 + [ctypes.c_void_p]),
+    "tcu_flash_attn_fwd_f16": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int,
+                                                                                           ctypes.c_void_p]),
+    "tcu_lstm_f16": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
+}
+
+
+class TcuError(RuntimeError):
+    """A C-ABI call returned a negative status (the reference op raises RuntimeError too)."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(f"tiledcuda_amd status {status}: {message}")
+        self.status = status
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    """Load the HIP extension (once). Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise ImportError(
+                f"{_LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(hipcc --offload-arch=gfx950). There is no fallback path.")
+        handle = ctypes.CDLL(_LIB_PATH)
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def last_error() -> str:
+    return lib().tcu_last_error().decode()
+
+
+def _check(status: int) -> None:
+    if status != TCU_OK:
+        raise TcuError(status, last_error())
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev_ptr(t: torch.Tensor | None, dtype: torch.dtype, name: str) -> int:
+    if t is None:
+        return 0
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live in device memory")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return t.data_ptr()
+
+
+def _out_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return TCU_DTYPE_F32
+    if dtype == torch.float16:
+        return TCU_DTYPE_F16
+    raise ValueError("out dtype must be torch.float32 or torch.float16")
+
+
+# ------------------------------------------------------------------------------ GEMM
+def gemm(a: torch.Tensor, b_t: torch.Tensor, out: torch.Tensor | None = None,
+         out_dtype: torch.dtype = torch.float16, algo: str = "auto") -> torch.Tensor:
+    """C[M, N] = A[M, K] · B with B column-major, i.e. ``b_t`` is the [N, K] array (``a @ b_t.T``).
+
+    Mirrors the reference's GEMM examples (A row-major, B column-major, f32 accumulate).
+    """
+    M, K = a.shape
+    N, K2 = b_t.shape
+    if K != K2:
+        raise ValueError("mismatched K dimension")
+    if out is None:
+        out = torch.empty(M, N, dtype=out_dtype, device=a.device)
+    elif tuple(out.shape) != (M, N):
+        raise ValueError("out has the wrong shape")
+    _check(lib().tcu_gemm_f16(_dev_ptr(a, torch.float16, "a"), _dev_ptr(b_t, torch.float16, "b_t"),
+                              _dev_ptr(out, out.dtype, "out"), M, N, K, _out_code(out.dtype), GEMM_ALGOS[algo],
+                              _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------ b2b GEMM
+def b2b_gemm(a: torch.Tensor, b_t: torch.Tensor, c_t: torch.Tensor, out: torch.Tensor | None = None,
+             out_dtype: torch.dtype = torch.float16) -> torch.Tensor:
+    """D = (A · B) · C per batch item; ``b_t`` [.., N, K] and ``c_t`` [.., P, N] are the
+    column-major operands of the reference's fused two-GEMM example stored as arrays."""
+    batched = a.dim() == 3
+    a3, b3, c3 = (t if batched else t.unsqueeze(0) for t in (a, b_t, c_t))
+    batch, M, K = a3.shape
+    _, N, _ = b3.shape
+    _, P, _ = c3.shape
+    if tuple(b3.shape) != (batch, N, K) or tuple(c3.shape) != (batch, P, N):
+        raise ValueError("operand shapes do not chain: A [b,M,K], b_t [b,N,K], c_t [b,P,N]")
+    if out is None:
+        out = torch.empty(batch, M, P, dtype=out_dtype, device=a.device)
+    _check(lib().tcu_b2b_gemm_f16(_dev_ptr(a3, torch.float16, "a"), _dev_ptr(b3, torch.float16, "b_t"),
+                                  _dev_ptr(c3, torch.float16, "c_t"), _dev_ptr(out, out.dtype, "out"), M, N, K, P,
+                                  batch, _out_code(out.dtype), _stream()))
+    return out if batched else out.view(M, P) if out.dim() == 3 else out
+
+
+# ------------------------------------------------------------------------------ attention
+def flash_attention_fwd(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, O: torch.Tensor, m: int, n: int, k: int,
+                        p: int, scale: float = 1.0, batch: int = 1) -> None:
+    """Same call shape as the reference's ``pytiledcuda.flash_attention_fwd`` (flattened fp16
+    device tensors; K as [n, k], V as [p, n]; O written in place; ``scale`` defaults to the
+    reference's 1).  Unsupported shapes raise ``RuntimeError`` like the reference op."""
+    _check(lib().tcu_flash_attn_fwd_f16(_dev_ptr(Q, torch.float16, "Q"), _dev_ptr(K, torch.float16, "K"),
+                                        _dev_ptr(V, torch.float16, "V"), _dev_ptr(O, torch.float16, "O"), batch, m, n,
+                                        k, p, float(scale), TCU_V_COL_MAJOR, _stream()))
+
+
+def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float | None = None,
+                    out: torch.Tensor | None = None) -> torch.Tensor:
+    """softmax(scale · q kᵀ) v for [..., S, D] tensors in the usual layout (V row-major [S, D]).
+    ``scale`` defaults to 1/sqrt(D)."""
+    *lead, M, D = q.shape
+    N = k.shape[-2]
+    P = v.shape[-1]
+    batch = int(math.prod(lead)) if lead else 1
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    if out is None:
+        out = torch.empty(*lead, M, P, dtype=torch.float16, device=q.device)
+    _check(lib().tcu_flash_attn_fwd_f16(_dev_ptr(q, torch.float16, "q"), _dev_ptr(k, torch.float16, "k"),
+                                        _dev_ptr(v, torch.float16, "v"), _dev_ptr(out, torch.float16, "out"), batch,
+                                        M, N, D, P, float(scale), TCU_V_ROW_MAJOR, _stream()))
+    return out
+
+
+class TiledFlashAttention:
+    """Mirror of the reference's ``pytiledcuda.TiledFlashAttention``: ``query`` [m, k],
+    ``key`` [k, n], ``value`` [n, p]; ``forward()`` returns O [m, p] in fp16 (scale 1)."""
+
+    def __init__(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, scale: float = 1.0):
+        self.m, self.k = query.size(-2), query.size(-1)
+        self.n, self.p = value.size(-2), value.size(-1)
+        self.scale = scale
+
+        self.query = query.half().flatten().contiguous()
+        # the kernel consumes K and V column-major: store their transposes
+        self.key = key.half().t().contiguous().flatten()
+        self.value = value.half().t().contiguous().flatten()
+
+        self.output = torch.empty(self.m, self.p, dtype=torch.half, device=query.device).flatten()
+
+    def forward(self) -> torch.Tensor:
+        flash_attention_fwd(self.query, self.key, self.value, self.output, self.m, self.n, self.k, self.p,
+                            scale=self.scale)
+        return self.output.view(self.m, self.p)
+
+
+# ------------------------------------------------------------------------------ LSTM
+def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor | None = None,
+         c0: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Fused LSTM layer. x [T, B, I] f16, W [4H, I+H] f16 (gate rows i,f,g,o), bias [4H] f16,
+    h0 [B, H] f16 / c0 [B, H] f32 (None = zeros). Returns (h_all [T, B, H] f16, c_T [B, H] f32)."""
+    T, B, I = x.shape
+    H = W.shape[0] // 4
+    if tuple(W.shape) != (4 * H, I + H) or tuple(bias.shape) != (4 * H,):
+        raise ValueError("W must be [4H, I+H] and bias [4H]")
+    h_all = torch.empty(T, B, H, dtype=torch.float16, device=x.device)
+    c_out = torch.empty(B, H, dtype=torch.float32, device=x.device)
+    _check(lib().tcu_lstm_f16(_dev_ptr(x, torch.float16, "x"), _dev_ptr(W, torch.float16, "W"),
+                              _dev_ptr(bias, torch.float16, "bias"), _dev_ptr(h0, torch.float16, "h0"),
+                              _dev_ptr(c0, torch.float32, "c0"), _dev_ptr(h_all, torch.float16, "h_all"),
+                              _dev_ptr(c_out, torch.float32, "c_out"), T, B, I, H, _stream()))
+    return h_all, c_out

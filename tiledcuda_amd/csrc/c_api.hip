@@ -1,0 +1,281 @@
+// Implementation of the C-ABI declared in include/tcu_c_api.h: argument checks, shape
+// dispatch and kernel launches. No device memory is allocated here and no stream is
+// synchronised; errors become status codes plus a thread-local message.
+#include "tcu_c_api.h"
+
+#include "kernels/gemm_pipelined.hpp"
+#include "kernels/mod.hpp"
+
+#include <string>
+
+using namespace tiledcuda;
+using namespace tiledcuda::kernels;
+namespace tl = tiledcuda::cell::tile_layout;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string& msg) {
+    g_last_error = msg;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    return fail(TCU_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+/// Launch with dynamic LDS; raises the limit when the kernel needs more than the default.
+template <typename Kernel, typename... Args>
+int launch(Kernel kernel, dim3 grid, dim3 block, int lds_bytes, hipStream_t stream, Args... args) {
+    if (lds_bytes > kMaxLdsBytes) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "kernel needs more LDS than a CU has");
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    }
+    hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args...);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, "kernel launch");
+    return TCU_OK;
+}
+
+bool positive(std::initializer_list<int> v) {
+    for (int x : v)
+        if (x <= 0) return false;
+    return true;
+}
+
+// ---------------------------------------------------------------------------- GEMM
+template <typename OutType, int kM, int kN, int kK, int kTM, int kTN, int kChunkK, typename WarpLayout>
+int launch_simple_gemm(const __half* A, const __half* B, OutType* C, hipStream_t stream) {
+    using Shape = GemmShape<kM, kN, kK>;
+    using Cfg = GemmTraits<__half, OutType, Shape, kTM, kTN, WarpLayout, kChunkK>;
+    auto kernel = &simple_gemm<__half, OutType, kM, kN, kK, kTM, kTN, typename Cfg::IteratorA, typename Cfg::RegA,
+                               typename Cfg::ALoader, typename Cfg::IteratorB, typename Cfg::RegB,
+                               typename Cfg::BLoader, typename Cfg::GlobalC, typename Cfg::RegC,
+                               typename Cfg::CStorer>;
+    return launch(kernel, dim3(kM / kTM, kN / kTN), dim3(Cfg::kThreads), 0, stream, A, B, C);
+}
+
+template <typename OutType, int kM, int kN, int kK, int kTM, int kTN, int kTK, int kRK, typename WarpLayout>
+int launch_all_mem_gemm(const __half* A, const __half* B, OutType* C, hipStream_t stream) {
+    using Cfg = KeGemmTraits<__half, OutType, GemmShape<kM, kN, kK>, GemmShape<kTM, kTN, kTK>, kRK, WarpLayout>;
+    auto kernel =
+        &gemm<__half, OutType, kM, kN, kK, kTM, kTN, kTK, typename Cfg::GIteratorA, typename Cfg::SIteratorA,
+              typename Cfg::SharedA, typename Cfg::RegA, typename Cfg::G2SLoaderA, typename Cfg::S2RLoaderA,
+              typename Cfg::GIteratorB, typename Cfg::SIteratorB, typename Cfg::SharedB, typename Cfg::RegB,
+              typename Cfg::G2SLoaderB, typename Cfg::S2RLoaderB, typename Cfg::GlobalC, typename Cfg::SharedC,
+              typename Cfg::RegC, typename Cfg::R2SStorerC, typename Cfg::S2GStorerC>;
+    return launch(kernel, dim3(kM / kTM, kN / kTN), dim3(Cfg::kThreads), Cfg::kShmBytes, stream, A, B, C);
+}
+
+template <typename Traits, typename OutType>
+int launch_pipelined(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    auto kernel = &gemm_pipelined<Traits, OutType>;
+    const int grid = (M / Traits::kBM) * (N / Traits::kBN);
+    return launch(kernel, dim3(grid), dim3(Traits::kThreads), Traits::template lds_bytes<OutType>(), stream, A, B, C,
+                  M, N, K);
+}
+
+using PipeLarge = PipelinedGemmTraits<256, 256, 64, 2, 2, 2>;
+using PipeMid = PipelinedGemmTraits<128, 128, 64, 2, 2, 2>;
+using PipeSmall = PipelinedGemmTraits<64, 64, 64, 2, 2, 2>;
+
+template <typename OutType>
+int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    if (K % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "pipelined GEMM needs K % 64 == 0");
+    const auto tiles = [&](int bm, int bn) { return (long)(M / bm) * (N / bn); };
+    if (M % 256 == 0 && N % 256 == 0 && tiles(256, 256) >= 128)
+        return launch_pipelined<PipeLarge>(A, B, C, M, N, K, stream);
+    if (M % 128 == 0 && N % 128 == 0 && tiles(128, 128) >= 64)
+        return launch_pipelined<PipeMid>(A, B, C, M, N, K, stream);
+    if (M % 64 == 0 && N % 64 == 0) return launch_pipelined<PipeSmall>(A, B, C, M, N, K, stream);
+    return fail(TCU_ERR_UNSUPPORTED_SHAPE, "pipelined GEMM needs M % 64 == 0 and N % 64 == 0");
+}
+
+template <typename OutType>
+int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, int algo, hipStream_t stream) {
+    using W22 = tl::RowMajor<2, 2>;
+    switch (algo) {
+        case TCU_GEMM_AUTO:
+        case TCU_GEMM_PIPELINED:
+            return gemm_pipelined_dispatch<OutType>(A, B, C, M, N, K, stream);
+        case TCU_GEMM_GLOBAL_REG:
+          if constexpr (std::is_same_v<OutType, float>) {
+            if (M == 128 && N == 64 && K == 256)  // the README shape of the reference
+                return launch_simple_gemm<OutType, 128, 64, 256, 128, 64, 32, W22>(A, B, C, stream);
+            if (M == 1024 && N == 1024 && K == 2048)  // the driver shape of 01_gemm_global_reg/main.cu:105-106
+                return launch_simple_gemm<OutType, 1024, 1024, 2048, 256, 128, 64, W22>(A, B, C, stream);
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE, "global->register GEMM is instantiated for 128x64x256 and "
+                                                   "1024x1024x2048 only");
+          }
+          [[fallthrough]];
+        case TCU_GEMM_ALL_MEM:
+          if constexpr (std::is_same_v<OutType, float>) {
+            if (algo == TCU_GEMM_ALL_MEM && M == 128 && N == 64 && K == 256)
+                return launch_all_mem_gemm<OutType, 128, 64, 256, 64, 64, 64, 32, W22>(A, B, C, stream);
+            if (algo == TCU_GEMM_ALL_MEM && M == 4096 && N == 4096 && K == 4096)  // the driver shape of 02_gemm_all_mem/main.cu:5-8
+                return launch_all_mem_gemm<OutType, 4096, 4096, 4096, 64, 256, 32, 32, W22>(A, B, C, stream);
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE, "single-stage LDS GEMM is instantiated for 128x64x256 and "
+                                                   "4096^3 only");
+          }
+          return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the reference-style GEMM kernels write f32 only");
+        default:
+            return fail(TCU_ERR_INVALID_ARGUMENT, "unknown GEMM algo");
+    }
+}
+
+// ---------------------------------------------------------------------------- b2b GEMM
+template <typename OutType, int kN, int kK, int kP, int kTM, int kTN, typename WarpLayout>
+int launch_b2b(const __half* A, const __half* B, const __half* C, OutType* D, int M, int batch, hipStream_t stream) {
+    using Traits = FusedGemmTraits<__half, float, OutType, FusedGemmShape<0, kN, kK, kP>,
+                                   FusedGemmShape<kTM, kTN, kK, kP>, WarpLayout>;
+    auto kernel = &KeFusedGemm<__half, OutType, Traits>;
+    return launch(kernel, dim3(M / kTM, 1, batch), dim3(Traits::kThreads), Traits::kShmBytes, stream, A, B, C, D, M);
+}
+
+template <typename OutType>
+int b2b_dispatch(const __half* A, const __half* B, const __half* C, OutType* D, int M, int N, int K, int P, int batch,
+                 hipStream_t stream) {
+    if (N == 256 && K == 128 && P == 128) {
+        // 32-row tiles keep all 256 CUs busy up to M * batch = 8192; 64-row tiles beyond that
+        if (M % 64 == 0 && (long)M * batch > 16384)
+            return launch_b2b<OutType, 256, 128, 128, 64, 64, tl::RowMajor<4, 1>>(A, B, C, D, M, batch, stream);
+        if (M % 32 == 0) return launch_b2b<OutType, 256, 128, 128, 32, 64, tl::RowMajor<2, 1>>(A, B, C, D, M, batch, stream);
+    }
+    if (N == 128 && K == 64 && P == 64 && M % 32 == 0)
+        return launch_b2b<OutType, 128, 64, 64, 32, 64, tl::RowMajor<2, 1>>(A, B, C, D, M, batch, stream);
+    if (N == 64 && K == 64 && P == 64 && M % 16 == 0)
+        return launch_b2b<OutType, 64, 64, 64, 16, 32, tl::RowMajor<1, 1>>(A, B, C, D, M, batch, stream);
+    return fail(TCU_ERR_UNSUPPORTED_SHAPE,
+                "b2b GEMM is instantiated for (N, K, P) in {(256,128,128), (128,64,64), (64,64,64)} with M a "
+                "multiple of 32 (16 for the last)");
+}
+
+// ---------------------------------------------------------------------------- attention
+template <int kNStatic, int kD, bool kVRowMajor, int kTM, int kTN, typename WarpLayout>
+int launch_fa(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
+              hipStream_t stream) {
+    using Traits = FlashAttentionTraits<__half, float, __half, FlashAttentionShape<0, kNStatic, kD, kD>,
+                                        FlashAttentionShape<kTM, kTN, kD, kD>, kVRowMajor, WarpLayout>;
+    auto kernel = &flash_attention<__half, __half, Traits>;
+    return launch(kernel, dim3(M / kTM, 1, batch), dim3(Traits::kThreads), Traits::kShmBytes, stream, Q, K, V, O, M, N,
+                  scale);
+}
+
+int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, int Kd, int P,
+                float scale, int v_layout, hipStream_t stream) {
+    using W41 = tl::RowMajor<4, 1>;
+    if (Kd != P) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs the query and value head sizes equal");
+    if (M % 64 != 0 || N % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs M % 64 == 0 and N % 64 == 0");
+    if (v_layout == TCU_V_ROW_MAJOR) {
+        if (Kd == 128) return launch_fa<0, 128, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+        if (Kd == 64) return launch_fa<0, 64, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
+    }
+    if (v_layout == TCU_V_COL_MAJOR) {
+        if (Kd != 128) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for head size 128");
+        // a column-major V has leading dimension N: one instantiation per N, as in the reference op
+        switch (N) {
+            case 64: return launch_fa<64, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+            case 128: return launch_fa<128, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+            case 256: return launch_fa<256, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+            case 2048: return launch_fa<2048, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+            default:
+                return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for N in {64, 128, 256, 2048}");
+        }
+    }
+    return fail(TCU_ERR_INVALID_ARGUMENT, "unknown v_layout");
+}
+
+// ---------------------------------------------------------------------------- LSTM
+template <int kI, int kH, int kTM, int kTH, int kTK, typename WarpLayout>
+int launch_lstm(const __half* x, const __half* W, const __half* bias, const __half* h0, const float* c0,
+                __half* h_all, float* c_out, int T, int B, hipStream_t stream) {
+    using Traits = LstmCellTraits<__half, float, kI, kH, kTM, kTH, kTK, WarpLayout>;
+    auto kernel = &lstm_cell<__half, Traits>;
+    for (int t = 0; t < T; ++t) {
+        const __half* x_t = x + size_t(t) * B * kI;
+        const __half* h_in = t == 0 ? h0 : h_all + size_t(t - 1) * B * kH;
+        const float* c_in = t == 0 ? c0 : c_out;
+        __half* h_out = h_all + size_t(t) * B * kH;
+        int rc = launch(kernel, dim3(B / kTM, kH / kTH), dim3(Traits::kThreads), Traits::kShmBytes, stream, x_t, h_in,
+                        W, bias, c_in, c_out, h_out);
+        if (rc != TCU_OK) return rc;
+    }
+    return TCU_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tcu_version(void) { return 100; }
+
+const char* tcu_last_error(void) { return g_last_error.c_str(); }
+
+int tcu_device_count(void) {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) return fail(TCU_ERR_NO_DEVICE, std::string("hipGetDeviceCount: ") + hipGetErrorString(e));
+    return n;
+}
+
+int tcu_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K, int out_dtype, int algo, void* stream) {
+    if (!A || !B || !C) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16: null pointer");
+    if (!positive({M, N, K})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16: sizes must be positive");
+    auto s = static_cast<hipStream_t>(stream);
+    auto a = static_cast<const __half*>(A), b = static_cast<const __half*>(B);
+    if (out_dtype == TCU_DTYPE_F32) return gemm_dispatch<float>(a, b, static_cast<float*>(C), M, N, K, algo, s);
+    if (out_dtype == TCU_DTYPE_F16) {
+        if (algo == TCU_GEMM_GLOBAL_REG || algo == TCU_GEMM_ALL_MEM)
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the reference-style GEMM kernels write f32 (their accumulator type)");
+        return gemm_dispatch<__half>(a, b, static_cast<__half*>(C), M, N, K, algo, s);
+    }
+    return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16: out_dtype must be TCU_DTYPE_F32 or TCU_DTYPE_F16");
+}
+
+int tcu_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D, int M, int N, int K, int P, int batch,
+                     int out_dtype, void* stream) {
+    if (!A || !B || !C || !D) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: null pointer");
+    if (!positive({M, N, K, P, batch}))
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: sizes must be positive");
+    auto s = static_cast<hipStream_t>(stream);
+    auto a = static_cast<const __half*>(A), b = static_cast<const __half*>(B), c = static_cast<const __half*>(C);
+    if (out_dtype == TCU_DTYPE_F32) return b2b_dispatch<float>(a, b, c, static_cast<float*>(D), M, N, K, P, batch, s);
+    if (out_dtype == TCU_DTYPE_F16) return b2b_dispatch<__half>(a, b, c, static_cast<__half*>(D), M, N, K, P, batch, s);
+    return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: out_dtype must be TCU_DTYPE_F32 or TCU_DTYPE_F16");
+}
+
+int tcu_flash_attn_fwd_f16(const void* Q, const void* K, const void* V, void* O, int batch, int M, int N, int Kdim,
+                           int P, float scale, int v_layout, void* stream) {
+    if (!Q || !K || !V || !O) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_flash_attn_fwd_f16: null pointer");
+    if (!positive({batch, M, N, Kdim, P}))
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_flash_attn_fwd_f16: sizes must be positive");
+    return fa_dispatch(static_cast<const __half*>(Q), static_cast<const __half*>(K), static_cast<const __half*>(V),
+                       static_cast<__half*>(O), batch, M, N, Kdim, P, scale, v_layout,
+                       static_cast<hipStream_t>(stream));
+}
+
+int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                 void* c_out, int T, int B, int I, int H, void* stream) {
+    if (!x || !W || !bias || !h_all || !c_out) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: null pointer");
+    if (!positive({T, B, I, H})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: sizes must be positive");
+    auto s = static_cast<hipStream_t>(stream);
+    auto xp = static_cast<const __half*>(x), wp = static_cast<const __half*>(W), bp = static_cast<const __half*>(bias);
+    auto h0p = static_cast<const __half*>(h0);
+    auto c0p = static_cast<const float*>(c0);
+    auto hp = static_cast<__half*>(h_all);
+    auto cp = static_cast<float*>(c_out);
+    if (B % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16: batch must be a multiple of 64");
+    if (I == 1024 && H == 1024)
+        return launch_lstm<1024, 1024, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+    if (I == 128 && H == 128)
+        return launch_lstm<128, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+    if (I == 64 && H == 128)
+        return launch_lstm<64, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+    return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16 is instantiated for (I, H) in {(1024,1024), (128,128), (64,128)}");
+}
+
+}  // extern "C"
