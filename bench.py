@@ -125,7 +125,7 @@ def main():
         d3a, d3b, d3c = to_dev(A3), to_dev(B3), to_dev(C3)
         d3d = torch.empty(1, M, P, dtype=torch.float16, device=dev)
         ms = time_kernel(lambda: tcu.b2b_gemm(d3a, d3b, d3c, out=d3d), args.steps, args.warmup)
-        err = oracle.max_rel_err(d3d[0].float().cpu().numpy(), oracle.b2b_gemm(A3, B3, C3))
+        err = oracle.max_rel_err(d3d[0].float().cpu().numpy(), oracle.b2b_gemm(A3, B3, C3), eps=1.0)
         flops = 2.0 * M * K * N + 2.0 * M * N * P
         nbytes = 2.0 * (M * K + N * K + P * N + M * P)
         configs.append({"name": "b2b_8192x256x128x128", "ms": ms, "us": ms * 1e3, "tflops": flops / (ms * 1e-3) / 1e12,

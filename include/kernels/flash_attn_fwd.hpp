@@ -1,0 +1,242 @@
+// FlashAttention-2 forward for gfx950, O = softmax(scale · Q·Kᵀ)·V, f16 in/out, f32 statistics.
+// The tuned counterpart of kernels/flash_attn.hpp (which composes the generic 16x16 tile
+// primitives, as the reference's src/kernels/flash_attn.cu:134-312 does). Layouts: Q [M, D],
+// K [N, D], V [N, D], O [M, D] row-major per batch item (the usual [seq, head_dim]).
+//
+// Design (per workgroup: kWaves wavefronts x 32 query rows; K/V streamed in blocks of kBN keys):
+//   * Sᵀ = K·Qᵀ with v_mfma_f32_32x32x16_f16: the accumulator of a 32x32 tile then gives every
+//     lane 16 keys of ONE query (column = lane % 32), so the online-softmax row maximum and
+//     row sum are in-lane reductions plus one exchange with lane ^ 32, and the rescale factor
+//     is a per-lane scalar;
+//   * Oᵀ = Vᵀ·Pᵀ: exp(Sᵀ - m) converted to f16 is directly the B operand (the contraction
+//     index of an MFMA may be permuted freely as long as both operands agree: slot e of k-step
+//     s of lane half h is key 16 s + 8 (e / 4) + 4 h + e % 4); Vᵀ comes from the row-major V
+//     tile in LDS through the transposing read ds_read_b64_tr_b16, two per operand;
+//   * Q stays in registers for the whole kernel (it is read from HBM once, where the
+//     reference re-reads it for every key block, flash_attn.cu:241);
+//   * K and V blocks go global -> LDS directly (16 B per lane, no register staging), double
+//     buffered: block j+1 is in flight while block j is consumed; one barrier per block;
+//   * LDS rows are 2 * kD bytes. K: the 16-byte chunks of a row are XOR-ed with the row index
+//     (ds_read_b128 of 16 consecutive rows at one chunk hits all 64 banks once). V: the
+//     32-byte units of a row are XOR-ed with a function of the row so that the 4 rows x 32 B
+//     read by each 16-lane group of a transposing read, and the two groups of a half-wave,
+//     fall on distinct banks. Both permutations are applied on the global-address side;
+//   * softmax runs in the log2 domain: p = exp2(s * scale * log2(e) - m).
+// M % (32 * kWaves) == 0 and N % kBN == 0 are required (checked by the host launcher).
+#pragma once
+
+#include "config.hpp"
+#include "hip_utils.hpp"
+#include "kernels/gemm_pipelined.hpp"  // detail::load_lds_16B
+
+namespace tiledcuda::kernels {
+
+template <const int kD_, const int kWaves_, const int kBN_ = 64>
+struct FlashFwdTraits {
+    static constexpr int kD = kD_, kWaves = kWaves_, kBN = kBN_;
+    static constexpr int kBM = 32 * kWaves;
+    static constexpr int kThreads = kWaves * kWaveSize;
+    static constexpr int kRowBytes = 2 * kD;             // 256 for D = 128
+    static constexpr int kTileBytes = kBN * kRowBytes;   // one K or V block
+    static constexpr int kStageBytes = 2 * kTileBytes;   // K + V
+    static constexpr int kRowsPerLoad = 1024 / kRowBytes;
+    static constexpr int kLoadsPerTile = kBN / kRowsPerLoad;  // 1 KiB instructions per K (or V) block
+    static constexpr int kDSteps = kD / 16;   // k-steps of Sᵀ = K Qᵀ
+    static constexpr int kDTiles = kD / 32;   // 32-row tiles of Oᵀ
+    static constexpr int kKvTiles = kBN / 32; // 32-row tiles of Sᵀ
+    static constexpr int kKvSteps = kBN / 16; // k-steps of Oᵀ = Vᵀ Pᵀ
+    static_assert(kD == 128 || kD == 64, "head size 64 or 128");
+    static_assert(kBN % 32 == 0);
+    static_assert((2 * kLoadsPerTile) % kWaves == 0 || kWaves % (2 * kLoadsPerTile) == 0);
+    static constexpr int kLdsBytes = 2 * kStageBytes > kBM * kRowBytes ? 2 * kStageBytes : kBM * kRowBytes;
+
+    /// XOR applied to the 16-byte chunk index of K row `row`.
+    HOST_DEVICE static constexpr int k_swz(int row) { return row & (kRowBytes / 16 - 1) & 15; }
+    /// XOR applied to the 32-byte unit index of V row `row`: rows 4 a .. 4 a + 3 at one unit, and the two
+    /// 16-lane groups of a half-wave (adjacent units), must fall on 8 distinct 32-byte bank slots.
+    /// 256-byte rows all start on bank 0: spread the 4 rows over units with 2 * (row % 4).
+    /// 128-byte rows alternate between the two halves of the banks: only rows 2 apart collide: row & 2.
+    HOST_DEVICE static constexpr int v_swz(int row) { return kRowBytes == 256 ? ((row & 3) << 1) : (row & 2); }
+};
+
+namespace detail {
+DEVICE float exchange32(float v) { return __shfl_xor(v, 32, 64); }
+}  // namespace detail
+
+/// grid = (M / kBM, batch), block = Traits::kThreads, dynamic LDS = Traits::kLdsBytes.
+template <typename Traits>
+__global__ void __launch_bounds__(Traits::kThreads)
+    flash_attention_fwd(const __half* __restrict__ Q, const __half* __restrict__ K, const __half* __restrict__ V,
+                        __half* __restrict__ O, int M, int N, float scale) {
+    constexpr int kD = Traits::kD, kBN = Traits::kBN, kWaves = Traits::kWaves;
+    constexpr int kRowBytes = Traits::kRowBytes;
+    constexpr int kChunks = kRowBytes / 16;  // 16-byte chunks per row
+    extern __shared__ __align__(1024) unsigned char lds[];
+
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+    const int q32 = lane & 31;  // query (column of Sᵀ / Oᵀ) owned by this lane
+    const int h = lane >> 5;    // lane half
+
+    const size_t head = blockIdx.y;
+    const int m0 = blockIdx.x * Traits::kBM + wave * 32;
+    const __half* Qh = Q + (head * M + m0) * kD;
+    const __half* Kh = K + head * size_t(N) * kD;
+    const __half* Vh = V + head * size_t(N) * kD;
+    __half* Oh = O + (head * M + m0) * kD;
+
+    // ---- Q fragments: B operand of Sᵀ = K Qᵀ: lane (q, h) holds Q[q][16 s + 8 h .. + 7] for k-step s
+    f16x8 qf[Traits::kDSteps];
+#pragma unroll
+    for (int s = 0; s < Traits::kDSteps; ++s)
+        qf[s] = *reinterpret_cast<const f16x8*>(Qh + size_t(q32) * kD + 16 * s + 8 * h);
+
+    // ---- global -> LDS for a K/V block. One instruction fills kRowsPerLoad rows.
+    // The 2 * kLoadsPerTile instructions of a block (K first, then V) are dealt round-robin to the wavefronts.
+    constexpr int kLoadsPerBlock = 2 * Traits::kLoadsPerTile;
+    constexpr int kLoadsPerWave = (kLoadsPerBlock + kWaves - 1) / kWaves;
+    const int lrow = lane / kChunks;  // row within the instruction's rows
+    const int lchk = lane % kChunks;  // physical 16-byte chunk
+    auto issue_block = [&](int stage, int n0) {
+        unsigned char* sk = lds + stage * Traits::kStageBytes;
+#pragma unroll
+        for (int j = 0; j < kLoadsPerWave; ++j) {
+            const int idx = wave + j * kWaves;  // wave-uniform
+            if (kLoadsPerBlock % kWaves == 0 || idx < kLoadsPerBlock) {
+                const bool is_v = idx >= Traits::kLoadsPerTile;
+                const int t = is_v ? idx - Traits::kLoadsPerTile : idx;
+                const int row = t * Traits::kRowsPerLoad + lrow;
+                // physical chunk lchk holds logical chunk (K: ^ row % 16; V: 32-byte unit ^ 2 * (row % 4))
+                const int chunk = is_v ? (lchk ^ (Traits::v_swz(row) << 1)) : (lchk ^ Traits::k_swz(row));
+                const __half* src = (is_v ? Vh : Kh) + size_t(n0 + row) * kD + chunk * 8;
+                detail::load_lds_16B(src, sk + (is_v ? Traits::kTileBytes : 0) + t * 1024);
+            }
+        }
+    };
+
+    // ---- accumulators and statistics (log2 domain)
+    f32x16 o_acc[Traits::kDTiles];
+#pragma unroll
+    for (int t = 0; t < Traits::kDTiles; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o_acc[t][e] = 0.f;
+    float m_run = -INFINITY;  // running max of s * c, shared by lanes l and l ^ 32
+    float l_run = 0.f;        // this lane's share of the running sum
+    const float c = scale * 1.4426950408889634f;
+
+    const int nblocks = N / kBN;
+    issue_block(0, 0);
+
+    for (int j = 0; j < nblocks; ++j) {
+        const int stage = j & 1;
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my share of block j has landed
+        __syncthreads();                      // everyone's share landed; everyone is done with block j-1
+        if (j + 1 < nblocks) issue_block(stage ^ 1, (j + 1) * kBN);
+
+        const unsigned char* sk = lds + stage * Traits::kStageBytes;
+        const unsigned char* sv = sk + Traits::kTileBytes;
+
+        // ---- Sᵀ[kv, q] = K[kv, :] · Q[q, :]
+        f32x16 s_acc[Traits::kKvTiles];
+#pragma unroll
+        for (int t = 0; t < Traits::kKvTiles; ++t) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s_acc[t][e] = 0.f;
+            const int row = t * 32 + q32;  // key row read by this lane (A operand: row = lane % 32)
+#pragma unroll
+            for (int s = 0; s < Traits::kDSteps; ++s) {
+                const int chunk = (2 * s + h) ^ Traits::k_swz(row);
+                const f16x8 kf = *reinterpret_cast<const f16x8*>(sk + row * kRowBytes + chunk * 16);
+                s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], s_acc[t], 0, 0, 0);
+            }
+        }
+
+        // ---- online softmax for query q32: this lane holds keys 32 t + 8 (r / 4) + 4 h + r % 4
+        float mx = s_acc[0][0];
+#pragma unroll
+        for (int t = 0; t < Traits::kKvTiles; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[t][e]);
+        mx = fmaxf(mx, detail::exchange32(mx));
+        const float m_new = fmaxf(m_run, mx * c);
+        const float alpha = exp2f(m_run - m_new);  // exp2(-inf) = 0 on the first block
+        m_run = m_new;
+        float psum = 0.f;
+        f16x8 pf[Traits::kKvSteps];
+#pragma unroll
+        for (int t = 0; t < Traits::kKvTiles; ++t) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float p = exp2f(s_acc[t][e] * c - m_new);
+                psum += p;
+                pf[2 * t + e / 8][e % 8] = static_cast<_Float16>(p);
+            }
+        }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int t = 0; t < Traits::kDTiles; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o_acc[t][e] *= alpha;
+
+        // ---- Oᵀ[d, q] += Vᵀ[d, kv] · Pᵀ[kv, q]
+        // A operand for (d tile dt, k-step s): lane (d = 32 dt + lane % 32, h), slot e = key 16 s + 8 (e / 4) + 4 h + e % 4,
+        // fetched with two transposing reads (4 consecutive keys of one d each). Within a 16-lane group, lane L
+        // supplies the address of row kv0 + L / 4, columns dbase + 4 (L % 4) .. + 3.
+        const int g = lane >> 4, L = lane & 15;
+        const int vrow_in = L >> 2;                    // 0..3: row within the 4-key group
+        const int vcol_b = (16 * (g & 1) + 4 * (L & 3)) * 2;  // byte offset of the lane's 4 columns inside the 32-d tile
+#pragma unroll
+        for (int dt = 0; dt < Traits::kDTiles; ++dt) {
+#pragma unroll
+            for (int s = 0; s < Traits::kKvSteps; ++s) {
+                f16x8 vf;
+#pragma unroll
+                for (int part = 0; part < 2; ++part) {
+                    const int row = 16 * s + 8 * part + 4 * h + vrow_in;
+                    const int byte_in_row = 64 * dt + vcol_b;  // multiple of 8
+                    const int unit = (byte_in_row >> 5) ^ Traits::v_swz(row);
+                    const unsigned char* p = sv + row * kRowBytes + unit * 32 + (byte_in_row & 31);
+                    using fp16x4 = __fp16 __attribute__((ext_vector_type(4)));
+                    const fp16x4 v4 = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+                        (fp16x4 __attribute__((address_space(3)))*)(p));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) vf[4 * part + e] = static_cast<_Float16>(v4[e]);
+                }
+                o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[s], o_acc[dt], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- epilogue: O[q, d] = Oᵀ[d, q] / l. acc[dt][r]: d = 32 dt + 8 (r / 4) + 4 h + r % 4, q = q32.
+    const float l_tot = l_run + detail::exchange32(l_run);
+    const float inv_l = 1.0f / l_tot;
+    __syncthreads();  // all wavefronts are done with the K/V stages: reuse LDS for staging
+    unsigned char* stg = lds + wave * (32 * kRowBytes);
+    // 8-byte slots of a staged row (4 consecutive d) are XOR-ed with 2 * (row % 16) within the row
+    constexpr int kSlotMask = (kRowBytes / 8 - 1) & ~1;
+#pragma unroll
+    for (int dt = 0; dt < Traits::kDTiles; ++dt) {
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            f16x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(o_acc[dt][4 * qd + e] * inv_l);
+            const int slot = (32 * dt + 8 * qd + 4 * h) >> 2;
+            const int pslot = slot ^ (((q32 & 15) << 1) & kSlotMask);
+            *reinterpret_cast<f16x4*>(stg + q32 * kRowBytes + pslot * 8) = v;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    constexpr int kLanesPerRow = kRowBytes / 16;
+    constexpr int kRowsPerIter = kWaveSize / kLanesPerRow;
+    const int rr = lane / kLanesPerRow, cc = lane % kLanesPerRow;
+#pragma unroll
+    for (int it = 0; it < 32 / kRowsPerIter; ++it) {
+        const int row = it * kRowsPerIter + rr;
+        const int pslot = (2 * cc) ^ (((row & 15) << 1) & kSlotMask);
+        const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kRowBytes + pslot * 8);
+        *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(Oh + size_t(row) * kD) + cc * 16) = v;
+    }
+}
+
+}  // namespace tiledcuda::kernels

@@ -236,7 +236,9 @@ __global__ void __launch_bounds__(Traits::kThreads)
         constexpr int kPitch = kWaveN * 2;  // bytes per staged row
         unsigned char* stg = lds + wave * (kWaveM * kPitch);
         // write: lane owns row (i*32 + frow); 4 halves (8 B) at column j*32 + 8*q + 4*fhalf.
-        // 8-byte slots of a row are XOR-ed with (row % 16) * 2 (bit 0 untouched) to spread banks.
+        // 8-byte slots of a row are XOR-ed with (row % 16) * 2 (bit 0 untouched, kept inside the row)
+        // to spread banks.
+        constexpr int kSlotMask = (kPitch / 8 - 1) & ~1;
 #pragma unroll
         for (int i = 0; i < kMT; ++i) {
             const int row = i * 32 + frow;
@@ -245,7 +247,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int slot = (j * 32 + 8 * q + 4 * fhalf) >> 2;  // 8-byte slot index in the row
-                    const int pslot = slot ^ ((row & 15) << 1);
+                    const int pslot = slot ^ (((row & 15) << 1) & kSlotMask);
                     f16x4 v;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc[i][j][4 * q + e]);
@@ -263,7 +265,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
 #pragma unroll
         for (int it = 0; it < kWaveM / kRowsPerIter; ++it) {
             const int row = it * kRowsPerIter + rr;
-            const int pslot = (2 * cc) ^ ((row & 15) << 1);
+            const int pslot = (2 * cc) ^ (((row & 15) << 1) & kSlotMask);
             const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kPitch + pslot * 8);
             *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(cbase + size_t(row) * N) + cc * 16) = v;
         }

@@ -40,6 +40,13 @@ typedef enum {
     TCU_V_ROW_MAJOR = 1  /* V stored [N, P] per batch item: the usual [seq, head_dim] */
 } tcu_v_layout;
 
+/* Which attention kernel to run (tcu_flash_attn_fwd_f16_algo). AUTO picks MFMA32 for a row-major V. */
+typedef enum {
+    TCU_ATTN_AUTO = 0,
+    TCU_ATTN_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, like the reference kernel */
+    TCU_ATTN_MFMA32 = 2        /* 32x32x16 MFMA, transposing LDS reads, direct-to-LDS K/V (row-major V only) */
+} tcu_attn_algo;
+
 /* Library version (major * 10000 + minor * 100 + patch). */
 int tcu_version(void);
 
@@ -77,6 +84,10 @@ int tcu_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D, int M
  */
 int tcu_flash_attn_fwd_f16(const void* Q, const void* K, const void* V, void* O, int batch, int M, int N, int Kdim,
                            int P, float scale, int v_layout, void* stream);
+
+/* tcu_flash_attn_fwd_f16 with an explicit kernel choice (tcu_attn_algo); same arguments otherwise. */
+int tcu_flash_attn_fwd_f16_algo(const void* Q, const void* K, const void* V, void* O, int batch, int M, int N,
+                                int Kdim, int P, float scale, int v_layout, int algo, void* stream);
 
 /*
  * Fused LSTM layer over T steps. x [T, B, I] f16; W [4H, I+H] f16 row-major, gate rows in the

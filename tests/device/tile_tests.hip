@@ -61,7 +61,6 @@ __global__ void __launch_bounds__(512) k_s2r_row_major(const Element* src, Eleme
     constexpr int kWR = tl::num_rows<WarpLayout>;
     constexpr int kMs = kRows / kWR / 16, kKs = kChunk / 16;
     using Reg = RegTile<BaseTileRowMajor<Element>, tl::RowMajor<kMs, kKs>>;
-    using OutGlobal = GlobalTile<Element, tl::RowMajor<kRows, kChunk, kCols>>;
 
     Global g_src(src);
     Shared s(smem);
@@ -77,16 +76,14 @@ __global__ void __launch_bounds__(512) k_s2r_row_major(const Element* src, Eleme
         Reg r;
         s2r(iter(k), r);
         if (Base::warp_col_id() == 0) {
-            // write this wavefront-row's block back with a single-column wavefront layout
-            using OutWarps = tl::RowMajor<kWR, 1>;
-            OutGlobal g_out(dst + k * kChunk);
-            // emulate a kWR x 1 layout: wavefront row = warp_row_id()
-            Element* p = g_out.mutable_data() + Base::warp_row_id() * (kRows / kWR) * kCols;
-            using Sub = GlobalTile<Element, tl::RowMajor<kRows / kWR, kChunk, kCols>>;
-            Sub sub(p);
-            RegToGlobalStorer<Sub, Reg, tl::RowMajor<1, 1>> r2g;
-            (void)sizeof(OutWarps);
-            r2g(r, sub);
+            // write this wavefront-row's block back, BaseTile by BaseTile (wavefronts of one row hold copies)
+            Element* block = dst + Base::warp_row_id() * (kRows / kWR) * kCols + k * kChunk;
+#pragma unroll
+            for (int i = 0; i < kMs; ++i)
+#pragma unroll
+                for (int j = 0; j < kKs; ++j)
+                    copy::detail::move_base_tile<Element, const typename Reg::DType, kCols, 1, false>(
+                        block + i * 16 * kCols + j * 16, r(i, j));
         }
     }
 }
@@ -117,10 +114,13 @@ __global__ void __launch_bounds__(512) k_s2r_col_major(const Element* src, Eleme
         Reg r;
         s2r(iter(k), r);
         if (Base::warp_row_id() == 0) {
-            using Sub = GlobalTile<Element, tl::ColMajor<kChunk, kCols / kWC, kRows>>;
-            Sub sub(dst + k * kChunk + Base::warp_col_id() * (kCols / kWC) * kRows);
-            RegToGlobalStorer<Sub, Reg, tl::RowMajor<1, 1>> r2g;
-            r2g(r, sub);
+            Element* block = dst + k * kChunk + Base::warp_col_id() * (kCols / kWC) * kRows;
+#pragma unroll
+            for (int i = 0; i < kKs; ++i)
+#pragma unroll
+                for (int j = 0; j < kNs; ++j)
+                    copy::detail::move_base_tile<Element, const typename Reg::DType, 1, kRows, false>(
+                        block + i * 16 + j * 16 * kRows, r(i, j));
         }
     }
 }

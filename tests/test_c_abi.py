@@ -20,7 +20,7 @@ def declared_symbols():
 
 def test_header_declares_the_entry_points():
     syms = declared_symbols()
-    for name in ("tcu_gemm_f16", "tcu_b2b_gemm_f16", "tcu_flash_attn_fwd_f16", "tcu_lstm_f16", "tcu_last_error",
+    for name in ("tcu_gemm_f16", "tcu_b2b_gemm_f16", "tcu_flash_attn_fwd_f16", "tcu_lstm_f16", "tcu_flash_attn_fwd_f16_algo", "tcu_last_error",
                  "tcu_version", "tcu_device_count"):
         assert name in syms
 
@@ -94,5 +94,7 @@ def test_tile_test_library_loads():
     path = os.path.join(ROOT, "tests", "device", "_build", "libtcu_tile_tests.so")
     if not os.path.exists(path):
         pytest.skip("device test library not built")
+    import torch  # noqa: F401  (load torch's HIP runtime first, as every user of the library does)
+
     handle = ctypes.CDLL(path)
     assert handle.tt_num_cases() > 50

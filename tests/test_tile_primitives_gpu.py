@@ -6,6 +6,7 @@ import os
 
 import numpy as np
 import pytest
+import torch  # before any HIP library is loaded: the process must share torch's HIP runtime
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "tests", "device", "_build", "libtcu_tile_tests.so")

@@ -18,7 +18,7 @@ import torch
 
 __all__ = [
     "TcuError", "library_path", "lib", "last_error", "gemm", "b2b_gemm", "flash_attention_fwd",
-    "flash_attention", "TiledFlashAttention", "lstm", "GEMM_ALGOS",
+    "flash_attention", "TiledFlashAttention", "lstm", "GEMM_ALGOS", "ATTN_ALGOS",
 ]
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -39,6 +39,8 @@ GEMM_ALGOS = {"auto": 0, "global_reg": 1, "all_mem": 2, "pipelined": 3}
 TCU_V_COL_MAJOR = 0
 TCU_V_ROW_MAJOR = 1
 
+ATTN_ALGOS = {"auto": 0, "tile_library": 1, "mfma32": 2}
+
 # every exported symbol with its ctypes signature (also what the symbol test checks)
 _SIGNATURES = {
     "tcu_version": (ctypes.c_int, []),
@@ -48,6 +50,8 @@ _SIGNATURES = {
     "tcu_b2b_gemm_f16": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 6 + [ctypes.c_void_p]),
     "tcu_flash_attn_fwd_f16": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int,
                                                                                            ctypes.c_void_p]),
+    "tcu_flash_attn_fwd_f16_algo": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int,
+                                                                                                ctypes.c_int, ctypes.c_void_p]),
     "tcu_lstm_f16": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
 }
 
@@ -167,7 +171,7 @@ def flash_attention_fwd(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, O: to
 
 
 def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float | None = None,
-                    out: torch.Tensor | None = None) -> torch.Tensor:
+                    out: torch.Tensor | None = None, algo: str = "auto") -> torch.Tensor:
     """softmax(scale · q kᵀ) v for [..., S, D] tensors in the usual layout (V row-major [S, D]).
     ``scale`` defaults to 1/sqrt(D)."""
     *lead, M, D = q.shape
@@ -178,9 +182,10 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: fl
         scale = 1.0 / math.sqrt(D)
     if out is None:
         out = torch.empty(*lead, M, P, dtype=torch.float16, device=q.device)
-    _check(lib().tcu_flash_attn_fwd_f16(_dev_ptr(q, torch.float16, "q"), _dev_ptr(k, torch.float16, "k"),
-                                        _dev_ptr(v, torch.float16, "v"), _dev_ptr(out, torch.float16, "out"), batch,
-                                        M, N, D, P, float(scale), TCU_V_ROW_MAJOR, _stream()))
+    _check(lib().tcu_flash_attn_fwd_f16_algo(_dev_ptr(q, torch.float16, "q"), _dev_ptr(k, torch.float16, "k"),
+                                             _dev_ptr(v, torch.float16, "v"), _dev_ptr(out, torch.float16, "out"),
+                                             batch, M, N, D, P, float(scale), TCU_V_ROW_MAJOR, ATTN_ALGOS[algo],
+                                             _stream()))
     return out
 
 

@@ -3,10 +3,14 @@
 // synchronised; errors become status codes plus a thread-local message.
 #include "tcu_c_api.h"
 
+#include "kernels/flash_attn_fwd.hpp"
 #include "kernels/gemm_pipelined.hpp"
 #include "kernels/mod.hpp"
 
+#include <mutex>
+#include <set>
 #include <string>
+#include <utility>
 
 using namespace tiledcuda;
 using namespace tiledcuda::kernels;
@@ -15,6 +19,10 @@ namespace tl = tiledcuda::cell::tile_layout;
 namespace {
 
 thread_local std::string g_last_error;
+
+// kernels whose dynamic-LDS limit has already been raised, per device
+std::mutex g_attr_mutex;
+std::set<std::pair<const void*, int>> g_attr_done;
 
 int fail(int code, const std::string& msg) {
     g_last_error = msg;
@@ -30,9 +38,22 @@ template <typename Kernel, typename... Args>
 int launch(Kernel kernel, dim3 grid, dim3 block, int lds_bytes, hipStream_t stream, Args... args) {
     if (lds_bytes > kMaxLdsBytes) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "kernel needs more LDS than a CU has");
     if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+        // once per kernel function (and per device: the attribute is per device)
+        int device = 0;
+        (void)hipGetDevice(&device);
+        const auto key = std::make_pair(reinterpret_cast<const void*>(kernel), device);
+        bool known;
+        {
+            std::lock_guard<std::mutex> lock(g_attr_mutex);
+            known = g_attr_done.count(key) != 0;
+        }
+        if (!known) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
+            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+            std::lock_guard<std::mutex> lock(g_attr_mutex);
+            g_attr_done.insert(key);
+        }
     }
     hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args...);
     hipError_t e = hipGetLastError();
@@ -78,7 +99,7 @@ int launch_pipelined(const __half* A, const __half* B, OutType* C, int M, int N,
                   M, N, K);
 }
 
-using PipeLarge = PipelinedGemmTraits<256, 256, 64, 2, 2, 2>;
+using PipeLarge = PipelinedGemmTraits<256, 256, 64, 4, 2, 2>;  // 8 wavefronts, 2 per SIMD
 using PipeMid = PipelinedGemmTraits<128, 128, 64, 2, 2, 2>;
 using PipeSmall = PipelinedGemmTraits<64, 64, 64, 2, 2, 2>;
 
@@ -164,11 +185,37 @@ int launch_fa(const __half* Q, const __half* K, const __half* V, __half* O, int 
                   scale);
 }
 
+template <int kD, int kWaves>
+int launch_fa_fwd(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
+                  hipStream_t stream) {
+    using Traits = FlashFwdTraits<kD, kWaves, 64>;
+    auto kernel = &flash_attention_fwd<Traits>;
+    return launch(kernel, dim3(M / Traits::kBM, batch), dim3(Traits::kThreads), Traits::kLdsBytes, stream, Q, K, V, O,
+                  M, N, scale);
+}
+
+template <int kD>
+int fa_fwd_by_rows(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
+                   hipStream_t stream) {
+    if (M % 256 == 0) return launch_fa_fwd<kD, 8>(Q, K, V, O, batch, M, N, scale, stream);
+    if (M % 128 == 0) return launch_fa_fwd<kD, 4>(Q, K, V, O, batch, M, N, scale, stream);
+    return launch_fa_fwd<kD, 2>(Q, K, V, O, batch, M, N, scale, stream);
+}
+
 int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, int Kd, int P,
-                float scale, int v_layout, hipStream_t stream) {
+                float scale, int v_layout, int algo, hipStream_t stream) {
     using W41 = tl::RowMajor<4, 1>;
     if (Kd != P) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs the query and value head sizes equal");
     if (M % 64 != 0 || N % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs M % 64 == 0 and N % 64 == 0");
+    if (algo != TCU_ATTN_AUTO && algo != TCU_ATTN_TILE_LIBRARY && algo != TCU_ATTN_MFMA32)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "unknown attention algo");
+    if (v_layout == TCU_V_ROW_MAJOR && algo != TCU_ATTN_TILE_LIBRARY) {
+        if (Kd == 128) return fa_fwd_by_rows<128>(Q, K, V, O, batch, M, N, scale, stream);
+        if (Kd == 64) return fa_fwd_by_rows<64>(Q, K, V, O, batch, M, N, scale, stream);
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
+    }
+    if (algo == TCU_ATTN_MFMA32)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 32x32x16 attention kernel takes a row-major V");
     if (v_layout == TCU_V_ROW_MAJOR) {
         if (Kd == 128) return launch_fa<0, 128, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
         if (Kd == 64) return launch_fa<0, 64, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
@@ -248,14 +295,19 @@ int tcu_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D, int M
     return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: out_dtype must be TCU_DTYPE_F32 or TCU_DTYPE_F16");
 }
 
-int tcu_flash_attn_fwd_f16(const void* Q, const void* K, const void* V, void* O, int batch, int M, int N, int Kdim,
-                           int P, float scale, int v_layout, void* stream) {
+int tcu_flash_attn_fwd_f16_algo(const void* Q, const void* K, const void* V, void* O, int batch, int M, int N,
+                                int Kdim, int P, float scale, int v_layout, int algo, void* stream) {
     if (!Q || !K || !V || !O) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_flash_attn_fwd_f16: null pointer");
     if (!positive({batch, M, N, Kdim, P}))
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_flash_attn_fwd_f16: sizes must be positive");
     return fa_dispatch(static_cast<const __half*>(Q), static_cast<const __half*>(K), static_cast<const __half*>(V),
-                       static_cast<__half*>(O), batch, M, N, Kdim, P, scale, v_layout,
+                       static_cast<__half*>(O), batch, M, N, Kdim, P, scale, v_layout, algo,
                        static_cast<hipStream_t>(stream));
+}
+
+int tcu_flash_attn_fwd_f16(const void* Q, const void* K, const void* V, void* O, int batch, int M, int N, int Kdim,
+                           int P, float scale, int v_layout, void* stream) {
+    return tcu_flash_attn_fwd_f16_algo(Q, K, V, O, batch, M, N, Kdim, P, scale, v_layout, TCU_ATTN_AUTO, stream);
 }
 
 int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
