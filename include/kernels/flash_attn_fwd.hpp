@@ -14,14 +14,21 @@
 //     tile in LDS through the transposing read ds_read_b64_tr_b16, two per operand;
 //   * Q stays in registers for the whole kernel (it is read from HBM once, where the
 //     reference re-reads it for every key block, flash_attn.cu:241);
-//   * K and V blocks go global -> LDS directly (16 B per lane, no register staging), double
-//     buffered: block j+1 is in flight while block j is consumed; one barrier per block;
+//   * K and V blocks go global -> LDS directly (16 B per lane, no register staging) into a ring of
+//     three stages; one barrier per block;
+//   * the two wavefronts that share a SIMD run an iteration in different orders (scores of block j+1
+//     first / last), so one of them feeds the matrix pipe while the other does the softmax VALU work;
 //   * LDS rows are 2 * kD bytes. K: the 16-byte chunks of a row are XOR-ed with the row index
 //     (ds_read_b128 of 16 consecutive rows at one chunk hits all 64 banks once). V: the
 //     32-byte units of a row are XOR-ed with a function of the row so that the 4 rows x 32 B
 //     read by each 16-lane group of a transposing read, and the two groups of a half-wave,
 //     fall on distinct banks. Both permutations are applied on the global-address side;
-//   * softmax runs in the log2 domain: p = exp2(s * scale * log2(e) - m).
+//   * softmax runs in the log2 domain with as few VALU operations per score as possible: Q is
+//     multiplied by scale * log2(e) once, when it is loaded; the accumulators of Sᵀ start at -m (the
+//     running maximum of that query) instead of 0, so p = exp2(acc) with no subtraction; the maximum
+//     is only moved when a block exceeds it by more than 2^8 ("lazy rescaling": a stale maximum is
+//     harmless, p <= 2^8 stays far inside f16 / f32 range and the final division cancels it), which
+//     makes the rescale of the output accumulators a rare, wave-uniform branch.
 // M % (32 * kWaves) == 0 and N % kBN == 0 are required (checked by the host launcher).
 #pragma once
 
@@ -36,6 +43,7 @@ struct FlashFwdTraits {
     static constexpr int kD = kD_, kWaves = kWaves_, kBN = kBN_;
     static constexpr int kBM = 32 * kWaves;
     static constexpr int kThreads = kWaves * kWaveSize;
+    static constexpr int kStages = 3;
     static constexpr int kRowBytes = 2 * kD;             // 256 for D = 128
     static constexpr int kTileBytes = kBN * kRowBytes;   // one K or V block
     static constexpr int kStageBytes = 2 * kTileBytes;   // K + V
@@ -47,8 +55,8 @@ struct FlashFwdTraits {
     static constexpr int kKvSteps = kBN / 16; // k-steps of Oᵀ = Vᵀ Pᵀ
     static_assert(kD == 128 || kD == 64, "head size 64 or 128");
     static_assert(kBN % 32 == 0);
-    static_assert((2 * kLoadsPerTile) % kWaves == 0 || kWaves % (2 * kLoadsPerTile) == 0);
-    static constexpr int kLdsBytes = 2 * kStageBytes > kBM * kRowBytes ? 2 * kStageBytes : kBM * kRowBytes;
+    static constexpr int kLdsMain = kStages * kStageBytes;
+    static constexpr int kLdsBytes = kLdsMain > kBM * kRowBytes ? kLdsMain : kBM * kRowBytes;
 
     /// XOR applied to the 16-byte chunk index of K row `row`.
     HOST_DEVICE static constexpr int k_swz(int row) { return row & (kRowBytes / 16 - 1) & 15; }
@@ -61,6 +69,8 @@ struct FlashFwdTraits {
 
 namespace detail {
 DEVICE float exchange32(float v) { return __shfl_xor(v, 32, 64); }
+/// 2^x as one v_exp_f32 (no range fix-ups: arguments here are <= 8 and results below 2^-126 may flush to 0).
+DEVICE float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
 }  // namespace detail
 
 /// grid = (M / kBM, batch), block = Traits::kThreads, dynamic LDS = Traits::kLdsBytes.
@@ -71,6 +81,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     constexpr int kD = Traits::kD, kBN = Traits::kBN, kWaves = Traits::kWaves;
     constexpr int kRowBytes = Traits::kRowBytes;
     constexpr int kChunks = kRowBytes / 16;  // 16-byte chunks per row
+    constexpr int kStages = Traits::kStages;
     extern __shared__ __align__(1024) unsigned char lds[];
 
     const int lane = lane_id();
@@ -85,11 +96,16 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const __half* Vh = V + head * size_t(N) * kD;
     __half* Oh = O + (head * M + m0) * kD;
 
-    // ---- Q fragments: B operand of Sᵀ = K Qᵀ: lane (q, h) holds Q[q][16 s + 8 h .. + 7] for k-step s
+    // ---- Q fragments: B operand of Sᵀ = K Qᵀ: lane (q, h) holds Q[q][16 s + 8 h .. + 7] for k-step s,
+    // pre-multiplied by scale * log2(e) so that the scores come out of the MFMA in the log2 domain.
+    const float c = scale * 1.4426950408889634f;
     f16x8 qf[Traits::kDSteps];
 #pragma unroll
-    for (int s = 0; s < Traits::kDSteps; ++s)
-        qf[s] = *reinterpret_cast<const f16x8*>(Qh + size_t(q32) * kD + 16 * s + 8 * h);
+    for (int s = 0; s < Traits::kDSteps; ++s) {
+        const f16x8 raw = *reinterpret_cast<const f16x8*>(Qh + size_t(q32) * kD + 16 * s + 8 * h);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<_Float16>(static_cast<float>(raw[e]) * c);
+    }
 
     // ---- global -> LDS for a K/V block. One instruction fills kRowsPerLoad rows.
     // The 2 * kLoadsPerTile instructions of a block (K first, then V) are dealt round-robin to the wavefronts.
@@ -106,10 +122,27 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 const bool is_v = idx >= Traits::kLoadsPerTile;
                 const int t = is_v ? idx - Traits::kLoadsPerTile : idx;
                 const int row = t * Traits::kRowsPerLoad + lrow;
-                // physical chunk lchk holds logical chunk (K: ^ row % 16; V: 32-byte unit ^ 2 * (row % 4))
+                // physical chunk lchk holds logical chunk lchk ^ swizzle(row)
                 const int chunk = is_v ? (lchk ^ (Traits::v_swz(row) << 1)) : (lchk ^ Traits::k_swz(row));
                 const __half* src = (is_v ? Vh : Kh) + size_t(n0 + row) * kD + chunk * 8;
                 detail::load_lds_16B(src, sk + (is_v ? Traits::kTileBytes : 0) + t * 1024);
+            }
+        }
+    };
+
+    // ---- Sᵀ[kv, q] - m_init = K[kv, :] · (c Q[q, :]) - m_init: accumulators start at -m_init
+    auto qk_block = [&](int stage, float m_init, f32x16 (&s_acc)[Traits::kKvTiles]) {
+        const unsigned char* sk = lds + stage * Traits::kStageBytes;
+#pragma unroll
+        for (int t = 0; t < Traits::kKvTiles; ++t) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s_acc[t][e] = -m_init;
+            const int row = t * 32 + q32;  // key row read by this lane (A operand: row = lane % 32)
+#pragma unroll
+            for (int s = 0; s < Traits::kDSteps; ++s) {
+                const int chunk = (2 * s + h) ^ Traits::k_swz(row);
+                const f16x8 kf = *reinterpret_cast<const f16x8*>(sk + row * kRowBytes + chunk * 16);
+                s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], s_acc[t], 0, 0, 0);
             }
         }
     };
@@ -120,71 +153,108 @@ __global__ void __launch_bounds__(Traits::kThreads)
     for (int t = 0; t < Traits::kDTiles; ++t)
 #pragma unroll
         for (int e = 0; e < 16; ++e) o_acc[t][e] = 0.f;
-    float m_run = -INFINITY;  // running max of s * c, shared by lanes l and l ^ 32
+    float m_run = -INFINITY;  // reference maximum of this lane's query (same in lanes l and l ^ 32)
     float l_run = 0.f;        // this lane's share of the running sum
-    const float c = scale * 1.4426950408889634f;
 
     const int nblocks = N / kBN;
     issue_block(0, 0);
+    if (nblocks > 1) issue_block(1, kBN);
+    if (nblocks > 1) __builtin_amdgcn_s_waitcnt(0x0070 | (kLoadsPerWave & 0xF));  // block 0 landed, block 1 in flight
+    else __builtin_amdgcn_s_waitcnt(0x0070);
+    __syncthreads();
 
-    for (int j = 0; j < nblocks; ++j) {
-        const int stage = j & 1;
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my share of block j has landed
-        __syncthreads();                      // everyone's share landed; everyone is done with block j-1
-        if (j + 1 < nblocks) issue_block(stage ^ 1, (j + 1) * kBN);
+    f32x16 s_cur[Traits::kKvTiles], s_nxt[Traits::kKvTiles];
+    float m_init_cur = 0.f, m_init_nxt = 0.f;  // what the accumulators of s_cur / s_nxt were started at (negated)
+    qk_block(0, m_init_cur, s_cur);
 
-        const unsigned char* sk = lds + stage * Traits::kStageBytes;
-        const unsigned char* sv = sk + Traits::kTileBytes;
+    constexpr float kLazy = 8.0f;
+    const int g = lane >> 4, L = lane & 15;
+    const int vrow_in = L >> 2;                            // 0..3: row within the 4-key group
+    const int vcol_b = (16 * (g & 1) + 4 * (L & 3)) * 2;  // byte offset of the lane's 4 columns inside a 32-d tile
 
-        // ---- Sᵀ[kv, q] = K[kv, :] · Q[q, :]
-        f32x16 s_acc[Traits::kKvTiles];
-#pragma unroll
-        for (int t = 0; t < Traits::kKvTiles; ++t) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) s_acc[t][e] = 0.f;
-            const int row = t * 32 + q32;  // key row read by this lane (A operand: row = lane % 32)
-#pragma unroll
-            for (int s = 0; s < Traits::kDSteps; ++s) {
-                const int chunk = (2 * s + h) ^ Traits::k_swz(row);
-                const f16x8 kf = *reinterpret_cast<const f16x8*>(sk + row * kRowBytes + chunk * 16);
-                s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], s_acc[t], 0, 0, 0);
-            }
-        }
-
-        // ---- online softmax for query q32: this lane holds keys 32 t + 8 (r / 4) + 4 h + r % 4
+    // block maximum of s (relative to its m_init) for the query of this lane
+    auto block_max = [&](const f32x16 (&s_acc)[Traits::kKvTiles]) -> float {
         float mx = s_acc[0][0];
 #pragma unroll
         for (int t = 0; t < Traits::kKvTiles; ++t)
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[t][e]);
-        mx = fmaxf(mx, detail::exchange32(mx));
-        const float m_new = fmaxf(m_run, mx * c);
-        const float alpha = exp2f(m_run - m_new);  // exp2(-inf) = 0 on the first block
-        m_run = m_new;
+        return fmaxf(mx, detail::exchange32(mx));
+    };
+    // Is the general path needed for a block whose accumulators started at m_init and whose maximum is mx?
+    // Yes if the reference maximum must move (lazy rescaling) or if it moved after the accumulators were started.
+    auto needs_general = [&](float m_init, float mx) -> bool {
+        return __any((m_init + mx - m_run > kLazy) || (m_init != m_run));
+    };
+
+    float mx_cur = block_max(s_cur);
+    bool general_cur = true;  // first block: m_run = -inf
+
+    // The wavefronts of a workgroup run the three pieces of an iteration in two different orders, so that
+    // the two wavefronts sharing a SIMD are out of phase: while one does softmax (VALU, transcendental),
+    // the other feeds the matrix pipe.
+    //   wavefronts 0-3: scores of block j+1 (MFMA), softmax of block j (VALU), output update with block j (MFMA)
+    //   wavefronts 4-7: softmax of block j, output update with block j, scores of block j+1
+    // (the wavefronts of a workgroup are dealt to the 4 SIMDs round-robin: w and w + 4 share one).
+    const bool scores_first = ((wave >> 2) & 1) == 0;
+
+    int stage = 0;
+    for (int j = 0; j < nblocks; ++j) {
+        const int stage_nxt = stage + 1 == kStages ? 0 : stage + 1;
+        const bool has_next = j + 1 < nblocks;
+        if (has_next) {
+            __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): my share of block j+1 (issued one iteration ago) landed
+            __syncthreads();                      // everyone's share landed; everyone is done with block j-1
+            if (j + 2 < nblocks) issue_block(stage_nxt + 1 == kStages ? 0 : stage_nxt + 1, (j + 2) * kBN);
+        }
+
+        if (has_next && scores_first) {
+            m_init_nxt = (m_run == -INFINITY) ? 0.f : m_run;
+            qk_block(stage_nxt, m_init_nxt, s_nxt);
+        }
+
+        // ---- probabilities of block j. This lane holds keys 32 t + 8 (r / 4) + 4 h + r % 4; s_cur = score - m_init_cur.
         float psum = 0.f;
         f16x8 pf[Traits::kKvSteps];
+        if (general_cur) {
+            // move the reference maximum if needed, rescale the output, exponentiate with the correction
+            const float m_blk = m_init_cur + mx_cur;
+            const bool upd = m_blk - m_run > kLazy;
+            const float m_new = upd ? m_blk : m_run;
+            const float alpha = detail::exp2_raw(m_run - m_new);  // exp2(-inf) = 0, exp2(0) = 1
+            l_run *= alpha;
 #pragma unroll
-        for (int t = 0; t < Traits::kKvTiles; ++t) {
+            for (int t = 0; t < Traits::kDTiles; ++t)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const float p = exp2f(s_acc[t][e] * c - m_new);
-                psum += p;
-                pf[2 * t + e / 8][e % 8] = static_cast<_Float16>(p);
-            }
+                for (int e = 0; e < 16; ++e) o_acc[t][e] *= alpha;
+            m_run = m_new;
+            const float delta = m_init_cur - m_run;
+#pragma unroll
+            for (int t = 0; t < Traits::kKvTiles; ++t)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float p = detail::exp2_raw(s_cur[t][e] + delta);
+                    psum += p;
+                    pf[2 * t + e / 8][e % 8] = static_cast<_Float16>(p);
+                }
+        } else {
+            // common case: m_init_cur == m_run and the maximum stays: p = exp2(s_cur)
+#pragma unroll
+            for (int t = 0; t < Traits::kKvTiles; ++t)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float p = detail::exp2_raw(s_cur[t][e]);
+                    psum += p;
+                    pf[2 * t + e / 8][e % 8] = static_cast<_Float16>(p);
+                }
         }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int t = 0; t < Traits::kDTiles; ++t)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o_acc[t][e] *= alpha;
+        l_run += psum;
 
         // ---- Oᵀ[d, q] += Vᵀ[d, kv] · Pᵀ[kv, q]
         // A operand for (d tile dt, k-step s): lane (d = 32 dt + lane % 32, h), slot e = key 16 s + 8 (e / 4) + 4 h + e % 4,
         // fetched with two transposing reads (4 consecutive keys of one d each). Within a 16-lane group, lane L
         // supplies the address of row kv0 + L / 4, columns dbase + 4 (L % 4) .. + 3.
-        const int g = lane >> 4, L = lane & 15;
-        const int vrow_in = L >> 2;                    // 0..3: row within the 4-key group
-        const int vcol_b = (16 * (g & 1) + 4 * (L & 3)) * 2;  // byte offset of the lane's 4 columns inside the 32-d tile
+        const unsigned char* sv = lds + stage * Traits::kStageBytes + Traits::kTileBytes;
 #pragma unroll
         for (int dt = 0; dt < Traits::kDTiles; ++dt) {
 #pragma unroll
@@ -205,6 +275,20 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[s], o_acc[dt], 0, 0, 0);
             }
         }
+
+        if (has_next) {
+            if (scores_first) {
+#pragma unroll
+                for (int t = 0; t < Traits::kKvTiles; ++t) s_cur[t] = s_nxt[t];
+                m_init_cur = m_init_nxt;
+            } else {
+                m_init_cur = m_run;  // m_run is finite here: at least one block has been processed
+                qk_block(stage_nxt, m_init_cur, s_cur);
+            }
+            mx_cur = block_max(s_cur);
+            general_cur = needs_general(m_init_cur, mx_cur);
+        }
+        stage = stage_nxt;
     }
 
     // ---- epilogue: O[q, d] = Oᵀ[d, q] / l. acc[dt][r]: d = 32 dt + 8 (r / 4) + 4 h + r % 4, q = q32.

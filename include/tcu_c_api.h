@@ -47,6 +47,13 @@ typedef enum {
     TCU_ATTN_MFMA32 = 2        /* 32x32x16 MFMA, transposing LDS reads, direct-to-LDS K/V (row-major V only) */
 } tcu_attn_algo;
 
+/* Which LSTM step kernel to run (tcu_lstm_f16_algo). AUTO picks STREAMING. */
+typedef enum {
+    TCU_LSTM_AUTO = 0,
+    TCU_LSTM_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, single LDS stage */
+    TCU_LSTM_STREAMING = 2     /* 32x32x16 MFMA, multi-stage direct-to-LDS ring, k split over two wavefront groups */
+} tcu_lstm_algo;
+
 /* Library version (major * 10000 + minor * 100 + patch). */
 int tcu_version(void);
 
@@ -99,6 +106,10 @@ int tcu_flash_attn_fwd_f16_algo(const void* Q, const void* K, const void* V, voi
  */
 int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
                  void* c_out, int T, int B, int I, int H, void* stream);
+
+/* tcu_lstm_f16 with an explicit kernel choice (tcu_lstm_algo); same arguments otherwise. */
+int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                      void* c_out, int T, int B, int I, int H, int algo, void* stream);
 
 #ifdef __cplusplus
 }

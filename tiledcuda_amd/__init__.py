@@ -18,7 +18,7 @@ import torch
 
 __all__ = [
     "TcuError", "library_path", "lib", "last_error", "gemm", "b2b_gemm", "flash_attention_fwd",
-    "flash_attention", "TiledFlashAttention", "lstm", "GEMM_ALGOS", "ATTN_ALGOS",
+    "flash_attention", "TiledFlashAttention", "lstm", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS",
 ]
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -40,6 +40,7 @@ TCU_V_COL_MAJOR = 0
 TCU_V_ROW_MAJOR = 1
 
 ATTN_ALGOS = {"auto": 0, "tile_library": 1, "mfma32": 2}
+LSTM_ALGOS = {"auto": 0, "tile_library": 1, "streaming": 2}
 
 # every exported symbol with its ctypes signature (also what the symbol test checks)
 _SIGNATURES = {
@@ -53,6 +54,7 @@ _SIGNATURES = {
     "tcu_flash_attn_fwd_f16_algo": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int,
                                                                                                 ctypes.c_int, ctypes.c_void_p]),
     "tcu_lstm_f16": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
+    "tcu_lstm_f16_algo": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 5 + [ctypes.c_void_p]),
 }
 
 
@@ -213,7 +215,7 @@ class TiledFlashAttention:
 
 # ------------------------------------------------------------------------------ LSTM
 def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor | None = None,
-         c0: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+         c0: torch.Tensor | None = None, algo: str = "auto") -> tuple[torch.Tensor, torch.Tensor]:
     """Fused LSTM layer. x [T, B, I] f16, W [4H, I+H] f16 (gate rows i,f,g,o), bias [4H] f16,
     h0 [B, H] f16 / c0 [B, H] f32 (None = zeros). Returns (h_all [T, B, H] f16, c_T [B, H] f32)."""
     T, B, I = x.shape
@@ -222,8 +224,8 @@ def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor 
         raise ValueError("W must be [4H, I+H] and bias [4H]")
     h_all = torch.empty(T, B, H, dtype=torch.float16, device=x.device)
     c_out = torch.empty(B, H, dtype=torch.float32, device=x.device)
-    _check(lib().tcu_lstm_f16(_dev_ptr(x, torch.float16, "x"), _dev_ptr(W, torch.float16, "W"),
-                              _dev_ptr(bias, torch.float16, "bias"), _dev_ptr(h0, torch.float16, "h0"),
-                              _dev_ptr(c0, torch.float32, "c0"), _dev_ptr(h_all, torch.float16, "h_all"),
-                              _dev_ptr(c_out, torch.float32, "c_out"), T, B, I, H, _stream()))
+    _check(lib().tcu_lstm_f16_algo(_dev_ptr(x, torch.float16, "x"), _dev_ptr(W, torch.float16, "W"),
+                                   _dev_ptr(bias, torch.float16, "bias"), _dev_ptr(h0, torch.float16, "h0"),
+                                   _dev_ptr(c0, torch.float32, "c0"), _dev_ptr(h_all, torch.float16, "h_all"),
+                                   _dev_ptr(c_out, torch.float32, "c_out"), T, B, I, H, LSTM_ALGOS[algo], _stream()))
     return h_all, c_out

@@ -5,6 +5,7 @@
 
 #include "kernels/flash_attn_fwd.hpp"
 #include "kernels/gemm_pipelined.hpp"
+#include "kernels/lstm_fwd.hpp"
 #include "kernels/mod.hpp"
 
 #include <mutex>
@@ -254,6 +255,24 @@ int launch_lstm(const __half* x, const __half* W, const __half* bias, const __ha
     return TCU_OK;
 }
 
+template <int kI, int kH>
+int launch_lstm_fwd(const __half* x, const __half* W, const __half* bias, const __half* h0, const float* c0,
+                    __half* h_all, float* c_out, int T, int B, hipStream_t stream) {
+    using Traits = LstmFwdTraits<kI, kH>;
+    auto kernel = &lstm_cell_fwd<Traits>;
+    const int grid = (B / Traits::kTM) * (kH / Traits::kTH);
+    for (int t = 0; t < T; ++t) {
+        const __half* x_t = x + size_t(t) * B * kI;
+        const __half* h_in = t == 0 ? h0 : h_all + size_t(t - 1) * B * kH;
+        const float* c_in = t == 0 ? c0 : c_out;
+        __half* h_out = h_all + size_t(t) * B * kH;
+        int rc = launch(kernel, dim3(grid), dim3(Traits::kThreads), Traits::kLdsBytes, stream, x_t, h_in, W, bias, c_in,
+                        c_out, h_out, B);
+        if (rc != TCU_OK) return rc;
+    }
+    return TCU_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -312,6 +331,11 @@ int tcu_flash_attn_fwd_f16(const void* Q, const void* K, const void* V, void* O,
 
 int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
                  void* c_out, int T, int B, int I, int H, void* stream) {
+    return tcu_lstm_f16_algo(x, W, bias, h0, c0, h_all, c_out, T, B, I, H, TCU_LSTM_AUTO, stream);
+}
+
+int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                      void* c_out, int T, int B, int I, int H, int algo, void* stream) {
     if (!x || !W || !bias || !h_all || !c_out) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: null pointer");
     if (!positive({T, B, I, H})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: sizes must be positive");
     auto s = static_cast<hipStream_t>(stream);
@@ -321,13 +345,24 @@ int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0,
     auto hp = static_cast<__half*>(h_all);
     auto cp = static_cast<float*>(c_out);
     if (B % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16: batch must be a multiple of 64");
+    if (algo != TCU_LSTM_AUTO && algo != TCU_LSTM_TILE_LIBRARY && algo != TCU_LSTM_STREAMING)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: unknown algo");
+    if (algo != TCU_LSTM_TILE_LIBRARY) {
+        if (I == 1024 && H == 1024) return launch_lstm_fwd<1024, 1024>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+        if (I == 128 && H == 128) return launch_lstm_fwd<128, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+        if (I == 256 && H == 128) return launch_lstm_fwd<256, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+        if (algo == TCU_LSTM_STREAMING)
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE,
+                        "the streaming LSTM kernel is instantiated for (I, H) in {(1024,1024), (128,128), (256,128)}");
+    }
     if (I == 1024 && H == 1024)
         return launch_lstm<1024, 1024, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
     if (I == 128 && H == 128)
         return launch_lstm<128, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
     if (I == 64 && H == 128)
         return launch_lstm<64, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
-    return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16 is instantiated for (I, H) in {(1024,1024), (128,128), (64,128)}");
+    return fail(TCU_ERR_UNSUPPORTED_SHAPE,
+                "tcu_lstm_f16 is instantiated for (I, H) in {(1024,1024), (128,128), (256,128), (64,128)}");
 }
 
 }  // extern "C"
