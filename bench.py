@@ -49,6 +49,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--only", default="", help="comma-separated subset of gemm,c1,b2b,attn,lstm (gemm always runs)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain device copy of 128 MiB (read 128 MiB, write 128 MiB) a few times, so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command has a kernel of known traffic to "
+                         "scale the counters by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
@@ -72,6 +76,14 @@ def main():
         return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
 
     configs = []
+
+    if args.calibrate_copy:
+        src = torch.arange(64 * 1024 * 1024, device=dev, dtype=torch.int16)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---------------------------------------------------------------- C2: GEMM 4096^3 (headline)
     n = 4096

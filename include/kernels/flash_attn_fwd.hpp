@@ -73,11 +73,14 @@ DEVICE float exchange32(float v) { return __shfl_xor(v, 32, 64); }
 DEVICE float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
 }  // namespace detail
 
-/// grid = (M / kBM, batch), block = Traits::kThreads, dynamic LDS = Traits::kLdsBytes.
+/// grid = (M / kBM) * batch workgroups (1-D), block = Traits::kThreads, dynamic LDS = Traits::kLdsBytes.
+/// Workgroup ids that are congruent modulo 8 land on the same XCD (and share its L2): when the batch
+/// count is a multiple of 8 the query blocks of one (batch, head) item all get such ids, so its K and V
+/// are fetched from HBM once instead of once per XCD.
 template <typename Traits>
 __global__ void __launch_bounds__(Traits::kThreads)
     flash_attention_fwd(const __half* __restrict__ Q, const __half* __restrict__ K, const __half* __restrict__ V,
-                        __half* __restrict__ O, int M, int N, float scale) {
+                        __half* __restrict__ O, int batch, int M, int N, float scale) {
     constexpr int kD = Traits::kD, kBN = Traits::kBN, kWaves = Traits::kWaves;
     constexpr int kRowBytes = Traits::kRowBytes;
     constexpr int kChunks = kRowBytes / 16;  // 16-byte chunks per row
@@ -89,8 +92,18 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int q32 = lane & 31;  // query (column of Sᵀ / Oᵀ) owned by this lane
     const int h = lane >> 5;    // lane half
 
-    const size_t head = blockIdx.y;
-    const int m0 = blockIdx.x * Traits::kBM + wave * 32;
+    const int q_blocks = M / Traits::kBM;
+    int head_i, q_block;
+    if (batch % 8 == 0) {
+        const int xcd = blockIdx.x & 7, rest = blockIdx.x >> 3;
+        q_block = rest % q_blocks;
+        head_i = (rest / q_blocks) * 8 + xcd;
+    } else {
+        q_block = blockIdx.x % q_blocks;
+        head_i = blockIdx.x / q_blocks;
+    }
+    const size_t head = head_i;
+    const int m0 = q_block * Traits::kBM + wave * 32;
     const __half* Qh = Q + (head * M + m0) * kD;
     const __half* Kh = K + head * size_t(N) * kD;
     const __half* Vh = V + head * size_t(N) * kD;

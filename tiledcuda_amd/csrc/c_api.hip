@@ -191,8 +191,8 @@ int launch_fa_fwd(const __half* Q, const __half* K, const __half* V, __half* O, 
                   hipStream_t stream) {
     using Traits = FlashFwdTraits<kD, kWaves, 64>;
     auto kernel = &flash_attention_fwd<Traits>;
-    return launch(kernel, dim3(M / Traits::kBM, batch), dim3(Traits::kThreads), Traits::kLdsBytes, stream, Q, K, V, O,
-                  M, N, scale);
+    return launch(kernel, dim3((M / Traits::kBM) * batch), dim3(Traits::kThreads), Traits::kLdsBytes, stream, Q, K, V,
+                  O, batch, M, N, scale);
 }
 
 template <int kD>
