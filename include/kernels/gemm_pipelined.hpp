@@ -2,19 +2,21 @@
 // [N, K]), f32 accumulate, C row-major in f16 or f32. This is the multi-stage kernel the
 // reference's examples/cpp/01_gemm/02_gemm_all_mem/gemm.hpp:103-155 lacks (it has one LDS
 // stage and waits for every load), built for the CDNA4 execution model:
-//   * one workgroup of kWM x kWN wavefronts per kBM x kBN tile of C, v_mfma_f32_32x32x16_f16,
-//     accumulators resident in registers for the whole K loop;
+//   * one workgroup of kWM x kWN wavefronts per kBM x kBN tile of C, accumulators resident in
+//     registers for the whole K loop; the MFMA is v_mfma_f32_16x16x32_f16: on random operands the
+//     matrix pipe is power-limited, and this shape sustains a ~12 % higher clock than
+//     v_mfma_f32_32x32x16_f16 at the same LDS traffic (the kernel measured 15-20 % faster with it);
 //   * A and B tiles go global -> LDS directly (global_load_lds_dwordx4, 16 B per lane, no
 //     VGPR staging; staging through registers measured 10 % slower), kStages LDS buffers; the
-//     loads of tile k+1 are issued in three portions between the MFMA groups of tile k (an
-//     even stream on the vector-memory path measured 3-5 % faster than one burst per tile);
+//     loads of tile k+1 are issued during the first k-substep of tile k and awaited before the
+//     last, which leaves them half a tile of MFMA time to land;
 //   * LDS rows are kBK halves (128 B for kBK = 64); the 16-byte chunks of a row are
-//     XOR-permuted with (row / 2) % 8 so that the ds_read_b128 of 32 consecutive rows at one
+//     XOR-permuted with (row / 2) % 8 so that the ds_read_b128 of 16 consecutive rows at one
 //     k-offset is bank-conflict free; the permutation is applied on the global-address side
 //     because a direct-to-LDS load writes 64 lanes x 16 B contiguously;
 //   * register double-buffering of the MFMA operands: the ds_reads of k-substep kk+1 are
 //     issued before the MFMAs of substep kk; the barrier that hands over an LDS stage sits
-//     before the last substep so its latency hides under 16 MFMAs;
+//     before the last substep so its latency hides under that substep's MFMAs;
 //   * the result is staged through LDS so that global stores are full 16-byte, row-contiguous;
 //   * workgroup ids are remapped so that the 32 workgroups an XCD receives (ids congruent
 //     modulo 8) form a compact block of tiles and share A / B panels in that XCD's L2.
@@ -34,13 +36,13 @@ struct PipelinedGemmTraits {
 
     static constexpr int kWaveM = kBM / kWM;  // rows of C per wavefront
     static constexpr int kWaveN = kBN / kWN;
-    static constexpr int kMT = kWaveM / 32;  // 32x32 MFMA tiles per wavefront along M
-    static constexpr int kNT = kWaveN / 32;
-    static constexpr int kKS = kBK / 16;  // MFMA k-substeps per LDS tile
+    static constexpr int kMT = kWaveM / 16;  // 16x16 MFMA tiles per wavefront along M
+    static constexpr int kNT = kWaveN / 16;
+    static constexpr int kKS = kBK / 32;  // MFMA k-substeps (32 wide) per LDS tile
 
     static_assert(kBK == 64, "LDS rows are 128 bytes: kBK must be 64 halves");
     static_assert(kStages == 2, "two LDS stages: a 256 x 256 x 64 stage is 64 KiB of the CU's 160 KiB");
-    static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0, "a wavefront owns whole 32x32 MFMA tiles");
+    static_assert(kWaveM % 16 == 0 && kWaveN % 16 == 0, "a wavefront owns whole 16x16 MFMA tiles");
 
     static constexpr int kRowBytes = kBK * 2;                    // 128
     static constexpr int kABytes = kBM * kRowBytes;              // one stage of A
@@ -155,22 +157,22 @@ __global__ void __launch_bounds__(Traits::kThreads)
     auto issue_stage = [&](int stage, int k0) { issue_part(stage, k0, 0, 1); };
 
     // ---- LDS -> register addressing -----------------------------------------------------
-    // 32x32x16 operand: lane l holds row l % 32, k = 8 * (l / 32) .. +7 of the 16-wide substep,
-    // i.e. logical chunk 2 * kk + l / 32 of its row.
-    const int frow = lane & 31;
-    const int fhalf = lane >> 5;
+    // 16x16x32 operand: lane l holds row l % 16, k = 8 * (l / 16) .. +7 of the 32-wide substep,
+    // i.e. logical chunk 4 * kk + l / 16 of its row.
+    const int frow = lane & 15;
+    const int fquad = lane >> 4;
     auto read_frag = [&](const unsigned char* base, int row, int kk) -> f16x8 {
-        const int chunk = (2 * kk + fhalf) ^ ((row >> 1) & 7);
+        const int chunk = (4 * kk + fquad) ^ ((row >> 1) & 7);
         return *reinterpret_cast<const f16x8*>(base + row * Traits::kRowBytes + chunk * 16);
     };
 
-    f32x16 acc[kMT][kNT];
+    f32x4 acc[kMT][kNT];
 #pragma unroll
     for (int i = 0; i < kMT; ++i)
 #pragma unroll
         for (int j = 0; j < kNT; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+            for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
     f16x8 fa[2][kMT], fb[2][kNT];
 
@@ -178,18 +180,18 @@ __global__ void __launch_bounds__(Traits::kThreads)
         const unsigned char* sa = lds + stage * Traits::kStageBytes;
         const unsigned char* sb = sa + Traits::kABytes;
 #pragma unroll
-        for (int i = 0; i < kMT; ++i) fa[buf][i] = read_frag(sa, wave_m * Traits::kWaveM + i * 32 + frow, kk);
+        for (int i = 0; i < kMT; ++i) fa[buf][i] = read_frag(sa, wave_m * Traits::kWaveM + i * 16 + frow, kk);
 #pragma unroll
-        for (int j = 0; j < kNT; ++j) fb[buf][j] = read_frag(sb, wave_n * Traits::kWaveN + j * 32 + frow, kk);
+        for (int j = 0; j < kNT; ++j) fb[buf][j] = read_frag(sb, wave_n * Traits::kWaveN + j * 16 + frow, kk);
     };
     auto mma = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < kMT; ++i)
 #pragma unroll
             for (int j = 0; j < kNT; ++j)
-                // operands swapped: the accumulator then holds C (not C^T) with 4 consecutive
-                // columns per register quad
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+                // operands swapped: the accumulator then holds C (not C^T): row l % 16, the 4 consecutive
+                // columns 4 * (l / 16) .. +3
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
     };
 
     const int ktiles = K / kBK;
@@ -206,7 +208,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
 #pragma unroll
         for (int kk = 0; kk < kKS - 1; ++kk) {
             // tile kt+1 goes to the other stage, which everyone left at the barrier of iteration kt-1;
-            // its loads are spread over this iteration's first kKS-1 substeps
+            // its loads are issued during this iteration's first kKS-1 substeps
             if (kt + 1 < ktiles) issue_part(next_stage, (kt + 1) * kBK, kk, kKS - 1);
             load_frags((kk + 1) & 1, stage, kk + 1);
             mma(kk & 1);
@@ -223,30 +225,27 @@ __global__ void __launch_bounds__(Traits::kThreads)
     }
 
     // ---- epilogue -----------------------------------------------------------------------
-    // acc[i][j][r]: row = lane % 32, col = 8 * (r / 4) + 4 * (lane / 32) + r % 4 of the 32x32 tile.
+    // acc[i][j][r]: row = lane % 16, col = 4 * (lane / 16) + r of the 16x16 tile.
     if constexpr (sizeof(OutType) == 2) {
         __syncthreads();  // everyone is done with the operand stages
         constexpr int kWaveN = Traits::kWaveN, kWaveM = Traits::kWaveM;
         constexpr int kPitch = kWaveN * 2;  // bytes per staged row
         unsigned char* stg = lds + wave * (kWaveM * kPitch);
-        // write: lane owns row (i*32 + frow); 4 halves (8 B) at column j*32 + 8*q + 4*fhalf.
+        // write: lane owns row i*16 + frow; 4 halves (8 B) at column j*16 + 4*fquad.
         // 8-byte slots of a row are XOR-ed with (row % 16) * 2 (bit 0 untouched, kept inside the row)
         // to spread banks.
         constexpr int kSlotMask = (kPitch / 8 - 1) & ~1;
 #pragma unroll
         for (int i = 0; i < kMT; ++i) {
-            const int row = i * 32 + frow;
+            const int row = i * 16 + frow;
 #pragma unroll
             for (int j = 0; j < kNT; ++j) {
+                const int slot = (j * 16 + 4 * fquad) >> 2;  // 8-byte slot index in the row
+                const int pslot = slot ^ (((row & 15) << 1) & kSlotMask);
+                f16x4 v;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int slot = (j * 32 + 8 * q + 4 * fhalf) >> 2;  // 8-byte slot index in the row
-                    const int pslot = slot ^ (((row & 15) << 1) & kSlotMask);
-                    f16x4 v;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc[i][j][4 * q + e]);
-                    *reinterpret_cast<f16x4*>(stg + row * kPitch + pslot * 8) = v;
-                }
+                for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc[i][j][e]);
+                *reinterpret_cast<f16x4*>(stg + row * kPitch + pslot * 8) = v;
             }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's staging writes are done
@@ -269,13 +268,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         for (int i = 0; i < kMT; ++i) {
 #pragma unroll
             for (int j = 0; j < kNT; ++j) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    f32x4 v;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
-                    *reinterpret_cast<f32x4*>(cbase + size_t(i * 32 + frow) * N + j * 32 + 8 * q + 4 * fhalf) = v;
-                }
+                *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * N + j * 16 + 4 * fquad) = acc[i][j];
             }
         }
     }

@@ -31,7 +31,7 @@ typedef enum {
     TCU_GEMM_AUTO = 0,
     TCU_GEMM_GLOBAL_REG = 1, /* global -> register -> MFMA (README kernel of the reference) */
     TCU_GEMM_ALL_MEM = 2,    /* global -> LDS -> register -> MFMA, single stage */
-    TCU_GEMM_PIPELINED = 3   /* direct-to-LDS, multi-stage, 32x32x16 MFMA */
+    TCU_GEMM_PIPELINED = 3   /* direct-to-LDS, double-buffered, 16x16x32 MFMA */
 } tcu_gemm_algo;
 
 /* Layout of V in tcu_flash_attn_fwd_f16. */

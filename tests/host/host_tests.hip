@@ -216,13 +216,13 @@ static void test_shared_tile_views() {
 
 static void test_pipelined_gemm_maps() {
     // LDS rows of 128 B, 16-byte chunk c of row r stored at chunk c ^ ((r / 2) % 8): any 16 consecutive
-    // lanes of a 32x32x16 operand read (rows r0..r0+15, one k-chunk) must touch 16 distinct 16-byte bank slots
-    for (int kk = 0; kk < 4; ++kk)
-        for (int half = 0; half < 2; ++half)
+    // lanes of a 16x16x32 operand read (rows r0..r0+15, one k-chunk) must touch 16 distinct 16-byte bank slots
+    for (int kk = 0; kk < 2; ++kk)
+        for (int quad = 0; quad < 4; ++quad)
             for (int r0 = 0; r0 < 64; r0 += 16) {
                 std::set<int> slots;
                 for (int r = r0; r < r0 + 16; ++r) {
-                    const int chunk = (2 * kk + half) ^ ((r >> 1) & 7);
+                    const int chunk = (4 * kk + quad) ^ ((r >> 1) & 7);
                     slots.insert(((r * 128 + chunk * 16) / 16) % 16);
                 }
                 CHECK(slots.size() == 16);
