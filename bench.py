@@ -6,7 +6,10 @@ configurations (GEMM 128x64x256, back-to-back GEMM, FlashAttention-2 forward, fu
 are timed in the same run and reported under "configs".
 
 Prints ONE JSON line: the driver's contract fields plus
-  roofline     -- dominant kernel vs the MFMA fp16 dense peak (2.5 PFLOP/s) / HBM (8 TB/s)
+  roofline     -- dominant kernel vs the MFMA fp16 dense peak (2.5 PFLOP/s) / HBM (8 TB/s); its
+                  "sustained_mfma" entry is the rate and core clock the GPU holds on a loop of nothing but
+                  MFMAs fed with the same operand distribution (the matrix pipe is power-managed, so this
+                  is the practical ceiling; the published peak assumes 2.4 GHz)
   cpu_baseline -- the CPU oracle (OpenMP, f32) timed on this host for the same workload
 """
 from __future__ import annotations
@@ -45,6 +48,32 @@ def time_kernel(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def probe_mfma(torch, operands, shape, waves=8, iters=20000):
+    """Sustained MFMA rate on `operands` (fp16 device tensor, >= 256*waves*4096 halves): TFLOP/s and core MHz."""
+    import ctypes
+
+    lib = ctypes.CDLL(os.path.join(ROOT, "tiledcuda_amd", "lib", "libtcu_probe.so"))
+    lib.tcu_probe_mfma_f16.restype = ctypes.c_int
+    lib.tcu_probe_mfma_f16.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4 + [ctypes.c_void_p]
+    wgs = 256
+    assert operands.numel() >= wgs * waves * 64 * 64
+    clocks = torch.zeros(2 * wgs, dtype=torch.int64, device=operands.device)
+    sink = torch.zeros(1, dtype=torch.float32, device=operands.device)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = lib.tcu_probe_mfma_f16(operands.data_ptr(), clocks.data_ptr(), sink.data_ptr(), shape, wgs, waves, iters, stream)
+        if rc != 0:
+            raise RuntimeError(f"tcu_probe_mfma_f16 failed with hipError {rc}")
+
+    ms = time_kernel(launch, 3, 1)
+    ticks = clocks.cpu().numpy().reshape(wgs, 2).astype("float64")
+    flops = wgs * waves * iters * 4.0 * (16384.0 if shape == 1 else 32768.0)
+    return {"tflops": flops / (ms * 1e-3) / 1e12, "core_clock_mhz": 100.0 * ticks[:, 0].sum() / ticks[:, 1].sum(),
+            "instruction": "v_mfma_f32_16x16x32_f16" if shape == 1 else "v_mfma_f32_32x32x16_f16",
+            "wavefronts_per_cu": waves}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -52,6 +81,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--only", default="", help="comma-separated subset of gemm,c1,b2b,attn,lstm (gemm always runs)")
+    ap.add_argument("--no-mfma-probe", action="store_true", help="skip the sustained-MFMA-rate measurement")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 128 MiB (read 128 MiB, write 128 MiB) a few times, so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command has a kernel of known traffic to "
@@ -118,6 +148,15 @@ def main():
     gemm_err = oracle.max_rel_err(dC[rows[0]:rows[1]].float().cpu().numpy(), ref[rows[0]:rows[1]])
     configs.append({"name": "gemm_4096", "ms": gemm_ms, "tflops": gemm_tflops,
                     "frac_mfma_peak": gemm_tflops / MFMA_F16_PEAK_TFLOPS, "max_rel_err": gemm_err})
+
+    # sustained MFMA rate on the same operand distribution (U[-1,1] fp16), the kernel's MFMA shape, 8 wavefronts per CU
+    sustained = None
+    if not args.no_mfma_probe:
+        sustained = probe_mfma(torch, dA, shape=1)
+        sustained["operands"] = "the GEMM's A matrix (U[-1,1] fp16)"
+        zeros = probe_mfma(torch, torch.zeros(1 << 23, dtype=torch.float16, device=dev), shape=1)
+        sustained["tflops_on_zero_operands"] = zeros["tflops"]
+        sustained["core_clock_mhz_on_zero_operands"] = zeros["core_clock_mhz"]
 
     # ---------------------------------------------------------------- C1: GEMM 128x64x256
     if want("c1"):
@@ -216,7 +255,8 @@ def main():
         "roofline": {"bound": "mfma", "achieved": gemm_tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": gemm_tflops / MFMA_F16_PEAK_TFLOPS, "traffic": GEMM_4096_TRAFFIC_BYTES,
                      "kernel": "gemm_pipelined<256x256x64, 4x2 wavefronts>", "flops_per_launch": gemm_flops,
-                     "avg_launch_us": gemm_ms * 1e3},
+                     "avg_launch_us": gemm_ms * 1e3, "sustained_mfma": sustained,
+                     "frac_of_sustained_mfma": (gemm_tflops / sustained["tflops"]) if sustained else None},
         "cpu_baseline": cpu,
         "max_rel_err": gemm_err,
         "configs": configs,
