@@ -80,7 +80,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
-    ap.add_argument("--only", default="", help="comma-separated subset of gemm,c1,b2b,attn,lstm (gemm always runs)")
+    ap.add_argument("--only", default="", help="comma-separated subset of gemm,c1,b2b,attn,lstm,scatter (gemm always runs)")
     ap.add_argument("--no-mfma-probe", action="store_true", help="skip the sustained-MFMA-rate measurement")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 128 MiB (read 128 MiB, write 128 MiB) a few times, so that a "
@@ -224,6 +224,20 @@ def main():
                         "gbs": step_bytes * T / (ms * 1e-3) / 1e9,
                         "frac_hbm_peak": step_bytes * T / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                         "tflops": flops / (ms * 1e-3) / 1e12, "max_abs_err": err})
+
+    # ---------------------------------------------------------------- scatter_nd (HBM-bound)
+    if want("scatter"):
+        rows, width = 65536, 1024
+        gen = torch.Generator(device="cpu").manual_seed(1240)
+        perm = torch.randperm(rows, generator=gen).to(dev).view(rows, 1)
+        upd = torch.randn(rows, width, device=dev)
+        data = torch.zeros(rows, width, device=dev)
+        ms = time_kernel(lambda: tcu.scatter_nd(data, perm, upd), max(5, args.steps // 2), max(2, args.warmup // 2))
+        ok = bool(torch.equal(data[perm.view(-1)], upd))
+        nbytes = 2.0 * rows * width * 4 + rows * 8
+        configs.append({"name": "scatter_nd_f32_65536x1024_rows_permuted", "ms": ms, "gbs": nbytes / (ms * 1e-3) / 1e9,
+                        "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "round_trip_exact": ok})
+        del upd, data
 
     # ---------------------------------------------------------------- CPU baseline (oracle, bounded)
     cpu = None

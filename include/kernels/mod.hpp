@@ -4,3 +4,4 @@
 #include "kernels/flash_attn.hpp"
 #include "kernels/gemm.hpp"
 #include "kernels/lstm.hpp"
+#include "kernels/scatter_nd.hpp"

@@ -1,0 +1,89 @@
+// scatter_nd for gfx950: data[indices[i, 0], ..., indices[i, k-1], :] (=|+=) updates[i, :] for i in [0, n).
+// The reference's kernel (src/kernels/scatter_nd.cu:25-55) runs one thread per index row that walks its whole
+// slice with scalar atomicAdds; its host code passes the index buffer as the update source (:104-107), leaks the
+// device stride array it allocates per call (:72-75) and its own test expects assignment, not accumulation
+// (tests/python/test_scatter_nd.py:47-56). Here: the strides travel by value in the kernel arguments (no
+// allocation), one lane per 16-byte piece of a slice (or per element when a slice is not a multiple of 16 bytes)
+// so that a wavefront writes contiguous memory, and the mode is explicit: assign (what the reference's test
+// checks; duplicate index rows then leave one of their updates, unspecified which) or atomic add (what the
+// reference's kernel body does).
+#pragma once
+
+#include "config.hpp"
+#include "hip_utils.hpp"
+
+#include <cstdint>
+
+namespace tiledcuda::kernels {
+
+constexpr int kScatterMaxRank = 8;
+
+struct ScatterNdShape {
+    int64_t strides[kScatterMaxRank];  // element strides of the first k dimensions of `data`
+    int64_t dims[kScatterMaxRank];     // their extents (indices are checked against them)
+    int64_t n;                         // index rows
+    int64_t slice;                     // elements per slice
+    int k;                             // index components per row
+};
+
+enum class ScatterMode : int { kAssign = 0, kAdd = 1 };
+
+namespace detail {
+DEVICE void atomic_add_elem(float* p, float v) { atomicAdd(p, v); }
+DEVICE void atomic_add_elem(__half* p, __half v) {
+    // 16-bit atomic add through a compare-and-swap on the aligned 32-bit word that holds the element
+    auto* word = reinterpret_cast<unsigned int*>(reinterpret_cast<uintptr_t>(p) & ~uintptr_t(3));
+    const bool high = (reinterpret_cast<uintptr_t>(p) & 2) != 0;
+    unsigned int old = *word, assumed;
+    do {
+        assumed = old;
+        const unsigned short cur = high ? (assumed >> 16) : (assumed & 0xffffu);
+        const __half sum = __float2half(__half2float(__ushort_as_half(cur)) + __half2float(v));
+        const unsigned int repl = high ? ((assumed & 0xffffu) | (unsigned(__half_as_ushort(sum)) << 16))
+                                       : ((assumed & 0xffff0000u) | __half_as_ushort(sum));
+        old = atomicCAS(word, assumed, repl);
+    } while (old != assumed);
+}
+}  // namespace detail
+
+/// One lane per group of kVec elements of one slice. kVec * sizeof(T) is 16 (vector path, assign mode only,
+/// slice % kVec == 0 and 16-byte aligned bases) or sizeof(T) (kVec = 1).
+/// Rows with an index component outside its extent are skipped and counted in *bad_rows (if not null).
+template <typename T, const int kVec, const ScatterMode kMode>
+__global__ void __launch_bounds__(256)
+    scatter_nd_kernel(T* __restrict__ data, const T* __restrict__ updates, const int64_t* __restrict__ indices,
+                      const ScatterNdShape shape, unsigned int* __restrict__ bad_rows) {
+    const int64_t groups_per_slice = shape.slice / kVec;
+    const int64_t total = shape.n * groups_per_slice;
+    for (int64_t g = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; g < total; g += int64_t(gridDim.x) * blockDim.x) {
+        const int64_t row = g / groups_per_slice;
+        const int64_t off = (g - row * groups_per_slice) * kVec;
+        const int64_t* idx = indices + row * shape.k;
+        int64_t base = 0;
+        bool ok = true;
+#pragma unroll 4
+        for (int c = 0; c < shape.k; ++c) {
+            const int64_t v = idx[c];
+            ok = ok && v >= 0 && v < shape.dims[c];
+            base += v * shape.strides[c];
+        }
+        if (!ok) {
+            if (bad_rows != nullptr && off == 0) atomicAdd(bad_rows, 1u);
+            continue;
+        }
+        const T* src = updates + row * shape.slice + off;
+        T* dst = data + base + off;
+        if constexpr (kMode == ScatterMode::kAssign) {
+            if constexpr (kVec == 1) {
+                *dst = *src;
+            } else {
+                *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src);
+            }
+        } else {
+            static_assert(kMode == ScatterMode::kAssign || kVec == 1, "atomic add is per element");
+            detail::atomic_add_elem(dst, *src);
+        }
+    }
+}
+
+}  // namespace tiledcuda::kernels

@@ -111,6 +111,25 @@ int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0,
 int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
                       void* c_out, int T, int B, int I, int H, int algo, void* stream);
 
+/* How tcu_scatter_nd combines an update with the data it lands on. */
+typedef enum {
+    TCU_SCATTER_ASSIGN = 0, /* data[...] = update: what the reference's test checks (tests/python/test_scatter_nd.py:47-56) */
+    TCU_SCATTER_ADD = 1     /* data[...] += update, atomically: what the reference's kernel body does (src/kernels/scatter_nd.cu:48-51) */
+} tcu_scatter_mode;
+
+/*
+ * data[idx[i,0], ..., idx[i,k-1], :] (= | +=) updates[i, :] for the n index rows of `indices`.
+ * data: device tensor of `rank` dimensions `data_dims` (HOST array of rank int64 values), row-major, dtype f32 or
+ * f16; indices: device int64 [n, k], k <= rank <= 8; updates: device [n, prod(data_dims[k:])], same dtype as data.
+ * Rows with a component outside [0, data_dims[c]) are skipped; if skipped_rows (device uint32, may be NULL) is
+ * given, it is incremented once per skipped row (the caller zeroes it). With TCU_SCATTER_ASSIGN, duplicate index
+ * rows leave one of their updates (unspecified which).
+ * Replaces custom_scatter_op / scatter_nd<T> of the reference's src/kernels/scatter_nd.cu:57-120 (the body of
+ * torch.ops.tiledcuda.scatter_nd, src/torch_bind.cc:9); unlike it, no device memory is allocated per call.
+ */
+int tcu_scatter_nd(void* data, const void* updates, const void* indices, const long long* data_dims, int rank,
+                   long long n, int k, int dtype, int mode, void* skipped_rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -169,6 +169,37 @@ def lstm(x: np.ndarray, W: np.ndarray, bias: np.ndarray, h0: np.ndarray | None =
     return h_all, c_out
 
 
+def scatter_nd(data: np.ndarray, indices: np.ndarray, updates: np.ndarray, mode: str = "assign") -> np.ndarray:
+    """data[indices[i, 0], ..., indices[i, k-1], ...] (= | +=) updates[i] over the index rows in order; returns a copy.
+    Offset arithmetic as the reference computes it (src/kernels/scatter_nd.cu:37-46: out_index = sum_c idx[c] *
+    strides[c], slice of prod(data.shape[k:]) elements, strides from :66-70); "assign" is the semantics its test
+    checks (tests/python/test_scatter_nd.py:47-56), "add" the accumulation its kernel body performs (:48-51).
+    A plain loop over rows on the flattened array: later rows win in "assign" mode. Rows with an index outside the
+    data are skipped."""
+    out = np.array(data, copy=True)
+    flat = out.reshape(-1)
+    k = indices.shape[-1]
+    rank = data.ndim
+    strides = [1] * rank
+    for d in range(rank - 2, -1, -1):
+        strides[d] = strides[d + 1] * data.shape[d + 1]
+    slice_size = int(np.prod(data.shape[k:], dtype=np.int64)) if k < rank else 1
+    idx = np.asarray(indices, dtype=np.int64).reshape(-1, k)
+    upd = np.asarray(updates).reshape(idx.shape[0], slice_size)
+    for i in range(idx.shape[0]):
+        if any(idx[i, c] < 0 or idx[i, c] >= data.shape[c] for c in range(k)):
+            continue
+        base = sum(int(idx[i, c]) * strides[c] for c in range(k))
+        if mode == "assign":
+            flat[base:base + slice_size] = upd[i]
+        elif mode == "add":
+            flat[base:base + slice_size] = (flat[base:base + slice_size].astype(np.float32) +
+                                            upd[i].astype(np.float32)).astype(flat.dtype)
+        else:
+            raise ValueError(mode)
+    return out
+
+
 # ---------------------------------------------------------------- error metrics
 def max_rel_err(x: np.ndarray, ref: np.ndarray, eps: float = 1e-2) -> float:
     """max |x-ref| / max(|ref|, eps·rms(ref)): relative error with a floor, so outputs that

@@ -58,6 +58,12 @@ def test_bad_sizes_and_enums_are_rejected(tcu):
     assert l.tcu_gemm_f16(p, p, p, 64, 64, 64, 0, 9, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
     assert l.tcu_b2b_gemm_f16(p, p, p, p, 64, 64, 64, 64, -1, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
     assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 64, 128, 128, 1.0, 5, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    dims = (ctypes.c_longlong * 2)(4, 4)
+    assert l.tcu_scatter_nd(0, p, p, dims, 2, 1, 1, 0, 0, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_scatter_nd(p, p, p, dims, 2, 1, 3, 0, 0, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT  # k > rank
+    assert l.tcu_scatter_nd(p, p, p, dims, 9, 1, 1, 0, 0, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT  # rank > 8
+    assert l.tcu_scatter_nd(p, p, p, dims, 2, 1, 1, 0, 7, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT  # mode
+    assert l.tcu_scatter_nd(p, p, p, dims, 2, 0, 1, 0, 0, 0, 0) == tcu.TCU_OK  # no rows: nothing to launch
     assert l.tcu_lstm_f16(p, p, p, 0, 0, p, p, 0, 64, 128, 128, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
 
 

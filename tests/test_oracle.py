@@ -280,3 +280,39 @@ def test_error_metric_floor(oracle):
     # the tiny reference value is floored at eps * rms, so the ratio stays bounded
     assert oracle.max_rel_err(x, ref) < 0.02
     assert oracle.max_rel_err(ref, ref) == 0.0
+
+
+# ---------------------------------------------------------------- scatter_nd
+def test_scatter_nd_oracle_matches_numpy_indexing(oracle):
+    """Pins the offset arithmetic: with distinct rows, "assign" equals numpy's advanced-index assignment (the
+    statement of the reference's own test, tests/python/test_scatter_nd.py:47: data[idx[:,0], idx[:,1]] = updates);
+    "add" equals numpy.add.at, duplicates included; later rows win in "assign"; k == rank scatters scalars."""
+    rng = np.random.default_rng(3)
+    data = rng.standard_normal((7, 8, 9, 10)).astype(np.float32)
+    rows = rng.permutation(56)[:20]
+    idx = np.stack(np.unravel_index(rows, (7, 8)), axis=1)
+    upd = rng.standard_normal((20, 9, 10)).astype(np.float32)
+    expect = data.copy()
+    expect[idx[:, 0], idx[:, 1]] = upd
+    assert np.array_equal(oracle.scatter_nd(data, idx, upd), expect)
+    # a wrong stride or a transposed index would move a slice: every other element must be untouched
+    untouched = np.ones((7, 8), bool)
+    untouched[idx[:, 0], idx[:, 1]] = False
+    assert np.array_equal(oracle.scatter_nd(data, idx, upd)[untouched], data[untouched])
+
+    idx_dup = rng.integers(0, 7, size=(50, 1))
+    upd_dup = rng.integers(-3, 4, size=(50, 8, 9, 10)).astype(np.float32)
+    expect = data.copy()
+    np.add.at(expect, (idx_dup[:, 0],), upd_dup)
+    np.testing.assert_allclose(oracle.scatter_nd(data, idx_dup, upd_dup, mode="add"), expect, rtol=0, atol=1e-4)
+
+    two = np.array([[2], [2]])
+    out = oracle.scatter_nd(np.zeros((4, 3), np.float32), two, np.array([[1, 1, 1], [2, 2, 2]], np.float32))
+    assert np.array_equal(out[2], [2, 2, 2])
+
+    full = np.array([[1, 2, 3], [0, 0, 0]])
+    out = oracle.scatter_nd(np.zeros((2, 3, 4), np.float32), full, np.array([5, 6], np.float32))
+    assert out[1, 2, 3] == 5 and out[0, 0, 0] == 6 and out.sum() == 11
+    # out-of-range rows are skipped
+    out = oracle.scatter_nd(np.zeros((2, 2), np.float32), np.array([[2], [-1], [1]]), np.ones((3, 2), np.float32))
+    assert np.array_equal(out, [[0, 0], [1, 1]])

@@ -18,7 +18,8 @@ import torch
 
 __all__ = [
     "TcuError", "library_path", "lib", "last_error", "gemm", "b2b_gemm", "flash_attention_fwd",
-    "flash_attention", "TiledFlashAttention", "lstm", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS",
+    "flash_attention", "TiledFlashAttention", "lstm", "scatter_nd", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS",
+    "SCATTER_MODES",
 ]
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -41,6 +42,7 @@ TCU_V_ROW_MAJOR = 1
 
 ATTN_ALGOS = {"auto": 0, "tile_library": 1, "mfma32": 2}
 LSTM_ALGOS = {"auto": 0, "tile_library": 1, "streaming": 2}
+SCATTER_MODES = {"assign": 0, "add": 1}
 
 # every exported symbol with its ctypes signature (also what the symbol test checks)
 _SIGNATURES = {
@@ -55,6 +57,9 @@ _SIGNATURES = {
                                                                                                 ctypes.c_int, ctypes.c_void_p]),
     "tcu_lstm_f16": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
     "tcu_lstm_f16_algo": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 5 + [ctypes.c_void_p]),
+    "tcu_scatter_nd": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.POINTER(ctypes.c_longlong), ctypes.c_int,
+                                                             ctypes.c_longlong, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                             ctypes.c_void_p, ctypes.c_void_p]),
 }
 
 
@@ -229,3 +234,35 @@ def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor 
                                    _dev_ptr(c0, torch.float32, "c0"), _dev_ptr(h_all, torch.float16, "h_all"),
                                    _dev_ptr(c_out, torch.float32, "c_out"), T, B, I, H, LSTM_ALGOS[algo], _stream()))
     return h_all, c_out
+
+
+# ------------------------------------------------------------------------------ scatter_nd
+def scatter_nd(scatter_data: torch.Tensor, scatter_indices: torch.Tensor, scatter_updates: torch.Tensor,
+               mode: str = "assign", skipped_rows: torch.Tensor | None = None) -> None:
+    """``data[indices[i, 0], ..., indices[i, k-1]] (= | +=) updates[i]`` in place, argument order of the
+    reference's ``pytiledcuda.scatter_nd(scatter_data, scatter_indices, scatter_updates)``.
+
+    ``scatter_data`` [d0, ..., d_{r-1}] f32 or f16, ``scatter_indices`` int64 [..., k], ``scatter_updates``
+    [..., d_k, ..., d_{r-1}]. (The reference wrapper is handed flattened tensors, which loses the shapes its op
+    reads them from; pass the shaped tensors here.) Rows with an out-of-range index are skipped; if
+    ``skipped_rows`` (uint32/int32 device tensor of one element, zeroed by the caller) is given it counts them."""
+    k = scatter_indices.shape[-1]
+    rank = scatter_data.dim()
+    n = scatter_indices.numel() // k if k else 0
+    slice_shape = tuple(scatter_data.shape[k:])
+    if k > rank or rank > 8:
+        raise ValueError("scatter_nd needs k <= rank(data) <= 8")
+    if scatter_updates.numel() != n * int(math.prod(slice_shape)):
+        raise ValueError("updates must have one slice data.shape[k:] per index row")
+    if scatter_data.dtype not in (torch.float32, torch.float16) or scatter_updates.dtype != scatter_data.dtype:
+        raise ValueError("data and updates must both be float32 or both float16")
+    dims = (ctypes.c_longlong * rank)(*scatter_data.shape)
+    skipped = 0
+    if skipped_rows is not None:
+        if not skipped_rows.is_cuda or skipped_rows.element_size() != 4 or skipped_rows.numel() != 1:
+            raise ValueError("skipped_rows must be a one-element 32-bit device tensor")
+        skipped = skipped_rows.data_ptr()
+    _check(lib().tcu_scatter_nd(_dev_ptr(scatter_data, scatter_data.dtype, "data"),
+                                _dev_ptr(scatter_updates, scatter_data.dtype, "updates"),
+                                _dev_ptr(scatter_indices, torch.int64, "indices"), dims, rank, n, k,
+                                _out_code(scatter_data.dtype), SCATTER_MODES[mode], skipped, _stream()))

@@ -365,4 +365,57 @@ int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void
                 "tcu_lstm_f16 is instantiated for (I, H) in {(1024,1024), (128,128), (256,128), (64,128)}");
 }
 
+int tcu_scatter_nd(void* data, const void* updates, const void* indices, const long long* data_dims, int rank,
+                   long long n, int k, int dtype, int mode, void* skipped_rows, void* stream) {
+    using namespace tiledcuda::kernels;
+    if (!data || !updates || !indices || !data_dims) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_scatter_nd: null pointer");
+    if (rank <= 0 || rank > kScatterMaxRank || k <= 0 || k > rank)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_scatter_nd: need 0 < k <= rank <= 8");
+    if (n < 0) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_scatter_nd: negative row count");
+    if (dtype != TCU_DTYPE_F32 && dtype != TCU_DTYPE_F16) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_scatter_nd: dtype must be f32 or f16");
+    if (mode != TCU_SCATTER_ASSIGN && mode != TCU_SCATTER_ADD) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_scatter_nd: unknown mode");
+    ScatterNdShape shape{};
+    int64_t stride = 1;
+    for (int d = rank - 1; d >= 0; --d) {
+        if (data_dims[d] <= 0) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_scatter_nd: dimensions must be positive");
+        if (d < k) {
+            shape.strides[d] = stride;
+            shape.dims[d] = data_dims[d];
+        }
+        stride *= data_dims[d];
+    }
+    shape.slice = 1;
+    for (int d = k; d < rank; ++d) shape.slice *= data_dims[d];
+    shape.n = n;
+    shape.k = k;
+    if (n == 0) return TCU_OK;
+    auto s = static_cast<hipStream_t>(stream);
+    auto idx = static_cast<const int64_t*>(indices);
+    auto bad = static_cast<unsigned int*>(skipped_rows);
+    const size_t elem = dtype == TCU_DTYPE_F32 ? 4 : 2;
+    const int vec = int(16 / elem);
+    const bool vec_ok = mode == TCU_SCATTER_ASSIGN && shape.slice % vec == 0 &&
+                        reinterpret_cast<uintptr_t>(data) % 16 == 0 && reinterpret_cast<uintptr_t>(updates) % 16 == 0;
+    const int64_t lanes = n * (vec_ok ? shape.slice / vec : shape.slice);
+    // enough workgroups to fill the chip several times over; the kernel strides over the rest
+    const int64_t want = (lanes + 255) / 256;
+    const dim3 grid(static_cast<unsigned>(want < 1 ? 1 : (want > 256 * 64 ? 256 * 64 : want))), block(256);
+    auto go = [&](auto* dptr, auto kernel) {
+        using T = std::remove_pointer_t<decltype(dptr)>;
+        hipLaunchKernelGGL(kernel, grid, block, 0, s, dptr, static_cast<const T*>(updates), idx, shape, bad);
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? int(TCU_OK) : hip_fail(e, "scatter_nd launch");
+    };
+    if (dtype == TCU_DTYPE_F32) {
+        auto* d = static_cast<float*>(data);
+        if (mode == TCU_SCATTER_ADD) return go(d, &scatter_nd_kernel<float, 1, ScatterMode::kAdd>);
+        return vec_ok ? go(d, &scatter_nd_kernel<float, 4, ScatterMode::kAssign>)
+                      : go(d, &scatter_nd_kernel<float, 1, ScatterMode::kAssign>);
+    }
+    auto* d = static_cast<__half*>(data);
+    if (mode == TCU_SCATTER_ADD) return go(d, &scatter_nd_kernel<__half, 1, ScatterMode::kAdd>);
+    return vec_ok ? go(d, &scatter_nd_kernel<__half, 8, ScatterMode::kAssign>)
+                  : go(d, &scatter_nd_kernel<__half, 1, ScatterMode::kAssign>);
+}
+
 }  // extern "C"
