@@ -250,9 +250,24 @@ __global__ void __launch_bounds__(512) k_row_ops(const Element* src, Element* ou
         op(r, v);
         compute::BroadcastSub<Vec, Reg, tl::Layout::kRowMajor> bs;
         bs(v, r);
-    } else {
+    } else if constexpr (kOp == 4) {
         compute::Softmax<Reg, tl::Layout::kRowMajor> sm;
         sm(r, v);
+    } else if constexpr (kOp == 5) {
+        compute::SumReduce<Reg, tl::Layout::kRowMajor> op;
+        op(r, v);
+        compute::BroadcastAdd<Vec, Reg, tl::Layout::kRowMajor> b;
+        b(v, r);
+    } else if constexpr (kOp == 6) {
+        compute::MaxReduce<Reg, tl::Layout::kRowMajor> op;
+        op(r, v);
+        compute::BroadcastMul<Vec, Reg, tl::Layout::kRowMajor> b;
+        b(v, r);
+    } else {
+        compute::SumReduce<Reg, tl::Layout::kRowMajor> op;
+        op(r, v);
+        compute::BroadcastDiv<Vec, Reg, tl::Layout::kRowMajor> b;
+        b(v, r);
     }
     // every lane of a row group holds the row value; lanes 0..15 of each wavefront write it
     const int lane = lane_id();
@@ -284,11 +299,24 @@ __global__ void __launch_bounds__(512) k_col_ops(const Element* src, Element* ou
     } else if constexpr (kOp == 1) {
         compute::MaxReduce<Reg, tl::Layout::kColMajor> op;
         op(r, v);
-    } else {
+    } else if constexpr (kOp == 2) {
         compute::MaxReduce<Reg, tl::Layout::kColMajor> op;
         op(r, v);
         compute::BroadcastSub<Vec, Reg, tl::Layout::kColMajor> bs;
         bs(v, r);
+    } else if constexpr (kOp == 3) {
+        compute::SumReduce<Reg, tl::Layout::kColMajor> op;
+        op(r, v);
+        compute::Broadcast<Vec, Reg, tl::Layout::kColMajor> bc;
+        bc(v, r);
+    } else if constexpr (kOp == 4) {
+        compute::Softmax<Reg, tl::Layout::kColMajor> sm;
+        sm(r, v);
+    } else {
+        compute::MaxReduce<Reg, tl::Layout::kColMajor> op;
+        op(r, v);
+        compute::BroadcastMul<Vec, Reg, tl::Layout::kColMajor> b;
+        b(v, r);
     }
     const int lane = lane_id();
     if (lane < 16) {
@@ -298,6 +326,49 @@ __global__ void __launch_bounds__(512) k_col_ops(const Element* src, Element* ou
     Global g_out(out_tile);
     RegToGlobalStorer<Global, Reg, WarpLayout> r2g;
     r2g(r, g_out);
+}
+
+// element-wise maps: out = op(a) or op(a, b) on [kRows, kCols] tiles in either orientation, kW wavefronts.
+// kOp: 0 exp, 1 log, 2 relu, 3 add, 4 sub, 5 mul, 6 div, 7 max, 8 min, 9 convert f32 -> f16 (out is __half)
+template <typename Element, bool kRowMajor, int kRows, int kCols, int kW, int kOp>
+__global__ void __launch_bounds__(512) k_elementwise(const Element* a, const Element* b, void* out) {
+    using WarpLayout = std::conditional_t<kRowMajor, tl::RowMajor<kW, 1>, tl::RowMajor<1, kW>>;
+    using GLayout = std::conditional_t<kRowMajor, tl::RowMajor<kRows, kCols>, tl::ColMajor<kRows, kCols>>;
+    constexpr int kRs = kRowMajor ? kRows / kW / 16 : kRows / 16;
+    constexpr int kCs = kRowMajor ? kCols / 16 : kCols / kW / 16;
+    using RLayout = std::conditional_t<kRowMajor, tl::RowMajor<kRs, kCs>, tl::ColMajor<kRs, kCs>>;
+    using Base = std::conditional_t<kRowMajor, BaseTileRowMajor<Element>, BaseTileColMajor<Element>>;
+    using Reg = RegTile<Base, RLayout>;
+    using Global = GlobalTile<Element, GLayout>;
+    Global ga(a), gb(b);
+    Reg ra, rb, rc;
+    GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
+    g2r(ga, ra);
+    g2r(gb, rb);
+    if constexpr (kOp == 9) {
+        using HBase = std::conditional_t<kRowMajor, BaseTileRowMajor<__half>, BaseTileColMajor<__half>>;
+        using HReg = RegTile<HBase, RLayout>;
+        using HGlobal = GlobalTile<__half, GLayout>;
+        HReg rh;
+        compute::RegTileConvert<Reg, HReg> cvt;
+        cvt(ra, rh);
+        HGlobal go(static_cast<__half*>(out));
+        RegToGlobalStorer<HGlobal, HReg, WarpLayout> r2g;
+        r2g(rh, go);
+    } else {
+        if constexpr (kOp == 0) { compute::RegTileExp<Reg> op; op(ra, rc); }
+        if constexpr (kOp == 1) { compute::RegTileLog<Reg> op; op(ra, rc); }
+        if constexpr (kOp == 2) { compute::RegTileRelu<Reg> op; op(ra, rc); }
+        if constexpr (kOp == 3) { compute::RegTileAdd<Reg> op; op(ra, rb, rc); }
+        if constexpr (kOp == 4) { compute::RegTileSub<Reg> op; op(ra, rb, rc); }
+        if constexpr (kOp == 5) { compute::RegTileMul<Reg> op; op(ra, rb, rc); }
+        if constexpr (kOp == 6) { compute::RegTileDiv<Reg> op; op(ra, rb, rc); }
+        if constexpr (kOp == 7) { compute::RegTileMax<Reg> op; op(ra, rb, rc); }
+        if constexpr (kOp == 8) { compute::RegTileMin<Reg> op; op(ra, rb, rc); }
+        Global go(static_cast<Element*>(out));
+        RegToGlobalStorer<Global, Reg, WarpLayout> r2g;
+        r2g(rc, go);
+    }
 }
 
 // ------------------------------------------------------------------ registry
@@ -407,7 +478,7 @@ void reg_gemm() {
 
 template <typename E, int kRows, int kCols, int kW, int kOp>
 void reg_row_op() {
-    static const char* names[] = {"sum", "max", "bcast_sum", "sub_max", "softmax"};
+    static const char* names[] = {"sum", "max", "bcast_sum", "sub_max", "softmax", "add_sum", "mul_max", "div_sum"};
     registry().push_back({"row_ops",
                           std::string(ename<E>()) + "_" + names[kOp] + "_" + std::to_string(kRows) + "x" +
                               std::to_string(kCols) + "_w" + std::to_string(kW),
@@ -419,7 +490,7 @@ void reg_row_op() {
 
 template <typename E, int kRows, int kCols, int kW, int kOp>
 void reg_col_op() {
-    static const char* names[] = {"sum", "max", "sub_max"};
+    static const char* names[] = {"sum", "max", "sub_max", "bcast_sum", "softmax", "mul_max"};
     registry().push_back({"col_ops",
                           std::string(ename<E>()) + "_" + names[kOp] + "_" + std::to_string(kRows) + "x" +
                               std::to_string(kCols) + "_w" + std::to_string(kW),
@@ -427,6 +498,23 @@ void reg_col_op() {
                           kW * 64,
                           0,
                           &launch_ops<k_col_ops<E, kRows, kCols, kW, kOp>, E>});
+}
+
+template <auto Kernel, typename E>
+void launch_elementwise(const void* a, const void* b, void* c, void*, int threads, int lds, hipStream_t s) {
+    hipLaunchKernelGGL(Kernel, dim3(1), dim3(threads), lds, s, static_cast<const E*>(a), static_cast<const E*>(b), c);
+}
+
+template <typename E, bool kRowMajor, int kRows, int kCols, int kW, int kOp>
+void reg_elementwise() {
+    static const char* names[] = {"exp", "log", "relu", "add", "sub", "mul", "div", "max", "min", "convert_f16"};
+    registry().push_back({"elementwise",
+                          std::string(ename<E>()) + "_" + names[kOp] + (kRowMajor ? "_row_" : "_col_") +
+                              std::to_string(kRows) + "x" + std::to_string(kCols) + "_w" + std::to_string(kW),
+                          {kRows, kCols, kOp, int(sizeof(E)), kRowMajor, 0, 0, 0},
+                          kW * 64,
+                          0,
+                          &launch_elementwise<k_elementwise<E, kRowMajor, kRows, kCols, kW, kOp>, E>});
 }
 
 template <typename E, bool kSwz>
@@ -540,6 +628,39 @@ void build_registry() {
     reg_col_op<float, 64, 32, 2, 1>();
     reg_col_op<float, 64, 32, 1, 2>();
     reg_col_op<__half, 32, 32, 1, 0>();
+    reg_row_op<float, 32, 64, 2, 5>();
+    reg_row_op<float, 32, 32, 1, 6>();
+    reg_row_op<float, 64, 32, 4, 7>();
+    reg_row_op<__half, 32, 32, 1, 7>();
+    reg_col_op<float, 32, 64, 2, 3>();
+    reg_col_op<float, 16, 16, 1, 4>();
+    reg_col_op<float, 64, 32, 2, 4>();
+    reg_col_op<__half, 32, 32, 1, 4>();
+    reg_col_op<float, 32, 32, 1, 5>();
+
+    // element-wise maps (reference: map.hpp:84-133, math_functor.hpp): every functor, both orientations
+    reg_elementwise<float, true, 32, 32, 1, 0>();
+    reg_elementwise<float, true, 32, 32, 1, 1>();
+    reg_elementwise<float, true, 32, 64, 2, 2>();
+    reg_elementwise<float, true, 64, 32, 4, 3>();
+    reg_elementwise<float, true, 32, 32, 1, 4>();
+    reg_elementwise<float, true, 32, 32, 1, 5>();
+    reg_elementwise<float, true, 32, 32, 1, 6>();
+    reg_elementwise<float, true, 32, 32, 2, 7>();
+    reg_elementwise<float, true, 32, 32, 2, 8>();
+    reg_elementwise<float, true, 32, 64, 2, 9>();
+    reg_elementwise<float, false, 32, 64, 2, 0>();
+    reg_elementwise<float, false, 64, 32, 1, 6>();
+    reg_elementwise<float, false, 32, 32, 1, 8>();
+    reg_elementwise<float, false, 32, 32, 1, 9>();
+    reg_elementwise<__half, true, 32, 32, 1, 0>();
+    reg_elementwise<__half, true, 32, 32, 1, 1>();
+    reg_elementwise<__half, true, 32, 32, 1, 2>();
+    reg_elementwise<__half, true, 32, 64, 2, 3>();
+    reg_elementwise<__half, true, 32, 32, 1, 5>();
+    reg_elementwise<__half, true, 32, 32, 1, 6>();
+    reg_elementwise<__half, false, 32, 32, 1, 7>();
+    reg_elementwise<__half, false, 32, 32, 1, 8>();
 }
 
 thread_local std::string g_err;
@@ -570,6 +691,7 @@ int tt_case_info(int id, const char** kind, const char** name, int* dims, int* t
 ///   copies:    a = src, c = dst
 ///   tile_gemm: a = A, b = B, c = C
 ///   row/col ops: a = src, c = per-line vector, d = tile output
+///   elementwise: a, b = operands, c = result
 int tt_run_case(int id, const void* a, const void* b, void* c, void* d, void* stream) {
     build_registry();
     if (id < 0 || id >= (int)registry().size()) return -1;

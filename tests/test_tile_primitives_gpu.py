@@ -47,7 +47,7 @@ def test_registry_is_populated():
     assert os.path.exists(LIB), "device test library missing: run __graft_entry__.build()"
     kinds = {c[1] for c in CASES}
     assert kinds == {"g2s_roundtrip", "s2r_identity", "store_roundtrip", "g2r_roundtrip", "tile_gemm", "row_ops",
-                     "col_ops"}
+                     "col_ops", "elementwise"}
 
 
 def _np_dtype(nbytes):
@@ -106,8 +106,10 @@ def test_tile_case(case, device, oracle):
         x64 = x.astype(np.float64)
         axis = 1 if row_major else 0
         tol = 1e-3 if dt == np.float32 else 0.15  # f16 sums of up to 64 values of magnitude 5
-        names = ["sum", "max", "bcast_sum", "sub_max", "softmax"] if row_major else ["sum", "max", "sub_max"]
+        names = (["sum", "max", "bcast_sum", "sub_max", "softmax", "add_sum", "mul_max", "div_sum"] if row_major
+                 else ["sum", "max", "sub_max", "bcast_sum", "softmax", "mul_max"])
         opname = names[op]
+        keep = dict(axis=axis, keepdims=True)
         if opname == "sum":
             assert np.allclose(v, x64.sum(axis), atol=tol)
             assert np.array_equal(t, x64)
@@ -115,11 +117,49 @@ def test_tile_case(case, device, oracle):
             assert np.array_equal(v, x64.max(axis))
         elif opname == "bcast_sum":
             assert np.allclose(v, x64.sum(axis), atol=tol)
-            assert np.allclose(t, np.repeat(x64.sum(1, keepdims=True), cols, 1), atol=tol)
+            assert np.allclose(t, np.broadcast_to(x64.sum(**keep), x64.shape), atol=tol)
         elif opname == "sub_max":
             assert np.allclose(t, x64 - x64.max(axis, keepdims=True), atol=1e-6 if dt == np.float32 else 1e-2)
         elif opname == "softmax":
-            e = np.exp(x64 - x64.max(1, keepdims=True))
-            assert np.allclose(t, e / e.sum(1, keepdims=True), atol=1e-3)  # the reference's tolerance
+            e = np.exp(x64 - x64.max(**keep))
+            assert np.allclose(t, e / e.sum(**keep), atol=1e-3)  # the reference's tolerance
+        elif opname == "add_sum":
+            assert np.allclose(t, x64 + x64.sum(**keep), atol=tol)
+        elif opname == "mul_max":
+            assert np.allclose(t, x64 * x64.max(**keep), atol=1e-5 if dt == np.float32 else 0.05)
+        elif opname == "div_sum":
+            # sums of U[-5, 5] values can come close to 0: compare x = t * sum instead of dividing
+            assert np.allclose(t * x64.sum(**keep), x64, atol=1e-3 if dt == np.float32 else 0.5)
+    elif kind == "elementwise":
+        rows, cols, op, nbytes, row_major = dims[:5]
+        dt = _np_dtype(nbytes)
+        rng = np.random.default_rng(77 + idx)
+        opname = ["exp", "log", "relu", "add", "sub", "mul", "div", "max", "min", "convert_f16"][op]
+        xa = rng.uniform(-4, 4, (rows, cols)).astype(dt)
+        xb = rng.uniform(-4, 4, (rows, cols)).astype(dt)
+        if opname == "log":
+            xa = np.abs(xa) + dt(0.05)
+        if opname == "div":
+            xb = (np.sign(xb) * (np.abs(xb) + dt(0.25))).astype(dt)
+        store = (lambda m: m) if row_major else (lambda m: np.ascontiguousarray(m.T))
+        a, b = (torch.from_numpy(store(m).copy()).to(device) for m in (xa, xb))
+        out_dt = torch.float16 if opname == "convert_f16" else a.dtype
+        c = torch.full(store(xa).shape, float("nan"), dtype=out_dt, device=device)
+        run(a, b, c, None)
+        got = c.cpu().numpy()
+        got = (got if row_major else got.T).astype(np.float64)
+        a64, b64 = xa.astype(np.float64), xb.astype(np.float64)
+        exact = {"relu": np.maximum(a64, 0), "max": np.maximum(a64, b64), "min": np.minimum(a64, b64)}
+        if opname in exact:
+            assert np.array_equal(got, exact[opname])
+        elif opname == "convert_f16":
+            assert np.array_equal(got, xa.astype(np.float16).astype(np.float64))  # round-to-nearest-even
+        else:
+            want = {"exp": lambda: np.exp(a64), "log": lambda: np.log(a64), "add": lambda: a64 + b64,
+                    "sub": lambda: a64 - b64, "mul": lambda: a64 * b64, "div": lambda: a64 / b64}[opname]()
+            # f32: the fast-math exp/log/div of the reference's functors (__expf, __logf) are good to ~1e-6 relative;
+            # f16: one rounding of the result (2^-11) plus the rounding inside hexp/hlog
+            rtol = 2e-6 if dt == np.float32 else 2e-3
+            assert np.allclose(got, want, rtol=rtol, atol=rtol)
     else:
         raise AssertionError(kind)
