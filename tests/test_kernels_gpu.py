@@ -199,7 +199,34 @@ def test_flash_attention_reference_shapes(tcu, oracle, device, n):
     assert oracle.max_abs_err(host(O), ref) <= ABS_TOL
 
 
-@pytest.mark.parametrize("algo", ["tile_library", "mfma32"])
+@pytest.mark.parametrize("algo", ["tile_library", "mfma32", "mfma32_fused"])
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("q_gain,k_growth,tol", [(2.0, 3.0, ABS_TOL), (4.0, 8.0, 5e-2)])
+def test_flash_attention_growing_maxima(tcu, oracle, device, algo, D, q_gain, k_growth, tol):
+    """Keys whose norm grows along the sequence and large queries: the row maxima move in many key blocks, so the
+    rescale path of mfma32 and the failed-speculation path of mfma32_fused run all the time; also a block of
+    keys far *below* the maximum (probabilities that underflow) and one query row of zeros (uniform weights).
+    First setting: logits up to about +-30, the usual tolerance. Second setting: logits up to about +-150, where
+    near-ties between the top keys are decided by the rounding of the scores themselves (the tuned kernels take
+    Q pre-multiplied by scale * log2(e) in f16: relative error 2^-11 per product term), hence the looser bound."""
+    import torch
+
+    batch, M, N = 2, 256, 1024
+    q = oracle.fill_normal(batch * M * D, 51).reshape(batch, M, D).astype(np.float32) * q_gain
+    k = oracle.fill_normal(batch * N * D, 52).reshape(batch, N, D).astype(np.float32)
+    k *= (1.0 + k_growth * np.arange(N, dtype=np.float32) / N)[None, :, None]
+    k[:, 512:576] *= 0.01
+    q[:, 7] = 0.0
+    v = oracle.fill_normal(batch * N * D, 53).reshape(batch, N, D)
+    q, k = q.astype(np.float16), k.astype(np.float16)
+    O = tcu.flash_attention(dev(q, device), dev(k, device), dev(v, device), algo=algo)
+    torch.cuda.synchronize()
+    ref = oracle.attention(q, k, v, 1.0 / math.sqrt(D))
+    assert np.isfinite(host(O)).all()
+    assert oracle.max_abs_err(host(O), ref) <= tol
+
+
+@pytest.mark.parametrize("algo", ["tile_library", "mfma32", "mfma32_fused"])
 @pytest.mark.parametrize("batch,M,N,D", [(1, 64, 64, 128), (3, 128, 192, 128), (2, 256, 512, 128), (2, 128, 256, 64),
                                          (1, 512, 1024, 128), (2, 192, 64, 64)])
 def test_flash_attention_row_major_v(tcu, oracle, device, batch, M, N, D, algo):
@@ -232,6 +259,9 @@ def test_flash_attention_properties(tcu, oracle, device):
     O1 = tcu.flash_attention(q, k, v)
     O2 = tcu.flash_attention(q, k[:, perm].contiguous(), v[:, perm].contiguous())
     assert torch.allclose(O1.float(), O2.float(), atol=4e-3)
+    # the two tuned kernels compute the same thing
+    O3 = tcu.flash_attention(q, k, v, algo="mfma32")
+    assert torch.allclose(O1.float(), O3.float(), atol=2e-3)
 
 
 def test_flash_attention_config4(tcu, oracle, device):

@@ -186,21 +186,21 @@ int launch_fa(const __half* Q, const __half* K, const __half* V, __half* O, int 
                   scale);
 }
 
-template <int kD, int kWaves>
+template <int kD, int kWaves, bool kFused>
 int launch_fa_fwd(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
                   hipStream_t stream) {
     using Traits = FlashFwdTraits<kD, kWaves, 64>;
-    auto kernel = &flash_attention_fwd<Traits>;
+    auto kernel = kFused ? &flash_attention_fwd_fused<Traits> : &flash_attention_fwd<Traits>;
     return launch(kernel, dim3((M / Traits::kBM) * batch), dim3(Traits::kThreads), Traits::kLdsBytes, stream, Q, K, V,
                   O, batch, M, N, scale);
 }
 
-template <int kD>
+template <int kD, bool kFused>
 int fa_fwd_by_rows(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
                    hipStream_t stream) {
-    if (M % 256 == 0) return launch_fa_fwd<kD, 8>(Q, K, V, O, batch, M, N, scale, stream);
-    if (M % 128 == 0) return launch_fa_fwd<kD, 4>(Q, K, V, O, batch, M, N, scale, stream);
-    return launch_fa_fwd<kD, 2>(Q, K, V, O, batch, M, N, scale, stream);
+    if (M % 256 == 0) return launch_fa_fwd<kD, 8, kFused>(Q, K, V, O, batch, M, N, scale, stream);
+    if (M % 128 == 0) return launch_fa_fwd<kD, 4, kFused>(Q, K, V, O, batch, M, N, scale, stream);
+    return launch_fa_fwd<kD, 2, kFused>(Q, K, V, O, batch, M, N, scale, stream);
 }
 
 int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, int Kd, int P,
@@ -208,15 +208,18 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     using W41 = tl::RowMajor<4, 1>;
     if (Kd != P) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs the query and value head sizes equal");
     if (M % 64 != 0 || N % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs M % 64 == 0 and N % 64 == 0");
-    if (algo != TCU_ATTN_AUTO && algo != TCU_ATTN_TILE_LIBRARY && algo != TCU_ATTN_MFMA32)
+    if (algo != TCU_ATTN_AUTO && algo != TCU_ATTN_TILE_LIBRARY && algo != TCU_ATTN_MFMA32 && algo != TCU_ATTN_MFMA32_FUSED)
         return fail(TCU_ERR_INVALID_ARGUMENT, "unknown attention algo");
     if (v_layout == TCU_V_ROW_MAJOR && algo != TCU_ATTN_TILE_LIBRARY) {
-        if (Kd == 128) return fa_fwd_by_rows<128>(Q, K, V, O, batch, M, N, scale, stream);
-        if (Kd == 64) return fa_fwd_by_rows<64>(Q, K, V, O, batch, M, N, scale, stream);
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
+        if (Kd != 128 && Kd != 64) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
+        if (algo == TCU_ATTN_MFMA32)
+            return Kd == 128 ? fa_fwd_by_rows<128, false>(Q, K, V, O, batch, M, N, scale, stream)
+                             : fa_fwd_by_rows<64, false>(Q, K, V, O, batch, M, N, scale, stream);
+        return Kd == 128 ? fa_fwd_by_rows<128, true>(Q, K, V, O, batch, M, N, scale, stream)
+                         : fa_fwd_by_rows<64, true>(Q, K, V, O, batch, M, N, scale, stream);
     }
-    if (algo == TCU_ATTN_MFMA32)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 32x32x16 attention kernel takes a row-major V");
+    if (algo == TCU_ATTN_MFMA32 || algo == TCU_ATTN_MFMA32_FUSED)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 32x32x16 attention kernels take a row-major V");
     if (v_layout == TCU_V_ROW_MAJOR) {
         if (Kd == 128) return launch_fa<0, 128, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
         if (Kd == 64) return launch_fa<0, 64, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
