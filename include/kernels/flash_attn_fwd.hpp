@@ -15,7 +15,10 @@
 //   * Q stays in registers for the whole kernel (it is read from HBM once, where the
 //     reference re-reads it for every key block, flash_attn.cu:241);
 //   * K and V blocks go global -> LDS directly (16 B per lane, no register staging) into a ring of
-//     three stages; one barrier per block;
+//     three stages; one barrier per block; the loads are issued through inline assembly
+//     (detail::load_lds_16B_untracked): with the builtin the compiler waits for the block just requested
+//     (s_waitcnt vmcnt(0)) before the next LDS read, because it cannot prove that the read does not alias
+//     the stage being filled, and the ring degenerates to one block at a time;
 //   * the two wavefronts that share a SIMD run an iteration in different orders (scores of block j+1
 //     first / last), so one of them feeds the matrix pipe while the other does the softmax VALU work;
 //   * LDS rows are 2 * kD bytes. K: the 16-byte chunks of a row are XOR-ed with the row index
@@ -138,7 +141,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 // physical chunk lchk holds logical chunk lchk ^ swizzle(row)
                 const int chunk = is_v ? (lchk ^ (Traits::v_swz(row) << 1)) : (lchk ^ Traits::k_swz(row));
                 const __half* src = (is_v ? Vh : Kh) + size_t(n0 + row) * kD + chunk * 8;
-                detail::load_lds_16B(src, sk + (is_v ? Traits::kTileBytes : 0) + t * 1024);
+                detail::load_lds_16B_untracked(src, sk + (is_v ? Traits::kTileBytes : 0) + t * 1024);
             }
         }
     };
@@ -406,7 +409,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 const int row = t * Traits::kRowsPerLoad + lrow;
                 const int chunk = is_v ? (lchk ^ (Traits::v_swz(row) << 1)) : (lchk ^ Traits::k_swz(row));
                 const __half* src = (is_v ? Vh : Kh) + size_t(n0 + row) * kD + chunk * 8;
-                detail::load_lds_16B(src, sk + (is_v ? Traits::kTileBytes : 0) + t * 1024);
+                detail::load_lds_16B_untracked(src, sk + (is_v ? Traits::kTileBytes : 0) + t * 1024);
             }
         }
     };

@@ -79,6 +79,22 @@ DEVICE void load_lds_16B(const void* gptr, void* lds_wave_base) {
     __builtin_amdgcn_global_load_lds((glb_ptr_t)gptr, (lds_ptr_t)lds_wave_base, 16, 0, 0);
 }
 
+/// Direct-to-LDS load of 16 bytes per lane (lane i's data lands at lds_wave_base + 16 i) issued as inline assembly, so
+/// that the compiler does not know it writes LDS. With the builtin, the compiler makes every later LDS read (and every
+/// barrier fence) wait for *all* outstanding direct-to-LDS loads (s_waitcnt vmcnt(0)), because it cannot prove that the
+/// read does not alias a tile still in flight; that serialises a ring of stages to one tile at a time. Here the
+/// kernel's own s_waitcnt vmcnt(N) before the barrier that hands a stage over is the only synchronisation.
+/// kAgentScope: request at agent scope (sc1), past this XCD's L2, for data written by other workgroups in this launch.
+template <bool kAgentScope = false>
+DEVICE void load_lds_16B_untracked(const void* gptr, const void* lds_wave_base) {
+    const unsigned int lds_addr = __builtin_amdgcn_readfirstlane(
+        static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds_wave_base)));
+    if constexpr (kAgentScope)
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off sc1" ::"v"(gptr), "s"(lds_addr) : "m0", "memory");
+    else
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "m0", "memory");
+}
+
 /// Tile coordinates for workgroup `bid` of a grid of tiles_m x tiles_n tiles: ids that are
 /// congruent modulo 8 (same XCD) are gathered into compact blocks of tiles.
 HOST_DEVICE void xcd_tile_coords(int bid, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {

@@ -59,6 +59,15 @@ template <int N>
 DEVICE void wait_vmcnt_lgkm0() {
     __builtin_amdgcn_s_waitcnt(0x0070 | (N & 0xF) | ((N >> 4) << 14));
 }
+
+/// Workgroup barrier that orders LDS accesses only. __syncthreads() also waits for every outstanding global memory
+/// operation of the wavefront (s_waitcnt vmcnt(0)), which would drain the ring of direct-to-LDS loads at every tile:
+/// the tiles requested ahead must stay in flight across the barrier.
+DEVICE void lds_barrier() {
+    // (a workgroup-scope fence restricted to LDS still waits for vmcnt(0): direct-to-LDS loads count as LDS writes)
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS reads and writes are done
+    __builtin_amdgcn_s_barrier();
+}
 }  // namespace detail
 
 /// grid = (B / 64) * (H / 16) workgroups (1-D), block = 512, dynamic LDS = Traits::kLdsBytes.
@@ -109,7 +118,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 const int wrow = ((row >> 3) & 3) * kH + hid0 + 8 * (row >> 5) + (row & 7);
                 src = W + size_t(wrow) * kKK + k0 + chunk * 8;
             }
-            detail::load_lds_16B(src, sbase + t * 1024);
+            detail::load_lds_16B_untracked(src, sbase + t * 1024);
         }
     };
 
@@ -148,7 +157,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         // stages of L loads each; in the tail (fewer stages issued after p) wait for everything.
         if (p + S - 2 <= ktiles - 1) detail::wait_vmcnt_lgkm0<(S - 2) * L>();
         else detail::wait_vmcnt_lgkm0<0>();
-        __syncthreads();  // everyone's share of stage p landed; everyone finished reading stage p-1 (= `fill`)
+        detail::lds_barrier();  // everyone's share of stage p landed; everyone finished reading stage p-1 (= `fill`)
         if (p + S - 1 < ktiles) issue_stage(fill, p + S - 1);
 
         {
@@ -174,7 +183,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     for (int e = 0; e < 16; ++e) acc[e] = acc0[e] + acc1[e];
 
     // ---- add the two groups' partial sums: group 1 parks its accumulators in LDS (16 f32 per lane)
-    __syncthreads();  // all reads of the last stage are done
+    detail::lds_barrier();  // all reads of the last stage are done
     float* park = reinterpret_cast<float*>(lds) + ((wave & 3) * 64 + lane) * 16;
     if (group == 1) {
 #pragma unroll
@@ -183,7 +192,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
             *reinterpret_cast<f32x4*>(park + 4 * q) = v;
         }
     }
-    __syncthreads();
+    detail::lds_barrier();
     if (group == 1) return;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {

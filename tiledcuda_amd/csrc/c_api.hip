@@ -49,8 +49,10 @@ int launch(Kernel kernel, dim3 grid, dim3 block, int lds_bytes, hipStream_t stre
             known = g_attr_done.count(key) != 0;
         }
         if (!known) {
+            // (every instantiation is launched with one fixed size; asking for the CU's whole LDS would be refused
+            // for a kernel that also has static LDS)
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
             if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
             std::lock_guard<std::mutex> lock(g_attr_mutex);
             g_attr_done.insert(key);
