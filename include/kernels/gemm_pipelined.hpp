@@ -95,6 +95,20 @@ DEVICE void load_lds_16B_untracked(const void* gptr, const void* lds_wave_base) 
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "m0", "memory");
 }
 
+/// Workgroup barrier that orders LDS accesses only. __syncthreads() also waits for every outstanding global memory
+/// operation of the wavefront (s_waitcnt vmcnt(0): its workgroup fence covers the LDS writes of direct-to-LDS loads),
+/// which would drain a ring of stages at every hand-over: tiles requested ahead must stay in flight across the barrier.
+/// kVmcnt: additionally wait until at most that many of this wavefront's vector-memory operations are outstanding.
+/// The empty asm statements keep the compiler from moving LDS accesses across the sequence (the two builtins are
+/// declared as not touching memory).
+template <int kVmcnt = 63>
+DEVICE void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070 | (kVmcnt & 0xF) | ((kVmcnt >> 4) << 14));  // vmcnt(kVmcnt) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 /// Tile coordinates for workgroup `bid` of a grid of tiles_m x tiles_n tiles: ids that are
 /// congruent modulo 8 (same XCD) are gathered into compact blocks of tiles.
 HOST_DEVICE void xcd_tile_coords(int bid, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {

@@ -60,14 +60,6 @@ DEVICE void wait_vmcnt_lgkm0() {
     __builtin_amdgcn_s_waitcnt(0x0070 | (N & 0xF) | ((N >> 4) << 14));
 }
 
-/// Workgroup barrier that orders LDS accesses only. __syncthreads() also waits for every outstanding global memory
-/// operation of the wavefront (s_waitcnt vmcnt(0)), which would drain the ring of direct-to-LDS loads at every tile:
-/// the tiles requested ahead must stay in flight across the barrier.
-DEVICE void lds_barrier() {
-    // (a workgroup-scope fence restricted to LDS still waits for vmcnt(0): direct-to-LDS loads count as LDS writes)
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS reads and writes are done
-    __builtin_amdgcn_s_barrier();
-}
 }  // namespace detail
 
 /// grid = (B / 64) * (H / 16) workgroups (1-D), block = 512, dynamic LDS = Traits::kLdsBytes.

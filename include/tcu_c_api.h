@@ -34,6 +34,13 @@ typedef enum {
     TCU_GEMM_PIPELINED = 3   /* direct-to-LDS, double-buffered, 16x16x32 MFMA */
 } tcu_gemm_algo;
 
+/* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks RESIDENT where it is instantiated. */
+typedef enum {
+    TCU_B2B_AUTO = 0,
+    TCU_B2B_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, the reference kernel's structure */
+    TCU_B2B_RESIDENT = 2      /* A tile, B, C and the intermediate all resident in LDS, one round of loads */
+} tcu_b2b_algo;
+
 /* Layout of V in tcu_flash_attn_fwd_f16. */
 typedef enum {
     TCU_V_COL_MAJOR = 0, /* V stored [P, N] per batch item: the reference op's convention */
@@ -84,6 +91,10 @@ int tcu_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K, int
  */
 int tcu_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D, int M, int N, int K, int P, int batch,
                      int out_dtype, void* stream);
+
+/* tcu_b2b_gemm_f16 with an explicit kernel choice (tcu_b2b_algo); same arguments otherwise. */
+int tcu_b2b_gemm_f16_algo(const void* A, const void* B, const void* C, void* D, int M, int N, int K, int P, int batch,
+                          int out_dtype, int algo, void* stream);
 
 /*
  * O[b, M, P] = softmax(scale · Q[b, M, K] · K[b]) · V[b], f16 in / f16 out, f32 softmax

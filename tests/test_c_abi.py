@@ -57,6 +57,8 @@ def test_bad_sizes_and_enums_are_rejected(tcu):
     assert "out_dtype" in tcu.last_error()
     assert l.tcu_gemm_f16(p, p, p, 64, 64, 64, 0, 9, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
     assert l.tcu_b2b_gemm_f16(p, p, p, p, 64, 64, 64, 64, -1, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_b2b_gemm_f16_algo(p, p, p, p, 64, 256, 128, 128, 1, 0, 9, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_b2b_gemm_f16_algo(p, p, p, p, 64, 64, 64, 64, 1, 0, 2, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 64, 128, 128, 1.0, 5, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
     dims = (ctypes.c_longlong * 2)(4, 4)
     assert l.tcu_scatter_nd(0, p, p, dims, 2, 1, 1, 0, 0, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT

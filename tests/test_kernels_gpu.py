@@ -159,6 +159,38 @@ def test_b2b_gemm_shapes(tcu, oracle, device, M, N, K, P, batch, out_dtype):
     assert oracle.max_rel_err(host(D), ref, eps=1.0) <= REL_TOL
 
 
+@pytest.mark.parametrize("algo", ["tile_library", "resident"])
+@pytest.mark.parametrize("M,batch,out_dtype", [(32, 1, "f32"), (96, 3, "f16"), (8192, 1, "f16"), (16384, 2, "f32")])
+def test_b2b_gemm_both_kernels_at_256x128x128(tcu, oracle, device, algo, M, batch, out_dtype):
+    """(N, K, P) = (256, 128, 128): the tile-library kernel and the LDS-resident kernel against the oracle, one
+    workgroup, ragged workgroup counts, the C3 size and a two-item batch; plus a one-hot probe of the index maps."""
+    import torch
+
+    print(f"b2b {algo} M{M} b{batch} {out_dtype}", flush=True)
+    N, K, P = 256, 128, 128
+    A = oracle.fill_normal(batch * M * K, 71, 0, 0.1).reshape(batch, M, K)
+    Bt = oracle.fill_normal(batch * N * K, 72, 0, 0.1).reshape(batch, N, K)
+    Ct = oracle.fill_normal(batch * P * N, 73, 0, 0.1).reshape(batch, P, N)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    D = tcu.b2b_gemm(dev(A, device), dev(Bt, device), dev(Ct, device), out_dtype=dt, algo=algo)
+    torch.cuda.synchronize()
+    rows = slice(0, M) if M <= 256 else slice(M // 2 - 48, M // 2 + 48)
+    ref = oracle.b2b_gemm(np.ascontiguousarray(A[:, rows]), Bt, Ct)
+    assert oracle.max_rel_err(host(D)[:, rows], ref, eps=1.0) <= REL_TOL
+    if M == 96:
+        # D[m, p] = A[m, k] B[k, n] C[n, p] with one-hot operands: exact, and wrong if any index is permuted
+        A1 = torch.zeros(1, 96, K, dtype=torch.float16, device=device)
+        B1 = torch.zeros(1, N, K, dtype=torch.float16, device=device)
+        C1 = torch.zeros(1, P, N, dtype=torch.float16, device=device)
+        for i, (m, k, n, p) in enumerate([(0, 0, 0, 0), (95, 127, 255, 127), (37, 5, 200, 66), (64, 77, 13, 1)]):
+            A1[0, m, k] = 1.0 + i
+            B1[0, n, k] = 2.0
+            C1[0, p, n] = 0.5
+        D1 = tcu.b2b_gemm(A1, B1, C1, out_dtype=torch.float32, algo=algo)
+        want = (A1[0].float() @ B1[0].float().T) @ C1[0].float().T
+        assert torch.equal(D1[0], want)
+
+
 def test_b2b_gemm_config3(tcu, oracle, device):
     """C3: A [8192x128], B [128x256], C [256x128], N(0, 0.1), f16 D."""
     import torch

@@ -18,7 +18,7 @@ import torch
 
 __all__ = [
     "TcuError", "library_path", "lib", "last_error", "gemm", "b2b_gemm", "flash_attention_fwd",
-    "flash_attention", "TiledFlashAttention", "lstm", "scatter_nd", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS",
+    "flash_attention", "TiledFlashAttention", "lstm", "scatter_nd", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS", "B2B_ALGOS",
     "SCATTER_MODES",
 ]
 
@@ -42,6 +42,7 @@ TCU_V_ROW_MAJOR = 1
 
 ATTN_ALGOS = {"auto": 0, "tile_library": 1, "mfma32": 2, "mfma32_fused": 3}
 LSTM_ALGOS = {"auto": 0, "tile_library": 1, "streaming": 2}
+B2B_ALGOS = {"auto": 0, "tile_library": 1, "resident": 2}
 SCATTER_MODES = {"assign": 0, "add": 1}
 
 # every exported symbol with its ctypes signature (also what the symbol test checks)
@@ -51,6 +52,7 @@ _SIGNATURES = {
     "tcu_device_count": (ctypes.c_int, []),
     "tcu_gemm_f16": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int] * 5 + [ctypes.c_void_p]),
     "tcu_b2b_gemm_f16": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 6 + [ctypes.c_void_p]),
+    "tcu_b2b_gemm_f16_algo": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7 + [ctypes.c_void_p]),
     "tcu_flash_attn_fwd_f16": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int,
                                                                                            ctypes.c_void_p]),
     "tcu_flash_attn_fwd_f16_algo": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int,
@@ -148,7 +150,7 @@ def gemm(a: torch.Tensor, b_t: torch.Tensor, out: torch.Tensor | None = None,
 
 # ------------------------------------------------------------------------------ b2b GEMM
 def b2b_gemm(a: torch.Tensor, b_t: torch.Tensor, c_t: torch.Tensor, out: torch.Tensor | None = None,
-             out_dtype: torch.dtype = torch.float16) -> torch.Tensor:
+             out_dtype: torch.dtype = torch.float16, algo: str = "auto") -> torch.Tensor:
     """D = (A · B) · C per batch item; ``b_t`` [.., N, K] and ``c_t`` [.., P, N] are the
     column-major operands of the reference's fused two-GEMM example stored as arrays."""
     batched = a.dim() == 3
@@ -160,9 +162,9 @@ def b2b_gemm(a: torch.Tensor, b_t: torch.Tensor, c_t: torch.Tensor, out: torch.T
         raise ValueError("operand shapes do not chain: A [b,M,K], b_t [b,N,K], c_t [b,P,N]")
     if out is None:
         out = torch.empty(batch, M, P, dtype=out_dtype, device=a.device)
-    _check(lib().tcu_b2b_gemm_f16(_dev_ptr(a3, torch.float16, "a"), _dev_ptr(b3, torch.float16, "b_t"),
-                                  _dev_ptr(c3, torch.float16, "c_t"), _dev_ptr(out, out.dtype, "out"), M, N, K, P,
-                                  batch, _out_code(out.dtype), _stream()))
+    _check(lib().tcu_b2b_gemm_f16_algo(_dev_ptr(a3, torch.float16, "a"), _dev_ptr(b3, torch.float16, "b_t"),
+                                       _dev_ptr(c3, torch.float16, "c_t"), _dev_ptr(out, out.dtype, "out"), M, N, K, P,
+                                       batch, _out_code(out.dtype), B2B_ALGOS[algo], _stream()))
     return out if batched else out.view(M, P) if out.dim() == 3 else out
 
 

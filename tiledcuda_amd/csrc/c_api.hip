@@ -3,6 +3,7 @@
 // synchronised; errors become status codes plus a thread-local message.
 #include "tcu_c_api.h"
 
+#include "kernels/b2b_gemm_fwd.hpp"
 #include "kernels/flash_attn_fwd.hpp"
 #include "kernels/gemm_pipelined.hpp"
 #include "kernels/lstm_fwd.hpp"
@@ -161,7 +162,17 @@ int launch_b2b(const __half* A, const __half* B, const __half* C, OutType* D, in
 
 template <typename OutType>
 int b2b_dispatch(const __half* A, const __half* B, const __half* C, OutType* D, int M, int N, int K, int P, int batch,
-                 hipStream_t stream) {
+                 int algo, hipStream_t stream) {
+    if (algo != TCU_B2B_AUTO && algo != TCU_B2B_TILE_LIBRARY && algo != TCU_B2B_RESIDENT)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: unknown algo");
+    if (algo != TCU_B2B_TILE_LIBRARY) {
+        if (N == 256 && K == 128 && P == 128 && M % 32 == 0)
+            return launch(&b2b_gemm_resident<OutType>, dim3(M / B2bResidentTraits::kTM, batch),
+                          dim3(B2bResidentTraits::kThreads), B2bResidentTraits::kLdsBytes, stream, A, B, C, D, M);
+        if (algo == TCU_B2B_RESIDENT)
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE,
+                        "the LDS-resident b2b kernel is instantiated for (N, K, P) = (256, 128, 128) with M a multiple of 32");
+    }
     if (N == 256 && K == 128 && P == 128) {
         // 32-row tiles keep all 256 CUs busy up to M * batch = 8192; 64-row tiles beyond that
         if (M % 64 == 0 && (long)M * batch > 16384)
@@ -309,13 +320,18 @@ int tcu_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K, int
 
 int tcu_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D, int M, int N, int K, int P, int batch,
                      int out_dtype, void* stream) {
+    return tcu_b2b_gemm_f16_algo(A, B, C, D, M, N, K, P, batch, out_dtype, TCU_B2B_AUTO, stream);
+}
+
+int tcu_b2b_gemm_f16_algo(const void* A, const void* B, const void* C, void* D, int M, int N, int K, int P, int batch,
+                          int out_dtype, int algo, void* stream) {
     if (!A || !B || !C || !D) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: null pointer");
     if (!positive({M, N, K, P, batch}))
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: sizes must be positive");
     auto s = static_cast<hipStream_t>(stream);
     auto a = static_cast<const __half*>(A), b = static_cast<const __half*>(B), c = static_cast<const __half*>(C);
-    if (out_dtype == TCU_DTYPE_F32) return b2b_dispatch<float>(a, b, c, static_cast<float*>(D), M, N, K, P, batch, s);
-    if (out_dtype == TCU_DTYPE_F16) return b2b_dispatch<__half>(a, b, c, static_cast<__half*>(D), M, N, K, P, batch, s);
+    if (out_dtype == TCU_DTYPE_F32) return b2b_dispatch<float>(a, b, c, static_cast<float*>(D), M, N, K, P, batch, algo, s);
+    if (out_dtype == TCU_DTYPE_F16) return b2b_dispatch<__half>(a, b, c, static_cast<__half*>(D), M, N, K, P, batch, algo, s);
     return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: out_dtype must be TCU_DTYPE_F32 or TCU_DTYPE_F16");
 }
 
