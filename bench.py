@@ -27,8 +27,8 @@ sys.path.insert(0, ROOT)
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
 HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per launch of the 4096^3 GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# plain 128 MiB copy (profiles/gemm_pipelined_f16_4096x4096x4096.md): 196674 KiB fetched + 32768 KiB written.
-GEMM_4096_TRAFFIC_BYTES = (196674 + 32768) * 1024
+# plain 128 MiB copy (profiles/gemm_w128_f16_4096x4096x4096.md): 196801 KiB fetched + 32768 KiB written.
+GEMM_4096_TRAFFIC_BYTES = (196801 + 32768) * 1024
 
 
 def time_kernel(fn, steps, warmup):
@@ -273,7 +273,7 @@ def main():
                                "(BASELINE configs[1])"},
         "roofline": {"bound": "mfma", "achieved": gemm_tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": gemm_tflops / MFMA_F16_PEAK_TFLOPS, "traffic": GEMM_4096_TRAFFIC_BYTES,
-                     "kernel": "gemm_pipelined<256x256x64, 4x2 wavefronts>", "flops_per_launch": gemm_flops,
+                     "kernel": "gemm_w128<256x256x64, 2x2 wavefronts>", "flops_per_launch": gemm_flops,
                      "avg_launch_us": gemm_ms * 1e3, "sustained_mfma": sustained,
                      "frac_of_sustained_mfma": (gemm_tflops / sustained["tflops"]) if sustained else None},
         "cpu_baseline": cpu,

@@ -1,0 +1,241 @@
+// fp16 GEMM for gfx950 with one wavefront per SIMD: C[M, N] = A[M, K] · B, A row-major, B column-major (stored
+// [N, K]), f32 accumulate, C row-major in f16 or f32. Same contract as kernels/gemm_pipelined.hpp (the multi-stage
+// counterpart of the reference's examples/cpp/01_gemm/02_gemm_all_mem/gemm.hpp:103-155) and bit-identical results;
+// what changes is how the 256 x 256 x 64 workgroup tile is mapped to the CU:
+//   * 4 wavefronts (2 x 2), one per SIMD, each owning a 128 x 128 block of C: 64 v_mfma_f32_16x16x32_f16 per
+//     32-wide k-substep for 16 ds_read_b128 (8 A + 8 B fragments) - a third less LDS traffic per MFMA than the
+//     64 x 128 blocks of the 8-wavefront kernel, and on this part the matrix pipe's clock is set by power, so every
+//     byte not moved is clock for the MFMAs;
+//   * the 256 f32 accumulators per lane live in the AGPR half of the wavefront's 512 registers for the whole kernel.
+//     The MFMAs are issued through inline assembly with AGPR-constrained operands: that pins the accumulators there
+//     (the compiler, left alone, moves them through VGPRs) and fixes the instruction order, which is the point of a
+//     one-wavefront-per-SIMD kernel - nothing else can fill the matrix pipe while this wavefront does something else;
+//   * a tile of K is two phases of 64 MFMAs. Phase 1 (substep 0) also issues the 16 fragment reads of substep 1, one
+//     per two MFMAs; then one LDS-only barrier per tile: tile kt+1 has landed, everyone has left tile kt's stage;
+//     phase 2 (substep 1) also issues the reads of tile kt+1 / substep 0 and this wavefront's 16 direct-to-LDS loads
+//     of tile kt+2 into the stage just vacated, one per four MFMAs (the CU's address unit takes one vector-memory
+//     instruction per ~14 cycles, and a wavefront that has to wait for it issues no MFMAs). A load has a full tile
+//     of MFMA time to land;
+//   * the loads address memory as scalar base + 32-bit lane offset (the k offset advances in scalar registers: no
+//     vector ALU work per load), and each load is one asm statement with the MFMA that precedes it, which is the
+//     wait state the load needs after the write of m0;
+//   * no branches inside the loop over k (the last two tiles are peeled): a taken branch stalls the one instruction
+//     stream that feeds the matrix pipe;
+//   * LDS layout, XOR swizzle, XCD-aware tile order and the LDS-staged 16-byte epilogue are those of
+//     gemm_pipelined.hpp.
+// Because the compiler does not know these asm statements are MFMAs it inserts none of the wait states MFMA results
+// need before other instructions read them; the only such reads are in the epilogue, and every accumulator passes
+// through a waiting statement first (see below). M % 256 == 0, N % 256 == 0, K % 64 == 0 (checked by the launcher).
+#pragma once
+
+#include <type_traits>
+
+#include "config.hpp"
+#include "hip_utils.hpp"
+#include "kernels/gemm_pipelined.hpp"  // detail::lds_barrier, detail::xcd_tile_coords
+
+namespace tiledcuda::kernels {
+
+struct GemmW128Traits {
+    static constexpr int kBM = 256, kBN = 256, kBK = 64;
+    static constexpr int kWaves = 4, kThreads = kWaves * kWaveSize;
+    static constexpr int kWaveM = 128, kWaveN = 128;
+    static constexpr int kMT = kWaveM / 16, kNT = kWaveN / 16;  // 8 x 8 MFMA tiles of 16 x 16 per wavefront
+    static constexpr int kRowBytes = kBK * 2;                   // 128
+    static constexpr int kABytes = kBM * kRowBytes, kBBytes = kBN * kRowBytes;
+    static constexpr int kStageBytes = kABytes + kBBytes;  // 64 KiB
+    static constexpr int kLoads = kBM / 8 / kWaves;        // 1 KiB load instructions per operand per wavefront per stage
+    static constexpr int kLdsBytes = 2 * kStageBytes;      // the f16 epilogue needs 4 x 128 x 256 B = the same
+    static_assert(kLoads == 8 && kMT == 8 && kNT == 8, "the phase schedule below is written for these counts");
+    static_assert(kLdsBytes <= kMaxLdsBytes);
+};
+
+namespace detail {
+
+/// acc += a · b on the matrix pipe, accumulator in AGPRs.
+DEVICE void mfma_16x16x32_agpr(f32x4& acc, const f16x8& a, const f16x8& b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
+/// The same MFMA, then a direct-to-LDS load of 16 bytes per lane from sbase + voff to lds_addr + 16 * lane. m0 is
+/// written before the MFMA, which thereby is the wait state required between the write of m0 and the load.
+DEVICE void mfma_16x16x32_agpr_then_load(f32x4& acc, const f16x8& a, const f16x8& b, unsigned int voff,
+                                         const void* sbase, unsigned int lds_addr) {
+    asm volatile(
+        "s_mov_b32 m0, %5\n\t"
+        "v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\t"
+        "global_load_lds_dwordx4 %3, %4"
+        : "+a"(acc)
+        : "v"(a), "v"(b), "v"(voff), "s"(sbase), "s"(lds_addr)
+        : "m0", "memory");
+}
+
+/// Direct-to-LDS load, scalar base + 32-bit lane offset (prologue only; inside the loop the fused form is used).
+DEVICE void load_lds_16B_sbase(unsigned int voff, const void* sbase, unsigned int lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
+                 : "m0", "memory");
+}
+
+}  // namespace detail
+
+/// grid = (M / 256) * (N / 256), block = 256, dynamic LDS = GemmW128Traits::kLdsBytes.
+template <typename OutType>
+__global__ void __launch_bounds__(GemmW128Traits::kThreads)
+    gemm_w128(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K) {
+    using T = GemmW128Traits;
+    extern __shared__ __align__(1024) unsigned char lds[];
+
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    int tile_m, tile_n;
+    detail::xcd_tile_coords(blockIdx.x, M / T::kBM, N / T::kBN, tile_m, tile_n);
+    const int m0 = tile_m * T::kBM, n0 = tile_n * T::kBN;
+
+    // ---- global -> LDS: load instruction q of this wavefront (q < 8: A, else B) fills 8 rows of 128 bytes; lane i
+    // writes physical 16-byte chunk i % 8 of row i / 8, which must hold logical chunk (i % 8) ^ ((row / 2) % 8)
+    const int lrow = lane >> 3, lchk = lane & 7;
+    unsigned int voff[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+        const int row = (wave * T::kLoads + (q & 7)) * 8 + lrow;
+        voff[q] = static_cast<unsigned int>(row) * static_cast<unsigned int>(K) * 2u + (lchk ^ ((row >> 1) & 7)) * 16;
+    }
+    const __half* a_base = A + size_t(m0) * K;
+    const __half* b_base = Bt + size_t(n0) * K;
+    const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
+    auto load_dst = [&](int stage, int q) -> unsigned int {
+        return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +
+                                              (wave * T::kLoads + (q & 7)) * 1024);
+    };
+    auto load_src = [&](int kt, int q) -> const __half* { return (q < 8 ? a_base : b_base) + kt * T::kBK; };
+
+    // ---- LDS -> registers: fragment r of a substep (r < 8: A rows 16 r.., else B rows 16 (r - 8)..); lane l holds
+    // row l % 16, k = 8 (l / 16) .. +7 of the 32-wide substep = logical chunk 4 kk + l / 16 of its row
+    const int frow = lane & 15, fquad = lane >> 4;
+    auto read_frag = [&](int stage, int kk, int r) -> f16x8 {
+        const int row = (r < 8 ? wave_m * T::kWaveM + r * 16 : wave_n * T::kWaveN + (r - 8) * 16) + frow;
+        const int chunk = (4 * kk + fquad) ^ ((row >> 1) & 7);
+        return *reinterpret_cast<const f16x8*>(lds + stage * T::kStageBytes + (r < 8 ? 0 : T::kABytes) +
+                                               row * T::kRowBytes + chunk * 16);
+    };
+
+    f32x4 acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    f16x8 fx[16], fy[16];  // fragments of substep 0 / substep 1: [0..7] A, [8..15] B
+
+    const int ktiles = K / T::kBK;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
+    if (ktiles > 1) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(1, q), load_dst(1, q));
+        detail::lds_barrier<16>();  // this wavefront's part of tile 0 has landed; then everyone's
+    } else {
+        detail::lds_barrier<0>();
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) fx[r] = read_frag(0, 0, r);
+
+    // Order of the 16 fragment reads of a phase: row group 0 of the next phase needs A fragment 0 and all B fragments.
+    constexpr int kOrder[16] = {0, 8, 9, 10, 11, 12, 13, 14, 15, 1, 2, 3, 4, 5, 6, 7};
+
+    // One tile of K. kMore: there is a tile kt+1 (read its substep 0 during phase 2); kMore2: there is a tile kt+2
+    // (load it during phase 2). Row group i = MFMA tiles (i, 0..7): the MFMA order is fixed by the asm statements, the
+    // fragment reads (plain loads) are written where they should issue and the compiler keeps them there.
+    auto tile = [&](int kt, auto more_c, auto more2_c) {
+        constexpr bool kMore = decltype(more_c)::value, kMore2 = decltype(more2_c)::value;
+        const int stage = kt & 1;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int r = 4 * i + (j >> 1);
+                if ((j & 1) == 0 && r < 16) fy[kOrder[r]] = read_frag(stage, 1, kOrder[r]);
+                detail::mfma_16x16x32_agpr(acc[i][j], fx[8 + j], fx[i]);
+            }
+        }
+        // this wavefront's part of tile kt+1 has landed and its reads of `stage` are done; then everyone's
+        detail::lds_barrier<0>();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int r = 4 * i + (j >> 1);
+                if (kMore && (j & 1) == 0 && r < 16) fx[kOrder[r]] = read_frag(stage ^ 1, 0, kOrder[r]);
+                if (kMore2 && (j & 3) == 1) {
+                    const int q = 2 * i + (j >> 2);
+                    detail::mfma_16x16x32_agpr_then_load(acc[i][j], fy[8 + j], fy[i], voff[q], load_src(kt + 2, q),
+                                                         load_dst(stage, q));
+                } else {
+                    detail::mfma_16x16x32_agpr(acc[i][j], fy[8 + j], fy[i]);
+                }
+            }
+        }
+    };
+    {
+        int kt = 0;
+        for (; kt + 2 < ktiles; ++kt) tile(kt, std::true_type{}, std::true_type{});
+        if (kt + 1 < ktiles) {
+            tile(kt, std::true_type{}, std::false_type{});
+            ++kt;
+        }
+        tile(kt, std::false_type{}, std::false_type{});
+    }
+
+    // MFMA results may be read by other instructions only a number of cycles after the MFMA was issued, and the
+    // compiler, not knowing the statements above are MFMAs, would not wait: every accumulator passes through a
+    // statement that waits first (32 wait states cover the longest requirement).
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        asm volatile("s_nop 15\n\ts_nop 15"
+                     : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),
+                       "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]));
+
+    // ---- epilogue: acc[i][j][e] = C[16 i + lane % 16][16 j + 4 (lane / 16) + e] of the wavefront's block
+    if constexpr (sizeof(OutType) == 2) {
+        __syncthreads();  // everyone is done with the operand stages
+        constexpr int kPitch = T::kWaveN * 2;  // bytes per staged row
+        unsigned char* stg = lds + wave * (T::kWaveM * kPitch);
+        // 8-byte slots of a row are XOR-ed with (row % 16) * 2 to spread banks
+        constexpr int kSlotMask = (kPitch / 8 - 1) & ~1;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = i * 16 + frow;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int slot = (j * 16 + 4 * fquad) >> 2;
+                const int pslot = slot ^ (((row & 15) << 1) & kSlotMask);
+                f16x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc[i][j][e]);
+                *reinterpret_cast<f16x4*>(stg + row * kPitch + pslot * 8) = v;
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's staging writes are done
+        constexpr int kLanesPerRow = T::kWaveN / 8;                // 16 lanes x 16 B per row
+        constexpr int kRowsPerIter = kWaveSize / kLanesPerRow;     // 4
+        const int rr = lane / kLanesPerRow, cc = lane % kLanesPerRow;
+        OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * N + n0 + wave_n * T::kWaveN;
+#pragma unroll 4
+        for (int it = 0; it < T::kWaveM / kRowsPerIter; ++it) {
+            const int row = it * kRowsPerIter + rr;
+            const int pslot = (2 * cc) ^ (((row & 15) << 1) & kSlotMask);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kPitch + pslot * 8);
+            *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(cbase + size_t(row) * N) + cc * 16) = v;
+        }
+    } else {
+        OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * N + n0 + wave_n * T::kWaveN;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * N + j * 16 + 4 * fquad) = acc[i][j];
+    }
+}
+
+}  // namespace tiledcuda::kernels

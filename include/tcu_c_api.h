@@ -26,12 +26,15 @@ typedef enum {
 
 typedef enum { TCU_DTYPE_F32 = 0, TCU_DTYPE_F16 = 1 } tcu_dtype;
 
-/* Which GEMM kernel to run. AUTO picks the pipelined kernel when the shape allows. */
+/* Which GEMM kernel to run. AUTO picks WAVE128 when M and N are multiples of 256 with at least 128 tiles of 256 x 256,
+ * else the pipelined kernel when the shape allows. */
 typedef enum {
     TCU_GEMM_AUTO = 0,
     TCU_GEMM_GLOBAL_REG = 1, /* global -> register -> MFMA (README kernel of the reference) */
     TCU_GEMM_ALL_MEM = 2,    /* global -> LDS -> register -> MFMA, single stage */
-    TCU_GEMM_PIPELINED = 3   /* direct-to-LDS, double-buffered, 16x16x32 MFMA */
+    TCU_GEMM_PIPELINED = 3,  /* direct-to-LDS, double-buffered, 16x16x32 MFMA, 2 wavefronts per SIMD */
+    TCU_GEMM_WAVE128 = 4     /* same pipeline, 256 x 256 tile on 4 wavefronts (one per SIMD, 128 x 128 each),
+                                accumulators in AGPRs; results identical to PIPELINED bit for bit */
 } tcu_gemm_algo;
 
 /* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks RESIDENT where it is instantiated. */

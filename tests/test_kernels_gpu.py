@@ -75,7 +75,36 @@ def test_gemm_pipelined_shapes(tcu, oracle, device, M, N, K, out_dtype):
     assert oracle.max_rel_err(host(C), oracle.gemm(A, Bt)) <= REL_TOL
 
 
-def test_gemm_one_hot_index_probe(tcu, device):
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 256, 128), (256, 512, 192), (512, 256, 256), (768, 1024, 320),
+                                   (2048, 2048, 1024)])
+@pytest.mark.parametrize("out_dtype", ["f32", "f16"])
+def test_gemm_wave128_shapes(tcu, oracle, device, M, N, K, out_dtype):
+    """The one-wavefront-per-SIMD kernel: one, two, three and many k-tiles (its last two tiles are peeled), one and many
+    workgroups, both output types; against the oracle and bit for bit against the pipelined kernel, whose arithmetic
+    (MFMA shape, order of the k-substeps) it shares."""
+    import torch
+
+    print(f"gemm wave128 {M}x{N}x{K} {out_dtype}", flush=True)
+    A = oracle.fill_uniform(M * K, 17 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 19 + N).reshape(N, K)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    dA, dB = dev(A, device), dev(Bt, device)
+    C = tcu.gemm(dA, dB, out_dtype=dt, algo="wave128")
+    torch.cuda.synchronize()
+    assert oracle.max_rel_err(host(C), oracle.gemm(A, Bt)) <= REL_TOL
+    assert torch.equal(C, tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))
+
+
+def test_gemm_wave128_rejects_other_shapes(tcu, device):
+    import torch
+
+    A = torch.zeros(128, 64, dtype=torch.float16, device=device)
+    with pytest.raises(RuntimeError):
+        tcu.gemm(A, A, algo="wave128")
+
+
+@pytest.mark.parametrize("algo", ["pipelined", "wave128"])
+def test_gemm_one_hot_index_probe(tcu, device, algo):
     """C[m, n] = A[m, k] * Bt[n, k] for one-hot operands: pins rows/cols/transposition exactly."""
     import torch
 
@@ -86,7 +115,7 @@ def test_gemm_one_hot_index_probe(tcu, device):
     for i, (m, n, k) in enumerate(picks):
         A[m, k] = 1.0 + i
         Bt[n, k] = 2.0
-    C = tcu.gemm(A, Bt, out_dtype=torch.float32, algo="pipelined").cpu().numpy()
+    C = tcu.gemm(A, Bt, out_dtype=torch.float32, algo=algo).cpu().numpy()
     want = A.float().cpu().numpy() @ Bt.float().cpu().numpy().T
     assert np.array_equal(C, want)
 
@@ -137,6 +166,9 @@ def test_gemm_config2_4096_cubed(tcu, oracle, device):
     # f32 output agrees with the f16 output to f16 rounding
     C32 = tcu.gemm(dA, dB, out_dtype=torch.float32)
     assert torch.equal(C32.half(), C)
+    # the two tuned kernels share their arithmetic: identical bit for bit
+    assert torch.equal(tcu.gemm(dA, dB, out_dtype=torch.float16, algo="pipelined"), C)
+    assert torch.equal(tcu.gemm(dA, dB, out_dtype=torch.float16, algo="wave128"), C)
 
 
 # ------------------------------------------------------------------------------ back-to-back GEMM

@@ -6,6 +6,7 @@
 #include "kernels/b2b_gemm_fwd.hpp"
 #include "kernels/flash_attn_fwd.hpp"
 #include "kernels/gemm_pipelined.hpp"
+#include "kernels/gemm_w128.hpp"
 #include "kernels/lstm_fwd.hpp"
 #include "kernels/mod.hpp"
 
@@ -120,10 +121,28 @@ int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M,
 }
 
 template <typename OutType>
+int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    using T = GemmW128Traits;
+    if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM needs M % 256 == 0, N % 256 == 0, K % 64 == 0");
+    if ((long)K * 2 * T::kBM >= (1l << 32))
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
+    return launch(&gemm_w128<OutType>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
+                  C, M, N, K);
+}
+
+template <typename OutType>
 int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, int algo, hipStream_t stream) {
     using W22 = tl::RowMajor<2, 2>;
     switch (algo) {
+        case TCU_GEMM_WAVE128:
+            return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_AUTO:
+            // where the 256 x 256 tile is the choice anyway, the one-wavefront-per-SIMD kernel is the faster one
+            if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) >= 128 &&
+                (long)K * 512 < (1l << 32))
+                return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
+            [[fallthrough]];
         case TCU_GEMM_PIPELINED:
             return gemm_pipelined_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_GLOBAL_REG:
