@@ -21,8 +21,9 @@
 //     wait state the load needs after the write of m0;
 //   * no branches inside the loop over k (the last two tiles are peeled): a taken branch stalls the one instruction
 //     stream that feeds the matrix pipe;
-//   * LDS layout, XOR swizzle, XCD-aware tile order and the LDS-staged 16-byte epilogue are those of
-//     gemm_pipelined.hpp.
+//   * LDS layout, XOR swizzle and XCD-aware tile order are those of gemm_pipelined.hpp; the f16 epilogue stages 16
+//     rows at a time through 8 KiB of LDS per wavefront beyond the operand stages (no workgroup barrier, staging
+//     overlapped with the 16-byte row-contiguous stores).
 // Because the compiler does not know these asm statements are MFMAs it inserts none of the wait states MFMA results
 // need before other instructions read them; the only such reads are in the epilogue, and every accumulator passes
 // through a waiting statement first (see below). M % 256 == 0, N % 256 == 0, K % 64 == 0 (checked by the launcher).
@@ -45,7 +46,9 @@ struct GemmW128Traits {
     static constexpr int kABytes = kBM * kRowBytes, kBBytes = kBN * kRowBytes;
     static constexpr int kStageBytes = kABytes + kBBytes;  // 64 KiB
     static constexpr int kLoads = kBM / 8 / kWaves;        // 1 KiB load instructions per operand per wavefront per stage
-    static constexpr int kLdsBytes = 2 * kStageBytes;      // the f16 epilogue needs 4 x 128 x 256 B = the same
+    static constexpr int kLdsBytesMain = 2 * kStageBytes;  // 128 KiB of operand stages
+    static constexpr int kEpilogueBytesPerWave = 2 * 16 * kWaveN * 2;  // f16 epilogue: two buffers of 16 rows
+    static constexpr int kLdsBytes = kLdsBytesMain + kWaves * kEpilogueBytesPerWave;  // 160 KiB
     static_assert(kLoads == 8 && kMT == 8 && kNT == 8, "the phase schedule below is written for these counts");
     static_assert(kLdsBytes <= kMaxLdsBytes);
 };
@@ -198,35 +201,34 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 
     // ---- epilogue: acc[i][j][e] = C[16 i + lane % 16][16 j + 4 (lane / 16) + e] of the wavefront's block
     if constexpr (sizeof(OutType) == 2) {
-        __syncthreads();  // everyone is done with the operand stages
-        constexpr int kPitch = T::kWaveN * 2;  // bytes per staged row
-        unsigned char* stg = lds + wave * (T::kWaveM * kPitch);
-        // 8-byte slots of a row are XOR-ed with (row % 16) * 2 to spread banks
-        constexpr int kSlotMask = (kPitch / 8 - 1) & ~1;
+        // f16: 16 rows at a time through a private LDS buffer (beyond the operand stages, so no workgroup barrier),
+        // so that global stores are 16 bytes per lane and row-contiguous; two buffers per wavefront, so the
+        // conversion and staging of rows 16 (i + 1).. overlap the stores of rows 16 i..
+        constexpr int kPitch = T::kWaveN * 2;              // 256 bytes per staged row
+        constexpr int kSlotMask = (kPitch / 8 - 1) & ~1;   // 8-byte slots of a row are XOR-ed with 2 * row
+        unsigned char* stg = lds + T::kLdsBytesMain + wave * T::kEpilogueBytesPerWave;
+        const int rr = lane >> 4, cc = lane & 15;  // read-back: 16 lanes x 16 B per row, 4 rows per instruction
+        OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * N + n0 + wave_n * T::kWaveN;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const int row = i * 16 + frow;
+            unsigned char* buf = stg + (i & 1) * (16 * kPitch);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int slot = (j * 16 + 4 * fquad) >> 2;
-                const int pslot = slot ^ (((row & 15) << 1) & kSlotMask);
+                const int pslot = slot ^ ((frow << 1) & kSlotMask);
                 f16x4 v;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc[i][j][e]);
-                *reinterpret_cast<f16x4*>(stg + row * kPitch + pslot * 8) = v;
+                *reinterpret_cast<f16x4*>(buf + frow * kPitch + pslot * 8) = v;
             }
-        }
-        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's staging writes are done
-        constexpr int kLanesPerRow = T::kWaveN / 8;                // 16 lanes x 16 B per row
-        constexpr int kRowsPerIter = kWaveSize / kLanesPerRow;     // 4
-        const int rr = lane / kLanesPerRow, cc = lane % kLanesPerRow;
-        OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * N + n0 + wave_n * T::kWaveN;
-#pragma unroll 4
-        for (int it = 0; it < T::kWaveM / kRowsPerIter; ++it) {
-            const int row = it * kRowsPerIter + rr;
-            const int pslot = (2 * cc) ^ (((row & 15) << 1) & kSlotMask);
-            const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kPitch + pslot * 8);
-            *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(cbase + size_t(row) * N) + cc * 16) = v;
+            // LDS operations of one wavefront execute in order: the reads below see the writes above
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int row = it * 4 + rr;
+                const int pslot = (2 * cc) ^ ((row << 1) & kSlotMask);
+                const u32x4 v = *reinterpret_cast<const u32x4*>(buf + row * kPitch + pslot * 8);
+                *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(cbase + size_t(i * 16 + row) * N) + cc * 16) = v;
+            }
         }
     } else {
         OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * N + n0 + wave_n * T::kWaveN;
