@@ -48,6 +48,40 @@ def time_kernel(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def time_graph(fn, steps, warmup, launches_per_graph=20):
+    """Average milliseconds per call of fn() when `launches_per_graph` calls are captured in one HIP graph and the
+    graph is replayed: what a launch-bound kernel costs once the host is out of the way. Every replay's result is
+    that of the eager call (same operands), which the caller checks afterwards. None if capture is refused."""
+    import torch
+
+    try:
+        fn()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()  # default priority
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            fn()
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(launches_per_graph):
+                    fn()
+        torch.cuda.synchronize()
+        replays = max(1, steps // launches_per_graph)
+        for _ in range(max(1, warmup // launches_per_graph)):
+            graph.replay()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(replays):
+            graph.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / (replays * launches_per_graph)
+    except Exception as exc:  # capture is optional; the eager figure stands
+        print(f"bench: HIP graph timing skipped ({exc})", file=sys.stderr)
+        return None
+
+
 def probe_mfma(torch, operands, shape, waves=8, iters=20000):
     """Sustained MFMA rate on `operands` (fp16 device tensor, >= 256*waves*4096 halves): TFLOP/s and core MHz."""
     import ctypes
@@ -166,8 +200,10 @@ def main():
         d1c = torch.empty(128, 64, dtype=torch.float32, device=dev)
         for algo in ("global_reg", "pipelined"):
             ms = time_kernel(lambda: tcu.gemm(d1a, d1b, out=d1c, algo=algo), args.steps, args.warmup)
+            gms = time_graph(lambda: tcu.gemm(d1a, d1b, out=d1c, algo=algo), 10 * args.steps, args.warmup)
             err = oracle.max_rel_err(d1c.cpu().numpy(), oracle.gemm(A1, B1))
             configs.append({"name": f"gemm_128x64x256_{algo}", "ms": ms, "us": ms * 1e3,
+                            "us_in_hip_graph": None if gms is None else gms * 1e3,
                             "tflops": 2.0 * 128 * 64 * 256 / (ms * 1e-3) / 1e12, "max_rel_err": err})
 
     # ---------------------------------------------------------------- C3: back-to-back GEMM
@@ -179,10 +215,13 @@ def main():
         d3a, d3b, d3c = to_dev(A3), to_dev(B3), to_dev(C3)
         d3d = torch.empty(1, M, P, dtype=torch.float16, device=dev)
         ms = time_kernel(lambda: tcu.b2b_gemm(d3a, d3b, d3c, out=d3d), args.steps, args.warmup)
+        gms = time_graph(lambda: tcu.b2b_gemm(d3a, d3b, d3c, out=d3d), 10 * args.steps, args.warmup)
         err = oracle.max_rel_err(d3d[0].float().cpu().numpy(), oracle.b2b_gemm(A3, B3, C3), eps=1.0)
         flops = 2.0 * M * K * N + 2.0 * M * N * P
         nbytes = 2.0 * (M * K + N * K + P * N + M * P)
-        configs.append({"name": "b2b_8192x256x128x128", "ms": ms, "us": ms * 1e3, "tflops": flops / (ms * 1e-3) / 1e12,
+        configs.append({"name": "b2b_8192x256x128x128", "ms": ms, "us": ms * 1e3,
+                        "us_in_hip_graph": None if gms is None else gms * 1e3,
+                        "gbs_in_hip_graph": None if gms is None else nbytes / (gms * 1e-3) / 1e9, "tflops": flops / (ms * 1e-3) / 1e12,
                         "gbs": nbytes / (ms * 1e-3) / 1e9, "frac_mfma_peak": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
                         "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "max_rel_err": err})
 

@@ -223,6 +223,38 @@ def test_b2b_gemm_both_kernels_at_256x128x128(tcu, oracle, device, algo, M, batc
         assert torch.equal(D1[0], want)
 
 
+def test_kernels_in_a_hip_graph_replay_like_eager(tcu, oracle, device):
+    """Launch-bound callers capture these entry points in HIP graphs: several replays, with eager work and
+    synchronisations in between, each give the eager result (operands changed between replays)."""
+    import torch
+
+    M, N, K, P = 1024, 256, 128, 128
+    A = dev(oracle.fill_normal(M * K, 81, 0, 0.1).reshape(1, M, K), device)
+    Bt = dev(oracle.fill_normal(N * K, 82, 0, 0.1).reshape(1, N, K), device)
+    Ct = dev(oracle.fill_normal(P * N, 83, 0, 0.1).reshape(1, P, N), device)
+    D = torch.empty(1, M, P, dtype=torch.float16, device=device)
+    G = torch.empty(M, N, dtype=torch.float16, device=device)
+    tcu.b2b_gemm(A, Bt, Ct, out=D)
+    tcu.gemm(A[0], Bt[0], out=G)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            tcu.b2b_gemm(A, Bt, Ct, out=D)
+            tcu.gemm(A[0], Bt[0], out=G)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        A.mul_(-0.5 if rep % 2 else 1.5)  # eager work between the replays
+        torch.cuda.synchronize()
+        D.zero_()
+        G.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(D, tcu.b2b_gemm(A, Bt, Ct)), f"replay {rep}"
+        assert torch.equal(G, tcu.gemm(A[0], Bt[0])), f"replay {rep}"
+
+
 def test_b2b_gemm_config3(tcu, oracle, device):
     """C3: A [8192x128], B [128x256], C [256x128], N(0, 0.1), f16 D."""
     import torch
