@@ -1,7 +1,8 @@
 /*
  * C-ABI of the MI355X tile-kernel library: the boundary a host program (C, C++, Python
  * ctypes, a torch op) binds to. Plain pointers and sizes only; every pointer is a device
- * pointer owned by the caller; nothing is allocated, freed or synchronised by the library;
+ * pointer owned by the caller and 16-byte aligned (the kernels move 16 bytes per lane);
+ * nothing is allocated, freed or synchronised by the library;
  * work is enqueued on the hipStream_t passed as `stream` (NULL = the default stream).
  * Every function returns 0 on success or a negative tcu_status; tcu_last_error() gives the
  * message of the last failure on the calling thread. No function ever calls exit().
@@ -18,7 +19,7 @@ extern "C" {
 
 typedef enum {
     TCU_OK = 0,
-    TCU_ERR_INVALID_ARGUMENT = -1,  /* null pointer, non-positive size, bad enum value */
+    TCU_ERR_INVALID_ARGUMENT = -1,  /* null or misaligned pointer, non-positive size, bad enum value */
     TCU_ERR_UNSUPPORTED_SHAPE = -2, /* shape not divisible by the tile / not instantiated */
     TCU_ERR_HIP = -3,               /* a HIP runtime call failed (message has the HIP error) */
     TCU_ERR_NO_DEVICE = -4          /* no HIP device is available to this process */

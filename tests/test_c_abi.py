@@ -49,6 +49,19 @@ def test_null_pointers_are_rejected(tcu, call):
     assert "null pointer" in tcu.last_error()
 
 
+def test_misaligned_operands_are_rejected(tcu):
+    """The kernels move 16 bytes per lane: an operand that does not start on a 16-byte boundary is refused before
+    anything is launched."""
+    l = tcu.lib()
+    p, q = 0x1000, 0x1002
+    assert l.tcu_gemm_f16(q, p, p, 64, 64, 64, 0, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert "16-byte aligned" in tcu.last_error()
+    assert l.tcu_b2b_gemm_f16(p, p, q, p, 64, 64, 64, 64, 1, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_flash_attn_fwd_f16(p, p, p, q, 1, 64, 64, 128, 128, 1.0, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_lstm_f16(p, p, p, 0, q, p, p, 1, 64, 128, 128, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert "16-byte aligned" in tcu.last_error()
+
+
 def test_bad_sizes_and_enums_are_rejected(tcu):
     l = tcu.lib()
     p = 0x1000  # never dereferenced: argument checks come first

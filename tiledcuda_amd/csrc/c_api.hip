@@ -72,6 +72,14 @@ bool positive(std::initializer_list<int> v) {
     return true;
 }
 
+/// The kernels move 16 bytes per lane (vector loads, direct-to-LDS loads, vector stores): operands must start on a
+/// 16-byte boundary (null = absent optional operand is fine here; required ones are checked for null separately).
+bool aligned16(std::initializer_list<const void*> v) {
+    for (const void* p : v)
+        if (reinterpret_cast<uintptr_t>(p) % 16 != 0) return false;
+    return true;
+}
+
 // ---------------------------------------------------------------------------- GEMM
 template <typename OutType, int kM, int kN, int kK, int kTM, int kTN, int kChunkK, typename WarpLayout>
 int launch_simple_gemm(const __half* A, const __half* B, OutType* C, hipStream_t stream) {
@@ -326,6 +334,7 @@ int tcu_device_count(void) {
 int tcu_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K, int out_dtype, int algo, void* stream) {
     if (!A || !B || !C) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16: null pointer");
     if (!positive({M, N, K})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16: sizes must be positive");
+    if (!aligned16({A, B, C})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16: operands must be 16-byte aligned");
     auto s = static_cast<hipStream_t>(stream);
     auto a = static_cast<const __half*>(A), b = static_cast<const __half*>(B);
     if (out_dtype == TCU_DTYPE_F32) return gemm_dispatch<float>(a, b, static_cast<float*>(C), M, N, K, algo, s);
@@ -347,6 +356,8 @@ int tcu_b2b_gemm_f16_algo(const void* A, const void* B, const void* C, void* D, 
     if (!A || !B || !C || !D) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: null pointer");
     if (!positive({M, N, K, P, batch}))
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: sizes must be positive");
+    if (!aligned16({A, B, C, D}))
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: operands must be 16-byte aligned");
     auto s = static_cast<hipStream_t>(stream);
     auto a = static_cast<const __half*>(A), b = static_cast<const __half*>(B), c = static_cast<const __half*>(C);
     if (out_dtype == TCU_DTYPE_F32) return b2b_dispatch<float>(a, b, c, static_cast<float*>(D), M, N, K, P, batch, algo, s);
@@ -359,6 +370,8 @@ int tcu_flash_attn_fwd_f16_algo(const void* Q, const void* K, const void* V, voi
     if (!Q || !K || !V || !O) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_flash_attn_fwd_f16: null pointer");
     if (!positive({batch, M, N, Kdim, P}))
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_flash_attn_fwd_f16: sizes must be positive");
+    if (!aligned16({Q, K, V, O}))
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_flash_attn_fwd_f16: operands must be 16-byte aligned");
     return fa_dispatch(static_cast<const __half*>(Q), static_cast<const __half*>(K), static_cast<const __half*>(V),
                        static_cast<__half*>(O), batch, M, N, Kdim, P, scale, v_layout, algo,
                        static_cast<hipStream_t>(stream));
@@ -378,6 +391,8 @@ int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void
                       void* c_out, int T, int B, int I, int H, int algo, void* stream) {
     if (!x || !W || !bias || !h_all || !c_out) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: null pointer");
     if (!positive({T, B, I, H})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: sizes must be positive");
+    if (!aligned16({x, W, bias, h0, c0, h_all, c_out}))
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: operands must be 16-byte aligned");
     auto s = static_cast<hipStream_t>(stream);
     auto xp = static_cast<const __half*>(x), wp = static_cast<const __half*>(W), bp = static_cast<const __half*>(bias);
     auto h0p = static_cast<const __half*>(h0);
