@@ -257,8 +257,23 @@ def main():
         h_ref, c_ref = oracle.lstm(x, W, b, rows=(0, 2))
         err = max(oracle.max_abs_err(out["h"][:, 0:2].float().cpu().numpy(), h_ref[:, 0:2]),
                   oracle.max_abs_err(out["c"][0:2].cpu().numpy(), c_ref[0:2]))
+        # the same layer with the input projection of all steps hoisted into one GEMM (caller-owned workspace)
+        ws = torch.empty(tcu.lstm_workspace_bytes(T, Bb, I, Hh), dtype=torch.uint8, device=dev)
+        outh = {}
+
+        def lstm_hoisted():
+            outh["h"], outh["c"] = tcu.lstm(dx, dW, db, algo="hoisted", workspace=ws)
+
+        ms_h = time_kernel(lstm_hoisted, max(5, args.steps // 2), max(2, args.warmup // 2))
+        err_h = max(oracle.max_abs_err(outh["h"][:, 0:2].float().cpu().numpy(), h_ref[:, 0:2]),
+                    oracle.max_abs_err(outh["c"][0:2].cpu().numpy(), c_ref[0:2]))
         step_bytes = 2.0 * (4 * Hh * (I + Hh) + 4 * Hh + Bb * I + 2 * Bb * Hh) + 4.0 * 2 * Bb * Hh
         flops = 2.0 * Bb * (I + Hh) * 4 * Hh * T
+        configs.append({"name": "lstm_b256_i1024_h1024_t16_hoisted_input_gemm", "ms": ms_h, "us_per_step": ms_h * 1e3 / T,
+                        "gbs": step_bytes * T / (ms_h * 1e-3) / 1e9,
+                        "frac_hbm_peak": step_bytes * T / (ms_h * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        "tflops": flops / (ms_h * 1e-3) / 1e12, "max_abs_err": err_h,
+                        "workspace_bytes": int(ws.numel())})
         configs.append({"name": "lstm_b256_i1024_h1024_t16", "ms": ms, "us_per_step": ms * 1e3 / T,
                         "gbs": step_bytes * T / (ms * 1e-3) / 1e9,
                         "frac_hbm_peak": step_bytes * T / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,

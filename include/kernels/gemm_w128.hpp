@@ -82,9 +82,12 @@ DEVICE void load_lds_16B_sbase(unsigned int voff, const void* sbase, unsigned in
 }  // namespace detail
 
 /// grid = (M / 256) * (N / 256), block = 256, dynamic LDS = GemmW128Traits::kLdsBytes.
+/// lda / ldb: elements between consecutive rows of A / of the stored [N, K] array (K for dense operands; larger when
+/// the operand is a column block of a wider matrix). C is dense.
 template <typename OutType>
 __global__ void __launch_bounds__(GemmW128Traits::kThreads)
-    gemm_w128(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K) {
+    gemm_w128(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
+              int lda, int ldb) {
     using T = GemmW128Traits;
     extern __shared__ __align__(1024) unsigned char lds[];
 
@@ -102,10 +105,11 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 #pragma unroll
     for (int q = 0; q < 16; ++q) {
         const int row = (wave * T::kLoads + (q & 7)) * 8 + lrow;
-        voff[q] = static_cast<unsigned int>(row) * static_cast<unsigned int>(K) * 2u + (lchk ^ ((row >> 1) & 7)) * 16;
+        voff[q] = static_cast<unsigned int>(row) * static_cast<unsigned int>(q < 8 ? lda : ldb) * 2u +
+                  (lchk ^ ((row >> 1) & 7)) * 16;
     }
-    const __half* a_base = A + size_t(m0) * K;
-    const __half* b_base = Bt + size_t(n0) * K;
+    const __half* a_base = A + size_t(m0) * lda;
+    const __half* b_base = Bt + size_t(n0) * ldb;
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
     auto load_dst = [&](int stage, int q) -> unsigned int {
         return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +

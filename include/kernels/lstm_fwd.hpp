@@ -64,11 +64,14 @@ DEVICE void wait_vmcnt_lgkm0() {
 
 /// grid = (B / 64) * (H / 16) workgroups (1-D), block = 512, dynamic LDS = Traits::kLdsBytes.
 /// h_in == nullptr: h_{t-1} = 0; c_in == nullptr: c_{t-1} = 0. h_out must not alias h_in.
-template <typename Traits>
+/// kHoisted: the input half of the gates, x_t · W[:, :I]ᵀ, was computed beforehand for the whole sequence (one large
+/// GEMM) and is passed as pre_t [B, 4H] f32; the step then streams only h_{t-1} and W[:, I:] (half the bytes) and x_t
+/// is not read.
+template <typename Traits, bool kHoisted = false>
 __global__ void __launch_bounds__(Traits::kThreads)
     lstm_cell_fwd(const __half* __restrict__ x_t, const __half* __restrict__ h_in, const __half* __restrict__ W,
                   const __half* __restrict__ bias, const float* c_in, float* c_out, __half* __restrict__ h_out,
-                  int B) {
+                  int B, const float* __restrict__ pre_t) {
     constexpr int kI = Traits::kI, kH = Traits::kH, kKK = Traits::kKK, kBK = Traits::kBK;
     constexpr int S = Traits::kStages, L = Traits::kLoadsPerWave;
     extern __shared__ __align__(1024) unsigned char lds[];
@@ -92,10 +95,11 @@ __global__ void __launch_bounds__(Traits::kThreads)
     // 32 wn + 8 gate + jj is weight row gate * H + hid0 + 8 wn + jj. Wavefront w issues t = 4 w .. 4 w + 3.
     // Physical 16-byte chunk p of row r holds logical chunk p ^ (r % 16).
     const int lrow = lane >> 4, lchk = lane & 15;
+    const int k_begin = kHoisted ? kI : 0;
     const int k_end = h_in ? kKK : kI;
-    const int ktiles = k_end / kBK;
+    const int ktiles = (k_end - k_begin) / kBK;
     auto issue_stage = [&](int stage, int kt) {
-        const int k0 = kt * kBK;
+        const int k0 = k_begin + kt * kBK;
         unsigned char* sbase = lds + stage * Traits::kStageBytes;
 #pragma unroll
         for (int j = 0; j < L; ++j) {
@@ -126,10 +130,14 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int hid = hid0 + 8 * wave_n + 4 * fhalf;
     f32x4 c_prev = {0.f, 0.f, 0.f, 0.f};
     f16x4 bias_v[4];
+    f32x4 pre_v[4];
     if (group == 0) {
         if (c_in) c_prev = *reinterpret_cast<const f32x4*>(c_in + size_t(b) * kH + hid);
 #pragma unroll
-        for (int g = 0; g < 4; ++g) bias_v[g] = *reinterpret_cast<const f16x4*>(bias + g * kH + hid);
+        for (int g = 0; g < 4; ++g) {
+            bias_v[g] = *reinterpret_cast<const f16x4*>(bias + g * kH + hid);
+            if constexpr (kHoisted) pre_v[g] = *reinterpret_cast<const f32x4*>(pre_t + size_t(b) * (4 * kH) + g * kH + hid);
+        }
     }
 
     // two accumulators: consecutive MFMAs do not depend on each other
@@ -199,10 +207,16 @@ __global__ void __launch_bounds__(Traits::kThreads)
     f16x4 h_new;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        const float gi = acc[0 + e] + static_cast<float>(bias_v[0][e]);
-        const float gf = acc[4 + e] + static_cast<float>(bias_v[1][e]);
-        const float gg = acc[8 + e] + static_cast<float>(bias_v[2][e]);
-        const float go = acc[12 + e] + static_cast<float>(bias_v[3][e]);
+        float gi = acc[0 + e] + static_cast<float>(bias_v[0][e]);
+        float gf = acc[4 + e] + static_cast<float>(bias_v[1][e]);
+        float gg = acc[8 + e] + static_cast<float>(bias_v[2][e]);
+        float go = acc[12 + e] + static_cast<float>(bias_v[3][e]);
+        if constexpr (kHoisted) {
+            gi += pre_v[0][e];
+            gf += pre_v[1][e];
+            gg += pre_v[2][e];
+            go += pre_v[3][e];
+        }
         const float cn = detail::sigmoid_fast(gf) * c_prev[e] + detail::sigmoid_fast(gi) * detail::tanh_fast(gg);
         c_new[e] = cn;
         h_new[e] = static_cast<_Float16>(detail::sigmoid_fast(go) * detail::tanh_fast(cn));

@@ -129,6 +129,20 @@ int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0,
 int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
                       void* c_out, int T, int B, int I, int H, int algo, void* stream);
 
+/*
+ * tcu_lstm_f16 with the input half of the gates hoisted out of the time loop: x · W[:, :I]^T for all T steps is one
+ * large GEMM into `workspace` ([T, B, 4H] f32), and each step then streams only h_{t-1} and W[:, I:] (half the bytes
+ * of a step, which is what bounds it). Same arguments and results (up to the order of the f32 summation) as
+ * tcu_lstm_f16. `workspace` is device memory of at least tcu_lstm_workspace_bytes(T, B, I, H) bytes, 16-byte aligned,
+ * owned by the caller and free to reuse once the work enqueued here has run. tcu_lstm_workspace_bytes returns 0 for
+ * shapes this path is not instantiated for ((I, H) in {(1024, 1024), (128, 128), (256, 128)}, T * B a multiple of
+ * 256); tcu_lstm_f16_ws then fails with TCU_ERR_UNSUPPORTED_SHAPE. No counterpart in the reference (it has no LSTM).
+ */
+unsigned long long tcu_lstm_workspace_bytes(int T, int B, int I, int H);
+int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                    void* c_out, int T, int B, int I, int H, void* workspace, unsigned long long workspace_bytes,
+                    void* stream);
+
 /* How tcu_scatter_nd combines an update with the data it lands on. */
 typedef enum {
     TCU_SCATTER_ASSIGN = 0, /* data[...] = update: what the reference's test checks (tests/python/test_scatter_nd.py:47-56) */

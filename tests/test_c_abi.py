@@ -20,7 +20,7 @@ def declared_symbols():
 
 def test_header_declares_the_entry_points():
     syms = declared_symbols()
-    for name in ("tcu_gemm_f16", "tcu_b2b_gemm_f16", "tcu_flash_attn_fwd_f16", "tcu_lstm_f16", "tcu_flash_attn_fwd_f16_algo", "tcu_lstm_f16_algo", "tcu_last_error",
+    for name in ("tcu_gemm_f16", "tcu_b2b_gemm_f16", "tcu_flash_attn_fwd_f16", "tcu_lstm_f16", "tcu_flash_attn_fwd_f16_algo", "tcu_lstm_f16_algo", "tcu_lstm_f16_ws", "tcu_lstm_workspace_bytes", "tcu_last_error",
                  "tcu_version", "tcu_device_count"):
         assert name in syms
 

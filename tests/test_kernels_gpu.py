@@ -424,6 +424,51 @@ def test_lstm_small(tcu, oracle, device, T, B, I, H, with_state, algo):
     assert oracle.max_abs_err(host(c_T), c_ref) <= ABS_TOL
 
 
+@pytest.mark.parametrize("T,B,I,H", [(4, 64, 128, 128), (2, 128, 256, 128), (8, 64, 128, 128)])
+@pytest.mark.parametrize("with_state", [False, True])
+def test_lstm_hoisted_input_projection(tcu, oracle, device, T, B, I, H, with_state):
+    """tcu_lstm_f16_ws: the input half of the gates from one GEMM over all steps, then steps over h only; against the
+    oracle, against the per-step streaming kernel, with a caller-owned workspace larger than needed, and twice in a row
+    on the same workspace."""
+    import torch
+
+    print(f"lstm hoisted T{T} B{B} I{I} H{H} state={with_state}", flush=True)
+    x = oracle.fill_normal(T * B * I, 51, 0, 0.5).reshape(T, B, I)
+    W = oracle.fill_normal(4 * H * (I + H), 52, 0, 0.1).reshape(4 * H, I + H)
+    b = oracle.fill_normal(4 * H, 53, 0, 0.1)
+    h0 = oracle.fill_normal(B * H, 54, 0, 0.5).reshape(B, H) if with_state else None
+    c0 = oracle.fill_normal(B * H, 55, 0, 0.5).reshape(B, H).astype(np.float32) if with_state else None
+    args = (dev(x, device), dev(W, device), dev(b, device), dev(h0, device) if with_state else None,
+            dev(c0, device) if with_state else None)
+    need = tcu.lstm_workspace_bytes(T, B, I, H)
+    assert need == T * B * 4 * H * 4
+    ws = torch.full((need + 4096,), 0xFF, dtype=torch.uint8, device=device)  # NaN patterns: nothing may be read unwritten
+    h_ref, c_ref = oracle.lstm(x, W, b, h0, c0)
+    h_str, c_str = tcu.lstm(*args, algo="streaming")
+    for rep in range(2):
+        h_all, c_T = tcu.lstm(*args, algo="hoisted", workspace=ws)
+        torch.cuda.synchronize()
+        assert oracle.max_abs_err(host(h_all), h_ref) <= ABS_TOL
+        assert oracle.max_abs_err(host(c_T), c_ref) <= ABS_TOL
+        assert float((h_all.float() - h_str.float()).abs().max()) <= 2e-3
+        assert float((c_T - c_str).abs().max()) <= 2e-3
+    assert bool((ws[need:] == 0xFF).all())  # nothing written past the stated size
+
+
+def test_lstm_hoisted_rejects_what_it_cannot_do(tcu, device):
+    import torch
+
+    assert tcu.lstm_workspace_bytes(3, 64, 128, 128) == 0  # T * B not a multiple of 256
+    assert tcu.lstm_workspace_bytes(4, 64, 64, 64) == 0    # shape not instantiated
+    x = torch.zeros(4, 64, 128, dtype=torch.float16, device=device)
+    W = torch.zeros(512, 256, dtype=torch.float16, device=device)
+    b = torch.zeros(512, dtype=torch.float16, device=device)
+    with pytest.raises(RuntimeError):
+        tcu.lstm(x, W, b, algo="hoisted", workspace=torch.empty(1024, dtype=torch.uint8, device=device))
+    with pytest.raises(RuntimeError):
+        tcu.lstm(x[:3].contiguous(), W, b, algo="hoisted")
+
+
 def test_lstm_zero_weights_closed_form(tcu, device):
     """W = 0: c_t = sigmoid(b_f) c_{t-1} + sigmoid(b_i) tanh(b_g), h_t = sigmoid(b_o) tanh(c_t)."""
     import torch
@@ -452,14 +497,16 @@ def test_lstm_config5(tcu, oracle, device):
     x = oracle.fill_normal(T * B * I, 1239, 0, 0.05).reshape(T, B, I)
     W = oracle.fill_normal(4 * H * (I + H), 2239, 0, 0.05).reshape(4 * H, I + H)
     b = oracle.fill_normal(4 * H, 3239, 0, 0.05)
-    h_all, c_T = tcu.lstm(dev(x, device), dev(W, device), dev(b, device))
-    torch.cuda.synchronize()
-    hh, cc = host(h_all), host(c_T)
-    assert np.isfinite(hh).all() and np.isfinite(cc).all()
-    for rows in [(0, 4), (252, 256)]:
-        h_ref, c_ref = oracle.lstm(x, W, b, rows=rows)
-        assert oracle.max_abs_err(hh[:, rows[0]:rows[1]], h_ref[:, rows[0]:rows[1]]) <= ABS_TOL
-        assert oracle.max_abs_err(cc[rows[0]:rows[1]], c_ref[rows[0]:rows[1]]) <= ABS_TOL
+    dx, dW, db = dev(x, device), dev(W, device), dev(b, device)
+    refs = {rows: oracle.lstm(x, W, b, rows=rows) for rows in [(0, 4), (252, 256)]}
+    for algo in ("auto", "hoisted"):
+        h_all, c_T = tcu.lstm(dx, dW, db, algo=algo)
+        torch.cuda.synchronize()
+        hh, cc = host(h_all), host(c_T)
+        assert np.isfinite(hh).all() and np.isfinite(cc).all()
+        for rows, (h_ref, c_ref) in refs.items():
+            assert oracle.max_abs_err(hh[:, rows[0]:rows[1]], h_ref[:, rows[0]:rows[1]]) <= ABS_TOL, algo
+            assert oracle.max_abs_err(cc[rows[0]:rows[1]], c_ref[rows[0]:rows[1]]) <= ABS_TOL, algo
 
 
 def test_smoke_entry(device):

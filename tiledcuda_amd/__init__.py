@@ -18,7 +18,7 @@ import torch
 
 __all__ = [
     "TcuError", "library_path", "lib", "last_error", "gemm", "b2b_gemm", "flash_attention_fwd",
-    "flash_attention", "TiledFlashAttention", "lstm", "scatter_nd", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS", "B2B_ALGOS",
+    "flash_attention", "TiledFlashAttention", "lstm", "lstm_workspace_bytes", "scatter_nd", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS", "B2B_ALGOS",
     "SCATTER_MODES",
 ]
 
@@ -59,6 +59,9 @@ _SIGNATURES = {
                                                                                                 ctypes.c_int, ctypes.c_void_p]),
     "tcu_lstm_f16": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
     "tcu_lstm_f16_algo": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 5 + [ctypes.c_void_p]),
+    "tcu_lstm_workspace_bytes": (ctypes.c_ulonglong, [ctypes.c_int] * 4),
+    "tcu_lstm_f16_ws": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_ulonglong,
+                                                                                     ctypes.c_void_p]),
     "tcu_scatter_nd": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.POINTER(ctypes.c_longlong), ctypes.c_int,
                                                              ctypes.c_longlong, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                              ctypes.c_void_p, ctypes.c_void_p]),
@@ -222,20 +225,42 @@ class TiledFlashAttention:
 
 # ------------------------------------------------------------------------------ LSTM
 def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor | None = None,
-         c0: torch.Tensor | None = None, algo: str = "auto") -> tuple[torch.Tensor, torch.Tensor]:
+         c0: torch.Tensor | None = None, algo: str = "auto",
+         workspace: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
     """Fused LSTM layer. x [T, B, I] f16, W [4H, I+H] f16 (gate rows i,f,g,o), bias [4H] f16,
-    h0 [B, H] f16 / c0 [B, H] f32 (None = zeros). Returns (h_all [T, B, H] f16, c_T [B, H] f32)."""
+    h0 [B, H] f16 / c0 [B, H] f32 (None = zeros). Returns (h_all [T, B, H] f16, c_T [B, H] f32).
+
+    ``algo="hoisted"`` computes the input half of the gates for all steps in one GEMM first (``tcu_lstm_f16_ws``); it
+    needs ``lstm_workspace_bytes(T, B, I, H)`` bytes of device memory, taken from ``workspace`` (any dtype) if given,
+    else allocated here."""
     T, B, I = x.shape
     H = W.shape[0] // 4
     if tuple(W.shape) != (4 * H, I + H) or tuple(bias.shape) != (4 * H,):
         raise ValueError("W must be [4H, I+H] and bias [4H]")
     h_all = torch.empty(T, B, H, dtype=torch.float16, device=x.device)
     c_out = torch.empty(B, H, dtype=torch.float32, device=x.device)
+    if algo == "hoisted":
+        need = lstm_workspace_bytes(T, B, I, H)
+        if workspace is None:
+            workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=x.device)
+        if not workspace.is_cuda or not workspace.is_contiguous():
+            raise ValueError("workspace must be a contiguous device tensor")
+        _check(lib().tcu_lstm_f16_ws(_dev_ptr(x, torch.float16, "x"), _dev_ptr(W, torch.float16, "W"),
+                                     _dev_ptr(bias, torch.float16, "bias"), _dev_ptr(h0, torch.float16, "h0"),
+                                     _dev_ptr(c0, torch.float32, "c0"), _dev_ptr(h_all, torch.float16, "h_all"),
+                                     _dev_ptr(c_out, torch.float32, "c_out"), T, B, I, H, workspace.data_ptr(),
+                                     workspace.numel() * workspace.element_size(), _stream()))
+        return h_all, c_out
     _check(lib().tcu_lstm_f16_algo(_dev_ptr(x, torch.float16, "x"), _dev_ptr(W, torch.float16, "W"),
                                    _dev_ptr(bias, torch.float16, "bias"), _dev_ptr(h0, torch.float16, "h0"),
                                    _dev_ptr(c0, torch.float32, "c0"), _dev_ptr(h_all, torch.float16, "h_all"),
                                    _dev_ptr(c_out, torch.float32, "c_out"), T, B, I, H, LSTM_ALGOS[algo], _stream()))
     return h_all, c_out
+
+
+def lstm_workspace_bytes(T: int, B: int, I: int, H: int) -> int:
+    """Device bytes ``lstm(..., algo="hoisted")`` needs; 0 if that path is not instantiated for the shape."""
+    return int(lib().tcu_lstm_workspace_bytes(T, B, I, H))
 
 
 # ------------------------------------------------------------------------------ scatter_nd

@@ -12,6 +12,7 @@
 
 #include <mutex>
 #include <set>
+#include <algorithm>
 #include <string>
 #include <utility>
 
@@ -129,14 +130,17 @@ int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M,
 }
 
 template <typename OutType>
-int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream,
+                       int lda = 0, int ldb = 0) {
     using T = GemmW128Traits;
+    if (lda == 0) lda = K;
+    if (ldb == 0) ldb = K;
     if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0)
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM needs M % 256 == 0, N % 256 == 0, K % 64 == 0");
-    if ((long)K * 2 * T::kBM >= (1l << 32))
+    if ((long)std::max(lda, ldb) * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
     return launch(&gemm_w128<OutType>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
-                  C, M, N, K);
+                  C, M, N, K, lda, ldb);
 }
 
 template <typename OutType>
@@ -299,6 +303,28 @@ int launch_lstm(const __half* x, const __half* W, const __half* bias, const __ha
 }
 
 template <int kI, int kH>
+int launch_lstm_hoisted(const __half* x, const __half* W, const __half* bias, const __half* h0, const float* c0,
+                        __half* h_all, float* c_out, int T, int B, float* pre, hipStream_t stream) {
+    using Traits = LstmFwdTraits<kI, kH>;
+    // pre[T * B, 4H] = x[T * B, I] . W[:, :I]^T: the stored [4H, I] operand is the first I columns of W's rows
+    int rc = gemm_w128_dispatch<float>(x, W, pre, T * B, 4 * kH, kI, stream, kI, kI + kH);
+    if (rc != TCU_OK) return rc;
+    auto kernel = &lstm_cell_fwd<Traits, true>;
+    const int grid = (B / Traits::kTM) * (kH / Traits::kTH);
+    for (int t = 0; t < T; ++t) {
+        const __half* x_t = x + size_t(t) * B * kI;
+        const __half* h_in = t == 0 ? h0 : h_all + size_t(t - 1) * B * kH;
+        const float* c_in = t == 0 ? c0 : c_out;
+        __half* h_out = h_all + size_t(t) * B * kH;
+        const float* pre_t = pre + size_t(t) * B * 4 * kH;
+        rc = launch(kernel, dim3(grid), dim3(Traits::kThreads), Traits::kLdsBytes, stream, x_t, h_in, W, bias, c_in,
+                    c_out, h_out, B, pre_t);
+        if (rc != TCU_OK) return rc;
+    }
+    return TCU_OK;
+}
+
+template <int kI, int kH>
 int launch_lstm_fwd(const __half* x, const __half* W, const __half* bias, const __half* h0, const float* c0,
                     __half* h_all, float* c_out, int T, int B, hipStream_t stream) {
     using Traits = LstmFwdTraits<kI, kH>;
@@ -310,7 +336,7 @@ int launch_lstm_fwd(const __half* x, const __half* W, const __half* bias, const 
         const float* c_in = t == 0 ? c0 : c_out;
         __half* h_out = h_all + size_t(t) * B * kH;
         int rc = launch(kernel, dim3(grid), dim3(Traits::kThreads), Traits::kLdsBytes, stream, x_t, h_in, W, bias, c_in,
-                        c_out, h_out, B);
+                        c_out, h_out, B, static_cast<const float*>(nullptr));
         if (rc != TCU_OK) return rc;
     }
     return TCU_OK;
@@ -418,6 +444,38 @@ int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void
         return launch_lstm<64, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
     return fail(TCU_ERR_UNSUPPORTED_SHAPE,
                 "tcu_lstm_f16 is instantiated for (I, H) in {(1024,1024), (128,128), (256,128), (64,128)}");
+}
+
+unsigned long long tcu_lstm_workspace_bytes(int T, int B, int I, int H) {
+    const bool shape_ok = (I == 1024 && H == 1024) || (I == 128 && H == 128) || (I == 256 && H == 128);
+    if (!shape_ok || T <= 0 || B <= 0 || B % 64 != 0 || ((long)T * B) % 256 != 0) return 0;
+    return (unsigned long long)T * B * 4 * H * sizeof(float);
+}
+
+int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                    void* c_out, int T, int B, int I, int H, void* workspace, unsigned long long workspace_bytes,
+                    void* stream) {
+    if (!x || !W || !bias || !h_all || !c_out || !workspace)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_ws: null pointer");
+    if (!positive({T, B, I, H})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_ws: sizes must be positive");
+    if (!aligned16({x, W, bias, h0, c0, h_all, c_out, workspace}))
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_ws: operands must be 16-byte aligned");
+    const unsigned long long need = tcu_lstm_workspace_bytes(T, B, I, H);
+    if (need == 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_ws: instantiated for (I, H) in {(1024,1024), (128,128), "
+                                               "(256,128)} with B % 64 == 0 and T * B % 256 == 0");
+    if (workspace_bytes < need)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_ws: workspace smaller than tcu_lstm_workspace_bytes()");
+    auto s = static_cast<hipStream_t>(stream);
+    auto xp = static_cast<const __half*>(x), wp = static_cast<const __half*>(W), bp = static_cast<const __half*>(bias);
+    auto h0p = static_cast<const __half*>(h0);
+    auto c0p = static_cast<const float*>(c0);
+    auto hp = static_cast<__half*>(h_all);
+    auto cp = static_cast<float*>(c_out);
+    auto pre = static_cast<float*>(workspace);
+    if (I == 1024 && H == 1024) return launch_lstm_hoisted<1024, 1024>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
+    if (I == 128 && H == 128) return launch_lstm_hoisted<128, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
+    return launch_lstm_hoisted<256, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
 }
 
 int tcu_scatter_nd(void* data, const void* updates, const void* indices, const long long* data_dims, int rank,
