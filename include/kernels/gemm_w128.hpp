@@ -127,12 +127,6 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
                                                row * T::kRowBytes + chunk * 16);
     };
 
-    f32x4 acc[8][8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
     f16x8 fx[16], fy[16];  // fragments of substep 0 / substep 1: [0..7] A, [8..15] B
 
     const int ktiles = K / T::kBK;
@@ -141,10 +135,20 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
     if (ktiles > 1) {
 #pragma unroll
         for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(1, q), load_dst(1, q));
-        detail::lds_barrier<16>();  // this wavefront's part of tile 0 has landed; then everyone's
-    } else {
-        detail::lds_barrier<0>();
     }
+    // the 256 accumulators are cleared while the first tiles are on their way (the empty asm statements keep the
+    // compiler from sinking the clears below the barrier, where nothing would hide them)
+    f32x4 acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        asm volatile(""
+                     : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),
+                       "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]));
+    }
+    if (ktiles > 1) detail::lds_barrier<16>();  // this wavefront's part of tile 0 has landed; then everyone's
+    else detail::lds_barrier<0>();
 #pragma unroll
     for (int r = 0; r < 16; ++r) fx[r] = read_frag(0, 0, r);
 
