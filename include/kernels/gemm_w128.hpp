@@ -217,25 +217,40 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
         unsigned char* stg = lds + T::kLdsBytesMain + wave * T::kEpilogueBytesPerWave;
         const int rr = lane >> 4, cc = lane & 15;  // read-back: 16 lanes x 16 B per row, 4 rows per instruction
         OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * N + n0 + wave_n * T::kWaveN;
+        // LDS addresses of this lane's 8 staging writes and 4 read-backs of a row group (the same for every group but
+        // for the buffer), computed once: with one wavefront per SIMD the epilogue is bound by instruction issue
+        unsigned int waddr[8], raddr[4];
+        const unsigned int stg_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(stg));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int slot = (j * 16 + 4 * fquad) >> 2;
+            waddr[j] = stg_base + frow * kPitch + (slot ^ ((frow << 1) & kSlotMask)) * 8;
+            asm volatile("" : "+v"(waddr[j]));
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int row = it * 4 + rr;
+            raddr[it] = stg_base + row * kPitch + ((2 * cc) ^ ((row << 1) & kSlotMask)) * 8;
+            asm volatile("" : "+v"(raddr[it]));
+        }
+        using lds_f16x4_ptr = __attribute__((address_space(3))) f16x4*;
+        using lds_u32x4_ptr = __attribute__((address_space(3))) const u32x4*;
+        unsigned char* crow = reinterpret_cast<unsigned char*>(cbase + size_t(rr) * N) + cc * 16;  // row rr of the block
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            unsigned char* buf = stg + (i & 1) * (16 * kPitch);
+            const unsigned int buf = (i & 1) * (16 * kPitch);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const int slot = (j * 16 + 4 * fquad) >> 2;
-                const int pslot = slot ^ ((frow << 1) & kSlotMask);
                 f16x4 v;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc[i][j][e]);
-                *reinterpret_cast<f16x4*>(buf + frow * kPitch + pslot * 8) = v;
+                *reinterpret_cast<lds_f16x4_ptr>(waddr[j] + buf) = v;
             }
             // LDS operations of one wavefront execute in order: the reads below see the writes above
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
-                const int row = it * 4 + rr;
-                const int pslot = (2 * cc) ^ ((row << 1) & kSlotMask);
-                const u32x4 v = *reinterpret_cast<const u32x4*>(buf + row * kPitch + pslot * 8);
-                *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(cbase + size_t(i * 16 + row) * N) + cc * 16) = v;
+                const u32x4 v = *reinterpret_cast<lds_u32x4_ptr>(raddr[it] + buf);
+                *reinterpret_cast<u32x4*>(crow + size_t(i * 16 + it * 4) * N * sizeof(OutType)) = v;
             }
         }
     } else {
