@@ -114,14 +114,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
 
     // ---- Q fragments: B operand of Sᵀ = K Qᵀ: lane (q, h) holds Q[q][16 s + 8 h .. + 7] for k-step s,
     // pre-multiplied by scale * log2(e) so that the scores come out of the MFMA in the log2 domain.
+    // (filled after the first K/V blocks have been requested, so that the two cold latencies overlap)
     const float c = scale * 1.4426950408889634f;
     f16x8 qf[Traits::kDSteps];
+    auto load_q = [&]() {
 #pragma unroll
-    for (int s = 0; s < Traits::kDSteps; ++s) {
-        const f16x8 raw = *reinterpret_cast<const f16x8*>(Qh + size_t(q32) * kD + 16 * s + 8 * h);
+        for (int s = 0; s < Traits::kDSteps; ++s) {
+            const f16x8 raw = *reinterpret_cast<const f16x8*>(Qh + size_t(q32) * kD + 16 * s + 8 * h);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<_Float16>(static_cast<float>(raw[e]) * c);
-    }
+            for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<_Float16>(static_cast<float>(raw[e]) * c);
+        }
+    };
 
     // ---- global -> LDS for a K/V block. One instruction fills kRowsPerLoad rows.
     // The 2 * kLoadsPerTile instructions of a block (K first, then V) are dealt round-robin to the wavefronts.
@@ -175,8 +178,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int nblocks = N / kBN;
     issue_block(0, 0);
     if (nblocks > 1) issue_block(1, kBN);
-    if (nblocks > 1) __builtin_amdgcn_s_waitcnt(0x0070 | (kLoadsPerWave & 0xF));  // block 0 landed, block 1 in flight
-    else __builtin_amdgcn_s_waitcnt(0x0070);
+    load_q();  // requested after the K/V blocks: by the time Q has arrived and is converted, so have they
+    __builtin_amdgcn_s_waitcnt(0x0070);
     __syncthreads();
 
     f32x16 s_cur[Traits::kKvTiles], s_nxt[Traits::kKvTiles];
@@ -384,14 +387,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
     __half* Oh = O + (head * M + m0) * kD;
 
     // Q fragments, pre-multiplied by scale * log2(e)
+    // (filled after the first K/V blocks have been requested, so that the two cold latencies overlap)
     const float c = scale * 1.4426950408889634f;
     f16x8 qf[Traits::kDSteps];
+    auto load_q = [&]() {
 #pragma unroll
-    for (int s = 0; s < Traits::kDSteps; ++s) {
-        const f16x8 raw = *reinterpret_cast<const f16x8*>(Qh + size_t(q32) * kD + 16 * s + 8 * h);
+        for (int s = 0; s < Traits::kDSteps; ++s) {
+            const f16x8 raw = *reinterpret_cast<const f16x8*>(Qh + size_t(q32) * kD + 16 * s + 8 * h);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<_Float16>(static_cast<float>(raw[e]) * c);
-    }
+            for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<_Float16>(static_cast<float>(raw[e]) * c);
+        }
+    };
 
     // global -> LDS for a K/V block (same dealing and swizzles as flash_attention_fwd)
     constexpr int kLoadsPerBlock = 2 * Traits::kLoadsPerTile;
@@ -443,8 +449,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int nblocks = N / kBN;
     issue_block(0, 0);
     if (nblocks > 1) issue_block(1, kBN);
-    if (nblocks > 1) __builtin_amdgcn_s_waitcnt(0x0070 | (kLoadsPerWave & 0xF));  // block 0 landed, block 1 in flight
-    else __builtin_amdgcn_s_waitcnt(0x0070);
+    load_q();  // requested after the K/V blocks: by the time Q has arrived and is converted, so have they
+    __builtin_amdgcn_s_waitcnt(0x0070);
     __syncthreads();
 
     constexpr float kLazy = 8.0f;
