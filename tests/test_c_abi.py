@@ -62,6 +62,26 @@ def test_misaligned_operands_are_rejected(tcu):
     assert "16-byte aligned" in tcu.last_error()
 
 
+def test_lstm_workspace_entry_point_checks_its_arguments(tcu):
+    """tcu_lstm_f16_ws / tcu_lstm_workspace_bytes: everything that can be refused is refused before a launch."""
+    l = tcu.lib()
+    p = 0x1000
+    assert l.tcu_lstm_workspace_bytes(16, 256, 1024, 1024) == 16 * 256 * 4096 * 4
+    assert l.tcu_lstm_workspace_bytes(4, 64, 128, 128) == 4 * 64 * 512 * 4
+    assert l.tcu_lstm_workspace_bytes(3, 64, 128, 128) == 0    # T * B not a multiple of 256
+    assert l.tcu_lstm_workspace_bytes(4, 32, 128, 128) == 0    # B not a multiple of 64
+    assert l.tcu_lstm_workspace_bytes(4, 64, 64, 128) == 0     # (I, H) not instantiated for this path
+    assert l.tcu_lstm_workspace_bytes(0, 64, 128, 128) == 0
+    need = 4 * 64 * 512 * 4
+    assert l.tcu_lstm_f16_ws(p, p, p, 0, 0, p, p, 4, 64, 128, 128, 0, need, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert "null pointer" in tcu.last_error()
+    assert l.tcu_lstm_f16_ws(p, p, p, 0, 0, p, p, 4, 64, 128, 128, p, need - 1, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert "workspace" in tcu.last_error()
+    assert l.tcu_lstm_f16_ws(p, p, p, 0, 0, p, p, 4, 64, 128, 128, p + 4, need, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_lstm_f16_ws(p, p, p, 0, 0, p, p, 3, 64, 128, 128, p, need, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_lstm_f16_ws(p, p, p, 0, 0, p, p, 4, 64, 128, -1, p, need, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+
+
 def test_bad_sizes_and_enums_are_rejected(tcu):
     l = tcu.lib()
     p = 0x1000  # never dereferenced: argument checks come first
