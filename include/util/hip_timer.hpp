@@ -37,6 +37,4 @@ class HipTimer {
     hipStream_t stream_{nullptr};
 };
 
-using CudaTimer = HipTimer;  // source-compatible spelling
-
 }  // namespace tiledcuda

@@ -132,6 +132,66 @@ def test_python_wrappers_validate_before_calling(tcu):
     assert isinstance(err, RuntimeError) and err.status == -2
 
 
+def test_python_wrappers_check_operand_shapes_against_each_other(tcu):
+    """A key/value tensor with fewer leading dimensions than the query (the MQA/GQA habit), a mismatched key count,
+    a wrongly shaped output or initial state would make a kernel read or write past an allocation: all of them are
+    refused on the host, before any pointer is taken (so CPU tensors suffice here)."""
+    import torch
+
+    f16 = torch.float16
+    q = torch.zeros(2, 4, 128, 64, dtype=f16)
+    kv = torch.zeros(2, 4, 256, 64, dtype=f16)
+    with pytest.raises(ValueError, match="k must be"):
+        tcu.flash_attention(q, torch.zeros(2, 1, 256, 64, dtype=f16), kv)
+    with pytest.raises(ValueError, match="k must be"):
+        tcu.flash_attention(q, torch.zeros(256, 64, dtype=f16), kv)
+    with pytest.raises(ValueError, match="k must be"):
+        tcu.flash_attention(q, torch.zeros(2, 4, 256, 128, dtype=f16), kv)
+    with pytest.raises(ValueError, match="v must be"):
+        tcu.flash_attention(q, kv, torch.zeros(2, 4, 128, 64, dtype=f16))
+    with pytest.raises(ValueError, match="v must be"):
+        tcu.flash_attention(q, kv, torch.zeros(4, 256, 64, dtype=f16))
+    with pytest.raises(ValueError, match="out must be"):
+        tcu.flash_attention(q, kv, kv, out=torch.zeros(2, 4, 64, 64, dtype=f16))
+    with pytest.raises(ValueError, match="device memory"):  # consistent shapes get as far as the device check
+        tcu.flash_attention(q, kv, kv)
+
+    # the reference's flattened call shape: every tensor must hold exactly batch * rows * cols elements
+    Q, K, V, O = (torch.zeros(n, dtype=f16) for n in (64 * 128, 256 * 128, 128 * 256, 64 * 128))
+    with pytest.raises(ValueError, match="K must hold"):
+        tcu.flash_attention_fwd(Q, K[:-128], V, O, 64, 256, 128, 128)
+    with pytest.raises(ValueError, match="V must hold"):
+        tcu.flash_attention_fwd(Q, K, V, O, 64, 256, 128, 64)
+    with pytest.raises(ValueError, match="Q must hold"):
+        tcu.flash_attention_fwd(Q, K, V, O, 64, 256, 128, 128, batch=2)
+    with pytest.raises(ValueError, match="O must hold"):
+        tcu.flash_attention_fwd(Q, K, V, O[:100], 64, 256, 128, 128)
+    with pytest.raises(ValueError, match="positive"):
+        tcu.flash_attention_fwd(Q, K, V, O, 64, 0, 128, 128)
+    with pytest.raises(ValueError, match="device memory"):
+        tcu.flash_attention_fwd(Q, K, V, O, 64, 256, 128, 128)
+
+    a, b, c = torch.zeros(64, 64, dtype=f16), torch.zeros(128, 64, dtype=f16), torch.zeros(32, 128, dtype=f16)
+    with pytest.raises(ValueError, match="out must be"):
+        tcu.b2b_gemm(a, b, c, out=torch.zeros(1, 64, 64, dtype=f16))
+    with pytest.raises(ValueError, match="out must be"):
+        tcu.b2b_gemm(a.unsqueeze(0), b.unsqueeze(0), c.unsqueeze(0), out=torch.zeros(64, 32, dtype=f16))
+    with pytest.raises(ValueError, match="2-D or all be 3-D"):
+        tcu.b2b_gemm(a.unsqueeze(0), b, c)
+    with pytest.raises(ValueError, match="do not chain"):
+        tcu.b2b_gemm(a, b, torch.zeros(32, 64, dtype=f16))
+    with pytest.raises(ValueError, match="device memory"):
+        tcu.b2b_gemm(a, b, c, out=torch.zeros(64, 32, dtype=f16))
+
+    x, W, bias = torch.zeros(2, 64, 128, dtype=f16), torch.zeros(512, 256, dtype=f16), torch.zeros(512, dtype=f16)
+    with pytest.raises(ValueError, match="h0 must be"):
+        tcu.lstm(x, W, bias, h0=torch.zeros(32, 128, dtype=f16))
+    with pytest.raises(ValueError, match="c0 must be"):
+        tcu.lstm(x, W, bias, c0=torch.zeros(64, 64))
+    with pytest.raises(ValueError, match="x must be"):
+        tcu.lstm(x[0], W, bias)
+
+
 def test_tile_test_library_loads():
     path = os.path.join(ROOT, "tests", "device", "_build", "libtcu_tile_tests.so")
     if not os.path.exists(path):

@@ -28,6 +28,34 @@ def test_generated_sources_compile_and_export_kernel_entry(jit, tmp_path):
         assert b"kernel_entry_stream" in open(path, "rb").read()
 
 
+def test_cache_key_follows_the_source_and_cache_dir_is_private(jit, tmp_path, monkeypatch):
+    """The library name carries a digest of the generated source and of the headers: a changed kernel header must
+    not resolve to the library built from the old one. The default cache directory is private to the user."""
+    import stat
+    import subprocess
+
+    calls = []
+
+    def fake_run(cmd, **kw):
+        calls.append(cmd)
+        open(cmd[-1], "wb").close()
+        return subprocess.CompletedProcess(cmd, 0, "", "")
+
+    monkeypatch.setattr(jit.subprocess, "run", fake_run)
+    builder = jit.Compile(file_prefix="k", tmp_dir=str(tmp_path))
+    cfg = (256, 256, 256, 64, 64, 32, 2, 2)
+    first = builder.compile(*cfg)
+    assert builder.compile(*cfg) == first and len(calls) == 1
+    monkeypatch.setattr(jit, "_headers_digest", lambda: "a different set of headers")
+    second = builder.compile(*cfg)
+    assert second != first and len(calls) == 2
+
+    monkeypatch.setenv("XDG_CACHE_HOME", str(tmp_path / "cache"))
+    path = jit.Compile().tmp_dir
+    assert path.startswith(str(tmp_path / "cache"))
+    assert stat.S_IMODE(os.stat(path).st_mode) == 0o700
+
+
 def test_bad_instantiation_raises(jit, tmp_path):
     builder = jit.Compile(file_prefix="bad", tmp_dir=str(tmp_path))
     with pytest.raises(RuntimeError, match="Compilation failed"):

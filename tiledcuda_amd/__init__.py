@@ -157,6 +157,8 @@ def b2b_gemm(a: torch.Tensor, b_t: torch.Tensor, c_t: torch.Tensor, out: torch.T
     """D = (A · B) · C per batch item; ``b_t`` [.., N, K] and ``c_t`` [.., P, N] are the
     column-major operands of the reference's fused two-GEMM example stored as arrays."""
     batched = a.dim() == 3
+    if any(t.dim() != a.dim() for t in (b_t, c_t)) or a.dim() not in (2, 3):
+        raise ValueError("operands must all be 2-D or all be 3-D (batched)")
     a3, b3, c3 = (t if batched else t.unsqueeze(0) for t in (a, b_t, c_t))
     batch, M, K = a3.shape
     _, N, _ = b3.shape
@@ -165,6 +167,8 @@ def b2b_gemm(a: torch.Tensor, b_t: torch.Tensor, c_t: torch.Tensor, out: torch.T
         raise ValueError("operand shapes do not chain: A [b,M,K], b_t [b,N,K], c_t [b,P,N]")
     if out is None:
         out = torch.empty(batch, M, P, dtype=out_dtype, device=a.device)
+    elif tuple(out.shape) != (batch, M, P) and not (not batched and tuple(out.shape) == (M, P)):
+        raise ValueError(f"out must be [{batch}, {M}, {P}], got {tuple(out.shape)}")
     _check(lib().tcu_b2b_gemm_f16_algo(_dev_ptr(a3, torch.float16, "a"), _dev_ptr(b3, torch.float16, "b_t"),
                                        _dev_ptr(c3, torch.float16, "c_t"), _dev_ptr(out, out.dtype, "out"), M, N, K, P,
                                        batch, _out_code(out.dtype), B2B_ALGOS[algo], _stream()))
@@ -177,6 +181,12 @@ def flash_attention_fwd(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, O: to
     """Same call shape as the reference's ``pytiledcuda.flash_attention_fwd`` (flattened fp16
     device tensors; K as [n, k], V as [p, n]; O written in place; ``scale`` defaults to the
     reference's 1).  Unsupported shapes raise ``RuntimeError`` like the reference op."""
+    if min(m, n, k, p, batch) <= 0:
+        raise ValueError("m, n, k, p and batch must be positive")
+    for name, t, want in (("Q", Q, batch * m * k), ("K", K, batch * n * k), ("V", V, batch * p * n),
+                          ("O", O, batch * m * p)):
+        if t.numel() != want:
+            raise ValueError(f"{name} must hold batch*rows*cols = {want} elements, got {t.numel()}")
     _check(lib().tcu_flash_attn_fwd_f16(_dev_ptr(Q, torch.float16, "Q"), _dev_ptr(K, torch.float16, "K"),
                                         _dev_ptr(V, torch.float16, "V"), _dev_ptr(O, torch.float16, "O"), batch, m, n,
                                         k, p, float(scale), TCU_V_COL_MAJOR, _stream()))
@@ -186,14 +196,24 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: fl
                     out: torch.Tensor | None = None, algo: str = "auto") -> torch.Tensor:
     """softmax(scale · q kᵀ) v for [..., S, D] tensors in the usual layout (V row-major [S, D]).
     ``scale`` defaults to 1/sqrt(D)."""
+    if q.dim() < 2 or k.dim() < 2 or v.dim() < 2:
+        raise ValueError("q, k and v must be [..., S, D]")
     *lead, M, D = q.shape
     N = k.shape[-2]
     P = v.shape[-1]
+    # the kernel strides every operand by the same leading index: broadcast (MQA/GQA-style) operands would be read
+    # past their end
+    if tuple(k.shape) != (*lead, N, D):
+        raise ValueError(f"k must be {(*lead, N, D)} (same leading dimensions and head size as q), got {tuple(k.shape)}")
+    if tuple(v.shape) != (*lead, N, P):
+        raise ValueError(f"v must be {(*lead, N, P)} (same leading dimensions and key count as k), got {tuple(v.shape)}")
     batch = int(math.prod(lead)) if lead else 1
     if scale is None:
         scale = 1.0 / math.sqrt(D)
     if out is None:
         out = torch.empty(*lead, M, P, dtype=torch.float16, device=q.device)
+    elif tuple(out.shape) != (*lead, M, P):
+        raise ValueError(f"out must be {(*lead, M, P)}, got {tuple(out.shape)}")
     _check(lib().tcu_flash_attn_fwd_f16_algo(_dev_ptr(q, torch.float16, "q"), _dev_ptr(k, torch.float16, "k"),
                                              _dev_ptr(v, torch.float16, "v"), _dev_ptr(out, torch.float16, "out"),
                                              batch, M, N, D, P, float(scale), TCU_V_ROW_MAJOR, ATTN_ALGOS[algo],
@@ -233,10 +253,16 @@ def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor 
     ``algo="hoisted"`` computes the input half of the gates for all steps in one GEMM first (``tcu_lstm_f16_ws``); it
     needs ``lstm_workspace_bytes(T, B, I, H)`` bytes of device memory, taken from ``workspace`` (any dtype) if given,
     else allocated here."""
+    if x.dim() != 3 or W.dim() != 2:
+        raise ValueError("x must be [T, B, I] and W [4H, I+H]")
     T, B, I = x.shape
     H = W.shape[0] // 4
     if tuple(W.shape) != (4 * H, I + H) or tuple(bias.shape) != (4 * H,):
         raise ValueError("W must be [4H, I+H] and bias [4H]")
+    if h0 is not None and tuple(h0.shape) != (B, H):
+        raise ValueError(f"h0 must be [{B}, {H}], got {tuple(h0.shape)}")
+    if c0 is not None and tuple(c0.shape) != (B, H):
+        raise ValueError(f"c0 must be [{B}, {H}], got {tuple(c0.shape)}")
     h_all = torch.empty(T, B, H, dtype=torch.float16, device=x.device)
     c_out = torch.empty(B, H, dtype=torch.float32, device=x.device)
     if algo == "hoisted":

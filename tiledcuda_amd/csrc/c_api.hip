@@ -10,6 +10,7 @@
 #include "kernels/lstm_fwd.hpp"
 #include "kernels/mod.hpp"
 
+#include <climits>
 #include <mutex>
 #include <set>
 #include <algorithm>
@@ -61,10 +62,18 @@ int launch(Kernel kernel, dim3 grid, dim3 block, int lds_bytes, hipStream_t stre
             g_attr_done.insert(key);
         }
     }
-    hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args...);
-    hipError_t e = hipGetLastError();
+    // the launch's own return value: an error left behind earlier by unrelated code of the calling thread is neither
+    // reported as this launch's nor cleared
+    void* argv[] = {static_cast<void*>(&args)...};
+    hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, size_t(lds_bytes), stream);
     if (e != hipSuccess) return hip_fail(e, "kernel launch");
     return TCU_OK;
+}
+
+/// Adds which of the T step launches of an LSTM layer failed to the message (steps before it are enqueued).
+int lstm_step_failed(int rc, int t, int T) {
+    return fail(rc, g_last_error + " (LSTM step " + std::to_string(t) + " of " + std::to_string(T) +
+                        "; the steps before it were enqueued)");
 }
 
 bool positive(std::initializer_list<int> v) {
@@ -297,7 +306,7 @@ int launch_lstm(const __half* x, const __half* W, const __half* bias, const __ha
         __half* h_out = h_all + size_t(t) * B * kH;
         int rc = launch(kernel, dim3(B / kTM, kH / kTH), dim3(Traits::kThreads), Traits::kShmBytes, stream, x_t, h_in,
                         W, bias, c_in, c_out, h_out);
-        if (rc != TCU_OK) return rc;
+        if (rc != TCU_OK) return lstm_step_failed(rc, t, T);
     }
     return TCU_OK;
 }
@@ -307,7 +316,9 @@ int launch_lstm_hoisted(const __half* x, const __half* W, const __half* bias, co
                         __half* h_all, float* c_out, int T, int B, float* pre, hipStream_t stream) {
     using Traits = LstmFwdTraits<kI, kH>;
     // pre[T * B, 4H] = x[T * B, I] . W[:, :I]^T: the stored [4H, I] operand is the first I columns of W's rows
-    int rc = gemm_w128_dispatch<float>(x, W, pre, T * B, 4 * kH, kI, stream, kI, kI + kH);
+    const long rows = long(T) * B;
+    if (rows > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_ws: T * B exceeds the 32-bit row count");
+    int rc = gemm_w128_dispatch<float>(x, W, pre, int(rows), 4 * kH, kI, stream, kI, kI + kH);
     if (rc != TCU_OK) return rc;
     auto kernel = &lstm_cell_fwd<Traits, true>;
     const int grid = (B / Traits::kTM) * (kH / Traits::kTH);
@@ -319,7 +330,7 @@ int launch_lstm_hoisted(const __half* x, const __half* W, const __half* bias, co
         const float* pre_t = pre + size_t(t) * B * 4 * kH;
         rc = launch(kernel, dim3(grid), dim3(Traits::kThreads), Traits::kLdsBytes, stream, x_t, h_in, W, bias, c_in,
                     c_out, h_out, B, pre_t);
-        if (rc != TCU_OK) return rc;
+        if (rc != TCU_OK) return lstm_step_failed(rc, t, T);
     }
     return TCU_OK;
 }
@@ -337,7 +348,7 @@ int launch_lstm_fwd(const __half* x, const __half* W, const __half* bias, const 
         __half* h_out = h_all + size_t(t) * B * kH;
         int rc = launch(kernel, dim3(grid), dim3(Traits::kThreads), Traits::kLdsBytes, stream, x_t, h_in, W, bias, c_in,
                         c_out, h_out, B, static_cast<const float*>(nullptr));
-        if (rc != TCU_OK) return rc;
+        if (rc != TCU_OK) return lstm_step_failed(rc, t, T);
     }
     return TCU_OK;
 }
@@ -426,6 +437,7 @@ int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void
     auto hp = static_cast<__half*>(h_all);
     auto cp = static_cast<float*>(c_out);
     if (B % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16: batch must be a multiple of 64");
+    if (long(T) * B > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16: T * B exceeds the 32-bit row count");
     if (algo != TCU_LSTM_AUTO && algo != TCU_LSTM_TILE_LIBRARY && algo != TCU_LSTM_STREAMING)
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: unknown algo");
     if (algo != TCU_LSTM_TILE_LIBRARY) {
@@ -443,7 +455,10 @@ int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void
     if (I == 64 && H == 128)
         return launch_lstm<64, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
     return fail(TCU_ERR_UNSUPPORTED_SHAPE,
-                "tcu_lstm_f16 is instantiated for (I, H) in {(1024,1024), (128,128), (256,128), (64,128)}");
+                algo == TCU_LSTM_TILE_LIBRARY
+                    ? "the tile-library LSTM kernel is instantiated for (I, H) in {(1024,1024), (128,128), (64,128)}"
+                    : "tcu_lstm_f16 is instantiated for (I, H) in {(1024,1024), (128,128), (256,128)} (streaming "
+                      "kernel) and (64,128) (tile-library kernel)");
 }
 
 unsigned long long tcu_lstm_workspace_bytes(int T, int B, int I, int H) {
@@ -515,9 +530,7 @@ int tcu_scatter_nd(void* data, const void* updates, const void* indices, const l
     const dim3 grid(static_cast<unsigned>(want < 1 ? 1 : (want > 256 * 64 ? 256 * 64 : want))), block(256);
     auto go = [&](auto* dptr, auto kernel) {
         using T = std::remove_pointer_t<decltype(dptr)>;
-        hipLaunchKernelGGL(kernel, grid, block, 0, s, dptr, static_cast<const T*>(updates), idx, shape, bad);
-        hipError_t e = hipGetLastError();
-        return e == hipSuccess ? int(TCU_OK) : hip_fail(e, "scatter_nd launch");
+        return launch(kernel, grid, block, 0, s, dptr, static_cast<const T*>(updates), idx, shape, bad);
     };
     if (dtype == TCU_DTYPE_F32) {
         auto* d = static_cast<float*>(data);

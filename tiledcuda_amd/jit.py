@@ -12,6 +12,7 @@ operand), C is [M, N] fp32.
 from __future__ import annotations
 
 import ctypes
+import hashlib
 import os
 import shutil
 import subprocess
@@ -71,6 +72,31 @@ extern "C" int kernel_entry_stream(__half* parameter1, __half* parameter2, float
 """
 
 
+def _default_cache_dir() -> str:
+    """A directory only this user can write (mode 0700): the libraries in it are loaded into the process, so a
+    world-writable location would let another user of the host plant one."""
+    base = os.environ.get("XDG_CACHE_HOME") or os.path.join(os.path.expanduser("~"), ".cache")
+    path = os.path.join(base, "tiledcuda_amd", "jit")
+    try:
+        os.makedirs(path, mode=0o700, exist_ok=True)
+        if os.stat(path).st_uid == os.getuid() and os.access(path, os.W_OK):
+            return path
+    except OSError:
+        pass
+    return tempfile.mkdtemp(prefix="tiledcuda_amd_jit_")  # created 0700, unique to this process
+
+
+def _headers_digest() -> str:
+    """Digest of the contents of every header under include/ (the generated sources include them)."""
+    h = hashlib.sha256()
+    for root, _dirs, files in sorted(os.walk(INCLUDE_DIR)):
+        for name in sorted(files):
+            if name.endswith((".hpp", ".h")):
+                with open(os.path.join(root, name), "rb") as f:
+                    h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
+
+
 def _find_hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"),
                  os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "hipcc")):
@@ -86,10 +112,10 @@ class Compile:
     def __init__(self, file_prefix: str = "gemm", tmp_dir: str | None = None, kernel: str = "tile_library"):
         if kernel not in ("tile_library", "pipelined"):
             raise ValueError("kernel must be 'tile_library' or 'pipelined'")
-        self.tmp_dir = tmp_dir or os.path.join(tempfile.gettempdir(), "tiledcuda_amd_jit")
+        self.tmp_dir = tmp_dir or _default_cache_dir()
         self.file_prefix = file_prefix
         self.kernel = kernel
-        os.makedirs(self.tmp_dir, exist_ok=True)
+        os.makedirs(self.tmp_dir, mode=0o700, exist_ok=True)
         self.hipcc_path = _find_hipcc()
         self._libs: dict[str, ctypes.CDLL] = {}
 
@@ -101,13 +127,18 @@ class Compile:
                 timeout: float | None = None) -> str | None:
         """Returns the library path, None on a compiler timeout; raises RuntimeError (with the compiler's
         output) if the instantiation does not compile, e.g. a tile that does not divide over the wavefronts."""
-        file_name = f"{self.file_prefix}_{self.kernel}_{M}_{N}_{K}_{TM}_{TN}_{kChunkK}_{warp_per_row}_{warp_per_col}"
+        source = self._create_entry_code(M, N, K, TM, TN, kChunkK, warp_per_row, warp_per_col)
+        # the name carries a digest of the generated source and of every header it can include, so that an edited
+        # kernel header never resolves to a library built from the old one
+        digest = hashlib.sha256((source + _headers_digest()).encode()).hexdigest()[:16]
+        file_name = (f"{self.file_prefix}_{self.kernel}_{M}_{N}_{K}_{TM}_{TN}_{kChunkK}_{warp_per_row}_{warp_per_col}"
+                     f"_{digest}")
         lib_path = os.path.join(self.tmp_dir, f"{file_name}.so")
         if os.path.exists(lib_path):
             return lib_path
         source_path = os.path.join(self.tmp_dir, f"{file_name}.hip")
         with open(source_path, "w") as f:
-            f.write(self._create_entry_code(M, N, K, TM, TN, kChunkK, warp_per_row, warp_per_col))
+            f.write(source)
         tmp_out = lib_path + f".{os.getpid()}.tmp"
         command = [self.hipcc_path, "--offload-arch=gfx950", "-std=c++20", "-O3", "-fPIC", "-shared",
                    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", f"-I{INCLUDE_DIR}",
