@@ -145,6 +145,21 @@ int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* 
                     void* c_out, int T, int B, int I, int H, void* workspace, unsigned long long workspace_bytes,
                     void* stream);
 
+/*
+ * tcu_lstm_f16_ws for callers that can neither allocate device memory nor bring a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. No counterpart in the reference. The [T, B, 4H] f32
+ * gate pre-activations go to a buffer of tcu_lstm_noalloc_max_bytes() (64 MiB) that is part of the library's device
+ * image (each GPU the library is used on holds its own copy until the process ends); the call allocates and frees
+ * nothing. Same arguments, shape rules and results as tcu_lstm_f16_ws; shapes with T * B * 4H * 4 bytes above the
+ * maximum fail with TCU_ERR_UNSUPPORTED_SHAPE (the C5 layer, T 16 x B 256 x H 1024, fits exactly). Every call on one
+ * GPU uses that GPU's one buffer: calls whose work overlaps in time on one GPU (different streams, or different host
+ * threads) race on it; calls on one stream are ordered and safe. Nothing in the buffer has to start at zero (the
+ * projection GEMM overwrites every element a step kernel reads), and it keeps the last call's contents.
+ */
+unsigned long long tcu_lstm_noalloc_max_bytes(void);
+int tcu_lstm_f16_noalloc(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                         void* c_out, int T, int B, int I, int H, void* stream);
+
 /* How tcu_scatter_nd combines an update with the data it lands on. */
 typedef enum {
     TCU_SCATTER_ASSIGN = 0, /* data[...] = update: what the reference's test checks (tests/python/test_scatter_nd.py:47-56) */

@@ -20,7 +20,7 @@ def declared_symbols():
 
 def test_header_declares_the_entry_points():
     syms = declared_symbols()
-    for name in ("tcu_gemm_f16", "tcu_b2b_gemm_f16", "tcu_flash_attn_fwd_f16", "tcu_lstm_f16", "tcu_flash_attn_fwd_f16_algo", "tcu_lstm_f16_algo", "tcu_lstm_f16_ws", "tcu_lstm_workspace_bytes", "tcu_last_error",
+    for name in ("tcu_gemm_f16", "tcu_b2b_gemm_f16", "tcu_flash_attn_fwd_f16", "tcu_lstm_f16", "tcu_flash_attn_fwd_f16_algo", "tcu_lstm_f16_algo", "tcu_lstm_f16_ws", "tcu_lstm_workspace_bytes", "tcu_lstm_f16_noalloc", "tcu_lstm_noalloc_max_bytes", "tcu_last_error",
                  "tcu_version", "tcu_device_count"):
         assert name in syms
 
@@ -80,6 +80,21 @@ def test_lstm_workspace_entry_point_checks_its_arguments(tcu):
     assert l.tcu_lstm_f16_ws(p, p, p, 0, 0, p, p, 4, 64, 128, 128, p + 4, need, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
     assert l.tcu_lstm_f16_ws(p, p, p, 0, 0, p, p, 3, 64, 128, 128, p, need, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_lstm_f16_ws(p, p, p, 0, 0, p, p, 4, 64, 128, -1, p, need, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+
+
+def test_no_alloc_lstm_entry_point_checks_its_arguments(tcu):
+    """tcu_lstm_f16_noalloc refuses, before any device call, what its fixed buffer cannot hold."""
+    l = tcu.lib()
+    p = 0x1000
+    limit = l.tcu_lstm_noalloc_max_bytes()
+    assert limit == 64 << 20 == l.tcu_lstm_workspace_bytes(16, 256, 1024, 1024)
+    assert l.tcu_lstm_f16_noalloc(p, p, p, 0, 0, p, p, 32, 256, 1024, 1024, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert "static scratch buffer" in tcu.last_error() and str(limit) in tcu.last_error()
+    assert l.tcu_lstm_f16_noalloc(p, p, p, 0, 0, p, p, 3, 64, 128, 128, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_lstm_f16_noalloc(p, p, 0, 0, 0, p, p, 4, 64, 128, 128, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert "null pointer" in tcu.last_error()
+    assert l.tcu_lstm_f16_noalloc(p, p, p, 0, 0, p + 2, p, 4, 64, 128, 128, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
+    assert l.tcu_lstm_f16_noalloc(p, p, p, 0, 0, p, p, 4, 64, 128, 0, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
 
 
 def test_bad_sizes_and_enums_are_rejected(tcu):

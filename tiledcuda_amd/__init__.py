@@ -62,6 +62,8 @@ _SIGNATURES = {
     "tcu_lstm_workspace_bytes": (ctypes.c_ulonglong, [ctypes.c_int] * 4),
     "tcu_lstm_f16_ws": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_ulonglong,
                                                                                      ctypes.c_void_p]),
+    "tcu_lstm_noalloc_max_bytes": (ctypes.c_ulonglong, []),
+    "tcu_lstm_f16_noalloc": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
     "tcu_scatter_nd": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.POINTER(ctypes.c_longlong), ctypes.c_int,
                                                              ctypes.c_longlong, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                              ctypes.c_void_p, ctypes.c_void_p]),

@@ -90,6 +90,36 @@ bool aligned16(std::initializer_list<const void*> v) {
     return true;
 }
 
+// ---------------------------------------------------------------------------- static scratch
+// Device memory owned by the library for the entry point that may not allocate (tcu_lstm_f16_noalloc): every device
+// the library runs on holds one copy of this array, at its own address, until the process ends. In host code the
+// array's name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr unsigned long long kScratchBytes = 64ull << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+/// Device address of `scratch` on the current device, looked up once per device.
+int scratch_address(void** out) {
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (device < 0 || device >= kMaxDevices) return fail(TCU_ERR_HIP, "device ordinal beyond the scratch table");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        if (!ptr || reinterpret_cast<uintptr_t>(ptr) % 256 != 0)
+            return fail(TCU_ERR_HIP, "hipGetSymbolAddress(scratch) returned an unusable address");
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return TCU_OK;
+}
+
 // ---------------------------------------------------------------------------- GEMM
 template <typename OutType, int kM, int kN, int kK, int kTM, int kTN, int kChunkK, typename WarpLayout>
 int launch_simple_gemm(const __half* A, const __half* B, OutType* C, hipStream_t stream) {
@@ -491,6 +521,28 @@ int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* 
     if (I == 1024 && H == 1024) return launch_lstm_hoisted<1024, 1024>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
     if (I == 128 && H == 128) return launch_lstm_hoisted<128, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
     return launch_lstm_hoisted<256, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
+}
+
+unsigned long long tcu_lstm_noalloc_max_bytes(void) { return kScratchBytes; }
+
+int tcu_lstm_f16_noalloc(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                         void* c_out, int T, int B, int I, int H, void* stream) {
+    if (!x || !W || !bias || !h_all || !c_out) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_noalloc: null pointer");
+    if (!positive({T, B, I, H})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_noalloc: sizes must be positive");
+    if (!aligned16({x, W, bias, h0, c0, h_all, c_out}))
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_noalloc: operands must be 16-byte aligned");
+    const unsigned long long need = tcu_lstm_workspace_bytes(T, B, I, H);
+    if (need == 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_noalloc: instantiated for (I, H) in {(1024,1024), (128,128), "
+                                               "(256,128)} with B % 64 == 0 and T * B % 256 == 0");
+    if (need > kScratchBytes)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE,
+                    "tcu_lstm_f16_noalloc: the gate pre-activations need " + std::to_string(need) +
+                        " bytes, more than the library's static scratch buffer of " + std::to_string(kScratchBytes) +
+                        " bytes (T * B * 4H * 4 must not exceed it); use tcu_lstm_f16_ws with a caller-owned workspace");
+    void* ws = nullptr;
+    if (int rc = scratch_address(&ws); rc != TCU_OK) return rc;
+    return tcu_lstm_f16_ws(x, W, bias, h0, c0, h_all, c_out, T, B, I, H, ws, kScratchBytes, stream);
 }
 
 int tcu_scatter_nd(void* data, const void* updates, const void* indices, const long long* data_dims, int rank,
