@@ -1,0 +1,610 @@
+// FlashAttention-2 forward for gfx950 with one wavefront per SIMD: O = softmax(scale · Q·Kᵀ)·V, f16 in/out, f32
+// accumulation and statistics. Same contract and layouts as kernels/flash_attn_fwd.hpp (Q [M, D], K [N, D], V [N, D],
+// O [M, D] row-major per batch item; the tuned counterpart of the reference's src/kernels/flash_attn.cu:134-312).
+// What changes is how the work is mapped to the CU:
+//   * a workgroup is 4 wavefronts, one per SIMD, each owning 64 query rows (two 32-query column tiles of Sᵀ / Oᵀ):
+//     every K fragment and every Vᵀ fragment read from LDS feeds two MFMAs, which halves the LDS traffic per MFMA
+//     against 32 queries per wavefront (there the LDS read rate, not the matrix pipe, was the limit);
+//   * all matrix instructions are inline assembly. The 128 f32 accumulators of Oᵀ and the Q fragments live in
+//     AGPRs, the score tiles and the probabilities in VGPRs; the instruction order is the one written here.
+//     The compiler does not know these statements are MFMAs and inserts none of the wait states MFMA results need
+//     before other instructions read them; the schedule below keeps every such read at least two MFMAs behind
+//     the write, and the rare paths wait explicitly;
+//   * the key sequence is processed in halves of 32 keys, software-pipelined inside the one instruction stream:
+//     step i issues the 16 MFMAs of Sᵀ(i+1) = K·Qᵀ and the 16 MFMAs of Oᵀ += Vᵀ(i-1)·Pᵀ(i-1), interleaved
+//     with the VALU work of the softmax of half i (per MFMA: one v_exp_f32, half a conversion, half a dot2), so
+//     the matrix pipe and the vector ALU are both busy all the time and neither waits for the other;
+//   * softmax without a running maximum in the common path: the score accumulators start at -m (m = reference
+//     maximum of the query, handed to the first MFMA of a tile as its C operand), p = exp2(acc) is converted to
+//     f16 and summed from the f16 values (v_dot2_f32_f16, so numerator and denominator see the same rounding);
+//     only the sum of a half is checked: while it stays below 2^14 no probability can exceed 2^14, far inside f16
+//     range, and a stale reference maximum is harmless (the final division cancels it). If the check fails (a score
+//     more than 14 above its reference in the log2 domain), the maxima are moved, Oᵀ and the sums are rescaled, the
+//     scores already computed for the next half are re-biased and the probabilities are recomputed;
+//   * K/V blocks of 64 keys go global -> LDS directly into a ring of four stages, requested two blocks ahead, one
+//     LDS-only barrier per block; swizzles and the transposing V reads are those of flash_attn_fwd.hpp.
+// M % 256 == 0 and N % 64 == 0 are required (checked by the host launcher).
+#pragma once
+
+#include <type_traits>
+#include <utility>
+
+#include "config.hpp"
+#include "hip_utils.hpp"
+#include "kernels/flash_attn_fwd.hpp"  // FlashFwdTraits swizzles, detail::exchange32, detail::exp2_raw
+#include "kernels/gemm_w128.hpp"       // detail::load_lds_16B_sbase, detail::lds_barrier
+
+namespace tiledcuda::kernels {
+
+template <const int kD_>
+struct FlashW64Traits {
+    static constexpr int kD = kD_, kWaves = 4, kBN = 64;
+    static constexpr int kBM = 64 * kWaves;
+    static constexpr int kThreads = kWaves * kWaveSize;
+    static constexpr int kStages = 5;
+    using Swz = FlashFwdTraits<kD, 8, kBN>;               // row size and swizzle functions
+    static constexpr int kRowBytes = 2 * kD;
+    static constexpr int kTileBytes = kBN * kRowBytes;    // one K or V block
+    static constexpr int kHalfBytes = 32 * kRowBytes;     // 32 keys of it
+    static constexpr int kStageBytes = 2 * kTileBytes;    // K + V
+    static constexpr int kRowsPerLoad = 1024 / kRowBytes;
+    static constexpr int kLoadsPerTile = kBN / kRowsPerLoad;
+    static constexpr int kLoadsPerWave = 2 * kLoadsPerTile / kWaves;  // per block: K and V
+    static constexpr int kDSteps = kD / 16;  // k-steps of Sᵀ = K Qᵀ
+    static constexpr int kDTiles = kD / 32;  // 32-row tiles of Oᵀ
+    static constexpr int kFragAhead = 3;     // d-steps between the request of a K / V fragment and its MFMAs
+    static_assert(kD == 128, "the step schedule below is written for head size 128");
+    static_assert(kLoadsPerWave == 8 && kDSteps == 8 && kDTiles == 4);
+    static constexpr int kLdsBytes = kStages * kStageBytes;  // 160 KiB; the epilogue reuses 64 KiB of it
+    static_assert(kLdsBytes <= kMaxLdsBytes);
+};
+
+namespace detail {
+
+using f16x2 = _Float16 __attribute__((ext_vector_type(2)));
+
+/// d = a · b + c, all of d and c in VGPRs, b in AGPRs (first MFMA of a score tile: c carries -m).
+DEVICE void mfma32_score_first(f32x16& d, const f16x8& a, const f16x8& b, const f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
+}
+/// d += a · b, d in VGPRs, b in AGPRs.
+DEVICE void mfma32_score(f32x16& d, const f16x8& a, const f16x8& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+}
+/// d += a · b, d in AGPRs.
+DEVICE void mfma32_out(f32x16& d, const f16x8& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(d) : "v"(a), "v"(b));
+}
+/// f(integral_constant<int, 0>) ... f(integral_constant<int, kN - 1>): a loop whose index is a constant expression
+/// (wait counts and instruction offsets below are immediates).
+template <int kN, typename F, int... kIs>
+DEVICE void static_for_impl(F&& f, std::integer_sequence<int, kIs...>) {
+    (f(std::integral_constant<int, kIs>{}), ...);
+}
+template <int kN, typename F>
+DEVICE void static_for(F&& f) {
+    static_for_impl<kN>(f, std::make_integer_sequence<int, kN>{});
+}
+
+/// LDS fragment reads issued as inline assembly, so that the waits are the kernel's own: the compiler's waits for LDS
+/// reads it knows about are exact only inside a basic block; for fragments requested in one step of the pipeline
+/// and consumed in the next (across loop back edges and the branch of the rare path) it falls back to waiting for
+/// every read in flight, including the ones just issued for the following d-step. LDS reads return in order, so
+/// lds_wait<N>() (at most N reads outstanding) before the MFMAs of a d-step waits for exactly that d-step's fragments.
+DEVICE f16x8 lds_read_b128_untracked(unsigned int addr) {
+    f16x8 r;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr));
+    return r;
+}
+/// Two transposing 8-byte reads (addr + kOff0, addr + kOff1) forming one 16-byte MFMA operand.
+template <int kOff0, int kOff1>
+DEVICE f16x8 lds_read_tr_pair_untracked(unsigned int addr) {
+    f16x4 lo, hi;
+    asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                 : "=&v"(lo), "=&v"(hi)
+                 : "v"(addr), "n"(kOff0), "n"(kOff1));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+template <int kOutstanding>
+DEVICE void lds_wait() {
+    __builtin_amdgcn_s_waitcnt(0xC07F | (kOutstanding << 8));  // lgkmcnt(kOutstanding), nothing else
+}
+
+/// Two f32 -> one register of two f16 (round to nearest even), issued where it is written: left to the compiler, the
+/// conversions of a whole step sink to their first use and run as one block that no MFMA hides. The sources may be
+/// results of v_exp_f32: at least one other instruction must have been issued since (the callers' MFMAs are).
+DEVICE unsigned int cvt_pk_f16_here(float a, float b) {
+    unsigned int r;
+    asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+DEVICE unsigned int pack_f16x2(float a, float b) {
+    const f16x2 pk = {static_cast<_Float16>(a), static_cast<_Float16>(b)};
+    return __builtin_bit_cast(unsigned int, pk);
+}
+
+/// Wait long enough for every MFMA issued so far to have written its result (32 wait states cover the longest
+/// requirement) before `x` is touched by anything else.
+DEVICE void mfma_settle_v(f32x16& x) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(x)); }
+DEVICE void mfma_settle_a(f32x16& x) { asm volatile("s_nop 15\n\ts_nop 15" : "+a"(x)); }
+
+}  // namespace detail
+
+/// grid = (M / 256) * batch workgroups (1-D), block = 256, dynamic LDS = Traits::kLdsBytes.
+/// Workgroup ids congruent modulo 8 land on the same XCD: when the batch count is a multiple of 8 the query blocks
+/// of one (batch, head) item all get such ids, so its K and V are fetched from HBM once.
+template <typename Traits>
+__global__ void __launch_bounds__(Traits::kThreads)
+    flash_attention_fwd_w64(const __half* __restrict__ Q, const __half* __restrict__ K, const __half* __restrict__ V,
+                            __half* __restrict__ O, int batch, int M, int N, float scale) {
+    using Swz = typename Traits::Swz;
+    constexpr int kD = Traits::kD, kBN = Traits::kBN;
+    constexpr int kRowBytes = Traits::kRowBytes;
+    constexpr int kChunks = kRowBytes / 16;
+    constexpr int kStages = Traits::kStages;
+    constexpr int kL = Traits::kLoadsPerWave;
+    extern __shared__ __align__(1024) unsigned char lds[];
+
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+    const int q32 = lane & 31;  // query (column of Sᵀ / Oᵀ) of this lane within a 32-query tile
+    const int h = lane >> 5;    // lane half
+
+    const int q_blocks = M / Traits::kBM;
+    int head_i, q_block;
+    if (batch % 8 == 0) {
+        const int xcd = blockIdx.x & 7, rest = blockIdx.x >> 3;
+        q_block = rest % q_blocks;
+        head_i = (rest / q_blocks) * 8 + xcd;
+    } else {
+        q_block = blockIdx.x % q_blocks;
+        head_i = blockIdx.x / q_blocks;
+    }
+    const size_t head = head_i;
+    const int m0 = q_block * Traits::kBM + wave * 64;
+    const __half* Qh = Q + (head * M + m0) * kD;
+    const __half* Kh = K + head * size_t(N) * kD;
+    const __half* Vh = V + head * size_t(N) * kD;
+    __half* Oh = O + (head * M + m0) * kD;
+
+    const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
+
+    // ---- global -> LDS: load instruction j of this wavefront for a block (j < kL / 2: K, else V) fills
+    // kRowsPerLoad rows; the instructions of a block are dealt round-robin to the wavefronts
+    const int lrow = lane / kChunks, lchk = lane % kChunks;
+    unsigned int goff[kL];     // byte offset of this lane's 16 bytes inside the K (or V) block
+    unsigned int ldst[kL];     // LDS byte offset of the instruction's 1 KiB inside a stage
+#pragma unroll
+    for (int j = 0; j < kL; ++j) {
+        const bool is_v = j >= kL / 2;
+        const int t = wave + Traits::kWaves * (is_v ? j - kL / 2 : j);  // 1 KiB slot of the tile
+        const int row = t * Traits::kRowsPerLoad + lrow;
+        const int chunk = is_v ? (lchk ^ (Swz::v_swz(row) << 1)) : (lchk ^ Swz::k_swz(row));
+        goff[j] = static_cast<unsigned int>(row * kD + chunk * 8) * 2u;
+        ldst[j] = (is_v ? Traits::kTileBytes : 0) + t * 1024;
+    }
+    auto issue_load = [&](int block, int j) {
+        const bool is_v = j >= kL / 2;
+        const __half* src = (is_v ? Vh : Kh) + size_t(block) * kBN * kD;
+        const unsigned int dst =
+            __builtin_amdgcn_readfirstlane(lds_base + (block % kStages) * Traits::kStageBytes + ldst[j]);
+        detail::load_lds_16B_sbase(goff[j], src, dst);
+    };
+
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using Yes = std::true_type;
+    using No = std::false_type;
+
+    // ---- LDS -> registers. Addresses are 32-bit LDS offsets: a per-lane part computed once (below) plus the
+    // wave-uniform offset of the half being read (a scalar), so a fragment read costs one address addition.
+    using lds_f16x8_ptr = const f16x8 __attribute__((address_space(3)))*;
+    using fp16x4 = __fp16 __attribute__((ext_vector_type(4)));
+    using lds_fp16x4_ptr = fp16x4 __attribute__((address_space(3)))*;
+    // K fragment (A operand of Sᵀ = K Qᵀ) for d-step s: lane (row = lane % 32, h) holds K[row][16 s + 8 h .. + 7]
+    unsigned int koff[Traits::kDSteps];
+#pragma unroll
+    for (int s = 0; s < Traits::kDSteps; ++s) {
+        const int chunk = (2 * s + h) ^ Swz::k_swz(q32);  // the swizzle depends on row % 16 only
+        koff[s] = lds_base + q32 * kRowBytes + chunk * 16;
+        asm volatile("" : "+v"(koff[s]));  // keep the eight offsets in registers (not rematerialised per use)
+    }
+    auto read_k = [&](unsigned int k_half_off, int s) -> f16x8 {
+        return *reinterpret_cast<lds_f16x8_ptr>(koff[s] + k_half_off);
+    };
+    // Vᵀ fragment (A operand of Oᵀ += Vᵀ Pᵀ) for d tile dt and k-step s2 of the half: lane (d = 32 dt + lane % 32,
+    // h), slot e = key 16 s2 + 8 (e / 4) + 4 h + e % 4, fetched with two transposing reads. Within a 16-lane group,
+    // lane L supplies the address of row kv0 + L / 4, columns dbase + 4 (L % 4) .. + 3.
+    const int g = lane >> 4, L16 = lane & 15;
+    const int vrow_in = L16 >> 2;
+    const int vcol_b = (16 * (g & 1) + 4 * (L16 & 3)) * 2;
+    unsigned int voff[Traits::kDTiles];
+#pragma unroll
+    for (int dt = 0; dt < Traits::kDTiles; ++dt) {
+        const int byte_in_row = 64 * dt + vcol_b;
+        const int unit = (byte_in_row >> 5) ^ Swz::v_swz(vrow_in);  // every row read by this lane has row % 4 == vrow_in
+        voff[dt] = lds_base + (4 * h + vrow_in) * kRowBytes + unit * 32 + (byte_in_row & 31);
+        asm volatile("" : "+v"(voff[dt]));
+    }
+    auto read_v = [&](unsigned int v_half_off, int s2, int dt) -> f16x8 {
+        f16x8 vf;
+#pragma unroll
+        for (int part = 0; part < 2; ++part) {
+            const fp16x4 v4 = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+                reinterpret_cast<lds_fp16x4_ptr>(voff[dt] + v_half_off + (16 * s2 + 8 * part) * kRowBytes));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vf[4 * part + e] = static_cast<_Float16>(v4[e]);
+        }
+        return vf;
+    };
+    auto read_k_untracked = [&](unsigned int k_half_off, int s) -> f16x8 {
+        return detail::lds_read_b128_untracked(koff[s] + k_half_off);
+    };
+    auto read_v_untracked = [&](unsigned int v_half_off, auto s2_c, int dt) -> f16x8 {
+        constexpr int s2 = decltype(s2_c)::value;
+        return detail::lds_read_tr_pair_untracked<16 * s2 * kRowBytes, (16 * s2 + 8) * kRowBytes>(voff[dt] + v_half_off);
+    };
+    // LDS offset (relative to the ring) of the K rows of half `half_i` of the key sequence; V is kTileBytes further
+    auto k_half = [&](int half_i) -> unsigned int {
+        return ((half_i >> 1) % kStages) * Traits::kStageBytes + (half_i & 1) * Traits::kHalfBytes;
+    };
+    auto v_half = [&](int half_i) -> unsigned int { return k_half(half_i) + Traits::kTileBytes; };
+
+    // ---- prologue: Q and the first K/V blocks are requested together (so that the cold latencies overlap).
+    // Q fragments (B operand of Sᵀ = K Qᵀ): lane (q, h) of column tile c holds Q[32 c + q][16 s + 8 h .. + 7].
+    // Read straight from global memory that is 32 bytes from each of 32 rows per instruction; for sequences long
+    // enough to matter the wavefront instead stages its 64 contiguous rows (16 KiB) through LDS like a K block
+    // (coalesced 1 KiB loads, same swizzle, same fragment reads), in the two ring stages (3 and 4) that the K/V
+    // blocks reach last; those two blocks are then requested in the first block-iteration.
+    const int nb = N / kBN;
+    const bool q_via_lds = nb >= kStages;
+    f16x8 qraw[2][Traits::kDSteps];
+    if (q_via_lds) {
+        const unsigned int q_stage = 3 * Traits::kStageBytes + wave * (64 * kRowBytes);
+#pragma unroll
+        for (int t = 0; t < 64 / Traits::kRowsPerLoad; ++t) {
+            const int row = t * Traits::kRowsPerLoad + lrow;
+            const unsigned int off = static_cast<unsigned int>(row * kD + (lchk ^ Swz::k_swz(row)) * 8) * 2u;
+            detail::load_lds_16B_sbase(off, Qh, __builtin_amdgcn_readfirstlane(lds_base + q_stage + t * 1024));
+        }
+#pragma unroll
+        for (int j = 0; j < kL; ++j) {
+            issue_load(0, j);
+        }
+        // Only Q and block 0 are requested before the first scores: all workgroups of a round start together, and
+        // what they request at once arrives at the rate of the memory system (three more blocks per workgroup
+        // would be 20 MB more, and issuing a load blocks while the queues are full); blocks 1 and 2 are requested
+        // under the first two score computations below, blocks 3 and 4 in the first block-iteration.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_s_barrier();
+
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int s = 0; s < Traits::kDSteps; ++s) qraw[c][s] = read_k(q_stage + c * Traits::kHalfBytes, s);
+    } else {
+#pragma unroll
+        for (int b = 0; b < kStages - 1; ++b)
+            if (b < nb) {
+#pragma unroll
+                for (int j = 0; j < kL; ++j) issue_load(b, j);
+            }
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int s = 0; s < Traits::kDSteps; ++s)
+                qraw[c][s] = *reinterpret_cast<const f16x8*>(Qh + size_t(32 * c + q32) * kD + 16 * s + 8 * h);
+    }
+    // pre-multiplied by scale * log2(e): the scores come out of the MFMA in the log2 domain
+    const float cscale = scale * 1.4426950408889634f;
+    f16x8 qf[2][Traits::kDSteps];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int s = 0; s < Traits::kDSteps; ++s) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qf[c][s][e] = static_cast<_Float16>(static_cast<float>(qraw[c][s][e]) * cscale);
+        }
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int s = 0; s < Traits::kDSteps; ++s) asm volatile("" : "+a"(qf[c][s]));
+
+    f32x16 o_acc[Traits::kDTiles][2];  // Oᵀ tiles (d tile, query tile), AGPRs
+#pragma unroll
+    for (int dt = 0; dt < Traits::kDTiles; ++dt)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o_acc[dt][c][e] = 0.f;
+            asm volatile("" : "+a"(o_acc[dt][c]));
+        }
+
+    f32x16 s_acc[2][2];   // score tiles: [buffer][query tile], relative to the reference maximum
+    u32x4 pf[2][2][2];    // probabilities as B operands, two f16 per element: [buffer][query tile][k-step of the half]
+    f32x16 negm[2];       // -m of this lane's query of tile c, in all 16 slots (C operand of a tile's first MFMA)
+    float m_run[2], l_run[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) negm[c][e] = 0.f;
+
+    if (!q_via_lds) detail::lds_barrier<0>();  // everything requested so far has landed, for everyone
+
+
+    // scores of half `half_i` into buffer `buf` (MFMAs only; used before the pipeline is running)
+    auto qk_only = [&](int half_i, auto buf_c, int load_block) {
+        constexpr int buf = decltype(buf_c)::value;
+        const unsigned int sk = k_half(half_i);
+        f16x8 kf[2];
+        kf[0] = read_k(sk, 0);
+#pragma unroll
+        for (int s = 0; s < Traits::kDSteps; ++s) {
+            if (s + 1 < Traits::kDSteps) kf[(s + 1) & 1] = read_k(sk, s + 1);
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                if (s == 0) detail::mfma32_score_first(s_acc[buf][c], kf[s & 1], qf[c][s], negm[c]);
+                else detail::mfma32_score(s_acc[buf][c], kf[s & 1], qf[c][s]);
+            }
+            if (load_block > 0 && load_block < nb) issue_load(load_block, s);
+        }
+    };
+
+    // ---- half 0: exact maximum
+    qk_only(0, std::integral_constant<int, 0>{}, q_via_lds ? 1 : 0);
+    detail::mfma_settle_v(s_acc[0][0]);
+    detail::mfma_settle_v(s_acc[0][1]);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        float mx = s_acc[0][c][0];
+#pragma unroll
+        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s_acc[0][c][e]);
+        mx = fmaxf(mx, detail::exchange32(mx));
+        m_run[c] = mx;
+        float lsum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) {
+            const float p0 = detail::exp2_raw(s_acc[0][c][e] - mx);
+            const float p1 = detail::exp2_raw(s_acc[0][c][e + 1] - mx);
+            pf[0][c][e / 8][(e % 8) / 2] = detail::pack_f16x2(p0, p1);
+            lsum += p0 + p1;
+        }
+        l_run[c] = lsum;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) negm[c][e] = -mx;
+    }
+    qk_only(1, std::integral_constant<int, 1>{}, q_via_lds ? 2 : 0);
+
+    // ---- one pipelined step: softmax of half i (buffer kCur), scores of half i + 1 (if kQk) into the other
+    // buffer, output update with half i - 1 (probabilities of the other buffer). kLoads: this wavefront also issues
+    // its loads of block `load_block`, one per d-step. Fragments are requested kAhead d-steps before the MFMAs that
+    // use them, across the boundaries between steps (with one wavefront per SIMD nothing else covers the LDS
+    // latency): the last d-steps of a step request the first fragments of the next one (K of half i + 2 if
+    // kNextQk, V of half i).
+    constexpr int kAhead = Traits::kFragAhead, kRing = kAhead + 1;
+    static_assert(8 % kRing == 0 && kAhead <= 3, "ring positions must repeat from one step to the next; the prefetch stays within the first k-step of the next half");
+    f16x8 kf[kRing], vf[kRing];
+    auto step = [&](int i, auto cur_c, auto qk_c, auto loads_c, auto next_qk_c, int load_block) {
+        constexpr int kCur = decltype(cur_c)::value, kNxt = kCur ^ 1;
+        constexpr bool kQk = decltype(qk_c)::value, kLoads = decltype(loads_c)::value;
+        constexpr bool kNextQk = decltype(next_qk_c)::value;
+        const unsigned int sk = __builtin_amdgcn_readfirstlane(k_half(i + 1));
+        const unsigned int sv = __builtin_amdgcn_readfirstlane(v_half(i - 1));
+        const unsigned int sk_next = __builtin_amdgcn_readfirstlane(k_half(i + 2));
+        const unsigned int sv_next = __builtin_amdgcn_readfirstlane(v_half(i));
+        float lh[2] = {0.f, 0.f}, lg[2] = {0.f, 0.f};  // two partial sums per query tile (independent add chains)
+        // VALU work of the same wavefront hides under its MFMAs only in small doses: one v_exp_f32 plus one or two
+        // plain instructions directly behind each MFMA cost 2-3 cycles per MFMA, the same instructions in groups of
+        // four or more cost their full issue time. So a d-step is four slots of one MFMA and its share of the
+        // softmax (the pair of query tile 1 is converted and summed one d-step later), fenced from each other.
+        float x0 = 0.f, x1 = 0.f, y0 = 0.f, y1 = 0.f;
+        auto pack_pair = [&](auto c_c, auto d_c, float a0, float a1) {
+            // probabilities of slots 2 d, 2 d + 1 of query tile c: to f16, into the B operand
+            constexpr int c = decltype(c_c)::value, d = decltype(d_c)::value;
+            pf[kCur][c][d >> 2][d & 3] = detail::cvt_pk_f16_here(a0, a1);
+        };
+        auto ex = [&](float v) { return detail::exp2_raw(v); };
+        detail::static_for<8>([&](auto s_c) {
+            constexpr int s = decltype(s_c)::value;
+            constexpr int sp = s + kAhead;
+            if constexpr (sp < 8) {
+                if (kQk) kf[sp % kRing] = read_k_untracked(sk, sp);
+                if (sp < 4) vf[sp % kRing] = read_v_untracked(sv, C0{}, sp & 3);
+                else vf[sp % kRing] = read_v_untracked(sv, C1{}, sp & 3);
+                detail::lds_wait<kAhead * (kQk ? 3 : 2)>();
+            } else {
+                if (kNextQk) kf[sp % kRing] = read_k_untracked(sk_next, sp - 8);
+                vf[sp % kRing] = read_v_untracked(sv_next, C0{}, (sp - 8) & 3);
+                // in flight after this wait: the fragments of the d-steps still ahead in this step (3 or 2 reads
+                // each) and those just requested for the next step
+                detail::lds_wait<(7 - s) * (kQk ? 3 : 2) + (sp - 7) * (kNextQk ? 3 : 2)>();
+            }
+            // slot A
+            if (kQk) {
+                if (s == 0) detail::mfma32_score_first(s_acc[kNxt][0], kf[s % kRing], qf[0][s], negm[0]);
+                else detail::mfma32_score(s_acc[kNxt][0], kf[s % kRing], qf[0][s]);
+            }
+            x0 = ex(s_acc[kCur][0][2 * s]);
+            if constexpr (s > 0) pack_pair(C1{}, std::integral_constant<int, s - 1>{}, y0, y1);
+            __builtin_amdgcn_sched_barrier(0);
+            // slot B
+            if (kQk) {
+                if (s == 0) detail::mfma32_score_first(s_acc[kNxt][1], kf[s % kRing], qf[1][s], negm[1]);
+                else detail::mfma32_score(s_acc[kNxt][1], kf[s % kRing], qf[1][s]);
+            }
+            x1 = ex(s_acc[kCur][0][2 * s + 1]);
+            if constexpr (s > 0) {
+                lh[1] += y0;
+                lg[1] += y1;
+            }
+            if (kLoads) issue_load(load_block, s);
+            __builtin_amdgcn_sched_barrier(0);
+            // slot C
+            detail::mfma32_out(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2]);
+            y0 = ex(s_acc[kCur][1][2 * s]);
+            pack_pair(C0{}, s_c, x0, x1);
+            __builtin_amdgcn_sched_barrier(0);
+            // slot D
+            detail::mfma32_out(o_acc[s & 3][1], vf[s % kRing], pf[kNxt][1][s >> 2]);
+            y1 = ex(s_acc[kCur][1][2 * s + 1]);
+            lh[0] += x0;
+            lg[0] += x1;
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        lh[1] += y0;
+        lg[1] += y1;
+        lh[0] += lg[0];
+        lh[1] += lg[1];
+        pack_pair(C1{}, std::integral_constant<int, 7>{}, y0, y1);
+        // the check: no probability of this half can have left f16 range while its sum stays below 2^14
+        constexpr float kLimit = 16384.f;
+        if (__any(!(fmaxf(lh[0], lh[1]) <= kLimit))) {
+            // rare path: move the reference maxima, rescale, re-bias, recompute
+            if (kQk) {
+                detail::mfma_settle_v(s_acc[kNxt][0]);
+                detail::mfma_settle_v(s_acc[kNxt][1]);
+            }
+#pragma unroll
+            for (int dt = 0; dt < Traits::kDTiles; ++dt)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) detail::mfma_settle_a(o_acc[dt][c]);
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                float mx = s_acc[kCur][c][0];
+#pragma unroll
+                for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s_acc[kCur][c][e]);
+                mx = fmaxf(mx, detail::exchange32(mx));
+                const float shift = mx > 8.0f ? mx : 0.f;  // queries whose scores stayed near their reference keep it
+                const float alpha = detail::exp2_raw(-shift);
+                m_run[c] += shift;
+                l_run[c] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < Traits::kDTiles; ++dt)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o_acc[dt][c][e] *= alpha;
+                if (kQk) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) s_acc[kNxt][c][e] -= shift;
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) negm[c][e] = -m_run[c];
+                float lsum = 0.f;
+#pragma unroll
+                for (int e = 0; e < 16; e += 2) {
+                    const float p0 = detail::exp2_raw(s_acc[kCur][c][e] - shift);
+                    const float p1 = detail::exp2_raw(s_acc[kCur][c][e + 1] - shift);
+                    pf[kCur][c][e / 8][(e % 8) / 2] = detail::pack_f16x2(p0, p1);
+                    lsum += p0 + p1;
+                }
+                lh[c] = lsum;
+            }
+#pragma unroll
+            for (int dt = 0; dt < Traits::kDTiles; ++dt)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) asm volatile("" : "+a"(o_acc[dt][c]));
+        }
+        l_run[0] += lh[0];
+        l_run[1] += lh[1];
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // Hand-over of a stage: this wavefront's loads up to and including block J + 2 have landed (kPending newer
+    // ones may stay in flight), then everyone's; and everyone has left block J - 1, whose stage block J + 4 goes to.
+    // LDS reads in flight are fragment requests for the next d-steps and belong to younger stages: no lgkmcnt wait.
+    auto hand_over = [&](auto pending_c) {
+        constexpr int kPending = decltype(pending_c)::value;
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00 | (kPending & 0xF) | ((kPending >> 4) << 14));  // vmcnt only
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+
+    // first fragments of step 1
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) {
+        if (nb > 1) kf[a] = read_k_untracked(k_half(2), a);
+        vf[a] = read_v_untracked(v_half(0), C0{}, a & 3);
+    }
+    // ---- block-iterations: J covers halves 2 J + 1 (odd) and 2 J + 2 (even)
+    int J = 0;
+    if (q_via_lds) {
+        // J = 0: blocks 3 and 4 go to the stages the Q tiles were staged in (everyone has read its Q by now)
+        hand_over(std::integral_constant<int, 0>{});
+        step(1, C1{}, Yes{}, Yes{}, Yes{}, 3);
+        step(2, C0{}, Yes{}, Yes{}, Yes{}, 4);
+        J = 1;
+    }
+    for (; J + 4 < nb; ++J) {
+        hand_over(std::integral_constant<int, kL>{});
+        step(2 * J + 1, C1{}, Yes{}, Yes{}, Yes{}, J + 4);
+        step(2 * J + 2, C0{}, Yes{}, No{}, Yes{}, 0);
+    }
+    for (; J + 2 < nb; ++J) {
+        hand_over(std::integral_constant<int, 0>{});
+        step(2 * J + 1, C1{}, Yes{}, No{}, Yes{}, 0);
+        step(2 * J + 2, C0{}, Yes{}, No{}, Yes{}, 0);
+    }
+    if (J + 1 < nb) {
+        step(2 * J + 1, C1{}, Yes{}, No{}, Yes{}, 0);
+        step(2 * J + 2, C0{}, Yes{}, No{}, No{}, 0);
+        ++J;
+    }
+    step(2 * J + 1, C1{}, No{}, No{}, No{}, 0);
+    {
+        // the output update with the last half (its first fragments were requested by the step before)
+        const unsigned int sv = v_half(2 * J + 1);
+        detail::static_for<8>([&](auto s_c) {
+            constexpr int s = decltype(s_c)::value;
+            constexpr int sp = s + kAhead;
+            if constexpr (sp < 8) {
+                if (sp < 4) vf[sp % kRing] = read_v_untracked(sv, C0{}, sp & 3);
+                else vf[sp % kRing] = read_v_untracked(sv, C1{}, sp & 3);
+                detail::lds_wait<kAhead * 2>();
+            } else {
+                detail::lds_wait<(7 - s) * 2>();
+            }
+#pragma unroll
+            for (int c = 0; c < 2; ++c) detail::mfma32_out(o_acc[s & 3][c], vf[s % kRing], pf[1][c][s >> 2]);
+        });
+    }
+
+    // ---- epilogue: O[q, d] = Oᵀ[d, q] / l. o_acc[dt][c][r]: d = 32 dt + 8 (r / 4) + 4 h + r % 4, q = 32 c + q32.
+#pragma unroll
+    for (int dt = 0; dt < Traits::kDTiles; ++dt)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) detail::mfma_settle_a(o_acc[dt][c]);
+    __syncthreads();  // all wavefronts are done with the K/V stages: reuse LDS for staging
+    unsigned char* stg = lds + wave * (64 * kRowBytes);
+    constexpr int kSlotMask = (kRowBytes / 8 - 1) & ~1;  // 8-byte slots of a staged row are XOR-ed with 2 * (row % 16)
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const float l_tot = l_run[c] + detail::exchange32(l_run[c]);
+        const float inv_l = 1.0f / l_tot;
+        const int row = 32 * c + q32;
+#pragma unroll
+        for (int dt = 0; dt < Traits::kDTiles; ++dt) {
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                f16x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(o_acc[dt][c][4 * qd + e] * inv_l);
+                const int slot = (32 * dt + 8 * qd + 4 * h) >> 2;
+                const int pslot = slot ^ (((row & 15) << 1) & kSlotMask);
+                *reinterpret_cast<f16x4*>(stg + row * kRowBytes + pslot * 8) = v;
+            }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // this wavefront's staging writes are done (it reads only its own rows)
+    constexpr int kLanesPerRow = kRowBytes / 16;
+    constexpr int kRowsPerIter = kWaveSize / kLanesPerRow;
+    const int rr = lane / kLanesPerRow, cc = lane % kLanesPerRow;
+#pragma unroll
+    for (int it = 0; it < 64 / kRowsPerIter; ++it) {
+        const int row = it * kRowsPerIter + rr;
+        const int pslot = (2 * cc) ^ (((row & 15) << 1) & kSlotMask);
+        const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kRowBytes + pslot * 8);
+        *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(Oh + size_t(row) * kD) + cc * 16) = v;
+    }
+}
+
+}  // namespace tiledcuda::kernels

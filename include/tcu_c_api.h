@@ -51,14 +51,18 @@ typedef enum {
     TCU_V_ROW_MAJOR = 1  /* V stored [N, P] per batch item: the usual [seq, head_dim] */
 } tcu_v_layout;
 
-/* Which attention kernel to run (tcu_flash_attn_fwd_f16_algo). AUTO picks MFMA32_FUSED for a row-major V. */
+/* Which attention kernel to run (tcu_flash_attn_fwd_f16_algo). For a row-major V, AUTO picks WAVE64 for long sequences
+ * (head size 128, M % 256 == 0, N >= 1024, at least 128 blocks of 256 queries) and MFMA32_FUSED otherwise. */
 typedef enum {
     TCU_ATTN_AUTO = 0,
     TCU_ATTN_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, like the reference kernel */
     TCU_ATTN_MFMA32 = 2,       /* 32x32x16 MFMA, transposing LDS reads, direct-to-LDS K/V (row-major V only) */
-    TCU_ATTN_MFMA32_FUSED = 3  /* MFMA32 with the softmax of block j+1 computed speculatively under the MFMAs of
+    TCU_ATTN_MFMA32_FUSED = 3, /* MFMA32 with the softmax of block j+1 computed speculatively under the MFMAs of
                                   block j: faster when row maxima settle early, up to ~10 % slower than MFMA32
                                   when they keep growing along the keys; same results up to rounding */
+    TCU_ATTN_WAVE64 = 4        /* 4 wavefronts x 64 queries, one per SIMD: half the LDS traffic per MFMA, all matrix
+                                  instructions placed by hand, softmax of 32 keys interleaved with the MFMAs of the
+                                  neighbouring 32; row-major V, head size 128, M % 256 == 0 */
 } tcu_attn_algo;
 
 /* Which LSTM step kernel to run (tcu_lstm_f16_algo). AUTO picks STREAMING. */

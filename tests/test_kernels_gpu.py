@@ -295,7 +295,7 @@ def test_flash_attention_reference_shapes(tcu, oracle, device, n):
     assert oracle.max_abs_err(host(O), ref) <= ABS_TOL
 
 
-@pytest.mark.parametrize("algo", ["tile_library", "mfma32", "mfma32_fused"])
+@pytest.mark.parametrize("algo", ["tile_library", "mfma32", "mfma32_fused", "wave64"])
 @pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("q_gain,k_growth,tol", [(2.0, 3.0, ABS_TOL), (4.0, 8.0, 5e-2)])
 def test_flash_attention_growing_maxima(tcu, oracle, device, algo, D, q_gain, k_growth, tol):
@@ -307,6 +307,8 @@ def test_flash_attention_growing_maxima(tcu, oracle, device, algo, D, q_gain, k_
     Q pre-multiplied by scale * log2(e) in f16: relative error 2^-11 per product term), hence the looser bound."""
     import torch
 
+    if algo == "wave64" and D != 128:
+        pytest.skip("the wave64 kernel is instantiated for head size 128")
     batch, M, N = 2, 256, 1024
     q = oracle.fill_normal(batch * M * D, 51).reshape(batch, M, D).astype(np.float32) * q_gain
     k = oracle.fill_normal(batch * N * D, 52).reshape(batch, N, D).astype(np.float32)
@@ -336,6 +338,48 @@ def test_flash_attention_row_major_v(tcu, oracle, device, batch, M, N, D, algo):
     torch.cuda.synchronize()
     ref = oracle.attention(q, k, v, 1.0 / math.sqrt(D))
     assert oracle.max_abs_err(host(O), ref) <= ABS_TOL
+
+
+@pytest.mark.parametrize("batch,M,N", [(1, 256, 64), (3, 256, 128), (2, 512, 192), (1, 256, 256), (2, 256, 320),
+                                       (1, 512, 384), (2, 256, 448), (1, 256, 576), (8, 512, 1024), (3, 768, 2112)])
+def test_flash_attention_wave64_sequence_lengths(tcu, oracle, device, batch, M, N):
+    """The kernel with 64 queries per wavefront, at every count of 64-key blocks that takes a different way through
+    its prologue, its ring of five LDS stages and its peeled last block-iterations (1 ... 7, 9, 16, 33 blocks)."""
+    import torch
+
+    print(f"attention wave64 b{batch} {M}x{N}", flush=True)
+    D = 128
+    q = oracle.fill_normal(batch * M * D, 61).reshape(batch, M, D)
+    k = oracle.fill_normal(batch * N * D, 62).reshape(batch, N, D)
+    v = oracle.fill_normal(batch * N * D, 63).reshape(batch, N, D)
+    O = tcu.flash_attention(dev(q, device), dev(k, device), dev(v, device), algo="wave64")
+    torch.cuda.synchronize()
+    ref = oracle.attention(q, k, v, 1.0 / math.sqrt(D))
+    assert np.isfinite(host(O)).all()
+    assert oracle.max_abs_err(host(O), ref) <= ABS_TOL
+
+
+def test_flash_attention_wave64_maximum_jumps_late(tcu, oracle, device):
+    """One key far above everything before it, placed in each half of a 64-key block and in the last block: the
+    check on the sum of a 32-key half fails there, and the reference maxima, the output accumulators, the running
+    sums and the scores already computed for the following half are all re-based. Also a key of +inf-like weight at
+    the very first position (nothing to rescale yet)."""
+    import torch
+
+    batch, M, N, D = 2, 256, 640, 128
+    q = oracle.fill_normal(batch * M * D, 71).reshape(batch, M, D).astype(np.float32)
+    k = oracle.fill_normal(batch * N * D, 72).reshape(batch, N, D).astype(np.float32)
+    v = oracle.fill_normal(batch * N * D, 73).reshape(batch, N, D)
+    qdir = q / np.linalg.norm(q, axis=-1, keepdims=True)
+    for pos, gain in ((0, 30.0), (200, 60.0), (225, 120.0), (300, 200.0), (639, 400.0)):
+        # key `pos` points along a different query each time: for that query its logit exceeds all earlier ones by far
+        k[:, pos] = qdir[:, pos % M] * gain
+    q, k = q.astype(np.float16), k.astype(np.float16)
+    O = tcu.flash_attention(dev(q, device), dev(k, device), dev(v, device), algo="wave64")
+    torch.cuda.synchronize()
+    ref = oracle.attention(q, k, v, 1.0 / math.sqrt(D))
+    assert np.isfinite(host(O)).all()
+    assert oracle.max_abs_err(host(O), ref) <= 2e-2  # logits of several hundred: see test_flash_attention_growing_maxima
 
 
 def test_flash_attention_properties(tcu, oracle, device):
@@ -372,15 +416,17 @@ def test_flash_attention_config4(tcu, oracle, device):
     k = oracle.fill_normal(n, 2238).reshape(B * H, S, D)
     v = oracle.fill_normal(n, 3238).reshape(B * H, S, D)
     dq, dk, dv = (dev(t.reshape(B, H, S, D), device) for t in (q, k, v))
-    O = tcu.flash_attention(dq, dk, dv)
-    torch.cuda.synchronize()
-    assert tuple(O.shape) == (B, H, S, D)
-    Oh = host(O).reshape(B * H, S, D)
-    assert np.isfinite(Oh).all()
     scale = 1.0 / math.sqrt(D)
-    for head, rows in [(0, (0, 128)), (17, (960, 1088)), (63, (1920, 2048))]:
-        ref = oracle.attention(q[head], k[head], v[head], scale, rows=rows)
-        assert oracle.max_abs_err(Oh[head, rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= ABS_TOL
+    samples = [(0, (0, 128)), (17, (960, 1088)), (63, (1920, 2048))]
+    refs = [oracle.attention(q[head], k[head], v[head], scale, rows=rows) for head, rows in samples]
+    for algo in ("auto", "wave64", "mfma32_fused"):  # auto is wave64 at this shape
+        O = tcu.flash_attention(dq, dk, dv, algo=algo)
+        torch.cuda.synchronize()
+        assert tuple(O.shape) == (B, H, S, D)
+        Oh = host(O).reshape(B * H, S, D)
+        assert np.isfinite(Oh).all()
+        for (head, rows), ref in zip(samples, refs):
+            assert oracle.max_abs_err(Oh[head, rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= ABS_TOL, algo
     vconst = dv[:, :, :1, :].expand(B, H, S, D).contiguous()
     Oc = tcu.flash_attention(dq, dk, vconst)
     assert torch.allclose(Oc.float(), vconst.float(), atol=2e-3)

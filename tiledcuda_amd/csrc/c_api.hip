@@ -5,6 +5,7 @@
 
 #include "kernels/b2b_gemm_fwd.hpp"
 #include "kernels/flash_attn_fwd.hpp"
+#include "kernels/flash_attn_w64.hpp"
 #include "kernels/gemm_pipelined.hpp"
 #include "kernels/gemm_w128.hpp"
 #include "kernels/lstm_fwd.hpp"
@@ -278,6 +279,13 @@ int launch_fa_fwd(const __half* Q, const __half* K, const __half* V, __half* O, 
                   O, batch, M, N, scale);
 }
 
+int launch_fa_w64(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
+                  hipStream_t stream) {
+    using Traits = FlashW64Traits<128>;
+    return launch(&flash_attention_fwd_w64<Traits>, dim3((M / Traits::kBM) * batch), dim3(Traits::kThreads),
+                  Traits::kLdsBytes, stream, Q, K, V, O, batch, M, N, scale);
+}
+
 template <int kD, bool kFused>
 int fa_fwd_by_rows(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
                    hipStream_t stream) {
@@ -291,10 +299,20 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     using W41 = tl::RowMajor<4, 1>;
     if (Kd != P) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs the query and value head sizes equal");
     if (M % 64 != 0 || N % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs M % 64 == 0 and N % 64 == 0");
-    if (algo != TCU_ATTN_AUTO && algo != TCU_ATTN_TILE_LIBRARY && algo != TCU_ATTN_MFMA32 && algo != TCU_ATTN_MFMA32_FUSED)
+    if (algo != TCU_ATTN_AUTO && algo != TCU_ATTN_TILE_LIBRARY && algo != TCU_ATTN_MFMA32 &&
+        algo != TCU_ATTN_MFMA32_FUSED && algo != TCU_ATTN_WAVE64)
         return fail(TCU_ERR_INVALID_ARGUMENT, "unknown attention algo");
+    if (algo == TCU_ATTN_WAVE64) {
+        if (v_layout != TCU_V_ROW_MAJOR || Kd != 128 || M % 256 != 0)
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel takes a row-major V, head "
+                                                   "size 128 and M % 256 == 0");
+        return launch_fa_w64(Q, K, V, O, batch, M, N, scale, stream);
+    }
     if (v_layout == TCU_V_ROW_MAJOR && algo != TCU_ATTN_TILE_LIBRARY) {
         if (Kd != 128 && Kd != 64) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
+        // long sequences with enough query blocks to fill the chip: the kernel with 64 queries per wavefront
+        if (algo == TCU_ATTN_AUTO && Kd == 128 && M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 128)
+            return launch_fa_w64(Q, K, V, O, batch, M, N, scale, stream);
         if (algo == TCU_ATTN_MFMA32)
             return Kd == 128 ? fa_fwd_by_rows<128, false>(Q, K, V, O, batch, M, N, scale, stream)
                              : fa_fwd_by_rows<64, false>(Q, K, V, O, batch, M, N, scale, stream);
