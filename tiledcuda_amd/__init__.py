@@ -247,14 +247,14 @@ class TiledFlashAttention:
 
 # ------------------------------------------------------------------------------ LSTM
 def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor | None = None,
-         c0: torch.Tensor | None = None, algo: str = "auto",
-         workspace: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+         c0: torch.Tensor | None = None, algo: str = "auto", workspace: torch.Tensor | None = None,
+         out: tuple[torch.Tensor, torch.Tensor] | None = None) -> tuple[torch.Tensor, torch.Tensor]:
     """Fused LSTM layer. x [T, B, I] f16, W [4H, I+H] f16 (gate rows i,f,g,o), bias [4H] f16,
     h0 [B, H] f16 / c0 [B, H] f32 (None = zeros). Returns (h_all [T, B, H] f16, c_T [B, H] f32).
 
     ``algo="hoisted"`` computes the input half of the gates for all steps in one GEMM first (``tcu_lstm_f16_ws``); it
     needs ``lstm_workspace_bytes(T, B, I, H)`` bytes of device memory, taken from ``workspace`` (any dtype) if given,
-    else allocated here."""
+    else allocated here. ``out`` = (h_all, c_T) tensors to write into instead of allocating them."""
     if x.dim() != 3 or W.dim() != 2:
         raise ValueError("x must be [T, B, I] and W [4H, I+H]")
     T, B, I = x.shape
@@ -265,8 +265,13 @@ def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor 
         raise ValueError(f"h0 must be [{B}, {H}], got {tuple(h0.shape)}")
     if c0 is not None and tuple(c0.shape) != (B, H):
         raise ValueError(f"c0 must be [{B}, {H}], got {tuple(c0.shape)}")
-    h_all = torch.empty(T, B, H, dtype=torch.float16, device=x.device)
-    c_out = torch.empty(B, H, dtype=torch.float32, device=x.device)
+    if out is None:
+        h_all = torch.empty(T, B, H, dtype=torch.float16, device=x.device)
+        c_out = torch.empty(B, H, dtype=torch.float32, device=x.device)
+    else:
+        h_all, c_out = out
+        if tuple(h_all.shape) != (T, B, H) or tuple(c_out.shape) != (B, H):
+            raise ValueError(f"out must be (h_all [{T}, {B}, {H}], c_T [{B}, {H}])")
     if algo == "hoisted":
         need = lstm_workspace_bytes(T, B, I, H)
         if workspace is None:
