@@ -7,10 +7,16 @@
 // The operands are passed to the instruction swapped (B's share as the first operand):
 // the instruction then produces C^T in its native accumulator distribution, which is C in
 // the row-major BaseTile distribution (lane l: row l % 16, columns 4 * (l / 16) .. +3).
+//
+// With MFMA-shaped operand tiles (types/mfma_tile.hpp) every (i, j, k) step is exactly one instruction:
+//   A 16 x 32, B 32 x 16, C 16 x 16 BaseTile  ->  v_mfma_f32_16x16x32_f16
+//   A 32 x 16, B 16 x 32, C 32 x 32           ->  v_mfma_f32_32x32x16_f16
+// (operands swapped as above, so the accumulator holds runs of consecutive columns of a row of C).
 #pragma once
 
 #include "cell/traits/base.hpp"
 #include "types/layout.hpp"
+#include "types/mfma_tile.hpp"
 #include "types/tile_shape.hpp"
 
 namespace tiledcuda::cell::compute {
@@ -88,12 +94,76 @@ struct Gemm {
     }
 };
 
+template <typename T>
+struct IsMfmaTile : std::false_type {};
+template <typename E, const int kR, const int kC, const tl::Layout kT>
+struct IsMfmaTile<MfmaTile<E, kR, kC, kT>> : std::true_type {};
+
+/// gemm over MFMA-shaped operand tiles: one matrix instruction per (i, j, k).
+template <typename RegTileA, typename RegTileB, typename RegTileC>
+struct GemmMfmaTiles {
+    using TileA = typename RegTileA::DType;
+    using TileB = typename RegTileB::DType;
+    using TileC = typename RegTileC::DType;
+    using InType = typename TileA::DType;
+
+    static_assert(traits::HalfType<InType> && std::is_same_v<InType, typename TileB::DType>,
+                  "This GEMM supports only half-precision input elements of one type.");
+    static_assert(std::is_same_v<typename TileC::DType, float>, "The output type must be float.");
+    static_assert(TileA::kType == tl::Layout::kRowMajor && TileB::kType == tl::Layout::kColMajor,
+                  "Operand A must be made of row-major tiles, operand B of column-major tiles.");
+    static constexpr bool k16 = TileA::kTileRows == 16 && TileA::kTileCols == 32;
+    static constexpr bool k32 = TileA::kTileRows == 32 && TileA::kTileCols == 16;
+    static_assert(k16 || k32, "operand A must be a 16 x 32 or a 32 x 16 tile");
+    static_assert(TileB::kTileRows == TileA::kTileCols && TileB::kTileCols == TileA::kTileRows,
+                  "operand B must be the 32 x 16 / 16 x 32 counterpart of operand A");
+    static_assert(traits::TileGeometry<TileC>::kRows == TileA::kTileRows &&
+                      traits::TileGeometry<TileC>::kCols == TileB::kTileCols &&
+                      traits::TileGeometry<TileC>::kRowMajor,
+                  "the accumulator must be the row-major 16 x 16 BaseTile or the 32 x 32 MFMA tile");
+
+    static constexpr int kMs = RegTileA::kRows, kNs = RegTileB::kCols, kKs = RegTileA::kCols;
+    static_assert(RegTileB::kRows == kKs, "Mismatched k-dimension for operand A and B.");
+    static_assert(RegTileC::kRows == kMs && RegTileC::kCols == kNs, "Mismatched accumulator shape.");
+
+    DEVICE void operator()(const RegTileA& a, const RegTileB& b, RegTileC& c) {
+#pragma unroll
+        for (int k = 0; k < kKs; ++k) {
+#pragma unroll
+            for (int i = 0; i < kMs; ++i) {
+#pragma unroll
+                for (int j = 0; j < kNs; ++j) {
+                    f16x8 av, bv;
+                    __builtin_memcpy(&av, a(i, k).data(), sizeof(av));
+                    __builtin_memcpy(&bv, b(k, j).data(), sizeof(bv));
+                    if constexpr (k16) {
+                        f32x4 acc;
+                        __builtin_memcpy(&acc, c(i, j).data(), sizeof(acc));
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bv, av, acc, 0, 0, 0);
+                        __builtin_memcpy(c(i, j).mutable_data(), &acc, sizeof(acc));
+                    } else {
+                        f32x16 acc;
+                        __builtin_memcpy(&acc, c(i, j).data(), sizeof(acc));
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(bv, av, acc, 0, 0, 0);
+                        __builtin_memcpy(c(i, j).mutable_data(), &acc, sizeof(acc));
+                    }
+                }
+            }
+        }
+    }
+};
+
 }  // namespace detail
 
 template <typename RegTileA, typename RegTileB, typename RegTileC>
 DEVICE void gemm(const RegTileA& a, const RegTileB& b, RegTileC& c) {
-    detail::Gemm<RegTileA, RegTileB, RegTileC> gemm;
-    gemm(a, b, c);
+    if constexpr (detail::IsMfmaTile<typename RegTileA::DType>::value) {
+        detail::GemmMfmaTiles<RegTileA, RegTileB, RegTileC> gemm;
+        gemm(a, b, c);
+    } else {
+        detail::Gemm<RegTileA, RegTileB, RegTileC> gemm;
+        gemm(a, b, c);
+    }
 }
 
 }  // namespace tiledcuda::cell::compute

@@ -45,6 +45,44 @@ DEVICE void move_base_tile(DType* tile_ptr, BaseTile& reg) {
     }
 }
 
+/// The same for any tile described by TileGeometry (16 x 16 BaseTile or MFMA-shaped tile): every run of the lane
+/// moves as one vector access when it lies along the contiguous dimension of the memory tile.
+template <typename DType, typename BaseTile, const int kRowStride, const int kColStride, const bool kLoad>
+DEVICE void move_tile(DType* tile_ptr, BaseTile& reg) {
+    using G = TileGeometry<std::remove_const_t<BaseTile>>;
+    using E = std::remove_const_t<DType>;
+    const int lane = lane_id();
+    const int major = lane % G::kLaneMajor;
+    const int minor0 = (lane / G::kLaneMajor) * G::kRunLen;
+    constexpr int kStep = G::kRowMajor ? kColStride : kRowStride;
+    constexpr int kLinePitch = G::kRowMajor ? kRowStride : kColStride;
+    constexpr int kPiece = G::kRunLen * sizeof(E) > 16 ? int(16 / sizeof(E)) : G::kRunLen;
+    auto* r = const_cast<E*>(reg.data());
+#pragma unroll
+    for (int run = 0; run < G::kRuns; ++run) {
+        const int minor = minor0 + run * G::kRunStride;
+        DType* p = tile_ptr + (G::kRowMajor ? major * kRowStride + minor * kColStride
+                                            : minor * kRowStride + major * kColStride);
+        if constexpr (kStep == 1 && kLinePitch % kPiece == 0) {
+#pragma unroll
+            for (int e = 0; e < G::kRunLen; e += kPiece) {
+                if constexpr (kLoad)
+                    vec_load<kPiece>(p + e, r + run * G::kRunLen + e);
+                else
+                    vec_store<kPiece>(r + run * G::kRunLen + e, const_cast<E*>(p) + e);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < G::kRunLen; ++e) {
+                if constexpr (kLoad)
+                    r[run * G::kRunLen + e] = p[e * kStep];
+                else
+                    const_cast<E*>(p)[e * kStep] = r[run * G::kRunLen + e];
+            }
+        }
+    }
+}
+
 }  // namespace detail
 
 /// Load this wavefront's share of a global tile into a register tile.
@@ -54,7 +92,7 @@ struct GlobalToRegLoader : public Base {
     using Reg = Reg_;
     using BaseTile = typename Reg::DType;
     using DType = typename BaseTile::DType;
-    using BaseShape = BaseTileShape<DType>;
+    using BaseShape = TileExtent<BaseTile>;
 
     using WarpLayout = WarpLayout_;
     static constexpr WarpReuse kMode = kMode_;
@@ -73,7 +111,7 @@ struct GlobalToRegLoader : public Base {
             for (int j = 0; j < kColExec; ++j) {
                 const DType* tile_ptr = warp_ptr + i * BaseShape::kRows * Global::kRowStride +
                                         j * BaseShape::kCols * Global::kColStride;
-                detail::move_base_tile<const DType, BaseTile, Global::kRowStride, Global::kColStride, true>(
+                detail::move_tile<const DType, BaseTile, Global::kRowStride, Global::kColStride, true>(
                     tile_ptr, dst(i, j));
             }
         }
@@ -88,7 +126,7 @@ struct RegToGlobalStorer : public Base {
     using Reg = Reg_;
     using BaseTile = typename Reg::DType;
     using DType = typename Global::DType;
-    using BaseShape = BaseTileShape<DType>;
+    using BaseShape = TileExtent<BaseTile>;
 
     using WarpLayout = WarpLayout_;
 
@@ -108,7 +146,7 @@ struct RegToGlobalStorer : public Base {
             for (int j = 0; j < kColExec; ++j) {
                 DType* tile_ptr = warp_ptr + i * BaseShape::kRows * Global::kRowStride +
                                   j * BaseShape::kCols * Global::kColStride;
-                detail::move_base_tile<DType, const BaseTile, Global::kRowStride, Global::kColStride, false>(
+                detail::move_tile<DType, const BaseTile, Global::kRowStride, Global::kColStride, false>(
                     tile_ptr, src(i, j));
             }
         }

@@ -25,4 +25,16 @@ DEVICE void __copy_async() {
     __builtin_amdgcn_s_waitcnt(0);
 }
 
+/// Wait until at most N of this wavefront's copies are outstanding, then a workgroup barrier that orders LDS accesses
+/// only: the hand-over of a stage of a SharedRing filled by GlobalToSharedDirectLoader. __syncthreads() would also
+/// wait for every copy still in flight (its fence covers the LDS writes of direct-to-LDS loads), which empties the
+/// pipeline at every hand-over.
+template <int N = 0>
+DEVICE void wait_group_and_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070 | (N & 0xF) | ((N >> 4) << 14));  // vmcnt(N) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 }  // namespace tiledcuda::cell

@@ -5,10 +5,17 @@
 //     kernel of examples/cpp/01_gemm/02_gemm_all_mem/gemm.hpp:15-155. A barrier is added
 //     at the end of each k-step: the reference overwrites the shared tiles of the next
 //     step while other warps may still be reading them.
+//   * PipelinedGemmTileTraits / gemm_tile_pipelined: the same all-memory kernel on the CDNA4 data path, still
+//     composed from tile-library functors only: direct-to-LDS loads into a two-stage SharedRing
+//     (GlobalToSharedDirectLoader), one ds_read_b128 per 16 x 32 / 32 x 16 operand tile (SharedToRegLoader on
+//     MfmaTile operands), one v_mfma_f32_16x16x32_f16 per gemm() step, register double-buffering of the operand
+//     tiles, XCD-aware tile order. It performs the arithmetic of kernels/gemm_pipelined.hpp in the same order
+//     (results identical bit for bit).
 // A is row-major [M, K], B is column-major [K, N] (stored [N, K]), C is row-major [M, N].
 #pragma once
 
 #include "cell/mod.hpp"
+#include "kernels/gemm_pipelined.hpp"  // detail::xcd_tile_coords
 #include "types/mod.hpp"
 
 namespace tiledcuda::kernels {
@@ -221,6 +228,140 @@ __global__ void __launch_bounds__(512) gemm(const InType* dA, const InType* dB, 
     r2s_c(acc, sC);
     __syncthreads();
     s2g_c(sC, gC);
+}
+
+template <typename InType, typename OutType, typename WholeShape, const int kTM_, const int kTN_, typename WarpLayout>
+struct PipelinedGemmTileTraits {
+    static constexpr int kThreads = tl::get_numel<WarpLayout> * kWaveSize;
+    static constexpr int kWarpPerRow = tl::num_rows<WarpLayout>;
+    static constexpr int kWarpPerCol = tl::num_cols<WarpLayout>;
+
+    static constexpr int kM = dim_size<0, WholeShape>;
+    static constexpr int kN = dim_size<1, WholeShape>;
+    static constexpr int kK = dim_size<2, WholeShape>;
+    static constexpr int kTM = kTM_, kTN = kTN_;
+    static constexpr int kTK = 64;  // one LDS stage: lines of 128 bytes
+    static constexpr int kRK = 32;  // one MFMA k-step
+    static constexpr int kStages = 2;
+    static_assert(kM % kTM == 0 && kN % kTN == 0 && kK % kTK == 0);
+
+    using Shape = traits::MfmaTileShape<InType, traits::MfmaShape::k16x16x32>;
+
+    // operand A
+    using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK, kK>>;
+    using GIteratorA = GTileIterator<GlobalA, TileShape<kTM, kTK>>;
+    using SharedA = SharedTile<InType, tl::RowMajor<kTM, kTK>, true>;
+    using RingA = SharedRing<SharedA, kStages>;
+    using SIteratorA = STileIterator<SharedA, TileShape<kTM, kRK>>;
+    using RegA = RegTile<typename Shape::TileA, tl::RowMajor<kTM / kWarpPerRow / Shape::kM, 1>>;
+    using G2SLoaderA = GlobalToSharedDirectLoader<SharedA, WarpLayout>;
+    using S2RLoaderA = SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
+
+    // operand B
+    using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kTN, kK>>;
+    using GIteratorB = GTileIterator<GlobalB, TileShape<kTK, kTN>>;
+    using SharedB = SharedTile<InType, tl::ColMajor<kTK, kTN>, true>;
+    using RingB = SharedRing<SharedB, kStages>;
+    using SIteratorB = STileIterator<SharedB, TileShape<kRK, kTN>>;
+    using RegB = RegTile<typename Shape::TileB, tl::ColMajor<1, kTN / kWarpPerCol / Shape::kN>>;
+    using G2SLoaderB = GlobalToSharedDirectLoader<SharedB, WarpLayout>;
+    using S2RLoaderB = SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
+
+    // output C
+    static constexpr int kCMs = kTM / kWarpPerRow / 16, kCNs = kTN / kWarpPerCol / 16;
+    using RegAcc = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kCMs, kCNs>>;
+    using RegC = RegTile<BaseTileRowMajor<OutType>, tl::RowMajor<kCMs, kCNs>>;
+    using SharedC = SharedTile<OutType, tl::RowMajor<kTM, kTN>, true>;
+    using GlobalC = GlobalTile<OutType, tl::RowMajor<kTM, kTN, kN>>;
+    using R2SStorerC = RegToSharedStorer<RegC, WarpLayout>;
+    using S2GStorerC = SharedToGlobalStorer<SharedC, WarpLayout>;
+
+    static constexpr int kShmInput = RingA::kBytes + RingB::kBytes;
+    // an f32 result goes from registers straight to global memory; only f16 is staged through LDS
+    static constexpr int kShmOutput = sizeof(OutType) == 2 ? kTM * kTN * int(sizeof(OutType)) : 0;
+    static constexpr int kShmBytes = kShmInput > kShmOutput ? kShmInput : kShmOutput;
+    static_assert(kShmBytes <= kMaxLdsBytes);
+};
+
+/// grid = (kM / kTM) * (kN / kTN) workgroups (1-D), block = Traits::kThreads, dynamic LDS = Traits::kShmBytes.
+template <typename InType, typename OutType, typename Traits>
+__global__ void __launch_bounds__(Traits::kThreads) gemm_tile_pipelined(const InType* dA, const InType* dB, OutType* dC) {
+    constexpr int kM = Traits::kM, kN = Traits::kN, kK = Traits::kK, kTM = Traits::kTM, kTN = Traits::kTN;
+    int tile_m, tile_n;
+    detail::xcd_tile_coords(blockIdx.x, kM / kTM, kN / kTN, tile_m, tile_n);
+
+    extern __shared__ __align__(1024) unsigned char buf[];
+    auto* sA_ptr = reinterpret_cast<InType*>(buf);
+    auto* sB_ptr = reinterpret_cast<InType*>(buf + Traits::RingA::kBytes);
+
+    typename Traits::GIteratorA gAs(dA + size_t(tile_m) * kTM * kK);
+    typename Traits::GIteratorB gBs(dB + size_t(tile_n) * kTN * kK);
+    typename Traits::RingA ringA(sA_ptr);
+    typename Traits::RingB ringB(sB_ptr);
+
+    typename Traits::G2SLoaderA g2s_a;
+    typename Traits::G2SLoaderB g2s_b;
+    typename Traits::S2RLoaderA s2r_a;
+    typename Traits::S2RLoaderB s2r_b;
+
+    typename Traits::RegA rA[2];  // operand tiles of the k-step being multiplied and of the next one
+    typename Traits::RegB rB[2];
+    typename Traits::RegAcc acc;
+
+    auto load_stage = [&](int k1, int stage) {
+        auto sA = ringA[stage];
+        auto sB = ringB[stage];
+        g2s_a(gAs(k1), sA);
+        g2s_b(gBs(k1), sB);
+    };
+    auto load_frags = [&](int stage, int k2, int which) {
+        typename Traits::SIteratorA sAs(ringA.stage_data(stage));
+        typename Traits::SIteratorB sBs(ringB.stage_data(stage));
+        s2r_a(sAs(k2), rA[which]);
+        s2r_b(sBs(k2), rB[which]);
+    };
+
+    constexpr int kTiles = Traits::GIteratorA::sc1;
+    load_stage(0, 0);
+    wait_group_and_barrier<0>();
+    load_frags(0, 0, 0);
+
+    int stage = 0;
+    for (int k1 = 0; k1 < kTiles; ++k1) {
+        const int next = Traits::RingA::next(stage);
+        // tile k1 + 1 goes to the other stage, which everyone left at the hand-over of the previous iteration
+        if (k1 + 1 < kTiles) load_stage(k1 + 1, next);
+        // the copies are issued here, ahead of this iteration's matrix work (the compiler is otherwise free to sink
+        // them below the MFMAs, right in front of the wait that needs them)
+        commit_copy_group();
+        load_frags(stage, 1, 1);
+        compute::gemm(rA[0], rB[0], acc);
+        commit_copy_group();
+        if (k1 + 1 < kTiles) {
+            // this wavefront's copies have landed and its reads of `stage` have returned; then everyone's
+            wait_group_and_barrier<0>();
+            load_frags(next, 0, 0);
+        }
+        compute::gemm(rA[1], rB[1], acc);
+        stage = next;
+    }
+
+    typename Traits::GlobalC gC(dC + size_t(tile_m) * kTM * kN + size_t(tile_n) * kTN);
+    if constexpr (std::is_same_v<OutType, float>) {
+        RegToGlobalStorer<typename Traits::GlobalC, typename Traits::RegAcc, typename Traits::R2SStorerC::WarpLayout> r2g;
+        r2g(acc, gC);
+    } else {
+        typename Traits::RegC out;
+        compute::RegTileConvert<typename Traits::RegAcc, typename Traits::RegC> convert;
+        convert(acc, out);
+        __syncthreads();  // everyone is done with the operand stages: the space is reused for C
+        typename Traits::SharedC sC(reinterpret_cast<OutType*>(buf));
+        typename Traits::R2SStorerC r2s_c;
+        typename Traits::S2GStorerC s2g_c;
+        r2s_c(out, sC);
+        __syncthreads();
+        s2g_c(sC, gC);
+    }
 }
 
 }  // namespace tiledcuda::kernels

@@ -34,8 +34,11 @@ typedef enum {
     TCU_GEMM_GLOBAL_REG = 1, /* global -> register -> MFMA (README kernel of the reference) */
     TCU_GEMM_ALL_MEM = 2,    /* global -> LDS -> register -> MFMA, single stage */
     TCU_GEMM_PIPELINED = 3,  /* direct-to-LDS, double-buffered, 16x16x32 MFMA, 2 wavefronts per SIMD */
-    TCU_GEMM_WAVE128 = 4     /* same pipeline, 256 x 256 tile on 4 wavefronts (one per SIMD, 128 x 128 each),
+    TCU_GEMM_WAVE128 = 4,    /* same pipeline, 256 x 256 tile on 4 wavefronts (one per SIMD, 128 x 128 each),
                                 accumulators in AGPRs; results identical to PIPELINED bit for bit */
+    TCU_GEMM_TILE_PIPELINED = 5 /* the PIPELINED kernel composed from tile-library functors only (direct-to-LDS loader,
+                                two-stage shared ring, ds_read_b128 operand tiles, gemm()); compile-time shapes:
+                                4096^3, 1024^3, 512x768x192, 256x256x64; results identical to PIPELINED bit for bit */
 } tcu_gemm_algo;
 
 /* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks RESIDENT where it is instantiated. */

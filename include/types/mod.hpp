@@ -3,6 +3,7 @@
 #include "types/global.hpp"
 #include "types/global_tile_iterator.hpp"
 #include "types/layout.hpp"
+#include "types/mfma_tile.hpp"
 #include "types/register.hpp"
 #include "types/shared.hpp"
 #include "types/shared_tile_iterator.hpp"

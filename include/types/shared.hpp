@@ -82,4 +82,26 @@ class SharedTile {
     int elem0_;
 };
 
+/// kStages copies of a shared tile laid out back to back: the LDS side of a multi-stage global -> LDS pipeline
+/// (the reference's kernels have one stage and wait for every load, examples/cpp/01_gemm/02_gemm_all_mem/gemm.hpp:139-143).
+/// ring[s] is a whole-tile view of stage s; stages advance modulo kStages.
+template <typename Shared_, const int kStages_>
+class SharedRing {
+  public:
+    using Shared = Shared_;
+    using DType = typename Shared::DType;
+    static constexpr int kStages = kStages_;
+    static constexpr int kStageNumel = Shared::kLines * Shared::kPitch;
+    static constexpr int kBytes = kStages * kStageNumel * int(sizeof(DType));
+
+    HOST_DEVICE explicit SharedRing(DType* base) : base_(base) {}
+
+    HOST_DEVICE Shared operator[](int stage) const { return Shared(base_ + stage * kStageNumel); }
+    HOST_DEVICE DType* stage_data(int stage) const { return base_ + stage * kStageNumel; }
+    HOST_DEVICE static constexpr int next(int stage) { return stage + 1 == kStages ? 0 : stage + 1; }
+
+  private:
+    DType* base_;
+};
+
 }  // namespace tiledcuda::cell

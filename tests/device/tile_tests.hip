@@ -10,6 +10,10 @@
 //   tile gemm               tests/cpp/cell/test_gemm.cu:306-351
 //   reduce / broadcast      tests/cpp/cell/test_reduce.cu, test_broadcast.cu (which only print)
 //   softmax                 tests/cpp/cell/test_softmax.cu:117-163
+// The CDNA4 data path of the library has the same kinds of cases: direct-to-LDS loads into a ring stage must
+// reproduce the source, MFMA-shaped operand tiles read with ds_read_b128 and with the transposing read must
+// reproduce the source (swizzled and plain), and gemm() on those tiles must match the oracle for both instruction
+// shapes, including a B operand stored row-major and transposed on the way to registers.
 // Every kernel is launched with one workgroup; the host side checks results against the
 // CPU oracle or against the identity.
 #include "cell/mod.hpp"
@@ -204,6 +208,178 @@ __global__ void __launch_bounds__(512) k_tile_gemm(const __half* dA, const __hal
     SIterB sBs(sB_ptr);
     SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont> s2r_a;
     SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont> s2r_b;
+    RegA rA;
+    RegB rB;
+    RegC acc;
+    for (int k = 0; k < SIterA::sc1; ++k) {
+        s2r_a(sAs(k), rA);
+        s2r_b(sBs(k), rB);
+        compute::gemm(rA, rB, acc);
+    }
+    GlobalC gC(dC);
+    RegToGlobalStorer<GlobalC, RegC, WarpLayout> r2g;
+    r2g(acc, gC);
+}
+
+// ------------------------------------------------------------------ CDNA4 data path
+// global -> (direct-to-LDS, stage kStage of a ring of 3) -> global
+template <bool kRowMajor, int kRows, int kCols, typename WarpLayout, bool kSwizzled>
+__global__ void __launch_bounds__(512) k_direct_ring_roundtrip(const __half* src, __half* dst) {
+    extern __shared__ __align__(1024) unsigned char buf[];
+    using Layout = LayoutOf<kRowMajor, kRows, kCols>;
+    using Global = GlobalTile<__half, Layout>;
+    using Shared = SharedTile<__half, Layout, kSwizzled>;
+    using Ring = SharedRing<Shared, 3>;
+    Ring ring(reinterpret_cast<__half*>(buf));
+    Global g_src(src);
+    Global g_dst(dst);
+    GlobalToSharedDirectLoader<Shared, WarpLayout> loader;
+    SharedToGlobalStorer<Shared, WarpLayout> storer;
+    auto stage = ring[Ring::next(0)];
+    loader(g_src, stage);
+    wait_group_and_barrier<0>();
+    storer(stage, g_dst);
+}
+
+// shared -> MFMA-shaped operand tiles -> global. kTileMajor x kTileMinor: 16 x 32 or 32 x 16 (major = rows of a
+// row-major operand, columns of a column-major one).
+template <bool kRowMajor, int kRows, int kCols, int kChunk, typename WarpLayout, bool kSwizzled, int kTileMajor>
+__global__ void __launch_bounds__(512) k_s2r_mfma_tiles(const __half* src, __half* dst) {
+    extern __shared__ __align__(1024) unsigned char buf[];
+    auto* smem = reinterpret_cast<__half*>(buf);
+    constexpr int kTileMinor = 512 / kTileMajor;
+    using Layout = LayoutOf<kRowMajor, kRows, kCols>;
+    using Global = GlobalTile<__half, Layout>;
+    using Shared = SharedTile<__half, Layout, kSwizzled>;
+    Global g_src(src);
+    Shared s(smem);
+    GlobalToSharedLoader<Shared, WarpLayout> g2s;
+    g2s(g_src, s);
+    __copy_async();
+    __syncthreads();
+    if constexpr (kRowMajor) {
+        using SIter = STileIterator<Shared, TileShape<kRows, kChunk>>;
+        constexpr int kWR = tl::num_rows<WarpLayout>;
+        using Tile = MfmaTile<__half, kTileMajor, kTileMinor, tl::Layout::kRowMajor>;
+        using Reg = RegTile<Tile, tl::RowMajor<kRows / kWR / kTileMajor, kChunk / kTileMinor>>;
+        SharedToRegLoader<Reg, WarpLayout, WarpReuse::kRowReuseCont> s2r;
+        using Base = warp::CopyBase<WarpLayout, WarpReuse::kRowReuseCont>;
+        SIter iter(smem);
+        for (int k = 0; k < SIter::sc1; ++k) {
+            Reg r;
+            s2r(iter(k), r);
+            if (Base::warp_col_id() == 0) {
+                __half* block = dst + Base::warp_row_id() * (kRows / kWR) * kCols + k * kChunk;
+#pragma unroll
+                for (int i = 0; i < Reg::kRows; ++i)
+#pragma unroll
+                    for (int j = 0; j < Reg::kCols; ++j)
+                        copy::detail::move_tile<__half, const Tile, kCols, 1, false>(
+                            block + i * kTileMajor * kCols + j * kTileMinor, r(i, j));
+            }
+        }
+    } else {
+        using SIter = STileIterator<Shared, TileShape<kChunk, kCols>>;
+        constexpr int kWC = tl::num_cols<WarpLayout>;
+        using Tile = MfmaTile<__half, kTileMinor, kTileMajor, tl::Layout::kColMajor>;
+        using Reg = RegTile<Tile, tl::ColMajor<kChunk / kTileMinor, kCols / kWC / kTileMajor>>;
+        SharedToRegLoader<Reg, WarpLayout, WarpReuse::kColReuseCont> s2r;
+        using Base = warp::CopyBase<WarpLayout, WarpReuse::kColReuseCont>;
+        SIter iter(smem);
+        for (int k = 0; k < SIter::sc0; ++k) {
+            Reg r;
+            s2r(iter(k), r);
+            if (Base::warp_row_id() == 0) {
+                __half* block = dst + k * kChunk + Base::warp_col_id() * (kCols / kWC) * kRows;
+#pragma unroll
+                for (int i = 0; i < Reg::kRows; ++i)
+#pragma unroll
+                    for (int j = 0; j < Reg::kCols; ++j)
+                        copy::detail::move_tile<__half, const Tile, 1, kRows, false>(
+                            block + i * kTileMinor + j * kTileMajor * kRows, r(i, j));
+            }
+        }
+    }
+}
+
+// row-major shared [kRows (contraction index), kCols] -> column-major operand tiles through the transposing read ->
+// global (row-major again: every element must come back to its place)
+template <int kRows, int kCols, int kChunk, typename WarpLayout, bool kSwizzled, int kTileCols>
+__global__ void __launch_bounds__(512) k_s2r_transposed(const __half* src, __half* dst) {
+    extern __shared__ __align__(1024) unsigned char buf[];
+    auto* smem = reinterpret_cast<__half*>(buf);
+    constexpr int kTileRows = 512 / kTileCols;  // 32 x 16 or 16 x 32
+    using Global = GlobalTile<__half, tl::RowMajor<kRows, kCols>>;
+    using Shared = SharedTile<__half, tl::RowMajor<kRows, kCols>, kSwizzled>;
+    using SIter = STileIterator<Shared, TileShape<kChunk, kCols>>;
+    constexpr int kWC = tl::num_cols<WarpLayout>;
+    using Tile = MfmaTile<__half, kTileRows, kTileCols, tl::Layout::kColMajor>;
+    using Reg = RegTile<Tile, tl::ColMajor<kChunk / kTileRows, kCols / kWC / kTileCols>>;
+    Global g_src(src);
+    Shared s(smem);
+    GlobalToSharedLoader<Shared, WarpLayout> g2s;
+    g2s(g_src, s);
+    __copy_async();
+    __syncthreads();
+    SharedToRegLoaderTr<Reg, WarpLayout, WarpReuse::kColReuseCont> s2r;
+    using Base = warp::CopyBase<WarpLayout, WarpReuse::kColReuseCont>;
+    SIter iter(smem);
+    for (int k = 0; k < SIter::sc0; ++k) {
+        Reg r;
+        s2r(iter(k), r);
+        if (Base::warp_row_id() == 0) {
+            __half* block = dst + k * kChunk * kCols + Base::warp_col_id() * (kCols / kWC);
+#pragma unroll
+            for (int i = 0; i < Reg::kRows; ++i)
+#pragma unroll
+                for (int j = 0; j < Reg::kCols; ++j)
+                    copy::detail::move_tile<__half, const Tile, kCols, 1, false>(
+                        block + i * kTileRows * kCols + j * kTileCols, r(i, j));
+        }
+    }
+}
+
+// C = A · B through direct-to-LDS loads and MFMA-shaped tiles, one workgroup. kShape32: v_mfma_f32_32x32x16_f16,
+// else v_mfma_f32_16x16x32_f16. kBRowMajor: B is stored row-major [kK, kN] and transposed by the loader.
+template <int kM, int kN, int kK, typename WarpLayout, bool kShape32, bool kBRowMajor>
+__global__ void __launch_bounds__(512) k_tile_gemm_mfma(const __half* dA, const __half* dB, float* dC) {
+    extern __shared__ __align__(1024) unsigned char buf[];
+    auto* sA_ptr = reinterpret_cast<__half*>(buf);
+    auto* sB_ptr = sA_ptr + kM * kK;
+    constexpr int kWR = tl::num_rows<WarpLayout>, kWC = tl::num_cols<WarpLayout>;
+    using Shape = traits::MfmaTileShape<__half, kShape32 ? traits::MfmaShape::k32x32x16 : traits::MfmaShape::k16x16x32>;
+    constexpr int kChunkK = 64 / Shape::kK * Shape::kK;  // 64
+
+    using GlobalA = GlobalTile<__half, tl::RowMajor<kM, kK>>;
+    using SharedA = SharedTile<__half, tl::RowMajor<kM, kK>, true>;
+    using SIterA = STileIterator<SharedA, TileShape<kM, kChunkK>>;
+    using RegA = RegTile<typename Shape::TileA, tl::RowMajor<kM / kWR / Shape::kM, kChunkK / Shape::kK>>;
+
+    using LayoutB = std::conditional_t<kBRowMajor, tl::RowMajor<kK, kN>, tl::ColMajor<kK, kN>>;
+    using GlobalB = GlobalTile<__half, LayoutB>;
+    using SharedB = SharedTile<__half, LayoutB, true>;
+    using SIterB = STileIterator<SharedB, TileShape<kChunkK, kN>>;
+    using RegB = RegTile<typename Shape::TileB, tl::ColMajor<kChunkK / Shape::kK, kN / kWC / Shape::kN>>;
+
+    using GlobalC = GlobalTile<float, tl::RowMajor<kM, kN>>;
+    using RegC = RegTile<typename Shape::TileC, tl::RowMajor<kM / kWR / Shape::kM, kN / kWC / Shape::kN>>;
+
+    GlobalA gA(dA);
+    GlobalB gB(dB);
+    SharedA sA(sA_ptr);
+    SharedB sB(sB_ptr);
+    GlobalToSharedDirectLoader<SharedA, WarpLayout> g2s_a;
+    GlobalToSharedDirectLoader<SharedB, WarpLayout> g2s_b;
+    g2s_a(gA, sA);
+    g2s_b(gB, sB);
+    wait_group_and_barrier<0>();
+
+    SIterA sAs(sA_ptr);
+    SIterB sBs(sB_ptr);
+    SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont> s2r_a;
+    std::conditional_t<kBRowMajor, SharedToRegLoaderTr<RegB, WarpLayout, WarpReuse::kColReuseCont>,
+                       SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>>
+        s2r_b;
     RegA rA;
     RegB rB;
     RegC acc;
@@ -476,6 +652,60 @@ void reg_gemm() {
                           &launch_gemm<k_tile_gemm<kM, kN, kK, W, kChunkK, kSwz>>});
 }
 
+template <bool kRowMajor, int kRows, int kCols, int kWR, int kWC, bool kSwz>
+void reg_direct() {
+    using W = tl::RowMajor<kWR, kWC>;
+    registry().push_back({"g2s_roundtrip",
+                          std::string("f16_direct_ring") + (kRowMajor ? "_row_" : "_col_") + std::to_string(kRows) + "x" +
+                              std::to_string(kCols) + "_w" + std::to_string(kWR) + "x" + std::to_string(kWC) +
+                              (kSwz ? "_swz" : "_plain"),
+                          {kRows, kCols, 0, 2, kRowMajor, 0, 0, 0},
+                          kWR * kWC * 64,
+                          int(3 * kRows * kCols * sizeof(__half)),
+                          &launch2<k_direct_ring_roundtrip<kRowMajor, kRows, kCols, W, kSwz>, __half>});
+}
+
+template <bool kRowMajor, int kRows, int kCols, int kChunk, int kWR, int kWC, bool kSwz, int kTileMajor>
+void reg_s2r_mfma() {
+    using W = tl::RowMajor<kWR, kWC>;
+    registry().push_back({"s2r_identity",
+                          std::string("f16_mfma") + std::to_string(kTileMajor) + "x" + std::to_string(512 / kTileMajor) +
+                              (kRowMajor ? "_row_" : "_col_") + std::to_string(kRows) + "x" + std::to_string(kCols) +
+                              "_c" + std::to_string(kChunk) + "_w" + std::to_string(kWR) + "x" + std::to_string(kWC) +
+                              (kSwz ? "_swz" : "_plain"),
+                          {kRows, kCols, kChunk, 2, kRowMajor, 0, 0, 0},
+                          kWR * kWC * 64,
+                          int(kRows * kCols * sizeof(__half)),
+                          &launch2<k_s2r_mfma_tiles<kRowMajor, kRows, kCols, kChunk, W, kSwz, kTileMajor>, __half>});
+}
+
+template <int kRows, int kCols, int kChunk, int kWR, int kWC, bool kSwz, int kTileCols>
+void reg_s2r_tr() {
+    using W = tl::RowMajor<kWR, kWC>;
+    registry().push_back({"s2r_identity",
+                          std::string("f16_transposed") + std::to_string(512 / kTileCols) + "x" + std::to_string(kTileCols) +
+                              "_row_" + std::to_string(kRows) + "x" + std::to_string(kCols) + "_c" +
+                              std::to_string(kChunk) + "_w" + std::to_string(kWR) + "x" + std::to_string(kWC) +
+                              (kSwz ? "_swz" : "_plain"),
+                          {kRows, kCols, kChunk, 2, 1, 0, 0, 0},
+                          kWR * kWC * 64,
+                          int(kRows * kCols * sizeof(__half)),
+                          &launch2<k_s2r_transposed<kRows, kCols, kChunk, W, kSwz, kTileCols>, __half>});
+}
+
+template <int kM, int kN, int kK, int kWR, int kWC, bool kShape32, bool kBRowMajor>
+void reg_gemm_mfma() {
+    using W = tl::RowMajor<kWR, kWC>;
+    registry().push_back({"tile_gemm",
+                          std::string(kShape32 ? "mfma32x32x16_" : "mfma16x16x32_") + std::to_string(kM) + "x" +
+                              std::to_string(kN) + "x" + std::to_string(kK) + "_w" + std::to_string(kWR) + "x" +
+                              std::to_string(kWC) + (kBRowMajor ? "_b_row_major" : ""),
+                          {kM, kN, kK, 64, kBRowMajor, 0, 0, 0},
+                          kWR * kWC * 64,
+                          int((kM * kK + kK * kN) * sizeof(__half)),
+                          &launch_gemm<k_tile_gemm_mfma<kM, kN, kK, W, kShape32, kBRowMajor>>});
+}
+
 template <typename E, int kRows, int kCols, int kW, int kOp>
 void reg_row_op() {
     static const char* names[] = {"sum", "max", "bcast_sum", "sub_max", "softmax", "add_sum", "mul_max", "div_sum"};
@@ -609,6 +839,45 @@ void build_registry() {
     reg_gemm<64, 128, 128, 2, 4, 128>();
     reg_gemm<64, 64, 64, 2, 2, 32, false>();
     reg_gemm<32, 32, 48, 1, 1, 48>();
+
+    // the CDNA4 data path: direct-to-LDS loads into a ring stage (lines of 64, 128, 256 and 512 bytes)
+    reg_direct<true, 64, 64, 2, 2, true>();
+    reg_direct<true, 64, 64, 2, 2, false>();
+    reg_direct<true, 256, 64, 4, 2, true>();
+    reg_direct<true, 128, 32, 2, 1, true>();
+    reg_direct<true, 32, 128, 1, 2, true>();
+    reg_direct<true, 16, 256, 1, 1, true>();
+    reg_direct<false, 64, 128, 2, 2, true>();
+    reg_direct<false, 64, 256, 4, 2, true>();
+    reg_direct<false, 128, 64, 1, 4, false>();
+    // MFMA-shaped operand tiles out of LDS (ds_read_b128): both instruction shapes, both operands
+    reg_s2r_mfma<true, 64, 64, 64, 2, 2, true, 16>();
+    reg_s2r_mfma<true, 64, 64, 32, 2, 2, false, 16>();
+    reg_s2r_mfma<true, 128, 128, 64, 4, 1, true, 16>();
+    reg_s2r_mfma<true, 256, 64, 32, 4, 2, true, 16>();
+    reg_s2r_mfma<true, 64, 64, 16, 2, 2, true, 32>();
+    reg_s2r_mfma<true, 128, 128, 64, 2, 2, true, 32>();
+    reg_s2r_mfma<false, 64, 64, 64, 2, 2, true, 16>();
+    reg_s2r_mfma<false, 64, 256, 32, 4, 2, true, 16>();
+    reg_s2r_mfma<false, 128, 64, 32, 2, 2, false, 16>();
+    reg_s2r_mfma<false, 64, 128, 16, 2, 2, true, 32>();
+    // column-major operand tiles out of a row-major shared tile (ds_read_b64_tr_b16)
+    reg_s2r_tr<64, 64, 32, 2, 2, true, 16>();
+    reg_s2r_tr<64, 64, 32, 2, 2, false, 16>();
+    reg_s2r_tr<128, 128, 64, 2, 4, true, 16>();
+    reg_s2r_tr<64, 128, 16, 2, 2, true, 32>();
+    reg_s2r_tr<128, 64, 32, 1, 1, true, 32>();
+    // gemm() on MFMA-shaped tiles, operands brought in by the direct loader
+    reg_gemm_mfma<64, 64, 64, 2, 2, false, false>();
+    reg_gemm_mfma<128, 128, 128, 2, 2, false, false>();
+    reg_gemm_mfma<64, 128, 128, 2, 4, false, false>();
+    reg_gemm_mfma<128, 64, 64, 4, 1, false, false>();
+    reg_gemm_mfma<64, 64, 64, 2, 2, true, false>();
+    reg_gemm_mfma<128, 128, 128, 2, 2, true, false>();
+    reg_gemm_mfma<128, 64, 128, 4, 1, true, false>();
+    reg_gemm_mfma<64, 64, 64, 2, 2, false, true>();
+    reg_gemm_mfma<128, 128, 64, 2, 2, false, true>();
+    reg_gemm_mfma<64, 64, 128, 2, 2, true, true>();
 
     // reductions, broadcasts, softmax (test_reduce.cu / test_broadcast.cu / test_softmax.cu shapes)
     reg_row_op<float, 16, 16, 1, 0>();

@@ -103,6 +103,27 @@ def test_gemm_wave128_rejects_other_shapes(tcu, device):
         tcu.gemm(A, A, algo="wave128")
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 768, 192), (1024, 1024, 1024), (4096, 4096, 4096)])
+@pytest.mark.parametrize("out_dtype", ["f16", "f32"])
+def test_gemm_tile_api_pipelined_is_the_pipelined_kernel(tcu, oracle, device, M, N, K, out_dtype):
+    """The multi-stage kernel written with tile-library functors only (GlobalToSharedDirectLoader into a SharedRing,
+    SharedToRegLoader on 16 x 32 / 32 x 16 MFMA operand tiles, gemm()) against the oracle and, bit for bit, against
+    the hand-indexed pipelined kernel, whose arithmetic it performs in the same order (1, 3, 16 and 64 k-tiles)."""
+    import torch
+
+    print(f"gemm tile_pipelined {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float16 if out_dtype == "f16" else torch.float32
+    A = oracle.fill_uniform(M * K, 7000 + K).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 8000 + K).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    C = tcu.gemm(dA, dB, out_dtype=dt, algo="tile_pipelined")
+    torch.cuda.synchronize()
+    rows = (0, M) if M <= 1024 else (M - 192, M)
+    ref = oracle.gemm(A, Bt, rows=rows)
+    assert oracle.max_rel_err(host(C)[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
+    assert torch.equal(C, tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))
+
+
 @pytest.mark.parametrize("algo", ["pipelined", "wave128"])
 def test_gemm_one_hot_index_probe(tcu, device, algo):
     """C[m, n] = A[m, k] * Bt[n, k] for one-hot operands: pins rows/cols/transposition exactly."""

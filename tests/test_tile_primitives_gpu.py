@@ -82,7 +82,9 @@ def test_tile_case(case, device, oracle):
         M, N, K = dims[:3]
         A = oracle.fill_uniform(M * K, 100 + idx).reshape(M, K)
         Bt = oracle.fill_uniform(N * K, 200 + idx).reshape(N, K)
-        a, b = torch.from_numpy(A).to(device), torch.from_numpy(Bt).to(device)
+        # dims[4] = 1: the kernel takes B stored row-major [K, N] (and transposes it on the way to registers)
+        b_mem = np.ascontiguousarray(Bt.T) if dims[4] else Bt
+        a, b = torch.from_numpy(A).to(device), torch.from_numpy(b_mem).to(device)
         c = torch.full((M, N), float("nan"), dtype=torch.float32, device=device)
         run(a, b, c, None)
         err = oracle.max_rel_err(c.cpu().numpy(), oracle.gemm(A, Bt))

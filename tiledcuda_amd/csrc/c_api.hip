@@ -183,10 +183,33 @@ int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int 
                   C, M, N, K, lda, ldb);
 }
 
+template <typename OutType, int kM, int kN, int kK, int kTM, int kTN, typename WarpLayout>
+int launch_tile_pipelined(const __half* A, const __half* B, OutType* C, hipStream_t stream) {
+    using Traits = PipelinedGemmTileTraits<__half, OutType, GemmShape<kM, kN, kK>, kTM, kTN, WarpLayout>;
+    auto kernel = &gemm_tile_pipelined<__half, OutType, Traits>;
+    return launch(kernel, dim3((kM / kTM) * (kN / kTN)), dim3(Traits::kThreads), Traits::kShmBytes, stream, A, B, C);
+}
+
+/// The pipelined kernel composed from tile-library functors has compile-time shapes, like every kernel written against
+/// the tile API: the instantiations below are the benchmark shape and the shapes its tests use.
+template <typename OutType>
+int gemm_tile_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    using W42 = tl::RowMajor<4, 2>;
+    using W22 = tl::RowMajor<2, 2>;
+    if (M == 4096 && N == 4096 && K == 4096) return launch_tile_pipelined<OutType, 4096, 4096, 4096, 256, 256, W42>(A, B, C, stream);
+    if (M == 1024 && N == 1024 && K == 1024) return launch_tile_pipelined<OutType, 1024, 1024, 1024, 256, 256, W42>(A, B, C, stream);
+    if (M == 512 && N == 768 && K == 192) return launch_tile_pipelined<OutType, 512, 768, 192, 128, 128, W22>(A, B, C, stream);
+    if (M == 256 && N == 256 && K == 64) return launch_tile_pipelined<OutType, 256, 256, 64, 64, 64, W22>(A, B, C, stream);
+    return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the tile-API pipelined GEMM is instantiated for 4096^3, 1024^3, 512x768x192 "
+                                           "and 256x256x64");
+}
+
 template <typename OutType>
 int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, int algo, hipStream_t stream) {
     using W22 = tl::RowMajor<2, 2>;
     switch (algo) {
+        case TCU_GEMM_TILE_PIPELINED:
+            return gemm_tile_pipelined_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_WAVE128:
             return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_AUTO:
