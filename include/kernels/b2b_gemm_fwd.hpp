@@ -14,7 +14,11 @@
 //   * LDS rows are 256 B (A, B) or 512 B (C, intermediate); the 16-byte chunks are XOR-ed with row % 16 inside
 //     every aligned group of 16 chunks, which makes the ds_read_b128 of 16 consecutive rows at one k-offset
 //     conflict-free; for the loads the permutation is applied on the global-address side.
-// The intermediate never leaves the chip. M % 32 == 0 is required (checked by the host launcher).
+// Longer N (any multiple of 256, the reference's example also runs N = 1024 and 2048,
+// examples/cpp/02_fused_two_gemms/fused_gemm.cu:236-259) is processed in blocks of 256 columns of B / rows of C through
+// the same LDS buffers: the B buffer is refilled with the next block while the second product of the current block
+// runs, the C buffer while the first product of the next block runs; the f32 accumulators of D stay in registers.
+// The intermediate never leaves the chip. M % 32 == 0 and N % 256 == 0 are required (checked by the host launcher).
 #pragma once
 
 #include "config.hpp"
@@ -39,13 +43,13 @@ struct B2bResidentTraits {
     HOST_DEVICE static constexpr int swz(int c, int row) { return (c & 16) | ((c & 15) ^ (row & 15)); }
 };
 
-/// grid = (M / 32, batch), block = 512, dynamic LDS = B2bResidentTraits::kLdsBytes.
+/// grid = (M / 32, batch), block = 512, dynamic LDS = B2bResidentTraits::kLdsBytes. N: columns of B = rows of C.
 template <typename OutType>
 __global__ void __launch_bounds__(B2bResidentTraits::kThreads)
     b2b_gemm_resident(const __half* __restrict__ A, const __half* __restrict__ B, const __half* __restrict__ C,
-                      OutType* __restrict__ D, int M) {
+                      OutType* __restrict__ D, int M, int N) {
     using T = B2bResidentTraits;
-    constexpr int kN = T::kN, kK = T::kK, kP = T::kP;
+    constexpr int kN = T::kN, kK = T::kK, kP = T::kP;  // kN: the block of N held in LDS at a time
     extern __shared__ __align__(1024) unsigned char lds[];
 
     const int lane = lane_id();
@@ -54,32 +58,47 @@ __global__ void __launch_bounds__(B2bResidentTraits::kThreads)
     const int m0 = blockIdx.x * T::kTM;
     const size_t batch = blockIdx.y;
     const __half* Ab = A + (batch * M + m0) * kK;
-    const __half* Bb = B + batch * size_t(kN) * kK;
-    const __half* Cb = C + batch * size_t(kP) * kN;
+    const __half* Bb = B + batch * size_t(N) * kK;
+    const __half* Cb = C + batch * size_t(kP) * N;
     OutType* Db = D + (batch * M + m0) * kP;
+    const int nblocks = N / kN;
 
-    // ---- everything in flight at once: A (1 instruction per wavefront), B (8), C (8), 1 KiB each
-    {
+    // block nb of B: rows 256 nb .. of the stored [N, K] array (8 instructions of 1 KiB per wavefront)
+    auto load_b = [&](int nb) {
         const int r4 = lane >> 4, c16 = lane & 15;  // 256-byte rows: 4 rows x 16 chunks per instruction
-        {
-            const int row = 4 * wave + r4;
-            detail::load_lds_16B_untracked(Ab + size_t(row) * kK + (c16 ^ (row & 15)) * 8, lds + T::kAOff + wave * 1024);
-        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int q = 8 * wave + j;
             const int row = 4 * q + r4;
-            detail::load_lds_16B_untracked(Bb + size_t(row) * kK + (c16 ^ (row & 15)) * 8, lds + T::kBOff + q * 1024);
+            detail::load_lds_16B_untracked(Bb + (size_t(nb) * kN + row) * kK + (c16 ^ (row & 15)) * 8,
+                                           lds + T::kBOff + q * 1024);
         }
+    };
+    // block nb of C: columns 256 nb .. of the stored [P, N] array (8 instructions per wavefront)
+    auto load_c = [&](int nb) {
         const int r2 = lane >> 5, c32 = lane & 31;  // 512-byte rows: 2 rows x 32 chunks per instruction
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int q = 8 * wave + j;
             const int row = 2 * q + r2;
-            detail::load_lds_16B_untracked(Cb + size_t(row) * kN + T::swz(c32, row) * 8, lds + T::kCOff + q * 1024);
+            detail::load_lds_16B_untracked(Cb + size_t(row) * N + size_t(nb) * kN + T::swz(c32, row) * 8,
+                                           lds + T::kCOff + q * 1024);
         }
+    };
+    // ---- everything of the first block in flight at once: A (1 instruction per wavefront), B (8), C (8)
+    {
+        const int r4 = lane >> 4, c16 = lane & 15;
+        const int row = 4 * wave + r4;
+        detail::load_lds_16B_untracked(Ab + size_t(row) * kK + (c16 ^ (row & 15)) * 8, lds + T::kAOff + wave * 1024);
     }
-    detail::lds_barrier<8>();  // vmcnt(8): this wavefront's shares of A and B have landed; then everyone's
+    load_b(0);
+    load_c(0);
+
+    f32x4 acc2[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    for (int nb = 0; nb < nblocks; ++nb) {
+    // the B block (and A) have landed - this wavefront's share (the 8 younger loads, of the C block, may still be in
+    // flight), then everyone's; everyone is done with the previous block's C and intermediate
+    detail::lds_barrier<8>();
 
     // ---- first product: acc1[nt][mt][r] = (A·B)[m = 16 mt + L][n = 32 wave + 16 nt + 4 g + r]
     f32x4 acc1[2][2];
@@ -118,10 +137,10 @@ __global__ void __launch_bounds__(B2bResidentTraits::kThreads)
             for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc1[nt][mt][e]);
             *reinterpret_cast<f16x4*>(lds + T::kSOff + m * T::kRowBytesN + T::swz(chunk, m) * 16 + (g & 1) * 8) = v;
         }
-    detail::lds_barrier<0>();  // C has landed, the intermediate is written; for everyone
+    detail::lds_barrier<0>();  // C has landed, the intermediate is written, the B buffer is free; for everyone
+    if (nb + 1 < nblocks) load_b(nb + 1);  // under the second product
 
-    // ---- second product: acc2[mt][r] = D[m = 16 mt + L][p = 16 wave + 4 g + r]
-    f32x4 acc2[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    // ---- second product: acc2[mt][r] += D[m = 16 mt + L][p = 16 wave + 4 g + r] over this block's n
     const int p_row = 16 * wave + L;
 #pragma unroll
     for (int s = 0; s < kN / 32; ++s) {
@@ -135,6 +154,13 @@ __global__ void __launch_bounds__(B2bResidentTraits::kThreads)
             acc2[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fc, fs, acc2[mt], 0, 0, 0);
         }
     }
+    if (nb + 1 < nblocks) {
+        // everyone is done with this block's C and intermediate: the C buffer is refilled under the next first product
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS reads have returned
+        __builtin_amdgcn_s_barrier();
+        load_c(nb + 1);
+    }
+    }  // blocks of N
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
         OutType* dst = Db + size_t(16 * mt + L) * kP + 16 * wave + 4 * g;

@@ -45,7 +45,8 @@ typedef enum {
 typedef enum {
     TCU_B2B_AUTO = 0,
     TCU_B2B_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, the reference kernel's structure */
-    TCU_B2B_RESIDENT = 2      /* A tile, B, C and the intermediate all resident in LDS, one round of loads */
+    TCU_B2B_RESIDENT = 2      /* A tile, 256-column blocks of B and C and the intermediate resident in LDS (K = P = 128,
+                                 N % 256 == 0, M % 32 == 0); one round of loads per block */
 } tcu_b2b_algo;
 
 /* Layout of V in tcu_flash_attn_fwd_f16. */

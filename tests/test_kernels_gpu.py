@@ -212,6 +212,31 @@ def test_b2b_gemm_shapes(tcu, oracle, device, M, N, K, P, batch, out_dtype):
     assert oracle.max_rel_err(host(D), ref, eps=1.0) <= REL_TOL
 
 
+# every uncommented run<...> of the reference's driver, examples/cpp/02_fused_two_gemms/fused_gemm.cu:212-259
+REFERENCE_B2B_SHAPES = [(16, 16, 16, 16, 1), (16, 32, 16, 32, 1), (32, 64, 32, 64, 1), (64, 64, 32, 64, 1),
+                        (256, 128, 64, 64, 1), (1024, 1024, 128, 128, 1), (16, 16, 16, 16, 2),
+                        (1024, 1024, 128, 128, 5), (64, 256, 128, 128, 1), (2048, 1024, 128, 128, 1),
+                        (1024, 2048, 128, 128, 1)]
+
+
+@pytest.mark.parametrize("M,N,K,P,batch", REFERENCE_B2B_SHAPES)
+@pytest.mark.parametrize("algo", ["tile_library", "auto"])
+def test_b2b_gemm_reference_shape_list(tcu, oracle, device, M, N, K, P, batch, algo):
+    """The shapes the reference's fused two-GEMM example runs, on the kernel composed from tile primitives and on
+    whatever AUTO picks (the LDS-resident kernel, streaming blocks of N, where K = P = 128 and N % 256 == 0)."""
+    import torch
+
+    print(f"b2b reference shape {M}x{N}x{K}x{P} batch {batch} {algo}", flush=True)
+    A = oracle.fill_normal(batch * M * K, 811, 0, 0.1).reshape(batch, M, K)
+    Bt = oracle.fill_normal(batch * N * K, 812, 0, 0.1).reshape(batch, N, K)
+    Ct = oracle.fill_normal(batch * P * N, 813, 0, 0.1).reshape(batch, P, N)
+    D = tcu.b2b_gemm(dev(A, device), dev(Bt, device), dev(Ct, device), out_dtype=torch.float32, algo=algo)
+    torch.cuda.synchronize()
+    got = host(D)
+    for b in range(batch):
+        assert oracle.max_rel_err(got[b], oracle.b2b_gemm(A[b], Bt[b], Ct[b]), eps=1.0) <= REL_TOL
+
+
 @pytest.mark.parametrize("algo", ["tile_library", "resident"])
 @pytest.mark.parametrize("M,batch,out_dtype", [(32, 1, "f32"), (96, 3, "f16"), (8192, 1, "f16"), (16384, 2, "f32")])
 def test_b2b_gemm_both_kernels_at_256x128x128(tcu, oracle, device, algo, M, batch, out_dtype):

@@ -260,12 +260,12 @@ int b2b_dispatch(const __half* A, const __half* B, const __half* C, OutType* D, 
     if (algo != TCU_B2B_AUTO && algo != TCU_B2B_TILE_LIBRARY && algo != TCU_B2B_RESIDENT)
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: unknown algo");
     if (algo != TCU_B2B_TILE_LIBRARY) {
-        if (N == 256 && K == 128 && P == 128 && M % 32 == 0)
+        if (N % 256 == 0 && K == 128 && P == 128 && M % 32 == 0)
             return launch(&b2b_gemm_resident<OutType>, dim3(M / B2bResidentTraits::kTM, batch),
-                          dim3(B2bResidentTraits::kThreads), B2bResidentTraits::kLdsBytes, stream, A, B, C, D, M);
+                          dim3(B2bResidentTraits::kThreads), B2bResidentTraits::kLdsBytes, stream, A, B, C, D, M, N);
         if (algo == TCU_B2B_RESIDENT)
-            return fail(TCU_ERR_UNSUPPORTED_SHAPE,
-                        "the LDS-resident b2b kernel is instantiated for (N, K, P) = (256, 128, 128) with M a multiple of 32");
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the LDS-resident b2b kernel takes K = P = 128, N a multiple of 256 "
+                                                   "and M a multiple of 32");
     }
     if (N == 256 && K == 128 && P == 128) {
         // 32-row tiles keep all 256 CUs busy up to M * batch = 8192; 64-row tiles beyond that
@@ -277,9 +277,22 @@ int b2b_dispatch(const __half* A, const __half* B, const __half* C, OutType* D, 
         return launch_b2b<OutType, 128, 64, 64, 32, 64, tl::RowMajor<2, 1>>(A, B, C, D, M, batch, stream);
     if (N == 64 && K == 64 && P == 64 && M % 16 == 0)
         return launch_b2b<OutType, 64, 64, 64, 16, 32, tl::RowMajor<1, 1>>(A, B, C, D, M, batch, stream);
+    // the rest of the shape list of the reference's driver (examples/cpp/02_fused_two_gemms/fused_gemm.cu:212-259),
+    // with its tile shapes and warp layouts
+    if (N == 16 && K == 16 && P == 16 && M % 16 == 0)
+        return launch_b2b<OutType, 16, 16, 16, 16, 16, tl::RowMajor<1, 1>>(A, B, C, D, M, batch, stream);
+    if (N == 32 && K == 16 && P == 32 && M % 16 == 0)
+        return launch_b2b<OutType, 32, 16, 32, 16, 16, tl::RowMajor<1, 1>>(A, B, C, D, M, batch, stream);
+    if (N == 64 && K == 32 && P == 64 && M % 32 == 0)
+        return launch_b2b<OutType, 64, 32, 64, 32, 32, tl::RowMajor<2, 1>>(A, B, C, D, M, batch, stream);
+    if (N == 1024 && K == 128 && P == 128 && M % 64 == 0)
+        return launch_b2b<OutType, 1024, 128, 128, 64, 64, tl::RowMajor<4, 1>>(A, B, C, D, M, batch, stream);
+    if (N == 2048 && K == 128 && P == 128 && M % 64 == 0)
+        return launch_b2b<OutType, 2048, 128, 128, 64, 128, tl::RowMajor<4, 1>>(A, B, C, D, M, batch, stream);
     return fail(TCU_ERR_UNSUPPORTED_SHAPE,
-                "b2b GEMM is instantiated for (N, K, P) in {(256,128,128), (128,64,64), (64,64,64)} with M a "
-                "multiple of 32 (16 for the last)");
+                "the tile-library b2b GEMM is instantiated for (N, K, P) in {(16,16,16), (32,16,32), (64,32,64), (64,64,64), "
+                "(128,64,64), (256,128,128), (1024,128,128), (2048,128,128)} with M a multiple of its row tile (16 ... 64); "
+                "the LDS-resident kernel takes K = P = 128, N % 256 == 0, M % 32 == 0");
 }
 
 // ---------------------------------------------------------------------------- attention
