@@ -23,7 +23,16 @@
 //     scores already computed for the next half are re-biased and the probabilities are recomputed;
 //   * K/V blocks of 64 keys go global -> LDS directly into a ring of four stages, requested two blocks ahead, one
 //     LDS-only barrier per block; swizzles and the transposing V reads are those of flash_attn_fwd.hpp.
-// M % 256 == 0 and N % 64 == 0 are required (checked by the host launcher).
+// kVColMajor: V is stored column-major [N, D], i.e. as the array Vᵀ [D, N] (the convention of the reference's op,
+// src/kernels/flash_attn.cu:424-456 with pytiledcuda/__init__.py:17-30). A row of Vᵀ then holds consecutive keys, and
+// the A operand of Oᵀ += Vᵀ Pᵀ could be a plain ds_read_b128 if a lane needed 8 consecutive keys - which the
+// accumulator of Sᵀ does not give (a lane half holds keys 4 h .. + 3 of every group of 8). So the keys are re-ordered
+// where it is free: row i of a 32-key score tile is fed with key 16 ((i / 4) % 2) + 4 (i / 8) + i % 4 (just another
+// row address for the K fragment read), which puts the 16 consecutive keys 16 h .. 16 h + 15 of the tile into lane
+// half h, 8 consecutive ones per MFMA k-step: one ds_read_b128 per Vᵀ fragment, no transposing read. The swizzle of
+// the K rows is chosen for that read order.
+// M % 64 == 0 and N % 64 == 0 are required (checked by the host launcher); wavefronts of the last workgroup whose
+// 64 queries lie beyond M take part in the loads and barriers and discard their result.
 #pragma once
 
 #include <type_traits>
@@ -133,7 +142,7 @@ DEVICE void mfma_settle_a(f32x16& x) { asm volatile("s_nop 15\n\ts_nop 15" : "+a
 /// grid = (M / 256) * batch workgroups (1-D), block = 256, dynamic LDS = Traits::kLdsBytes.
 /// Workgroup ids congruent modulo 8 land on the same XCD: when the batch count is a multiple of 8 the query blocks
 /// of one (batch, head) item all get such ids, so its K and V are fetched from HBM once.
-template <typename Traits>
+template <typename Traits, bool kVColMajor = false>
 __global__ void __launch_bounds__(Traits::kThreads)
     flash_attention_fwd_w64(const __half* __restrict__ Q, const __half* __restrict__ K, const __half* __restrict__ V,
                             __half* __restrict__ O, int batch, int M, int N, float scale) {
@@ -150,7 +159,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int q32 = lane & 31;  // query (column of Sᵀ / Oᵀ) of this lane within a 32-query tile
     const int h = lane >> 5;    // lane half
 
-    const int q_blocks = M / Traits::kBM;
+    const int q_blocks = (M + Traits::kBM - 1) / Traits::kBM;
     int head_i, q_block;
     if (batch % 8 == 0) {
         const int xcd = blockIdx.x & 7, rest = blockIdx.x >> 3;
@@ -162,10 +171,20 @@ __global__ void __launch_bounds__(Traits::kThreads)
     }
     const size_t head = head_i;
     const int m0 = q_block * Traits::kBM + wave * 64;
-    const __half* Qh = Q + (head * M + m0) * kD;
+    const bool active = m0 < M;  // wave-uniform: this wavefront's 64 queries exist
+    const __half* Qh = Q + (head * M + (active ? m0 : 0)) * kD;
     const __half* Kh = K + head * size_t(N) * kD;
     const __half* Vh = V + head * size_t(N) * kD;
-    __half* Oh = O + (head * M + m0) * kD;
+    __half* Oh = O + (head * M + (active ? m0 : 0)) * kD;
+
+    // Key order inside a 32-key half (see the header): score-tile row i holds key key_of_row(i); identity for a
+    // row-major V. k_swizzle: XOR applied to the 16-byte chunk index of K row `row` of a block, chosen so that the 16
+    // rows read by one pass of a fragment read (rows key_of_row(0..15) or (16..31)) get 16 different values.
+    auto key_of_row = [](int i) { return kVColMajor ? 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3) : i; };
+    auto k_swizzle = [](int row) {
+        return kVColMajor ? (((row >> 2) & 1) << 3) | (((row >> 4) & 1) << 2) | (row & 3) : Swz::k_swz(row);
+    };
+    const int nb = N / kBN;
 
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
 
@@ -179,13 +198,20 @@ __global__ void __launch_bounds__(Traits::kThreads)
         const bool is_v = j >= kL / 2;
         const int t = wave + Traits::kWaves * (is_v ? j - kL / 2 : j);  // 1 KiB slot of the tile
         const int row = t * Traits::kRowsPerLoad + lrow;
-        const int chunk = is_v ? (lchk ^ (Swz::v_swz(row) << 1)) : (lchk ^ Swz::k_swz(row));
-        goff[j] = static_cast<unsigned int>(row * kD + chunk * 8) * 2u;
+        if (is_v && kVColMajor) {
+            // the V block is kD rows (d) of 64 keys = 128 bytes: 8 rows per instruction, chunks XOR-ed with (d / 2) % 8
+            const int d = t * 8 + (lane >> 3);
+            const int chunk8 = (lane & 7) ^ ((d >> 1) & 7);
+            goff[j] = static_cast<unsigned int>(d * N + chunk8 * 8) * 2u;
+        } else {
+            const int chunk = is_v ? (lchk ^ (Swz::v_swz(row) << 1)) : (lchk ^ k_swizzle(row));
+            goff[j] = static_cast<unsigned int>(row * kD + chunk * 8) * 2u;
+        }
         ldst[j] = (is_v ? Traits::kTileBytes : 0) + t * 1024;
     }
     auto issue_load = [&](int block, int j) {
         const bool is_v = j >= kL / 2;
-        const __half* src = (is_v ? Vh : Kh) + size_t(block) * kBN * kD;
+        const __half* src = (is_v && kVColMajor) ? Vh + size_t(block) * kBN : (is_v ? Vh : Kh) + size_t(block) * kBN * kD;
         const unsigned int dst =
             __builtin_amdgcn_readfirstlane(lds_base + (block % kStages) * Traits::kStageBytes + ldst[j]);
         detail::load_lds_16B_sbase(goff[j], src, dst);
@@ -202,53 +228,66 @@ __global__ void __launch_bounds__(Traits::kThreads)
     using fp16x4 = __fp16 __attribute__((ext_vector_type(4)));
     using lds_fp16x4_ptr = fp16x4 __attribute__((address_space(3)))*;
     // K fragment (A operand of Sᵀ = K Qᵀ) for d-step s: lane (row = lane % 32, h) holds K[row][16 s + 8 h .. + 7]
+    // (of the key this lane's score-tile row stands for)
     unsigned int koff[Traits::kDSteps];
+    const int krow = key_of_row(q32);
 #pragma unroll
     for (int s = 0; s < Traits::kDSteps; ++s) {
-        const int chunk = (2 * s + h) ^ Swz::k_swz(q32);  // the swizzle depends on row % 16 only
-        koff[s] = lds_base + q32 * kRowBytes + chunk * 16;
+        const int chunk = (2 * s + h) ^ k_swizzle(krow);  // the swizzle depends on row % 32 only
+        koff[s] = lds_base + krow * kRowBytes + chunk * 16;
         asm volatile("" : "+v"(koff[s]));  // keep the eight offsets in registers (not rematerialised per use)
     }
     auto read_k = [&](unsigned int k_half_off, int s) -> f16x8 {
         return *reinterpret_cast<lds_f16x8_ptr>(koff[s] + k_half_off);
     };
-    // Vᵀ fragment (A operand of Oᵀ += Vᵀ Pᵀ) for d tile dt and k-step s2 of the half: lane (d = 32 dt + lane % 32,
-    // h), slot e = key 16 s2 + 8 (e / 4) + 4 h + e % 4, fetched with two transposing reads. Within a 16-lane group,
-    // lane L supplies the address of row kv0 + L / 4, columns dbase + 4 (L % 4) .. + 3.
+    // the same read of the staged Q rows (row = lane % 32 of a 32-query tile, swizzled like a K block of a row-major V)
+    auto read_q_staged = [&](unsigned int q_half_off, int s) -> f16x8 {
+        const int chunk = (2 * s + h) ^ Swz::k_swz(q32);
+        return *reinterpret_cast<lds_f16x8_ptr>(lds_base + q32 * kRowBytes + chunk * 16 + q_half_off);
+    };
+    // Vᵀ fragment (A operand of Oᵀ += Vᵀ Pᵀ) for d tile dt and k-step s2 of key half t of a block: lane
+    // (d = 32 dt + lane % 32, h).
+    // Row-major V: slot e = key 16 s2 + 8 (e / 4) + 4 h + e % 4 of the half, fetched with two transposing reads; within
+    // a 16-lane group, lane L supplies the address of row kv0 + L / 4, columns dbase + 4 (L % 4) .. + 3.
+    // Column-major V: slot e = key 16 h + 8 s2 + e of the half (the keys this lane half holds after the re-ordering),
+    // 16 contiguous bytes of row d of the Vᵀ block: chunk 4 t + 2 h + s2, XOR-ed with (d / 2) % 8.
     const int g = lane >> 4, L16 = lane & 15;
     const int vrow_in = L16 >> 2;
     const int vcol_b = (16 * (g & 1) + 4 * (L16 & 3)) * 2;
-    unsigned int voff[Traits::kDTiles];
+    unsigned int voff[Traits::kDTiles];  // row-major V: per d tile; column-major V: per (t, s2)
 #pragma unroll
     for (int dt = 0; dt < Traits::kDTiles; ++dt) {
-        const int byte_in_row = 64 * dt + vcol_b;
-        const int unit = (byte_in_row >> 5) ^ Swz::v_swz(vrow_in);  // every row read by this lane has row % 4 == vrow_in
-        voff[dt] = lds_base + (4 * h + vrow_in) * kRowBytes + unit * 32 + (byte_in_row & 31);
+        if (kVColMajor) {
+            const int chunk = (4 * (dt >> 1) + 2 * h + (dt & 1)) ^ ((q32 >> 1) & 7);
+            voff[dt] = lds_base + q32 * 128 + chunk * 16;
+        } else {
+            const int byte_in_row = 64 * dt + vcol_b;
+            const int unit = (byte_in_row >> 5) ^ Swz::v_swz(vrow_in);  // every row read by this lane has row % 4 == vrow_in
+            voff[dt] = lds_base + (4 * h + vrow_in) * kRowBytes + unit * 32 + (byte_in_row & 31);
+        }
         asm volatile("" : "+v"(voff[dt]));
     }
-    auto read_v = [&](unsigned int v_half_off, int s2, int dt) -> f16x8 {
-        f16x8 vf;
-#pragma unroll
-        for (int part = 0; part < 2; ++part) {
-            const fp16x4 v4 = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
-                reinterpret_cast<lds_fp16x4_ptr>(voff[dt] + v_half_off + (16 * s2 + 8 * part) * kRowBytes));
-#pragma unroll
-            for (int e = 0; e < 4; ++e) vf[4 * part + e] = static_cast<_Float16>(v4[e]);
-        }
-        return vf;
-    };
     auto read_k_untracked = [&](unsigned int k_half_off, int s) -> f16x8 {
         return detail::lds_read_b128_untracked(koff[s] + k_half_off);
     };
-    auto read_v_untracked = [&](unsigned int v_half_off, auto s2_c, int dt) -> f16x8 {
-        constexpr int s2 = decltype(s2_c)::value;
-        return detail::lds_read_tr_pair_untracked<16 * s2 * kRowBytes, (16 * s2 + 8) * kRowBytes>(voff[dt] + v_half_off);
+    // v_blk_off: LDS offset of the V tile of the block; t_c, s2_c: key half of the block and k-step of the half
+    auto read_v_untracked = [&](unsigned int v_blk_off, auto t_c, auto s2_c, int dt) -> f16x8 {
+        constexpr int t = decltype(t_c)::value, s2 = decltype(s2_c)::value;
+        if constexpr (kVColMajor) {
+            return detail::lds_read_b128_untracked(voff[2 * t + s2] + v_blk_off + dt * (32 * 128));
+        } else {
+            constexpr int kRow0 = 32 * t + 16 * s2;
+            return detail::lds_read_tr_pair_untracked<kRow0 * kRowBytes, (kRow0 + 8) * kRowBytes>(voff[dt] + v_blk_off);
+        }
     };
     // LDS offset (relative to the ring) of the K rows of half `half_i` of the key sequence; V is kTileBytes further
     auto k_half = [&](int half_i) -> unsigned int {
         return ((half_i >> 1) % kStages) * Traits::kStageBytes + (half_i & 1) * Traits::kHalfBytes;
     };
-    auto v_half = [&](int half_i) -> unsigned int { return k_half(half_i) + Traits::kTileBytes; };
+    // LDS offset of the V tile of the block that half `half_i` belongs to
+    auto v_block = [&](int half_i) -> unsigned int {
+        return ((half_i >> 1) % kStages) * Traits::kStageBytes + Traits::kTileBytes;
+    };
 
     // ---- prologue: Q and the first K/V blocks are requested together (so that the cold latencies overlap).
     // Q fragments (B operand of Sᵀ = K Qᵀ): lane (q, h) of column tile c holds Q[32 c + q][16 s + 8 h .. + 7].
@@ -256,16 +295,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
     // enough to matter the wavefront instead stages its 64 contiguous rows (16 KiB) through LDS like a K block
     // (coalesced 1 KiB loads, same swizzle, same fragment reads), in the two ring stages (3 and 4) that the K/V
     // blocks reach last; those two blocks are then requested in the first block-iteration.
-    const int nb = N / kBN;
     const bool q_via_lds = nb >= kStages;
     f16x8 qraw[2][Traits::kDSteps];
     if (q_via_lds) {
         const unsigned int q_stage = 3 * Traits::kStageBytes + wave * (64 * kRowBytes);
+        if (active) {
 #pragma unroll
-        for (int t = 0; t < 64 / Traits::kRowsPerLoad; ++t) {
-            const int row = t * Traits::kRowsPerLoad + lrow;
-            const unsigned int off = static_cast<unsigned int>(row * kD + (lchk ^ Swz::k_swz(row)) * 8) * 2u;
-            detail::load_lds_16B_sbase(off, Qh, __builtin_amdgcn_readfirstlane(lds_base + q_stage + t * 1024));
+            for (int t = 0; t < 64 / Traits::kRowsPerLoad; ++t) {
+                const int row = t * Traits::kRowsPerLoad + lrow;
+                const unsigned int off = static_cast<unsigned int>(row * kD + (lchk ^ Swz::k_swz(row)) * 8) * 2u;
+                detail::load_lds_16B_sbase(off, Qh, __builtin_amdgcn_readfirstlane(lds_base + q_stage + t * 1024));
+            }
         }
 #pragma unroll
         for (int j = 0; j < kL; ++j) {
@@ -281,7 +321,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
 #pragma unroll
         for (int c = 0; c < 2; ++c)
 #pragma unroll
-            for (int s = 0; s < Traits::kDSteps; ++s) qraw[c][s] = read_k(q_stage + c * Traits::kHalfBytes, s);
+            for (int s = 0; s < Traits::kDSteps; ++s) qraw[c][s] = read_q_staged(q_stage + c * Traits::kHalfBytes, s);
     } else {
 #pragma unroll
         for (int b = 0; b < kStages - 1; ++b)
@@ -294,6 +334,14 @@ __global__ void __launch_bounds__(Traits::kThreads)
 #pragma unroll
             for (int s = 0; s < Traits::kDSteps; ++s)
                 qraw[c][s] = *reinterpret_cast<const f16x8*>(Qh + size_t(32 * c + q32) * kD + 16 * s + 8 * h);
+    }
+    if (!active) {
+        // nothing of this wavefront's result is kept: feed zeros (what was read above is some other rows' data or,
+        // for the staged path, whatever the stage held)
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int s = 0; s < Traits::kDSteps; ++s) qraw[c][s] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
     // pre-multiplied by scale * log2(e): the scores come out of the MFMA in the log2 domain
     const float cscale = scale * 1.4426950408889634f;
@@ -382,6 +430,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
     // latency): the last d-steps of a step request the first fragments of the next one (K of half i + 2 if
     // kNextQk, V of half i).
     constexpr int kAhead = Traits::kFragAhead, kRing = kAhead + 1;
+    // LDS read instructions per d-step: the V fragment is two transposing reads or one ds_read_b128; plus the K one
+    constexpr int kReadsV = kVColMajor ? 1 : 2, kReadsQk = kReadsV + 1;
     static_assert(8 % kRing == 0 && kAhead <= 3, "ring positions must repeat from one step to the next; the prefetch stays within the first k-step of the next half");
     f16x8 kf[kRing], vf[kRing];
     auto step = [&](int i, auto cur_c, auto qk_c, auto loads_c, auto next_qk_c, int load_block) {
@@ -389,9 +439,9 @@ __global__ void __launch_bounds__(Traits::kThreads)
         constexpr bool kQk = decltype(qk_c)::value, kLoads = decltype(loads_c)::value;
         constexpr bool kNextQk = decltype(next_qk_c)::value;
         const unsigned int sk = __builtin_amdgcn_readfirstlane(k_half(i + 1));
-        const unsigned int sv = __builtin_amdgcn_readfirstlane(v_half(i - 1));
+        const unsigned int sv = __builtin_amdgcn_readfirstlane(v_block(i - 1));  // key half kNxt of that block
         const unsigned int sk_next = __builtin_amdgcn_readfirstlane(k_half(i + 2));
-        const unsigned int sv_next = __builtin_amdgcn_readfirstlane(v_half(i));
+        const unsigned int sv_next = __builtin_amdgcn_readfirstlane(v_block(i));  // key half kCur of that block
         float lh[2] = {0.f, 0.f}, lg[2] = {0.f, 0.f};  // two partial sums per query tile (independent add chains)
         // VALU work of the same wavefront hides under its MFMAs only in small doses: one v_exp_f32 plus one or two
         // plain instructions directly behind each MFMA cost 2-3 cycles per MFMA, the same instructions in groups of
@@ -409,15 +459,15 @@ __global__ void __launch_bounds__(Traits::kThreads)
             constexpr int sp = s + kAhead;
             if constexpr (sp < 8) {
                 if (kQk) kf[sp % kRing] = read_k_untracked(sk, sp);
-                if (sp < 4) vf[sp % kRing] = read_v_untracked(sv, C0{}, sp & 3);
-                else vf[sp % kRing] = read_v_untracked(sv, C1{}, sp & 3);
-                detail::lds_wait<kAhead * (kQk ? 3 : 2)>();
+                if (sp < 4) vf[sp % kRing] = read_v_untracked(sv, std::integral_constant<int, kNxt>{}, C0{}, sp & 3);
+                else vf[sp % kRing] = read_v_untracked(sv, std::integral_constant<int, kNxt>{}, C1{}, sp & 3);
+                detail::lds_wait<kAhead * (kQk ? kReadsQk : kReadsV)>();
             } else {
                 if (kNextQk) kf[sp % kRing] = read_k_untracked(sk_next, sp - 8);
-                vf[sp % kRing] = read_v_untracked(sv_next, C0{}, (sp - 8) & 3);
-                // in flight after this wait: the fragments of the d-steps still ahead in this step (3 or 2 reads
+                vf[sp % kRing] = read_v_untracked(sv_next, std::integral_constant<int, kCur>{}, C0{}, (sp - 8) & 3);
+                // in flight after this wait: the fragments of the d-steps still ahead in this step (kReadsQk or kReadsV reads
                 // each) and those just requested for the next step
-                detail::lds_wait<(7 - s) * (kQk ? 3 : 2) + (sp - 7) * (kNextQk ? 3 : 2)>();
+                detail::lds_wait<(7 - s) * (kQk ? kReadsQk : kReadsV) + (sp - 7) * (kNextQk ? kReadsQk : kReadsV)>();
             }
             // slot A
             if (kQk) {
@@ -523,7 +573,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
 #pragma unroll
     for (int a = 0; a < kAhead; ++a) {
         if (nb > 1) kf[a] = read_k_untracked(k_half(2), a);
-        vf[a] = read_v_untracked(v_half(0), C0{}, a & 3);
+        vf[a] = read_v_untracked(v_block(0), C0{}, C0{}, a & 3);
     }
     // ---- block-iterations: J covers halves 2 J + 1 (odd) and 2 J + 2 (even)
     int J = 0;
@@ -552,16 +602,16 @@ __global__ void __launch_bounds__(Traits::kThreads)
     step(2 * J + 1, C1{}, No{}, No{}, No{}, 0);
     {
         // the output update with the last half (its first fragments were requested by the step before)
-        const unsigned int sv = v_half(2 * J + 1);
+        const unsigned int sv = v_block(2 * J + 1);
         detail::static_for<8>([&](auto s_c) {
             constexpr int s = decltype(s_c)::value;
             constexpr int sp = s + kAhead;
             if constexpr (sp < 8) {
-                if (sp < 4) vf[sp % kRing] = read_v_untracked(sv, C0{}, sp & 3);
-                else vf[sp % kRing] = read_v_untracked(sv, C1{}, sp & 3);
-                detail::lds_wait<kAhead * 2>();
+                if (sp < 4) vf[sp % kRing] = read_v_untracked(sv, C1{}, C0{}, sp & 3);
+                else vf[sp % kRing] = read_v_untracked(sv, C1{}, C1{}, sp & 3);
+                detail::lds_wait<kAhead * kReadsV>();
             } else {
-                detail::lds_wait<(7 - s) * 2>();
+                detail::lds_wait<(7 - s) * kReadsV>();
             }
 #pragma unroll
             for (int c = 0; c < 2; ++c) detail::mfma32_out(o_acc[s & 3][c], vf[s % kRing], pf[1][c][s >> 2]);
@@ -603,7 +653,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         const int row = it * kRowsPerIter + rr;
         const int pslot = (2 * cc) ^ (((row & 15) << 1) & kSlotMask);
         const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kRowBytes + pslot * 8);
-        *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(Oh + size_t(row) * kD) + cc * 16) = v;
+        if (active) *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(Oh + size_t(row) * kD) + cc * 16) = v;
     }
 }
 

@@ -127,7 +127,9 @@ def test_unsupported_shapes_are_reported_not_launched(tcu):
     assert l.tcu_b2b_gemm_f16(p, p, p, p, 64, 96, 64, 64, 1, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 64, 128, 64, 1.0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 100, 128, 128, 1.0, 1, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
-    assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 192, 128, 128, 1.0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 192, 64, 64, 1.0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # col-major V: D 128 only
+    assert l.tcu_flash_attn_fwd_f16_algo(p, p, p, p, 1, 64, 192, 128, 128, 1.0, 0, 1, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # tile library: fixed N
+    assert l.tcu_flash_attn_fwd_f16_algo(p, p, p, p, 1, 256, 256, 64, 64, 1.0, 1, 4, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # wave64: D 128 only
     assert l.tcu_lstm_f16(p, p, p, 0, 0, p, p, 1, 64, 100, 128, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_lstm_f16(p, p, p, 0, 0, p, p, 1, 10, 128, 128, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
 

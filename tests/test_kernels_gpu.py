@@ -405,6 +405,52 @@ def test_flash_attention_wave64_sequence_lengths(tcu, oracle, device, batch, M, 
     assert oracle.max_abs_err(host(O), ref) <= ABS_TOL
 
 
+@pytest.mark.parametrize("batch,m,n", [(1, 64, 64), (1, 64, 192), (2, 128, 448), (3, 320, 256), (1, 256, 1088),
+                                       (8, 512, 2048), (64, 2048, 2048)])
+def test_flash_attention_fwd_op_convention_any_key_count(tcu, oracle, device, batch, m, n):
+    """The reference op's call shape (flattened tensors, K as [n, k], V column-major = stored [p, n], scale 1) at key
+    counts the reference op does not dispatch (it knows n in {64, 128, 256} at batch 1): the kernel with 64 queries per
+    wavefront in its column-major-V form (keys re-ordered inside the score tiles, plain 16-byte reads of V), also with
+    query counts that leave wavefronts of the last workgroup idle, up to the C4 problem in this layout."""
+    import torch
+
+    print(f"attention op convention b{batch} m{m} n{n}", flush=True)
+    k = p = 128
+    Q = oracle.fill_normal(batch * m * k, 81).reshape(batch, m, k) * np.float16(0.3)
+    Kn = oracle.fill_normal(batch * n * k, 82).reshape(batch, n, k) * np.float16(0.3)
+    V = oracle.fill_normal(batch * n * p, 83).reshape(batch, n, p)
+    Vt = np.ascontiguousarray(V.transpose(0, 2, 1))
+    O = torch.full((batch * m * p,), float("nan"), dtype=torch.float16, device=device)
+    tcu.flash_attention_fwd(dev(Q, device).flatten(), dev(Kn, device).flatten(), dev(Vt, device).flatten(), O, m, n, k, p,
+                            batch=batch)
+    torch.cuda.synchronize()
+    got = host(O).reshape(batch, m, p)
+    assert np.isfinite(got).all()
+    items = range(batch) if batch <= 8 else (0, 21, batch - 1)
+    for b in items:
+        rows = (0, m) if m <= 512 else (m - 160, m - 32)
+        ref = oracle.attention(Q[b], Kn[b], V[b], 1.0, rows=rows)
+        assert oracle.max_abs_err(got[b, rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= ABS_TOL
+
+
+@pytest.mark.parametrize("batch,M,N", [(2, 64, 128), (1, 192, 384), (3, 320, 64), (2, 448, 704)])
+def test_flash_attention_wave64_partial_workgroups(tcu, oracle, device, batch, M, N):
+    """Query counts that are multiples of 64 but not of 256: wavefronts of the last workgroup beyond M take part in the
+    loads and barriers and write nothing (the output buffer is followed by a guard region that must stay untouched)."""
+    import torch
+
+    D = 128
+    q = oracle.fill_normal(batch * M * D, 91).reshape(batch, M, D)
+    k = oracle.fill_normal(batch * N * D, 92).reshape(batch, N, D)
+    v = oracle.fill_normal(batch * N * D, 93).reshape(batch, N, D)
+    buf = torch.full((batch * M * D + 256 * D,), 7.0, dtype=torch.float16, device=device)
+    out = buf[:batch * M * D].view(batch, M, D)
+    tcu.flash_attention(dev(q, device), dev(k, device), dev(v, device), out=out, algo="wave64")
+    torch.cuda.synchronize()
+    assert oracle.max_abs_err(host(out), oracle.attention(q, k, v, 1.0 / math.sqrt(D))) <= ABS_TOL
+    assert bool((buf[batch * M * D:] == 7.0).all())
+
+
 def test_flash_attention_wave64_maximum_jumps_late(tcu, oracle, device):
     """One key far above everything before it, placed in each half of a 64-key block and in the last block: the
     check on the sum of a 32-key half fails there, and the reference maxima, the output accumulators, the running
@@ -483,10 +529,10 @@ def test_unsupported_shape_raises_runtime_error(tcu, device):
     import torch
 
     q = torch.zeros(64 * 128, dtype=torch.float16, device=device)
-    kk = torch.zeros(192 * 128, dtype=torch.float16, device=device)
+    kk = torch.zeros(100 * 128, dtype=torch.float16, device=device)
     o = torch.zeros(64 * 128, dtype=torch.float16, device=device)
     with pytest.raises(RuntimeError):
-        tcu.flash_attention_fwd(q, kk, kk, o, 64, 192, 128, 128)
+        tcu.flash_attention_fwd(q, kk, kk, o, 64, 100, 128, 128)  # the key count must be a multiple of 64
     with pytest.raises(RuntimeError):
         tcu.gemm(torch.zeros(100, 64, dtype=torch.float16, device=device),
                  torch.zeros(64, 64, dtype=torch.float16, device=device))

@@ -315,11 +315,14 @@ int launch_fa_fwd(const __half* Q, const __half* K, const __half* V, __half* O, 
                   O, batch, M, N, scale);
 }
 
+template <bool kVColMajor>
 int launch_fa_w64(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
                   hipStream_t stream) {
     using Traits = FlashW64Traits<128>;
-    return launch(&flash_attention_fwd_w64<Traits>, dim3((M / Traits::kBM) * batch), dim3(Traits::kThreads),
-                  Traits::kLdsBytes, stream, Q, K, V, O, batch, M, N, scale);
+    if ((long)N * 256 >= (1l << 32))
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel addresses a V block with 32-bit offsets");
+    return launch(&flash_attention_fwd_w64<Traits, kVColMajor>, dim3(((M + Traits::kBM - 1) / Traits::kBM) * batch),
+                  dim3(Traits::kThreads), Traits::kLdsBytes, stream, Q, K, V, O, batch, M, N, scale);
 }
 
 template <int kD, bool kFused>
@@ -338,17 +341,18 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     if (algo != TCU_ATTN_AUTO && algo != TCU_ATTN_TILE_LIBRARY && algo != TCU_ATTN_MFMA32 &&
         algo != TCU_ATTN_MFMA32_FUSED && algo != TCU_ATTN_WAVE64)
         return fail(TCU_ERR_INVALID_ARGUMENT, "unknown attention algo");
+    if (v_layout != TCU_V_ROW_MAJOR && v_layout != TCU_V_COL_MAJOR) return fail(TCU_ERR_INVALID_ARGUMENT, "unknown v_layout");
     if (algo == TCU_ATTN_WAVE64) {
-        if (v_layout != TCU_V_ROW_MAJOR || Kd != 128 || M % 256 != 0)
-            return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel takes a row-major V, head "
-                                                   "size 128 and M % 256 == 0");
-        return launch_fa_w64(Q, K, V, O, batch, M, N, scale, stream);
+        if (Kd != 128)
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel is instantiated for head size 128");
+        return v_layout == TCU_V_ROW_MAJOR ? launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream)
+                                           : launch_fa_w64<true>(Q, K, V, O, batch, M, N, scale, stream);
     }
     if (v_layout == TCU_V_ROW_MAJOR && algo != TCU_ATTN_TILE_LIBRARY) {
         if (Kd != 128 && Kd != 64) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
         // long sequences with enough query blocks to fill the chip: the kernel with 64 queries per wavefront
         if (algo == TCU_ATTN_AUTO && Kd == 128 && M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 128)
-            return launch_fa_w64(Q, K, V, O, batch, M, N, scale, stream);
+            return launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream);
         if (algo == TCU_ATTN_MFMA32)
             return Kd == 128 ? fa_fwd_by_rows<128, false>(Q, K, V, O, batch, M, N, scale, stream)
                              : fa_fwd_by_rows<64, false>(Q, K, V, O, batch, M, N, scale, stream);
@@ -362,19 +366,20 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
         if (Kd == 64) return launch_fa<0, 64, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
     }
-    if (v_layout == TCU_V_COL_MAJOR) {
-        if (Kd != 128) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for head size 128");
-        // a column-major V has leading dimension N: one instantiation per N, as in the reference op
-        switch (N) {
-            case 64: return launch_fa<64, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
-            case 128: return launch_fa<128, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
-            case 256: return launch_fa<256, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
-            case 2048: return launch_fa<2048, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
-            default:
-                return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for N in {64, 128, 256, 2048}");
-        }
+    // column-major V (the reference op's convention), any N % 64 == 0
+    if (Kd != 128) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for head size 128");
+    if (algo == TCU_ATTN_AUTO) return launch_fa_w64<true>(Q, K, V, O, batch, M, N, scale, stream);
+    // the kernel composed from tile primitives has the leading dimension of V (= N) as a compile-time constant, like
+    // the reference op: one instantiation per N
+    switch (N) {
+        case 64: return launch_fa<64, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+        case 128: return launch_fa<128, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+        case 256: return launch_fa<256, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+        case 2048: return launch_fa<2048, 128, false, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+        default:
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the tile-library attention kernel takes a column-major V for N in {64, 128, "
+                                                   "256, 2048}");
     }
-    return fail(TCU_ERR_INVALID_ARGUMENT, "unknown v_layout");
 }
 
 // ---------------------------------------------------------------------------- LSTM
