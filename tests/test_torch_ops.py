@@ -25,6 +25,20 @@ def test_ops_are_registered_with_the_reference_schemas(ops):
         assert hasattr(ops, name)
 
 
+def test_ops_come_from_the_cpp_library(ops):
+    """The registrations live in a shared library built from C++ (csrc/torch_bind.cc, the counterpart of the reference's
+    src/torch_bind.cc), loaded with torch.ops.load_library, as the reference's Python package does."""
+    import os
+
+    import tiledcuda_amd.torch_ops as torch_ops
+
+    path = torch_ops.library_path()
+    assert os.path.basename(path) == "libtiledcuda_torch.so" and os.path.exists(path)
+    assert path in torch.ops.loaded_libraries
+    blob = open(path, "rb").read()
+    assert b"tcu_flash_attn_fwd_f16" in blob and b"tcu_scatter_nd" in blob  # it calls the C-ABI, nothing else
+
+
 def test_ops_have_no_cpu_fallback(ops):
     with pytest.raises(NotImplementedError):
         ops.gemm(torch.zeros(64, 64, dtype=torch.float16), torch.zeros(64, 64, dtype=torch.float16),
@@ -49,6 +63,31 @@ def test_flash_attention_fwd_op_reference_shapes(ops, oracle, device, n):
     ops.flash_attention_fwd(q, key, val, out, m, n, k, p)
     ref = oracle.attention(Q.half().numpy(), Kmat.half().t().contiguous().numpy(), V.half().numpy(), 1.0)
     assert oracle.max_abs_err(out.view(m, p).float().cpu().numpy(), ref) <= 1e-2
+
+
+@pytest.mark.gpu
+def test_cpp_ops_check_their_operands(ops, device):
+    """dtype / shape / contiguity mistakes are refused by the C++ layer (TORCH_CHECK -> RuntimeError) before any
+    pointer reaches a kernel; the reference op checks nothing."""
+    h = dict(dtype=torch.half, device=device)
+    a = torch.zeros(64, 64, **h)
+    with pytest.raises(RuntimeError, match="must be"):
+        ops.gemm(a.float(), a, torch.zeros(64, 64, **h))
+    with pytest.raises(RuntimeError, match="mismatched K"):
+        ops.gemm(a, torch.zeros(64, 32, **h), torch.zeros(64, 64, **h))
+    with pytest.raises(RuntimeError, match=r"C must be \[M, N\]"):
+        ops.gemm(a, a, torch.zeros(64, 32, **h))
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ops.gemm(a.t(), a, torch.zeros(64, 64, **h))
+    q = torch.zeros(64 * 128, **h)
+    with pytest.raises(RuntimeError, match="K must hold"):
+        ops.flash_attention_fwd(q, q[:-128], q, q, 64, 64, 128, 128)
+    with pytest.raises(RuntimeError, match="h0 must be"):
+        ops.lstm(torch.zeros(2, 64, 128, **h), torch.zeros(512, 256, **h), torch.zeros(512, **h),
+                 torch.zeros(32, 128, **h), None)
+    with pytest.raises(RuntimeError, match="one slice"):
+        ops.scatter_nd(torch.zeros(8, 4, device=device), torch.zeros(3, 4, device=device),
+                       torch.zeros(2, 1, dtype=torch.int64, device=device))
 
 
 @pytest.mark.gpu
