@@ -8,6 +8,7 @@
 #include "types/shared.hpp"
 #include "types/shared_tile_iterator.hpp"
 #include "types/tile_shape.hpp"
+#include "util/tile_print.hpp"
 
 namespace tiledcuda::cell {
 

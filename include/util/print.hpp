@@ -1,4 +1,5 @@
-// Tile printers (device printf); the role of the reference's util/print.hpp:15-65.
+// Scalar tile printers (device printf); the role of the reference's util/print.hpp:15-65. The printers that show a
+// register tile in matrix order (the reference's RegTilePrinter / RegVecPrinter, :67-175) are in util/tile_print.hpp.
 #pragma once
 
 #include "config.hpp"

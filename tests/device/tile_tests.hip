@@ -934,6 +934,35 @@ void build_registry() {
 
 thread_local std::string g_err;
 
+// prints (device printf) a 32 x 48 f16 ramp held as 2 x 3 row-major BaseTiles, a 32 x 32 f32 MFMA accumulator tile and
+// the row maxima of the first, each in matrix order
+__global__ void __launch_bounds__(64) k_print_tiles(const __half* src) {
+    using Global = GlobalTile<__half, tl::RowMajor<32, 48>>;
+    using Reg = RegTile<BaseTileRowMajor<__half>, tl::RowMajor<2, 3>>;
+    Global g(src);
+    Reg r;
+    GlobalToRegLoader<Reg, tl::RowMajor<1, 1>, WarpReuse::kCont> g2r;
+    g2r(g, r);
+    RegTilePrinter<Reg> print;
+    print(r, threadIdx.x);
+
+    using Vec = RegTile<__half, tl::RowMajor<2, 1>>;
+    Vec v;
+    compute::MaxReduce<Reg, tl::Layout::kRowMajor> row_max;
+    row_max(r, v);
+    RegVecPrinter<Vec> print_vec;
+    print_vec(v, threadIdx.x);
+
+    using Acc = RegTile<MfmaTileC32x32<float>, tl::RowMajor<1, 1>>;
+    Acc acc;
+    // element (row, col) = row + col / 100: this lane holds row lane % 32, columns 8 q + 4 (lane / 32) + e
+    for (int q = 0; q < 4; ++q)
+        for (int e = 0; e < 4; ++e)
+            acc(0, 0)(4 * q + e) = float(threadIdx.x % 32) + float(8 * q + 4 * (threadIdx.x / 32) + e) * 0.01f;
+    RegTilePrinter<Acc> print_acc;
+    print_acc(acc, threadIdx.x);
+}
+
 }  // namespace
 
 extern "C" {
@@ -966,6 +995,18 @@ int tt_run_case(int id, const void* a, const void* b, void* c, void* d, void* st
     if (id < 0 || id >= (int)registry().size()) return -1;
     const Case& cs = registry()[id];
     cs.launch(a, b, c, d, cs.threads, cs.lds_bytes, static_cast<hipStream_t>(stream));
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        g_err = hipGetErrorString(e);
+        return -3;
+    }
+    return 0;
+}
+
+/// Launches the tile printer demonstration (one wavefront; output goes to the process's stdout at the next
+/// synchronisation). src: 32 x 48 f16, row-major.
+int tt_print_tiles(const void* src, void* stream) {
+    hipLaunchKernelGGL(k_print_tiles, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), static_cast<const __half*>(src));
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         g_err = hipGetErrorString(e);

@@ -165,3 +165,26 @@ def test_tile_case(case, device, oracle):
             assert np.allclose(got, want, rtol=rtol, atol=rtol)
     else:
         raise AssertionError(kind)
+
+
+def test_tile_printers_show_matrix_order(device, capfd):
+    """RegTilePrinter / RegVecPrinter (the reference's include/util/print.hpp:67-175): a register tile spread over the
+    64 lanes prints as the matrix it stands for - a 32 x 48 f16 tile of 2 x 3 BaseTiles, its row maxima, and a
+    32 x 32 MFMA accumulator tile whose element (r, c) was set to r + c / 100 in its lane-local layout."""
+    handle = _load()
+    handle.tt_print_tiles.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    src = (np.arange(32 * 48) % 2048).astype(np.float16).reshape(32, 48)
+    a = torch.from_numpy(src).to(device)
+    capfd.readouterr()
+    assert handle.tt_print_tiles(a.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0, handle.tt_last_error()
+    torch.cuda.synchronize()
+    out = capfd.readouterr().out
+    blocks = [b for b in out.strip().split("\n\n") if b.strip()]
+    assert len(blocks) == 3, out
+    rows = [[float(x) for x in line.rstrip(", ").split(", ")] for line in blocks[0].strip().split("\n")]
+    assert np.array_equal(np.array(rows), src.astype(np.float64))
+    vec = [float(x) for x in blocks[1].strip().rstrip(",").split(", ")]
+    assert np.array_equal(np.array(vec), src.max(axis=1).astype(np.float64))
+    acc = np.array([[float(x) for x in line.rstrip(", ").split(", ")] for line in blocks[2].strip().split("\n")])
+    want = np.arange(32)[:, None] + np.arange(32)[None, :] * 0.01
+    assert acc.shape == (32, 32) and np.allclose(acc, want, atol=6e-4)  # printed with three decimals
