@@ -28,7 +28,8 @@ typedef enum {
 typedef enum { TCU_DTYPE_F32 = 0, TCU_DTYPE_F16 = 1 } tcu_dtype;
 
 /* Which GEMM kernel to run. AUTO picks WAVE128 when M and N are multiples of 256 with at least 128 tiles of 256 x 256,
- * else the pipelined kernel when the shape allows. */
+ * else the pipelined kernel when M, N and K are multiples of 64, else RAGGED: every shape made of whole 16 x 16
+ * BaseTiles (M, N, K multiples of 16), the granularity of the reference's tile types, is accepted. */
 typedef enum {
     TCU_GEMM_AUTO = 0,
     TCU_GEMM_GLOBAL_REG = 1, /* global -> register -> MFMA (README kernel of the reference) */
@@ -36,9 +37,11 @@ typedef enum {
     TCU_GEMM_PIPELINED = 3,  /* direct-to-LDS, double-buffered, 16x16x32 MFMA, 2 wavefronts per SIMD */
     TCU_GEMM_WAVE128 = 4,    /* same pipeline, 256 x 256 tile on 4 wavefronts (one per SIMD, 128 x 128 each),
                                 accumulators in AGPRs; results identical to PIPELINED bit for bit */
-    TCU_GEMM_TILE_PIPELINED = 5 /* the PIPELINED kernel composed from tile-library functors only (direct-to-LDS loader,
+    TCU_GEMM_TILE_PIPELINED = 5, /* the PIPELINED kernel composed from tile-library functors only (direct-to-LDS loader,
                                 two-stage shared ring, ds_read_b128 operand tiles, gemm()); compile-time shapes:
                                 4096^3, 1024^3, 512x768x192, 256x256x64; results identical to PIPELINED bit for bit */
+    TCU_GEMM_RAGGED = 6       /* run-time M, N, K in multiples of 16: MFMA operand tiles filled from global memory,
+                                tiles beyond the edge skipped; the fallback for shapes the tiled kernels do not cover */
 } tcu_gemm_algo;
 
 /* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks RESIDENT where it is instantiated. */

@@ -122,6 +122,8 @@ def test_unsupported_shapes_are_reported_not_launched(tcu):
     p = 0x1000
     assert l.tcu_gemm_f16(p, p, p, 100, 64, 64, 0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_gemm_f16(p, p, p, 64, 64, 48, 0, 3, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_gemm_f16(p, p, p, 64, 72, 64, 0, 6, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # whole 16 x 16 tiles only
+    assert l.tcu_gemm_f16(p, p, p, 64, 64, 40, 0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_gemm_f16(p, p, p, 256, 256, 256, 0, 1, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_gemm_f16(p, p, p, 128, 256, 64, 0, 4, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_b2b_gemm_f16(p, p, p, p, 64, 96, 64, 64, 1, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE

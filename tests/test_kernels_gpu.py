@@ -95,6 +95,31 @@ def test_gemm_wave128_shapes(tcu, oracle, device, M, N, K, out_dtype):
     assert torch.equal(C, tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 16, 16), (16, 48, 32), (80, 16, 48), (48, 112, 80), (144, 208, 16), (64, 64, 64),
+                                   (1040, 528, 272), (4096, 16, 4096)])
+@pytest.mark.parametrize("out_dtype", ["f32", "f16"])
+def test_gemm_ragged_shapes(tcu, oracle, device, M, N, K, out_dtype):
+    """Every shape made of whole 16 x 16 BaseTiles (the granularity of the reference's tile types,
+    include/types/register.hpp:108-112) runs: blocks that hang over the edge in M, in N and in both, a last k-step of
+    16, one tile, a thin N; through AUTO (which must route them to the run-time-shape kernel) and by name. The output is
+    surrounded by a guard band that must stay untouched."""
+    import torch
+
+    print(f"gemm ragged {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    A = oracle.fill_uniform(M * K, 31 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 37 + N).reshape(N, K)
+    want = oracle.gemm(A, Bt)
+    dA, dB = dev(A, device), dev(Bt, device)
+    for algo in ("ragged", "auto"):
+        guard = torch.full((M + 2, N), -7.0, dtype=dt, device=device)
+        out = guard[1:M + 1]
+        tcu.gemm(dA, dB, out=out, algo=algo)
+        torch.cuda.synchronize()
+        assert oracle.max_rel_err(host(out), want) <= REL_TOL
+        assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
+
+
 def test_gemm_wave128_rejects_other_shapes(tcu, device):
     import torch
 

@@ -7,6 +7,7 @@
 #include "kernels/flash_attn_fwd.hpp"
 #include "kernels/flash_attn_w64.hpp"
 #include "kernels/gemm_pipelined.hpp"
+#include "kernels/gemm_ragged.hpp"
 #include "kernels/gemm_w128.hpp"
 #include "kernels/lstm_fwd.hpp"
 #include "kernels/mod.hpp"
@@ -205,6 +206,16 @@ int gemm_tile_pipelined_dispatch(const __half* A, const __half* B, OutType* C, i
 }
 
 template <typename OutType>
+int gemm_ragged_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    using T = RaggedGemmTraits;
+    if (M % 16 != 0 || N % 16 != 0 || K % 16 != 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM shapes are whole 16 x 16 tiles: M, N and K must be multiples of 16");
+    const long grid = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
+    if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many 64 x 64 blocks for one launch");
+    return launch(&gemm_ragged<OutType>, dim3(unsigned(grid)), dim3(T::kThreads), 0, stream, A, B, C, M, N, K);
+}
+
+template <typename OutType>
 int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, int algo, hipStream_t stream) {
     using W22 = tl::RowMajor<2, 2>;
     switch (algo) {
@@ -217,9 +228,12 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) >= 128 &&
                 (long)K * 512 < (1l << 32))
                 return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
+            if (M % 64 != 0 || N % 64 != 0 || K % 64 != 0) return gemm_ragged_dispatch<OutType>(A, B, C, M, N, K, stream);
             [[fallthrough]];
         case TCU_GEMM_PIPELINED:
             return gemm_pipelined_dispatch<OutType>(A, B, C, M, N, K, stream);
+        case TCU_GEMM_RAGGED:
+            return gemm_ragged_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_GLOBAL_REG:
           if constexpr (std::is_same_v<OutType, float>) {
             if (M == 128 && N == 64 && K == 256)  // the README shape of the reference
