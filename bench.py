@@ -284,6 +284,18 @@ def main():
         ms_h = time_kernel(lstm_hoisted, max(5, args.steps // 2), max(2, args.warmup // 2))
         err_h = max(oracle.max_abs_err(outh["h"][:, 0:2].float().cpu().numpy(), h_ref[:, 0:2]),
                     oracle.max_abs_err(outh["c"][0:2].cpu().numpy(), c_ref[0:2]))
+        # the time loop as one weight-stationary launch after the same GEMM (h exchanged inside each XCD)
+        wsp = torch.empty(tcu.lstm_persistent_workspace_bytes(T, Bb, I, Hh), dtype=torch.uint8, device=dev)
+        outp = {"h": torch.empty(T, Bb, Hh, dtype=torch.float16, device=dev),
+                "c": torch.empty(Bb, Hh, dtype=torch.float32, device=dev)}
+
+        def lstm_persistent():
+            tcu.lstm(dx, dW, db, algo="persistent", workspace=wsp, out=(outp["h"], outp["c"]), check=False)
+
+        ms_p = time_kernel(lstm_persistent, max(5, args.steps // 2), max(2, args.warmup // 2))
+        tcu.lstm_persistent_status(wsp)  # raises if a workgroup gave up waiting for its XCD
+        err_p = max(oracle.max_abs_err(outp["h"][:, 0:2].float().cpu().numpy(), h_ref[:, 0:2]),
+                    oracle.max_abs_err(outp["c"][0:2].cpu().numpy(), c_ref[0:2]))
         step_bytes = 2.0 * (4 * Hh * (I + Hh) + 4 * Hh + Bb * I + 2 * Bb * Hh) + 4.0 * 2 * Bb * Hh
         flops = 2.0 * Bb * (I + Hh) * 4 * Hh * T
         configs.append({"name": "lstm_b256_i1024_h1024_t16_hoisted_input_gemm", "ms": ms_h, "us_per_step": ms_h * 1e3 / T,
@@ -291,6 +303,11 @@ def main():
                         "frac_hbm_peak": step_bytes * T / (ms_h * 1e-3) / 1e9 / HBM_PEAK_GBS,
                         "tflops": flops / (ms_h * 1e-3) / 1e12, "max_abs_err": err_h,
                         "workspace_bytes": int(ws.numel())})
+        configs.append({"name": "lstm_b256_i1024_h1024_t16_persistent_single_launch", "ms": ms_p,
+                        "us_per_step": ms_p * 1e3 / T, "gbs": step_bytes * T / (ms_p * 1e-3) / 1e9,
+                        "frac_hbm_peak": step_bytes * T / (ms_p * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        "tflops": flops / (ms_p * 1e-3) / 1e12, "max_abs_err": err_p,
+                        "workspace_bytes": int(wsp.numel())})
         configs.append({"name": "lstm_b256_i1024_h1024_t16", "ms": ms, "us_per_step": ms * 1e3 / T,
                         "us_per_step_in_hip_graph": None if gms is None else gms * 1e3 / T,
                         "frac_hbm_peak_in_hip_graph": None if gms is None else step_bytes * T / (gms * 1e-3) / 1e9 / HBM_PEAK_GBS,

@@ -22,7 +22,8 @@ typedef enum {
     TCU_ERR_INVALID_ARGUMENT = -1,  /* null or misaligned pointer, non-positive size, bad enum value */
     TCU_ERR_UNSUPPORTED_SHAPE = -2, /* shape not divisible by the tile / not instantiated */
     TCU_ERR_HIP = -3,               /* a HIP runtime call failed (message has the HIP error) */
-    TCU_ERR_NO_DEVICE = -4          /* no HIP device is available to this process */
+    TCU_ERR_NO_DEVICE = -4,         /* no HIP device is available to this process */
+    TCU_ERR_INCOMPLETE = -5         /* a single-launch kernel gave up a bounded wait; its outputs are invalid */
 } tcu_status;
 
 typedef enum { TCU_DTYPE_F32 = 0, TCU_DTYPE_F16 = 1 } tcu_dtype;
@@ -155,6 +156,28 @@ unsigned long long tcu_lstm_workspace_bytes(int T, int B, int I, int H);
 int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
                     void* c_out, int T, int B, int I, int H, void* workspace, unsigned long long workspace_bytes,
                     void* stream);
+
+/*
+ * The LSTM layer with the whole time loop in ONE launch, for the large-hidden-size case where a step is bound by
+ * streaming the recurrent weights and by the cost of a dependent launch (H == 1024, I % 64 == 0, B % 32 == 0, B <= 256,
+ * T * B % 256 == 0; a device of 256 CUs in 8 XCDs). As in tcu_lstm_f16_ws the input half of the gates of all steps is
+ * one GEMM into the workspace; the recurrence then runs weight-stationary: every XCD keeps a copy of W[:, I:] in the
+ * registers of its 32 CUs and owns 32 batch rows, and h_t is exchanged between those CUs through the XCD's L2 only.
+ * Same arguments and results (up to the order of the f32 summation) as tcu_lstm_f16_ws. `workspace`: device memory of
+ * at least tcu_lstm_persistent_workspace_bytes(T, B, I, H) bytes (0 = shape not supported), 1 KiB-aligned, owned by
+ * the caller; its first 4 KiB are synchronisation words, cleared by the call.
+ * The launch needs all of its 256 workgroups resident at the same time, i.e. a GPU that is not occupied by another
+ * kernel for long; its waits are bounded (2 s; TCU_LSTM_PERSISTENT_SPIN_US in the environment overrides, in
+ * microseconds), and every workgroup exits normally when a wait expires. The call itself is asynchronous like all
+ * others; tcu_lstm_persistent_status(workspace, stream) synchronises the stream and returns TCU_OK, or
+ * TCU_ERR_INCOMPLETE when a wait expired (h_all and c_out are then invalid: run tcu_lstm_f16_ws instead).
+ * No counterpart in the reference (it has no LSTM).
+ */
+unsigned long long tcu_lstm_persistent_workspace_bytes(int T, int B, int I, int H);
+int tcu_lstm_f16_persistent(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                            void* c_out, int T, int B, int I, int H, void* workspace,
+                            unsigned long long workspace_bytes, void* stream);
+int tcu_lstm_persistent_status(const void* workspace, void* stream);
 
 /*
  * tcu_lstm_f16_ws for callers that can neither allocate device memory nor bring a workspace: code under HIP graph

@@ -662,7 +662,8 @@ def test_lstm_config5(tcu, oracle, device):
     b = oracle.fill_normal(4 * H, 3239, 0, 0.05)
     dx, dW, db = dev(x, device), dev(W, device), dev(b, device)
     refs = {rows: oracle.lstm(x, W, b, rows=rows) for rows in [(0, 4), (252, 256)]}
-    for algo in ("auto", "hoisted"):
+    for algo in ("auto", "hoisted", "persistent"):
+        print(f"lstm C5 {algo}", flush=True)
         h_all, c_T = tcu.lstm(dx, dW, db, algo=algo)
         torch.cuda.synchronize()
         hh, cc = host(h_all), host(c_T)
@@ -670,6 +671,82 @@ def test_lstm_config5(tcu, oracle, device):
         for rows, (h_ref, c_ref) in refs.items():
             assert oracle.max_abs_err(hh[:, rows[0]:rows[1]], h_ref[:, rows[0]:rows[1]]) <= ABS_TOL, algo
             assert oracle.max_abs_err(cc[rows[0]:rows[1]], c_ref[rows[0]:rows[1]]) <= ABS_TOL, algo
+
+
+@pytest.mark.parametrize("T,B,I", [(4, 64, 64), (8, 32, 192), (2, 128, 1024), (1, 256, 64)])
+@pytest.mark.parametrize("with_state", [False, True])
+def test_lstm_persistent_single_launch(tcu, oracle, device, T, B, I, with_state):
+    """tcu_lstm_f16_persistent (H = 1024): the time loop in one weight-stationary launch, h exchanged inside each XCD.
+    One to eight XCDs in use, one to eight steps, with and without an initial state; against the oracle and against
+    the hoisted per-step path (same projection GEMM, other summation order); twice on one workspace, whose bytes past
+    the stated size stay untouched."""
+    import torch
+
+    H = 1024
+    print(f"lstm persistent T{T} B{B} I{I} state={with_state}", flush=True)
+    x = oracle.fill_normal(T * B * I, 61, 0, 0.5).reshape(T, B, I)
+    W = oracle.fill_normal(4 * H * (I + H), 62, 0, 0.03).reshape(4 * H, I + H)
+    b = oracle.fill_normal(4 * H, 63, 0, 0.1)
+    h0 = oracle.fill_normal(B * H, 64, 0, 0.5).reshape(B, H) if with_state else None
+    c0 = oracle.fill_normal(B * H, 65, 0, 0.5).reshape(B, H).astype(np.float32) if with_state else None
+    args = (dev(x, device), dev(W, device), dev(b, device), dev(h0, device) if with_state else None,
+            dev(c0, device) if with_state else None)
+    need = tcu.lstm_persistent_workspace_bytes(T, B, I, H)
+    assert need == 4096 + T * B * 4 * H * 4
+    ws = torch.full((need + 4096,), 0xFF, dtype=torch.uint8, device=device)
+    refs = {rows: oracle.lstm(x, W, b, h0, c0, rows=rows) for rows in [(0, 3), (B - 3, B)]}  # first and last XCD in use
+    for rep in range(2):
+        h_all, c_T = tcu.lstm(*args, algo="persistent", workspace=ws)
+        torch.cuda.synchronize()
+        for (r0, r1), (h_ref, c_ref) in refs.items():
+            assert oracle.max_abs_err(host(h_all)[:, r0:r1], h_ref[:, r0:r1]) <= ABS_TOL
+            assert oracle.max_abs_err(host(c_T)[r0:r1], c_ref[r0:r1]) <= ABS_TOL
+    assert bool((ws[need:] == 0xFF).all())
+    if tcu.lstm_workspace_bytes(T, B, I, H):
+        h_hst, c_hst = tcu.lstm(*args, algo="hoisted")
+        assert float((h_all.float() - h_hst.float()).abs().max()) <= 2e-3
+        assert float((c_T - c_hst).abs().max()) <= 2e-3
+
+
+def test_lstm_persistent_bounded_wait(tcu, device, monkeypatch):
+    """A workgroup whose peers never all arrive gives up after the time limit, raises the error word and exits; so does
+    everyone waiting for it: the launch ends normally and the host is told. Forced from the host: the kernel is told to
+    wait for 33 arrivals per XCD where 32 workgroups exist. The next, ordinary call on the same workspace works."""
+    import torch
+
+    T, B, I, H = 4, 64, 64, 1024
+    g = torch.Generator(device="cpu").manual_seed(5)
+    x = (torch.randn(T, B, I, generator=g) * 0.5).half().to(device)
+    W = (torch.randn(4 * H, I + H, generator=g) * 0.03).half().to(device)
+    b = (torch.randn(4 * H, generator=g) * 0.1).half().to(device)
+    ws = torch.empty(tcu.lstm_persistent_workspace_bytes(T, B, I, H), dtype=torch.uint8, device=device)
+    good = tcu.lstm(x, W, b, algo="persistent", workspace=ws)
+    monkeypatch.setenv("TCU_LSTM_PERSISTENT_PEERS", "33")
+    monkeypatch.setenv("TCU_LSTM_PERSISTENT_SPIN_US", "2000")
+    print("lstm persistent: forced time-out", flush=True)
+    with pytest.raises(RuntimeError, match="waited"):
+        tcu.lstm(x, W, b, algo="persistent", workspace=ws)
+    monkeypatch.delenv("TCU_LSTM_PERSISTENT_PEERS")
+    monkeypatch.delenv("TCU_LSTM_PERSISTENT_SPIN_US")
+    again = tcu.lstm(x, W, b, algo="persistent", workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(good[0], again[0]) and torch.equal(good[1], again[1])
+
+
+def test_lstm_persistent_rejects_what_it_cannot_do(tcu, device):
+    import torch
+
+    assert tcu.lstm_persistent_workspace_bytes(4, 64, 64, 512) == 0    # H != 1024
+    assert tcu.lstm_persistent_workspace_bytes(4, 48, 64, 1024) == 0   # B not a multiple of 32
+    assert tcu.lstm_persistent_workspace_bytes(1, 512, 64, 1024) == 0  # more rows than 8 XCDs x 32
+    assert tcu.lstm_persistent_workspace_bytes(3, 64, 64, 1024) == 0   # T * B not a multiple of 256
+    x = torch.zeros(4, 64, 64, dtype=torch.float16, device=device)
+    W = torch.zeros(4096, 64 + 1024, dtype=torch.float16, device=device)
+    b = torch.zeros(4096, dtype=torch.float16, device=device)
+    with pytest.raises(RuntimeError):
+        tcu.lstm(x, W, b, algo="persistent", workspace=torch.empty(8192, dtype=torch.uint8, device=device))
+    with pytest.raises(RuntimeError):
+        tcu.lstm(x[:3].contiguous(), W, b, algo="persistent")
 
 
 def test_smoke_entry(device):

@@ -18,7 +18,7 @@ import torch
 
 __all__ = [
     "TcuError", "library_path", "lib", "last_error", "gemm", "b2b_gemm", "flash_attention_fwd",
-    "flash_attention", "TiledFlashAttention", "lstm", "lstm_workspace_bytes", "scatter_nd", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS", "B2B_ALGOS",
+    "flash_attention", "TiledFlashAttention", "lstm", "lstm_workspace_bytes", "lstm_persistent_workspace_bytes", "lstm_persistent_status", "scatter_nd", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS", "B2B_ALGOS",
     "SCATTER_MODES",
 ]
 
@@ -62,6 +62,10 @@ _SIGNATURES = {
     "tcu_lstm_workspace_bytes": (ctypes.c_ulonglong, [ctypes.c_int] * 4),
     "tcu_lstm_f16_ws": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_ulonglong,
                                                                                      ctypes.c_void_p]),
+    "tcu_lstm_persistent_workspace_bytes": (ctypes.c_ulonglong, [ctypes.c_int] * 4),
+    "tcu_lstm_f16_persistent": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_ulonglong,
+                                                                                          ctypes.c_void_p]),
+    "tcu_lstm_persistent_status": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p]),
     "tcu_lstm_noalloc_max_bytes": (ctypes.c_ulonglong, []),
     "tcu_lstm_f16_noalloc": (ctypes.c_int, [ctypes.c_void_p] * 7 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
     "tcu_scatter_nd": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.POINTER(ctypes.c_longlong), ctypes.c_int,
@@ -248,13 +252,19 @@ class TiledFlashAttention:
 # ------------------------------------------------------------------------------ LSTM
 def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor | None = None,
          c0: torch.Tensor | None = None, algo: str = "auto", workspace: torch.Tensor | None = None,
-         out: tuple[torch.Tensor, torch.Tensor] | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+         out: tuple[torch.Tensor, torch.Tensor] | None = None, check: bool = True
+         ) -> tuple[torch.Tensor, torch.Tensor]:
     """Fused LSTM layer. x [T, B, I] f16, W [4H, I+H] f16 (gate rows i,f,g,o), bias [4H] f16,
     h0 [B, H] f16 / c0 [B, H] f32 (None = zeros). Returns (h_all [T, B, H] f16, c_T [B, H] f32).
 
     ``algo="hoisted"`` computes the input half of the gates for all steps in one GEMM first (``tcu_lstm_f16_ws``); it
     needs ``lstm_workspace_bytes(T, B, I, H)`` bytes of device memory, taken from ``workspace`` (any dtype) if given,
-    else allocated here. ``out`` = (h_all, c_T) tensors to write into instead of allocating them."""
+    else allocated here. ``out`` = (h_all, c_T) tensors to write into instead of allocating them.
+
+    ``algo="persistent"`` runs the whole time loop in one weight-stationary launch after the same GEMM
+    (``tcu_lstm_f16_persistent``: H = 1024, B <= 256 in multiples of 32; ``lstm_persistent_workspace_bytes``). Its
+    workgroups wait for each other with a time limit; with ``check=True`` (the default) the stream is synchronised and
+    a RuntimeError raised if a wait expired, ``check=False`` leaves that to a later ``lstm_persistent_status(workspace)``."""
     if x.dim() != 3 or W.dim() != 2:
         raise ValueError("x must be [T, B, I] and W [4H, I+H]")
     T, B, I = x.shape
@@ -272,6 +282,20 @@ def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor 
         h_all, c_out = out
         if tuple(h_all.shape) != (T, B, H) or tuple(c_out.shape) != (B, H):
             raise ValueError(f"out must be (h_all [{T}, {B}, {H}], c_T [{B}, {H}])")
+    if algo == "persistent":
+        need = lstm_persistent_workspace_bytes(T, B, I, H)
+        if workspace is None:
+            workspace = torch.empty(max(need, 4096), dtype=torch.uint8, device=x.device)
+        if not workspace.is_cuda or not workspace.is_contiguous():
+            raise ValueError("workspace must be a contiguous device tensor")
+        _check(lib().tcu_lstm_f16_persistent(_dev_ptr(x, torch.float16, "x"), _dev_ptr(W, torch.float16, "W"),
+                                             _dev_ptr(bias, torch.float16, "bias"), _dev_ptr(h0, torch.float16, "h0"),
+                                             _dev_ptr(c0, torch.float32, "c0"), _dev_ptr(h_all, torch.float16, "h_all"),
+                                             _dev_ptr(c_out, torch.float32, "c_out"), T, B, I, H, workspace.data_ptr(),
+                                             workspace.numel() * workspace.element_size(), _stream()))
+        if check:
+            lstm_persistent_status(workspace)
+        return h_all, c_out
     if algo == "hoisted":
         need = lstm_workspace_bytes(T, B, I, H)
         if workspace is None:
@@ -294,6 +318,17 @@ def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor 
 def lstm_workspace_bytes(T: int, B: int, I: int, H: int) -> int:
     """Device bytes ``lstm(..., algo="hoisted")`` needs; 0 if that path is not instantiated for the shape."""
     return int(lib().tcu_lstm_workspace_bytes(T, B, I, H))
+
+
+def lstm_persistent_workspace_bytes(T: int, B: int, I: int, H: int) -> int:
+    """Device bytes ``lstm(..., algo="persistent")`` needs; 0 if that path does not take the shape."""
+    return int(lib().tcu_lstm_persistent_workspace_bytes(T, B, I, H))
+
+
+def lstm_persistent_status(workspace: torch.Tensor) -> None:
+    """Synchronise the current stream and raise RuntimeError if the last ``lstm(..., algo="persistent")`` call that used
+    ``workspace`` gave up a wait (its outputs are then invalid)."""
+    _check(lib().tcu_lstm_persistent_status(workspace.data_ptr(), _stream()))
 
 
 # ------------------------------------------------------------------------------ scatter_nd

@@ -1,6 +1,7 @@
 // Implementation of the C-ABI declared in include/tcu_c_api.h: argument checks, shape
 // dispatch and kernel launches. No device memory is allocated here and no stream is
-// synchronised; errors become status codes plus a thread-local message.
+// synchronised (but for tcu_lstm_persistent_status, whose purpose it is); errors become status codes plus a
+// thread-local message.
 #include "tcu_c_api.h"
 
 #include "kernels/b2b_gemm_fwd.hpp"
@@ -10,9 +11,11 @@
 #include "kernels/gemm_ragged.hpp"
 #include "kernels/gemm_w128.hpp"
 #include "kernels/lstm_fwd.hpp"
+#include "kernels/lstm_recurrent.hpp"
 #include "kernels/mod.hpp"
 
 #include <climits>
+#include <cstdlib>
 #include <mutex>
 #include <set>
 #include <algorithm>
@@ -97,6 +100,7 @@ bool aligned16(std::initializer_list<const void*> v) {
 // the library runs on holds one copy of this array, at its own address, until the process ends. In host code the
 // array's name is only a handle for hipGetSymbolAddress, never a device address.
 constexpr unsigned long long kScratchBytes = 64ull << 20;
+constexpr unsigned long long kPersistentSyncBytes = 4096;  // synchronisation words in front of the pre-activations
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 constexpr int kMaxDevices = 64;
@@ -594,6 +598,72 @@ int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* 
     if (I == 1024 && H == 1024) return launch_lstm_hoisted<1024, 1024>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
     if (I == 128 && H == 128) return launch_lstm_hoisted<128, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
     return launch_lstm_hoisted<256, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
+}
+
+unsigned long long tcu_lstm_persistent_workspace_bytes(int T, int B, int I, int H) {
+    using Traits = LstmRecurrentTraits<1024>;
+    if (T <= 0 || B <= 0 || I <= 0 || H != Traits::kH) return 0;
+    if (B % Traits::kRows != 0 || B > Traits::kRows * Traits::kXcds || I % 64 != 0) return 0;
+    if ((long)T * B % 256 != 0 || (long)T * B > INT_MAX) return 0;
+    return kPersistentSyncBytes + (unsigned long long)T * B * 4 * H * sizeof(float);
+}
+
+int tcu_lstm_f16_persistent(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                            void* c_out, int T, int B, int I, int H, void* workspace, unsigned long long workspace_bytes,
+                            void* stream) {
+    using Traits = LstmRecurrentTraits<1024>;
+    if (!x || !W || !bias || !h_all || !c_out || !workspace)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: null pointer");
+    if (!positive({T, B, I, H})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: sizes must be positive");
+    if (!aligned16({x, W, bias, h0, c0, h_all, c_out}) || reinterpret_cast<uintptr_t>(workspace) % 1024 != 0)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: operands must be 16-byte aligned, the workspace 1 KiB-aligned");
+    const unsigned long long need = tcu_lstm_persistent_workspace_bytes(T, B, I, H);
+    if (need == 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_persistent: needs H == 1024, I % 64 == 0, B % 32 == 0, B <= 256 "
+                                               "and T * B % 256 == 0");
+    if (workspace_bytes < need)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: workspace smaller than tcu_lstm_persistent_workspace_bytes()");
+    // one workgroup per CU, all resident at once, 32 per XCD: the grid is the chip
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
+        return fail(TCU_ERR_NO_DEVICE, "tcu_lstm_f16_persistent: no current HIP device");
+    if (cus != Traits::kGrid)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_persistent: written for a device of 256 CUs in 8 XCDs; this one has " +
+                                                   std::to_string(cus) + " CUs");
+    unsigned long long spin_us = 2000000;  // a wait is microseconds when every workgroup is resident
+    unsigned int peers = Traits::kCusPerXcd;
+    if (const char* e = std::getenv("TCU_LSTM_PERSISTENT_SPIN_US")) spin_us = std::strtoull(e, nullptr, 10);
+    if (const char* e = std::getenv("TCU_LSTM_PERSISTENT_PEERS")) peers = unsigned(std::strtoul(e, nullptr, 10));
+    auto s = static_cast<hipStream_t>(stream);
+    auto sync = static_cast<unsigned int*>(workspace);
+    auto pre = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + kPersistentSyncBytes);
+    auto xp = static_cast<const __half*>(x), wp = static_cast<const __half*>(W);
+    int rc = launch(&lstm_recurrent_clear_sync, dim3(1), dim3(Traits::kSyncWords), 0, s, sync);
+    if (rc != TCU_OK) return rc;
+    rc = gemm_w128_dispatch<float>(xp, wp, pre, T * B, 4 * H, I, s, I, I + H);
+    if (rc != TCU_OK) return rc;
+    return launch(&lstm_recurrent_xcd<Traits>, dim3(Traits::kGrid), dim3(Traits::kThreads), Traits::kLdsBytes, s,
+                  static_cast<const float*>(pre), wp, I + H, I, static_cast<const __half*>(bias),
+                  static_cast<const __half*>(h0), static_cast<const float*>(c0), static_cast<__half*>(h_all),
+                  static_cast<float*>(c_out), T, B, sync, spin_us * 100ull, peers);
+}
+
+int tcu_lstm_persistent_status(const void* workspace, void* stream) {
+    if (!workspace) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_persistent_status: null pointer");
+    auto s = static_cast<hipStream_t>(stream);
+    unsigned int word = 0;
+    hipError_t e = hipStreamSynchronize(s);
+    if (e == hipSuccess)
+        e = hipMemcpy(&word, static_cast<const unsigned int*>(workspace) + LstmRecurrentTraits<1024>::kErrorWord, sizeof(word),
+                      hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return fail(TCU_ERR_HIP, std::string("tcu_lstm_persistent_status: ") + hipGetErrorString(e));
+    if (word == 1)
+        return fail(TCU_ERR_INCOMPLETE, "tcu_lstm_f16_persistent: workgroups that exchange h through an L2 were placed on different XCDs; the outputs are invalid");
+    if (word != 0)
+        return fail(TCU_ERR_INCOMPLETE, "tcu_lstm_f16_persistent: a workgroup waited for its XCD longer than the limit (the grid "
+                                    "was not resident at once); the outputs are invalid");
+    return TCU_OK;
 }
 
 unsigned long long tcu_lstm_noalloc_max_bytes(void) { return kScratchBytes; }
