@@ -113,9 +113,43 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int unit0 = slot * Traits::kUnitsPerCu + wave * Traits::kUnitsPerWave;
     f16x8 wf[Traits::kKSteps];
     {
-        const __half* wrow = W + size_t((frow >> 3) * kH + unit0 + (frow & 7)) * ldw + w_col0 + 8 * fhalf;
+        // A lane's share of a fragment is 16 bytes of one weight row, so loading fragments straight from memory asks
+        // for 32-byte pieces of 32 rows per instruction; instead the wavefront's 32 rows x 2 KiB pass through its
+        // quarter of the LDS (not yet in use) in 8 chunks of 32 rows x 256 B (8 k-steps), loaded directly to LDS in
+        // runs of 256 contiguous bytes (4 rows per instruction), two chunks in flight, and read back as fragments.
+        // Physical 16-byte chunk p of row r holds logical chunk p ^ (r % 16) (conflict-free ds_read_b128).
+        constexpr int kChunks = Traits::kKSteps / 8, kChunkBytes = 32 * 256;
+        const unsigned int stage = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds)) + wave * (2 * kChunkBytes);
+        const int lr = lane >> 4, lc = lane & 15;
+        const __half* wsrc[8];  // this lane's source for load instruction q of a chunk: row 4 q + lr
 #pragma unroll
-        for (int ks = 0; ks < Traits::kKSteps; ++ks) wf[ks] = *reinterpret_cast<const f16x8*>(wrow + 16 * ks);
+        for (int q = 0; q < 8; ++q) {
+            const int n = 4 * q + lr;
+            wsrc[q] = W + size_t((n >> 3) * kH + unit0 + (n & 7)) * ldw + w_col0 + (lc ^ (n & 15)) * 8;
+        }
+        auto issue_chunk = [&](int c) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+                detail::load_lds_16B_untracked_sc1(wsrc[q] + c * 128,
+                                                   __builtin_amdgcn_readfirstlane(stage + (c & 1) * kChunkBytes + q * 1024));
+        };
+        issue_chunk(0);
+        issue_chunk(1);
+        using lds_ptr = __attribute__((address_space(3))) const f16x8*;
+#pragma unroll
+        for (int c = 0; c < kChunks; ++c) {
+            // chunk c has landed when at most the 8 loads of chunk c + 1 are outstanding
+            if (c + 1 < kChunks) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int s = 0; s < 8; ++s)
+                wf[8 * c + s] = *reinterpret_cast<lds_ptr>(stage + (c & 1) * kChunkBytes + frow * 256 +
+                                                           (((2 * s + fhalf) ^ (frow & 15)) * 16));
+            if (c + 2 < kChunks) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are done before the buffer is refilled
+                issue_chunk(c + 2);
+            }
+        }
         // into the AGPR half, where the MFMAs below take them from
 #pragma unroll
         for (int ks = 0; ks < Traits::kKSteps; ++ks) asm volatile("" : "+a"(wf[ks]));
