@@ -395,6 +395,27 @@ def test_flash_attention_growing_maxima(tcu, oracle, device, algo, D, q_gain, k_
     assert oracle.max_abs_err(host(O), ref) <= tol
 
 
+@pytest.mark.parametrize("q_gain,bound_tile,bound_tuned", [(1.0, 3e-4, 3e-4), (3.0, 1.5e-3, 3e-3), (6.0, 1.5e-3, 7e-3)])
+def test_flash_attention_prescaled_q_precision(tcu, oracle, device, q_gain, bound_tile, bound_tuned):
+    """The tuned kernels multiply Q by scale * log2(e) and round it to f16 *before* the score MFMAs (a relative error
+    of 2^-11 on every product term, so the error of a logit grows with its magnitude); the tile-library kernel, like
+    the reference, scales the f32 scores. Each path gets its own bound (about 1.6 x what is measured), at logits up to
+    about +-5, +-14 and +-29, so that a regression of either is visible: measured 1.4e-4 / 1.2e-4, 9.6e-4 / 1.7e-3,
+    9.9e-4 / 4.4e-3 (tile library / tuned)."""
+    import torch
+
+    batch, M, N, D = 2, 256, 1024, 128
+    q = (oracle.fill_normal(batch * M * D, 71).reshape(batch, M, D).astype(np.float32) * q_gain).astype(np.float16)
+    k = oracle.fill_normal(batch * N * D, 72).reshape(batch, N, D)
+    v = oracle.fill_normal(batch * N * D, 73).reshape(batch, N, D)
+    ref = oracle.attention(q, k, v, 1.0 / math.sqrt(D))
+    for algo in ("tile_library", "mfma32", "mfma32_fused", "wave64"):
+        O = tcu.flash_attention(dev(q, device), dev(k, device), dev(v, device), algo=algo)
+        torch.cuda.synchronize()
+        err = oracle.max_abs_err(host(O), ref)
+        assert err <= (bound_tile if algo == "tile_library" else bound_tuned), (algo, err)
+
+
 @pytest.mark.parametrize("algo", ["tile_library", "mfma32", "mfma32_fused"])
 @pytest.mark.parametrize("batch,M,N,D", [(1, 64, 64, 128), (3, 128, 192, 128), (2, 256, 512, 128), (2, 128, 256, 64),
                                          (1, 512, 1024, 128), (2, 192, 64, 64)])
