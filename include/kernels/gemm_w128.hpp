@@ -81,9 +81,32 @@ DEVICE void load_lds_16B_sbase(unsigned int voff, const void* sbase, unsigned in
 
 }  // namespace detail
 
-/// grid = (M / 256) * (N / 256), block = 256, dynamic LDS = GemmW128Traits::kLdsBytes.
+/// C[i] = sum over z of partial[z][i] (f32 partial sums of a split-K product), 4 elements per lane. n % 4 == 0.
+template <typename OutType>
+__global__ void __launch_bounds__(256) splitk_reduce(const float* __restrict__ partial, OutType* __restrict__ C,
+                                                     size_t n, int splits) {
+    const size_t i = (size_t(blockIdx.x) * 256 + threadIdx.x) * 4;
+    if (i >= n) return;
+    f32x4 acc = *reinterpret_cast<const f32x4*>(partial + i);
+    for (int z = 1; z < splits; ++z) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(partial + size_t(z) * n + i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += v[e];
+    }
+    if constexpr (sizeof(OutType) == 4) {
+        *reinterpret_cast<f32x4*>(C + i) = acc;
+    } else {
+        f16x4 h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[e]);
+        *reinterpret_cast<f16x4*>(C + i) = h;
+    }
+}
+
+/// grid = ((M / 256) * (N / 256), splits), block = 256, dynamic LDS = GemmW128Traits::kLdsBytes.
 /// lda / ldb: elements between consecutive rows of A / of the stored [N, K] array (K for dense operands; larger when
-/// the operand is a column block of a wider matrix). C is dense.
+/// the operand is a column block of a wider matrix). C is dense. With splits > 1 workgroup row z multiplies the
+/// K-range [z K, (z + 1) K) and writes plane z of C ([splits, M, N]; partial sums for splitk_reduce).
 template <typename OutType>
 __global__ void __launch_bounds__(GemmW128Traits::kThreads)
     gemm_w128(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
@@ -108,8 +131,12 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
         voff[q] = static_cast<unsigned int>(row) * static_cast<unsigned int>(q < 8 ? lda : ldb) * 2u +
                   (lchk ^ ((row >> 1) & 7)) * 16;
     }
-    const __half* a_base = A + size_t(m0) * lda;
-    const __half* b_base = Bt + size_t(n0) * ldb;
+    // blockIdx.y = z selects the z-th K-range of length K of wider operands (split-K: lda, ldb >= gridDim.y * K) and
+    // the z-th [M, N] plane of C; an ordinary launch has gridDim.y == 1
+    const size_t z = blockIdx.y;
+    const __half* a_base = A + size_t(m0) * lda + z * K;
+    const __half* b_base = Bt + size_t(n0) * ldb + z * K;
+    C += z * size_t(M) * N;
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
     auto load_dst = [&](int stage, int q) -> unsigned int {
         return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +

@@ -120,6 +120,36 @@ def test_gemm_ragged_shapes(tcu, oracle, device, M, N, K, out_dtype):
         assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
 
 
+@pytest.mark.parametrize("M,N,K,splits", [(1024, 1024, 8192, 16), (512, 512, 4096, 8), (256, 256, 1024, 2),
+                                          (1024, 2048, 2048, 4), (256, 512, 64 * 24, 2), (256, 512, 512, 1), (2048, 2048, 2048, 1)])
+@pytest.mark.parametrize("out_dtype", ["f32", "f16"])
+def test_gemm_split_k_with_workspace(tcu, oracle, device, M, N, K, splits, out_dtype):
+    """tcu_gemm_f16_ws: few output tiles and a long K are split over K (f32 partial products in the caller's workspace,
+    then a reduction); against the oracle and against the unsplit kernel; the workspace size is splits * M * N * 4, bytes
+    past it stay untouched; shapes that are not split (last two cases) take the ordinary path and need no workspace."""
+    import torch
+
+    print(f"gemm split-K {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    need = tcu.gemm_workspace_bytes(M, N, K)
+    assert need == (splits * M * N * 4 if splits > 1 else 0)
+    A = oracle.fill_uniform(M * K, 131 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 137 + N).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    ws = torch.full((need + 4096,), 0xFF, dtype=torch.uint8, device=device)
+    C = tcu.gemm(dA, dB, out_dtype=dt, workspace=ws)
+    torch.cuda.synchronize()
+    rows = slice(0, min(M, 192))
+    want = oracle.gemm(A[rows], Bt)
+    assert oracle.max_rel_err(host(C)[rows], want) <= REL_TOL
+    plain = tcu.gemm(dA, dB, out_dtype=dt)
+    assert oracle.max_rel_err(host(C), host(plain)) <= REL_TOL
+    assert bool((ws[need:] == 0xFF).all())
+    if splits > 1:
+        with pytest.raises(RuntimeError):
+            tcu.gemm(dA, dB, out_dtype=dt, workspace=ws[:need // 2])
+
+
 def test_gemm_wave128_rejects_other_shapes(tcu, device):
     import torch
 

@@ -17,7 +17,7 @@ import os
 import torch
 
 __all__ = [
-    "TcuError", "library_path", "lib", "last_error", "gemm", "b2b_gemm", "flash_attention_fwd",
+    "TcuError", "library_path", "lib", "last_error", "gemm", "gemm_workspace_bytes", "b2b_gemm", "flash_attention_fwd",
     "flash_attention", "TiledFlashAttention", "lstm", "lstm_workspace_bytes", "lstm_persistent_workspace_bytes", "lstm_persistent_status", "scatter_nd", "GEMM_ALGOS", "ATTN_ALGOS", "LSTM_ALGOS", "B2B_ALGOS",
     "SCATTER_MODES",
 ]
@@ -51,6 +51,9 @@ _SIGNATURES = {
     "tcu_last_error": (ctypes.c_char_p, []),
     "tcu_device_count": (ctypes.c_int, []),
     "tcu_gemm_f16": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int] * 5 + [ctypes.c_void_p]),
+    "tcu_gemm_workspace_bytes": (ctypes.c_ulonglong, [ctypes.c_int] * 3),
+    "tcu_gemm_f16_ws": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_ulonglong,
+                                                                                  ctypes.c_void_p]),
     "tcu_b2b_gemm_f16": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 6 + [ctypes.c_void_p]),
     "tcu_b2b_gemm_f16_algo": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7 + [ctypes.c_void_p]),
     "tcu_flash_attn_fwd_f16": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int,
@@ -138,10 +141,12 @@ def _out_code(dtype: torch.dtype) -> int:
 
 # ------------------------------------------------------------------------------ GEMM
 def gemm(a: torch.Tensor, b_t: torch.Tensor, out: torch.Tensor | None = None,
-         out_dtype: torch.dtype = torch.float16, algo: str = "auto") -> torch.Tensor:
+         out_dtype: torch.dtype = torch.float16, algo: str = "auto", workspace: torch.Tensor | None = None) -> torch.Tensor:
     """C[M, N] = A[M, K] · B with B column-major, i.e. ``b_t`` is the [N, K] array (``a @ b_t.T``).
 
-    Mirrors the reference's GEMM examples (A row-major, B column-major, f32 accumulate).
+    Mirrors the reference's GEMM examples (A row-major, B column-major, f32 accumulate). With ``workspace`` (a
+    contiguous device tensor of at least ``gemm_workspace_bytes(M, N, K)`` bytes; ``algo`` must be "auto") a product
+    with few output tiles and a long K is split over K (``tcu_gemm_f16_ws``).
     """
     M, K = a.shape
     N, K2 = b_t.shape
@@ -151,10 +156,24 @@ def gemm(a: torch.Tensor, b_t: torch.Tensor, out: torch.Tensor | None = None,
         out = torch.empty(M, N, dtype=out_dtype, device=a.device)
     elif tuple(out.shape) != (M, N):
         raise ValueError("out has the wrong shape")
+    if workspace is not None:
+        if algo != "auto":
+            raise ValueError("a workspace goes with algo='auto'")
+        if not workspace.is_cuda or not workspace.is_contiguous():
+            raise ValueError("workspace must be a contiguous device tensor")
+        _check(lib().tcu_gemm_f16_ws(_dev_ptr(a, torch.float16, "a"), _dev_ptr(b_t, torch.float16, "b_t"),
+                                     _dev_ptr(out, out.dtype, "out"), M, N, K, _out_code(out.dtype), workspace.data_ptr(),
+                                     workspace.numel() * workspace.element_size(), _stream()))
+        return out
     _check(lib().tcu_gemm_f16(_dev_ptr(a, torch.float16, "a"), _dev_ptr(b_t, torch.float16, "b_t"),
                               _dev_ptr(out, out.dtype, "out"), M, N, K, _out_code(out.dtype), GEMM_ALGOS[algo],
                               _stream()))
     return out
+
+
+def gemm_workspace_bytes(M: int, N: int, K: int) -> int:
+    """Device bytes ``gemm(..., workspace=...)`` uses for a split over K; 0 when the product is not split."""
+    return int(lib().tcu_gemm_workspace_bytes(M, N, K))
 
 
 # ------------------------------------------------------------------------------ b2b GEMM

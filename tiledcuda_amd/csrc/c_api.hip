@@ -209,6 +209,33 @@ int gemm_tile_pipelined_dispatch(const __half* A, const __half* B, OutType* C, i
                                            "and 256x256x64");
 }
 
+/// Number of K-ranges a product is split into when the caller brings a workspace: 1 unless 256 x 256 tiles would
+/// leave most of the chip idle (at most 32 tiles) and K is long enough to give every workgroup at least 512 of it.
+int gemm_split_count(int M, int N, int K) {
+    using T = GemmW128Traits;
+    if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0) return 1;
+    const long tiles = (long)(M / T::kBM) * (N / T::kBN);
+    if (tiles > 32) return 1;
+    int s = 1;
+    while (2 * s * tiles <= 256 && K % (2 * s * T::kBK) == 0 && K / (2 * s) >= 512) s *= 2;
+    return s;
+}
+
+template <typename OutType>
+int gemm_splitk(const __half* A, const __half* B, OutType* C, int M, int N, int K, int splits, float* partial,
+                hipStream_t stream) {
+    using T = GemmW128Traits;
+    if ((long)K * 2 * T::kBM >= (1l << 32))
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
+    const int tiles = (M / T::kBM) * (N / T::kBN);
+    int rc = launch(&gemm_w128<float>, dim3(tiles, splits), dim3(T::kThreads), T::kLdsBytes, stream, A, B, partial, M, N,
+                    K / splits, K, K);
+    if (rc != TCU_OK) return rc;
+    const size_t n = size_t(M) * N;
+    return launch(&splitk_reduce<OutType>, dim3(unsigned((n / 4 + 255) / 256)), dim3(256), 0, stream,
+                  static_cast<const float*>(partial), C, n, splits);
+}
+
 template <typename OutType>
 int gemm_ragged_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
     using T = RaggedGemmTraits;
@@ -488,6 +515,29 @@ int tcu_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K, int
         return gemm_dispatch<__half>(a, b, static_cast<__half*>(C), M, N, K, algo, s);
     }
     return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16: out_dtype must be TCU_DTYPE_F32 or TCU_DTYPE_F16");
+}
+
+unsigned long long tcu_gemm_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const int splits = gemm_split_count(M, N, K);
+    return splits > 1 ? (unsigned long long)splits * M * N * sizeof(float) : 0;
+}
+
+int tcu_gemm_f16_ws(const void* A, const void* B, void* C, int M, int N, int K, int out_dtype, void* workspace,
+                    unsigned long long workspace_bytes, void* stream) {
+    const unsigned long long need = (M > 0 && N > 0 && K > 0) ? tcu_gemm_workspace_bytes(M, N, K) : 0;
+    if (need == 0 || !workspace) return tcu_gemm_f16(A, B, C, M, N, K, out_dtype, TCU_GEMM_AUTO, stream);
+    if (!A || !B || !C) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16_ws: null pointer");
+    if (!aligned16({A, B, C, workspace})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16_ws: operands must be 16-byte aligned");
+    if (workspace_bytes < need)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16_ws: workspace smaller than tcu_gemm_workspace_bytes()");
+    auto a = static_cast<const __half*>(A), b = static_cast<const __half*>(B);
+    auto s = static_cast<hipStream_t>(stream);
+    auto ws = static_cast<float*>(workspace);
+    const int splits = gemm_split_count(M, N, K);
+    if (out_dtype == TCU_DTYPE_F32) return gemm_splitk<float>(a, b, static_cast<float*>(C), M, N, K, splits, ws, s);
+    if (out_dtype == TCU_DTYPE_F16) return gemm_splitk<__half>(a, b, static_cast<__half*>(C), M, N, K, splits, ws, s);
+    return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16_ws: out_dtype must be TCU_DTYPE_F32 or TCU_DTYPE_F16");
 }
 
 int tcu_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D, int M, int N, int K, int P, int batch,
