@@ -1,7 +1,7 @@
 """Benchmark of the tile-kernel hot path on one MI355X.
 
 One "step" is one launch of the headline workload: the fp16 GEMM M=N=K=4096 (A row-major,
-B column-major, f32 accumulate, f16 output), inputs resident in HBM. The other BASELINE
+B column-major, f32 accumulate, f16 output), inputs resident in HBM. The other benchmark
 configurations (GEMM 128x64x256, back-to-back GEMM, FlashAttention-2 forward, fused LSTM)
 are timed in the same run and reported under "configs".
 

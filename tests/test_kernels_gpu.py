@@ -1,7 +1,7 @@
 """Parity tests of the kernel entries, through the C-ABI (ctypes), against the CPU oracle on
 the same seeded inputs.
 
-Tolerances (BASELINE): GEMM / back-to-back GEMM max relative error <= 1e-3 against the
+Tolerances of the benchmark specification: GEMM / back-to-back GEMM max relative error <= 1e-3 against the
 f32-accumulated oracle, where "relative" is |x - ref| / max(|ref|, eps * rms(ref)) (outputs of a
 K-long dot product land arbitrarily close to zero, so a plain elementwise ratio is meaningless).
 eps = 0.01 for the single GEMM. eps = 1 for the back-to-back GEMM: its f16-rounded
