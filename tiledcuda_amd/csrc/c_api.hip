@@ -351,6 +351,16 @@ int launch_fa(const __half* Q, const __half* K, const __half* V, __half* O, int 
                   scale);
 }
 
+template <int kNStatic, int kD, bool kVRowMajor, int kTM, int kTN, typename WarpLayout>
+int launch_fa_pipelined(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
+                        hipStream_t stream) {
+    using Traits = FlashAttentionTraits<__half, float, __half, FlashAttentionShape<0, kNStatic, kD, kD>,
+                                        FlashAttentionShape<kTM, kTN, kD, kD>, kVRowMajor, WarpLayout>;
+    auto kernel = &flash_attention_pipelined<__half, __half, Traits>;
+    return launch(kernel, dim3(M / kTM, 1, batch), dim3(Traits::kThreads), Traits::kShmBytesPipelined, stream, Q, K, V, O,
+                  M, N, scale);
+}
+
 template <int kD, int kWaves, bool kFused>
 int launch_fa_fwd(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
                   hipStream_t stream) {
@@ -407,8 +417,10 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     if (algo == TCU_ATTN_MFMA32 || algo == TCU_ATTN_MFMA32_FUSED)
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 32x32x16 attention kernels take a row-major V");
     if (v_layout == TCU_V_ROW_MAJOR) {
-        if (Kd == 128) return launch_fa<0, 128, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
-        if (Kd == 64) return launch_fa<0, 64, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+        // row-major V: the double-buffered composition (direct-to-LDS ring); 32 query rows per wavefront where M allows
+        if (Kd == 128 && M % 128 == 0) return launch_fa_pipelined<0, 128, true, 128, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+        if (Kd == 128) return launch_fa_pipelined<0, 128, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
+        if (Kd == 64) return launch_fa_pipelined<0, 64, true, 64, 64, W41>(Q, K, V, O, batch, M, N, scale, stream);
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
     }
     // column-major V (the reference op's convention), any N % 64 == 0
