@@ -73,11 +73,15 @@ typedef enum {
                                   neighbouring 32; row-major V, head size 128, M % 256 == 0 */
 } tcu_attn_algo;
 
-/* Which LSTM step kernel to run (tcu_lstm_f16_algo). AUTO picks STREAMING. */
+/* Which LSTM step kernel to run (tcu_lstm_f16_algo). AUTO picks STREAMING where it is instantiated, else
+ * TILE_LIBRARY, else RAGGED: every B, I, H in multiples of 16 is accepted. */
 typedef enum {
     TCU_LSTM_AUTO = 0,
-    TCU_LSTM_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, single LDS stage */
-    TCU_LSTM_STREAMING = 2     /* 32x32x16 MFMA, multi-stage direct-to-LDS ring, k split over two wavefront groups */
+    TCU_LSTM_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, single LDS stage; (I, H) in {(1024,1024),
+                                  (128,128), (64,128)}, B % 64 == 0 */
+    TCU_LSTM_STREAMING = 2,    /* 32x32x16 MFMA, multi-stage direct-to-LDS ring, k split over two wavefront groups;
+                                  (I, H) in {(1024,1024), (128,128), (256,128)}, B % 64 == 0 */
+    TCU_LSTM_RAGGED = 3        /* run-time B, I, H in multiples of 16: MFMA operand tiles filled from global memory */
 } tcu_lstm_algo;
 
 /* Library version (major * 10000 + minor * 100 + patch). */

@@ -683,6 +683,44 @@ def test_lstm_hoisted_rejects_what_it_cannot_do(tcu, device):
         tcu.lstm(x[:3].contiguous(), W, b, algo="hoisted")
 
 
+@pytest.mark.parametrize("T,B,I,H", [(3, 16, 16, 16), (2, 48, 80, 112), (4, 32, 256, 64), (2, 64, 144, 272), (1, 80, 1024, 48)])
+@pytest.mark.parametrize("with_state", [False, True])
+def test_lstm_any_shape_of_whole_tiles(tcu, oracle, device, T, B, I, H, with_state):
+    """Every B, I, H in multiples of 16 runs (the granularity of the tile types): AUTO routes shapes no tuned kernel is
+    instantiated for to the run-time-shape step kernel; k ranges that end in a half-filled 32-wide operand tile, hidden
+    sizes that leave wavefronts of the last workgroup without work, batches that are not multiples of 64."""
+    import torch
+
+    print(f"lstm ragged T{T} B{B} I{I} H{H} state={with_state}", flush=True)
+    x = oracle.fill_normal(T * B * I, 81, 0, 0.5).reshape(T, B, I)
+    W = oracle.fill_normal(4 * H * (I + H), 82, 0, 0.1).reshape(4 * H, I + H)
+    b = oracle.fill_normal(4 * H, 83, 0, 0.1)
+    h0 = oracle.fill_normal(B * H, 84, 0, 0.5).reshape(B, H) if with_state else None
+    c0 = oracle.fill_normal(B * H, 85, 0, 0.5).reshape(B, H).astype(np.float32) if with_state else None
+    h_ref, c_ref = oracle.lstm(x, W, b, h0, c0)
+    for algo in ("auto", "ragged"):
+        h_all, c_T = tcu.lstm(dev(x, device), dev(W, device), dev(b, device),
+                              dev(h0, device) if with_state else None, dev(c0, device) if with_state else None, algo=algo)
+        torch.cuda.synchronize()
+        assert oracle.max_abs_err(host(h_all), h_ref) <= ABS_TOL
+        assert oracle.max_abs_err(host(c_T), c_ref) <= ABS_TOL
+
+
+def test_lstm_ragged_matches_streaming_kernel(tcu, device):
+    """Where both exist, the run-time-shape kernel and the streaming kernel agree to the order of the f32 summation."""
+    import torch
+
+    T, B, I, H = 3, 64, 256, 128
+    g = torch.Generator(device="cpu").manual_seed(9)
+    x = (torch.randn(T, B, I, generator=g) * 0.5).half().to(device)
+    W = (torch.randn(4 * H, I + H, generator=g) * 0.1).half().to(device)
+    b = (torch.randn(4 * H, generator=g) * 0.1).half().to(device)
+    h_a, c_a = tcu.lstm(x, W, b, algo="streaming")
+    h_b, c_b = tcu.lstm(x, W, b, algo="ragged")
+    assert float((h_a.float() - h_b.float()).abs().max()) <= 2e-3
+    assert float((c_a - c_b).abs().max()) <= 2e-3
+
+
 def test_lstm_zero_weights_closed_form(tcu, device):
     """W = 0: c_t = sigmoid(b_f) c_{t-1} + sigmoid(b_i) tanh(b_g), h_t = sigmoid(b_o) tanh(c_t)."""
     import torch

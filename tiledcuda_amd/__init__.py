@@ -41,7 +41,7 @@ TCU_V_COL_MAJOR = 0
 TCU_V_ROW_MAJOR = 1
 
 ATTN_ALGOS = {"auto": 0, "tile_library": 1, "mfma32": 2, "mfma32_fused": 3, "wave64": 4}
-LSTM_ALGOS = {"auto": 0, "tile_library": 1, "streaming": 2}
+LSTM_ALGOS = {"auto": 0, "tile_library": 1, "streaming": 2, "ragged": 3}
 B2B_ALGOS = {"auto": 0, "tile_library": 1, "resident": 2}
 SCATTER_MODES = {"assign": 0, "add": 1}
 

@@ -11,6 +11,7 @@
 #include "kernels/gemm_ragged.hpp"
 #include "kernels/gemm_w128.hpp"
 #include "kernels/lstm_fwd.hpp"
+#include "kernels/lstm_ragged.hpp"
 #include "kernels/lstm_recurrent.hpp"
 #include "kernels/mod.hpp"
 
@@ -481,6 +482,22 @@ int launch_lstm_hoisted(const __half* x, const __half* W, const __half* bias, co
     return TCU_OK;
 }
 
+int launch_lstm_ragged(const __half* x, const __half* W, const __half* bias, const __half* h0, const float* c0,
+                       __half* h_all, float* c_out, int T, int B, int I, int H, hipStream_t stream) {
+    using Traits = RaggedLstmTraits;
+    const dim3 grid((H + Traits::kUnits - 1) / Traits::kUnits, B / Traits::kRows);
+    for (int t = 0; t < T; ++t) {
+        const __half* x_t = x + size_t(t) * B * I;
+        const __half* h_in = t == 0 ? h0 : h_all + size_t(t - 1) * B * H;
+        const float* c_in = t == 0 ? c0 : c_out;
+        __half* h_out = h_all + size_t(t) * B * H;
+        int rc = launch(&lstm_cell_ragged, grid, dim3(Traits::kThreads), 0, stream, x_t, h_in, W, bias, c_in, c_out, h_out,
+                        B, I, H);
+        if (rc != TCU_OK) return lstm_step_failed(rc, t, T);
+    }
+    return TCU_OK;
+}
+
 template <int kI, int kH>
 int launch_lstm_fwd(const __half* x, const __half* W, const __half* bias, const __half* h0, const float* c0,
                     __half* h_all, float* c_out, int T, int B, hipStream_t stream) {
@@ -605,29 +622,34 @@ int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void
     auto c0p = static_cast<const float*>(c0);
     auto hp = static_cast<__half*>(h_all);
     auto cp = static_cast<float*>(c_out);
-    if (B % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16: batch must be a multiple of 64");
     if (long(T) * B > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16: T * B exceeds the 32-bit row count");
-    if (algo != TCU_LSTM_AUTO && algo != TCU_LSTM_TILE_LIBRARY && algo != TCU_LSTM_STREAMING)
+    if (algo != TCU_LSTM_AUTO && algo != TCU_LSTM_TILE_LIBRARY && algo != TCU_LSTM_STREAMING && algo != TCU_LSTM_RAGGED)
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16: unknown algo");
-    if (algo != TCU_LSTM_TILE_LIBRARY) {
+    if (B % 16 != 0 || I % 16 != 0 || H % 16 != 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16: shapes are whole 16 x 16 tiles: B, I and H must be multiples of 16");
+    if (algo == TCU_LSTM_RAGGED) return launch_lstm_ragged(xp, wp, bp, h0p, c0p, hp, cp, T, B, I, H, s);
+    const bool b64 = B % 64 == 0;
+    if (algo != TCU_LSTM_TILE_LIBRARY && b64) {
         if (I == 1024 && H == 1024) return launch_lstm_fwd<1024, 1024>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
         if (I == 128 && H == 128) return launch_lstm_fwd<128, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
         if (I == 256 && H == 128) return launch_lstm_fwd<256, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
-        if (algo == TCU_LSTM_STREAMING)
-            return fail(TCU_ERR_UNSUPPORTED_SHAPE,
-                        "the streaming LSTM kernel is instantiated for (I, H) in {(1024,1024), (128,128), (256,128)}");
     }
-    if (I == 1024 && H == 1024)
-        return launch_lstm<1024, 1024, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
-    if (I == 128 && H == 128)
-        return launch_lstm<128, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
-    if (I == 64 && H == 128)
-        return launch_lstm<64, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
-    return fail(TCU_ERR_UNSUPPORTED_SHAPE,
-                algo == TCU_LSTM_TILE_LIBRARY
-                    ? "the tile-library LSTM kernel is instantiated for (I, H) in {(1024,1024), (128,128), (64,128)}"
-                    : "tcu_lstm_f16 is instantiated for (I, H) in {(1024,1024), (128,128), (256,128)} (streaming "
-                      "kernel) and (64,128) (tile-library kernel)");
+    if (algo == TCU_LSTM_STREAMING)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE,
+                    "the streaming LSTM kernel is instantiated for (I, H) in {(1024,1024), (128,128), (256,128)}, B % 64 == 0");
+    if (b64) {
+        if (I == 1024 && H == 1024)
+            return launch_lstm<1024, 1024, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+        if (I == 128 && H == 128)
+            return launch_lstm<128, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+        if (I == 64 && H == 128)
+            return launch_lstm<64, 128, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+    }
+    if (algo == TCU_LSTM_TILE_LIBRARY)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE,
+                    "the tile-library LSTM kernel is instantiated for (I, H) in {(1024,1024), (128,128), (64,128)}, B % 64 == 0");
+    // every other shape made of whole 16 x 16 tiles: the run-time-shape kernel
+    return launch_lstm_ragged(xp, wp, bp, h0p, c0p, hp, cp, T, B, I, H, s);
 }
 
 unsigned long long tcu_lstm_workspace_bytes(int T, int B, int I, int H) {
