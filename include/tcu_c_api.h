@@ -155,9 +155,10 @@ int tcu_flash_attn_fwd_f16_algo(const void* Q, const void* K, const void* V, voi
  * order i, f, g, o, columns concat(x_t, h_{t-1}); bias [4H] f16; h0 [B, H] f16 or NULL (zeros);
  * c0 [B, H] f32 or NULL (zeros); h_all [T, B, H] f16 receives every h_t; c_out [B, H] f32
  * receives c_T (it is also the running cell state, so it must not alias c0 unless c0 == c_out).
- * One kernel per step (gate GEMM fused with the cell update). B must be a multiple of 64 and T * B fit in 31 bits.
- * Instantiated (I, H): streaming kernel (1024,1024), (128,128), (256,128); tile-library kernel (1024,1024), (128,128),
- * (64,128); AUTO takes the streaming kernel where it exists, else the tile-library one.
+ * One kernel per step (gate GEMM fused with the cell update). B, I and H must be multiples of 16 (whole tiles) and
+ * T * B fit in 31 bits. With B % 64 == 0 the streaming kernel is instantiated for (I, H) = (1024,1024), (128,128),
+ * (256,128) and the tile-library kernel for (1024,1024), (128,128), (64,128); AUTO takes the streaming kernel where it
+ * exists, else the tile-library one, else the run-time-shape kernel (TCU_LSTM_RAGGED), which takes every shape.
  * The reference snapshot has no LSTM entry (Makefile:3 names a test only).
  */
 int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
