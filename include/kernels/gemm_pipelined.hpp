@@ -132,7 +132,10 @@ HOST_DEVICE void xcd_tile_coords(int bid, int tiles_m, int tiles_n, int& tile_m,
 
 }  // namespace detail
 
-template <typename Traits, typename OutType>
+/// kEdges: M and N need not be multiples of the tile (multiples of 16 suffice): the grid covers ceil(M / kBM) x
+/// ceil(N / kBN) tiles, rows beyond the edge are loaded from the last valid row (their products are computed and
+/// dropped) and the stores are guarded. K % kBK == 0 in either case.
+template <typename Traits, typename OutType, bool kEdges = false>
 __global__ void __launch_bounds__(Traits::kThreads)
     gemm_pipelined(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N,
                    int K) {
@@ -147,7 +150,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int wave_n = wave % Traits::kWN;
 
     int tile_m, tile_n;
-    detail::xcd_tile_coords(blockIdx.x, M / kBM, N / kBN, tile_m, tile_n);
+    detail::xcd_tile_coords(blockIdx.x, kEdges ? (M + kBM - 1) / kBM : M / kBM, kEdges ? (N + kBN - 1) / kBN : N / kBN,
+                            tile_m, tile_n);
     const int m0 = tile_m * kBM;
     const int n0 = tile_n * kBN;
 
@@ -160,12 +164,14 @@ __global__ void __launch_bounds__(Traits::kThreads)
     auto a_src = [&](int j, int k0) -> const __half* {
         const int row = (wave * Traits::kALoads + j) * Traits::kRowsPerLoad + lrow;
         const int chunk = lchk ^ ((row >> 1) & 7);
-        return A + size_t(m0 + row) * K + k0 + chunk * 8;
+        const int grow = kEdges ? (m0 + row < M ? m0 + row : M - 1) : m0 + row;
+        return A + size_t(grow) * K + k0 + chunk * 8;
     };
     auto b_src = [&](int j, int k0) -> const __half* {
         const int row = (wave * Traits::kBLoads + j) * Traits::kRowsPerLoad + lrow;
         const int chunk = lchk ^ ((row >> 1) & 7);
-        return Bt + size_t(n0 + row) * K + k0 + chunk * 8;
+        const int grow = kEdges ? (n0 + row < N ? n0 + row : N - 1) : n0 + row;
+        return Bt + size_t(grow) * K + k0 + chunk * 8;
     };
     // Issue part `part` of `nparts` of the loads of one stage (A instructions first, then B). Splitting a stage's
     // loads over the k-substeps keeps the vector-memory path evenly busy instead of bursting after the barrier.
@@ -290,6 +296,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
             const int row = it * kRowsPerIter + rr;
             const int pslot = (2 * cc) ^ (((row & 15) << 1) & kSlotMask);
             const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kPitch + pslot * 8);
+            if (kEdges && (m0 + wave_m * kWaveM + row >= M || n0 + wave_n * kWaveN + cc * 8 >= N)) continue;
             *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(cbase + size_t(row) * N) + cc * 16) = v;
         }
     } else {
@@ -298,6 +305,9 @@ __global__ void __launch_bounds__(Traits::kThreads)
         for (int i = 0; i < kMT; ++i) {
 #pragma unroll
             for (int j = 0; j < kNT; ++j) {
+                if (kEdges && (m0 + wave_m * Traits::kWaveM + i * 16 + frow >= M ||
+                               n0 + wave_n * Traits::kWaveN + j * 16 + 4 * fquad >= N))
+                    continue;
                 *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * N + j * 16 + 4 * fquad) = acc[i][j];
             }
         }

@@ -150,6 +150,31 @@ def test_gemm_split_k_with_workspace(tcu, oracle, device, M, N, K, splits, out_d
             tcu.gemm(dA, dB, out_dtype=dt, workspace=ws[:need // 2])
 
 
+@pytest.mark.parametrize("M,N,K", [(80, 144, 64), (1040, 528, 256), (272, 4112, 128), (2064, 4080, 192), (4112, 4112, 64)])
+@pytest.mark.parametrize("out_dtype", ["f32", "f16"])
+def test_gemm_edge_tiles(tcu, oracle, device, M, N, K, out_dtype):
+    """M, N multiples of 16 but not of 64 with K % 64 == 0: AUTO runs the pipelined kernel with edge tiles (rows beyond
+    the edge loaded from the last valid row, stores guarded) in all three tile sizes; against the oracle on sampled rows
+    including the last ones, against the run-time-shape kernel everywhere, with guard bands around the output."""
+    import torch
+
+    print(f"gemm edge tiles {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    A = oracle.fill_uniform(M * K, 231 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 237 + N).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    guard = torch.full((M + 2, N), -7.0, dtype=dt, device=device)
+    out = guard[1:M + 1]
+    tcu.gemm(dA, dB, out=out, algo="auto")
+    torch.cuda.synchronize()
+    assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
+    rows = sorted(set(list(range(0, min(M, 48))) + list(range(max(0, M - 48), M))))
+    want = oracle.gemm(A[rows], Bt)
+    assert oracle.max_rel_err(host(out)[rows], want) <= REL_TOL
+    plain = tcu.gemm(dA, dB, out_dtype=dt, algo="ragged")
+    assert oracle.max_rel_err(host(out), host(plain)) <= REL_TOL
+
+
 def test_gemm_wave128_rejects_other_shapes(tcu, device):
     import torch
 

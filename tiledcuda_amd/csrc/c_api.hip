@@ -163,6 +163,21 @@ using PipeLarge = PipelinedGemmTraits<256, 256, 64, 4, 2, 2>;  // 8 wavefronts, 
 using PipeMid = PipelinedGemmTraits<128, 128, 64, 2, 2, 2>;
 using PipeSmall = PipelinedGemmTraits<64, 64, 64, 2, 2, 2>;
 
+/// M, N any multiples of 16 (K % 64 == 0): the pipelined kernel with edge tiles, the tile size chosen as for whole tiles.
+template <typename OutType>
+int gemm_pipelined_edges_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    auto go = [&](auto traits) {
+        using Traits = decltype(traits);
+        const long grid = (long)((M + Traits::kBM - 1) / Traits::kBM) * ((N + Traits::kBN - 1) / Traits::kBN);
+        return launch(&gemm_pipelined<Traits, OutType, true>, dim3(unsigned(grid)), dim3(Traits::kThreads),
+                      Traits::template lds_bytes<OutType>(), stream, A, B, C, M, N, K);
+    };
+    const auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    if (tiles(256, 256) >= 128) return go(PipeLarge{});
+    if (tiles(128, 128) >= 64) return go(PipeMid{});
+    return go(PipeSmall{});
+}
+
 template <typename OutType>
 int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
     if (K % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "pipelined GEMM needs K % 64 == 0");
@@ -260,6 +275,8 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) >= 128 &&
                 (long)K * 512 < (1l << 32))
                 return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
+            if (K % 64 == 0 && M % 16 == 0 && N % 16 == 0 && (M % 64 != 0 || N % 64 != 0) && (long)M * N >= 64 * 64)
+                return gemm_pipelined_edges_dispatch<OutType>(A, B, C, M, N, K, stream);
             if (M % 64 != 0 || N % 64 != 0 || K % 64 != 0) return gemm_ragged_dispatch<OutType>(A, B, C, M, N, K, stream);
             [[fallthrough]];
         case TCU_GEMM_PIPELINED:
