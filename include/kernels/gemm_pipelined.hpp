@@ -132,9 +132,11 @@ HOST_DEVICE void xcd_tile_coords(int bid, int tiles_m, int tiles_n, int& tile_m,
 
 }  // namespace detail
 
-/// kEdges: M and N need not be multiples of the tile (multiples of 16 suffice): the grid covers ceil(M / kBM) x
+/// kEdges: M, N and K need not be multiples of the tile (multiples of 16 suffice): the grid covers ceil(M / kBM) x
 /// ceil(N / kBN) tiles, rows beyond the edge are loaded from the last valid row (their products are computed and
-/// dropped) and the stores are guarded. K % kBK == 0 in either case.
+/// dropped) and the stores are guarded; the loop runs over ceil(K / kBK) tiles, and in the last one every lane loads
+/// the 16-byte pieces that lie beyond K from the start of its row instead and, once they have landed, overwrites them
+/// in LDS with zeros.
 template <typename Traits, typename OutType, bool kEdges = false>
 __global__ void __launch_bounds__(Traits::kThreads)
     gemm_pipelined(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N,
@@ -165,13 +167,15 @@ __global__ void __launch_bounds__(Traits::kThreads)
         const int row = (wave * Traits::kALoads + j) * Traits::kRowsPerLoad + lrow;
         const int chunk = lchk ^ ((row >> 1) & 7);
         const int grow = kEdges ? (m0 + row < M ? m0 + row : M - 1) : m0 + row;
-        return A + size_t(grow) * K + k0 + chunk * 8;
+        const int k = kEdges && k0 + chunk * 8 >= K ? 0 : k0 + chunk * 8;
+        return A + size_t(grow) * K + k;
     };
     auto b_src = [&](int j, int k0) -> const __half* {
         const int row = (wave * Traits::kBLoads + j) * Traits::kRowsPerLoad + lrow;
         const int chunk = lchk ^ ((row >> 1) & 7);
         const int grow = kEdges ? (n0 + row < N ? n0 + row : N - 1) : n0 + row;
-        return Bt + size_t(grow) * K + k0 + chunk * 8;
+        const int k = kEdges && k0 + chunk * 8 >= K ? 0 : k0 + chunk * 8;
+        return Bt + size_t(grow) * K + k;
     };
     // Issue part `part` of `nparts` of the loads of one stage (A instructions first, then B). Splitting a stage's
     // loads over the k-substeps keeps the vector-memory path evenly busy instead of bursting after the barrier.
@@ -191,6 +195,23 @@ __global__ void __launch_bounds__(Traits::kThreads)
         }
     };
     auto issue_stage = [&](int stage, int k0) { issue_part(stage, k0, 0, 1); };
+    // kEdges, last k-tile when K % kBK != 0: what this lane loaded from beyond K (it sits at 16 * lane of each of this
+    // wavefront's 1 KiB pieces) becomes zero. Call after the loads have landed, before the barrier that hands the stage over.
+    auto zero_k_tail = [&](int stage, int k0) {
+        unsigned char* sa = lds + stage * Traits::kStageBytes;
+        unsigned char* sb = sa + Traits::kABytes;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int q = 0; q < Traits::kALoads + Traits::kBLoads; ++q) {
+            const bool is_a = q < Traits::kALoads;
+            const int j = is_a ? q : q - Traits::kALoads;
+            const int row = (wave * (is_a ? Traits::kALoads : Traits::kBLoads) + j) * Traits::kRowsPerLoad + lrow;
+            const int chunk = lchk ^ ((row >> 1) & 7);
+            if (k0 + chunk * 8 >= K)
+                *reinterpret_cast<u32x4*>((is_a ? sa : sb) + (wave * (is_a ? Traits::kALoads : Traits::kBLoads) + j) * 1024 +
+                                          lane * 16) = zero;
+        }
+    };
 
     // ---- LDS -> register addressing -----------------------------------------------------
     // 16x16x32 operand: lane l holds row l % 16, k = 8 * (l / 16) .. +7 of the 32-wide substep,
@@ -230,11 +251,13 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
     };
 
-    const int ktiles = K / kBK;
+    const int ktiles = kEdges ? (K + kBK - 1) / kBK : K / kBK;
+    const bool k_tail = kEdges && K % kBK != 0;
 
     // prologue: tile 0 -> stage 0
     issue_stage(0, 0);
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    if (k_tail && ktiles == 1) zero_k_tail(0, 0);
     __syncthreads();
     load_frags(0, 0, 0);
 
@@ -253,6 +276,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         // wavefronts agree, the other stage can be read (and this one refilled in the next iteration).
         if (kt + 1 < ktiles) {
             __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+            if (k_tail && kt + 2 == ktiles) zero_k_tail(next_stage, (kt + 1) * kBK);
             __syncthreads();
             load_frags(kKS & 1, next_stage, 0);
         }

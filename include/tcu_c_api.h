@@ -29,9 +29,9 @@ typedef enum {
 typedef enum { TCU_DTYPE_F32 = 0, TCU_DTYPE_F16 = 1 } tcu_dtype;
 
 /* Which GEMM kernel to run. AUTO picks WAVE128 when M and N are multiples of 256 with at least 128 tiles of 256 x 256,
- * else the pipelined kernel when K is a multiple of 64 (with edge tiles when M or N are not multiples of 64), else
- * RAGGED: every shape made of whole 16 x 16 BaseTiles (M, N, K multiples of 16), the granularity of the reference's
- * tile types, is accepted. */
+ * else the pipelined kernel (with edge tiles and a zero-filled k tail when M, N or K are not multiples of 64), RAGGED
+ * for tiny problems: every shape made of whole 16 x 16 BaseTiles (M, N, K multiples of 16), the granularity of the
+ * reference's tile types, is accepted. */
 typedef enum {
     TCU_GEMM_AUTO = 0,
     TCU_GEMM_GLOBAL_REG = 1, /* global -> register -> MFMA (README kernel of the reference) */

@@ -150,12 +150,14 @@ def test_gemm_split_k_with_workspace(tcu, oracle, device, M, N, K, splits, out_d
             tcu.gemm(dA, dB, out_dtype=dt, workspace=ws[:need // 2])
 
 
-@pytest.mark.parametrize("M,N,K", [(80, 144, 64), (1040, 528, 256), (272, 4112, 128), (2064, 4080, 192), (4112, 4112, 64)])
+@pytest.mark.parametrize("M,N,K", [(80, 144, 64), (1040, 528, 256), (272, 4112, 128), (2064, 4080, 192), (4112, 4112, 64),
+                                   (1040, 528, 272), (2064, 1040, 1072), (256, 256, 48), (4096, 4096, 144), (144, 208, 16)])
 @pytest.mark.parametrize("out_dtype", ["f32", "f16"])
 def test_gemm_edge_tiles(tcu, oracle, device, M, N, K, out_dtype):
-    """M, N multiples of 16 but not of 64 with K % 64 == 0: AUTO runs the pipelined kernel with edge tiles (rows beyond
-    the edge loaded from the last valid row, stores guarded) in all three tile sizes; against the oracle on sampled rows
-    including the last ones, against the run-time-shape kernel everywhere, with guard bands around the output."""
+    """M, N, K multiples of 16 but not all of 64: AUTO runs the pipelined kernel with edge tiles (rows beyond the edge
+    loaded from the last valid row, stores guarded, the pieces of the last k-tile beyond K zeroed in LDS) in all three
+    tile sizes, with k tails of 16, 32 and 48 and a single partial k-tile; against the oracle on sampled rows including
+    the last ones, against the run-time-shape kernel everywhere, with guard bands around the output."""
     import torch
 
     print(f"gemm edge tiles {M}x{N}x{K} {out_dtype}", flush=True)

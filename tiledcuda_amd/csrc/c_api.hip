@@ -163,7 +163,7 @@ using PipeLarge = PipelinedGemmTraits<256, 256, 64, 4, 2, 2>;  // 8 wavefronts, 
 using PipeMid = PipelinedGemmTraits<128, 128, 64, 2, 2, 2>;
 using PipeSmall = PipelinedGemmTraits<64, 64, 64, 2, 2, 2>;
 
-/// M, N any multiples of 16 (K % 64 == 0): the pipelined kernel with edge tiles, the tile size chosen as for whole tiles.
+/// M, N, K any multiples of 16: the pipelined kernel with edge tiles, the tile size chosen as for whole tiles.
 template <typename OutType>
 int gemm_pipelined_edges_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
     auto go = [&](auto traits) {
@@ -275,7 +275,9 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) >= 128 &&
                 (long)K * 512 < (1l << 32))
                 return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
-            if (K % 64 == 0 && M % 16 == 0 && N % 16 == 0 && (M % 64 != 0 || N % 64 != 0) && (long)M * N >= 64 * 64)
+            // shapes of whole 16 x 16 tiles that are not whole 64 x 64 x 64 tiles: edge tiles, unless the problem is tiny
+            if (M % 16 == 0 && N % 16 == 0 && K % 16 == 0 && (M % 64 != 0 || N % 64 != 0 || K % 64 != 0) &&
+                (long)M * N >= 64 * 64)
                 return gemm_pipelined_edges_dispatch<OutType>(A, B, C, M, N, K, stream);
             if (M % 64 != 0 || N % 64 != 0 || K % 64 != 0) return gemm_ragged_dispatch<OutType>(A, B, C, M, N, K, stream);
             [[fallthrough]];
