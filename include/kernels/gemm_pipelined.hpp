@@ -163,19 +163,39 @@ __global__ void __launch_bounds__(Traits::kThreads)
     // p ^ ((row / 2) % 8).
     const int lrow = lane >> 3;  // row within the 8-row group
     const int lchk = lane & 7;   // physical 16-byte chunk
-    auto a_src = [&](int j, int k0) -> const __half* {
-        const int row = (wave * Traits::kALoads + j) * Traits::kRowsPerLoad + lrow;
-        const int chunk = lchk ^ ((row >> 1) & 7);
-        const int grow = kEdges ? (m0 + row < M ? m0 + row : M - 1) : m0 + row;
-        const int k = kEdges && k0 + chunk * 8 >= K ? 0 : k0 + chunk * 8;
-        return A + size_t(grow) * K + k;
+    // Each load's source is a wave-uniform base (the tile's first row at the k-tile, in scalar registers) plus a byte
+    // offset per lane that is fixed for the whole kernel: one 32-bit register per load instruction. Offsets stay below
+    // kBM * K * 2 bytes, so K up to 2^23 / (kBM / 256) fits.
+    auto row_chunk = [&](int loads_per_wave, int j) {
+        const int row = (wave * loads_per_wave + j) * Traits::kRowsPerLoad + lrow;
+        return lchk ^ ((row >> 1) & 7);
     };
-    auto b_src = [&](int j, int k0) -> const __half* {
+    unsigned int a_off[Traits::kALoads], b_off[Traits::kBLoads];
+#pragma unroll
+    for (int j = 0; j < Traits::kALoads; ++j) {
+        const int row = (wave * Traits::kALoads + j) * Traits::kRowsPerLoad + lrow;
+        a_off[j] = unsigned(kEdges && m0 + row >= M ? M - 1 - m0 : row) * unsigned(K) * 2u + row_chunk(Traits::kALoads, j) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < Traits::kBLoads; ++j) {
         const int row = (wave * Traits::kBLoads + j) * Traits::kRowsPerLoad + lrow;
-        const int chunk = lchk ^ ((row >> 1) & 7);
-        const int grow = kEdges ? (n0 + row < N ? n0 + row : N - 1) : n0 + row;
-        const int k = kEdges && k0 + chunk * 8 >= K ? 0 : k0 + chunk * 8;
-        return Bt + size_t(grow) * K + k;
+        b_off[j] = unsigned(kEdges && n0 + row >= N ? N - 1 - n0 : row) * unsigned(K) * 2u + row_chunk(Traits::kBLoads, j) * 16;
+    }
+    const unsigned char* a_tile = reinterpret_cast<const unsigned char*>(A + size_t(m0) * K);
+    const unsigned char* b_tile = reinterpret_cast<const unsigned char*>(Bt + size_t(n0) * K);
+    // kEdges: the k-tile that straddles K asks for pieces beyond the end of their row; those land in LDS and are
+    // overwritten with zeros there (zero_k_tail), so any readable address serves: the offset is limited to the last
+    // 16 bytes of the matrix, which only the last row's pieces exceed.
+    const size_t a_left = (size_t(M - m0) * K - 8) * 2, b_left = (size_t(N - n0) * K - 8) * 2;
+    const unsigned int a_limit = a_left < 0xfffffff0u ? unsigned(a_left) : 0xfffffff0u;
+    const unsigned int b_limit = b_left < 0xfffffff0u ? unsigned(b_left) : 0xfffffff0u;
+    auto a_src = [&](int j, int k0) -> const unsigned char* {
+        const unsigned int off = a_off[j] + unsigned(k0) * 2u;
+        return a_tile + (kEdges ? (off < a_limit ? off : a_limit) : off);
+    };
+    auto b_src = [&](int j, int k0) -> const unsigned char* {
+        const unsigned int off = b_off[j] + unsigned(k0) * 2u;
+        return b_tile + (kEdges ? (off < b_limit ? off : b_limit) : off);
     };
     // Issue part `part` of `nparts` of the loads of one stage (A instructions first, then B). Splitting a stage's
     // loads over the k-substeps keeps the vector-memory path evenly busy instead of bursting after the barrier.

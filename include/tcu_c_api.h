@@ -29,14 +29,16 @@ typedef enum {
 typedef enum { TCU_DTYPE_F32 = 0, TCU_DTYPE_F16 = 1 } tcu_dtype;
 
 /* Which GEMM kernel to run. AUTO picks WAVE128 when M and N are multiples of 256 with at least 128 tiles of 256 x 256,
- * else the pipelined kernel (with edge tiles and a zero-filled k tail when M, N or K are not multiples of 64), RAGGED
- * for tiny problems: every shape made of whole 16 x 16 BaseTiles (M, N, K multiples of 16), the granularity of the
- * reference's tile types, is accepted. */
+ * else PIPELINED, RAGGED for problems below 64 x 64: every shape made of whole 16 x 16 BaseTiles (M, N, K multiples of
+ * 16), the granularity of the reference's tile types, is accepted. */
 typedef enum {
     TCU_GEMM_AUTO = 0,
     TCU_GEMM_GLOBAL_REG = 1, /* global -> register -> MFMA (README kernel of the reference) */
     TCU_GEMM_ALL_MEM = 2,    /* global -> LDS -> register -> MFMA, single stage */
-    TCU_GEMM_PIPELINED = 3,  /* direct-to-LDS, double-buffered, 16x16x32 MFMA, 2 wavefronts per SIMD */
+    TCU_GEMM_PIPELINED = 3,  /* direct-to-LDS, double-buffered, 16x16x32 MFMA, 2 wavefronts per SIMD; M, N, K multiples
+                                of 16; tiles of 256 x 256, 128 x 128 or 64 x 64 by a cost model of the rounds of
+                                workgroups a launch takes; edge tiles (rows clamped, stores guarded, k tail zeroed in
+                                LDS) where the shape is not whole tiles */
     TCU_GEMM_WAVE128 = 4,    /* same pipeline, 256 x 256 tile on 4 wavefronts (one per SIMD, 128 x 128 each),
                                 accumulators in AGPRs; results identical to PIPELINED bit for bit */
     TCU_GEMM_TILE_PIPELINED = 5, /* the PIPELINED kernel composed from tile-library functors only (direct-to-LDS loader,

@@ -121,7 +121,7 @@ def test_unsupported_shapes_are_reported_not_launched(tcu):
     l = tcu.lib()
     p = 0x1000
     assert l.tcu_gemm_f16(p, p, p, 100, 64, 64, 0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
-    assert l.tcu_gemm_f16(p, p, p, 64, 64, 48, 0, 3, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_gemm_f16(p, p, p, 64, 64, 40, 0, 3, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_gemm_f16(p, p, p, 64, 72, 64, 0, 6, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # whole 16 x 16 tiles only
     assert l.tcu_gemm_f16(p, p, p, 64, 64, 40, 0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_gemm_f16(p, p, p, 256, 256, 256, 0, 1, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE

@@ -151,43 +151,40 @@ int launch_all_mem_gemm(const __half* A, const __half* B, OutType* C, hipStream_
     return launch(kernel, dim3(kM / kTM, kN / kTN), dim3(Cfg::kThreads), Cfg::kShmBytes, stream, A, B, C);
 }
 
-template <typename Traits, typename OutType>
-int launch_pipelined(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
-    auto kernel = &gemm_pipelined<Traits, OutType>;
-    const int grid = (M / Traits::kBM) * (N / Traits::kBN);
-    return launch(kernel, dim3(grid), dim3(Traits::kThreads), Traits::template lds_bytes<OutType>(), stream, A, B, C,
-                  M, N, K);
-}
-
 using PipeLarge = PipelinedGemmTraits<256, 256, 64, 4, 2, 2>;  // 8 wavefronts, 2 per SIMD
 using PipeMid = PipelinedGemmTraits<128, 128, 64, 2, 2, 2>;
 using PipeSmall = PipelinedGemmTraits<64, 64, 64, 2, 2, 2>;
 
-/// M, N, K any multiples of 16: the pipelined kernel with edge tiles, the tile size chosen as for whole tiles.
+/// The pipelined kernel for M, N, K any multiples of 16. The tile size comes from a cost model: a launch runs
+/// ceil(tiles / capacity) rounds of workgroups, capacity = 256 CUs x the workgroups of that size a CU holds (1, 2, 4),
+/// and a round costs K / 1024 x 25.5, 16 or 13 us for 256 x 256, 128 x 128 and 64 x 64 tiles (measured on full rounds at
+/// K = 1024 .. 4096); the larger tile wins a tie. Edge tiles (rows clamped, stores guarded, the K tail zeroed in LDS)
+/// are compiled in only where the shape is not a whole number of the chosen tiles.
 template <typename OutType>
-int gemm_pipelined_edges_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    if (M % 16 != 0 || N % 16 != 0 || K % 16 != 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM shapes are whole 16 x 16 tiles: M, N and K must be multiples of 16");
+    if ((long)K * 512 >= (1l << 32))
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "pipelined GEMM addresses a tile's rows with 32-bit offsets: K < 2^23");
     auto go = [&](auto traits) {
         using Traits = decltype(traits);
         const long grid = (long)((M + Traits::kBM - 1) / Traits::kBM) * ((N + Traits::kBN - 1) / Traits::kBN);
+        if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many tiles for one launch");
+        if (M % Traits::kBM == 0 && N % Traits::kBN == 0 && K % Traits::kBK == 0)
+            return launch(&gemm_pipelined<Traits, OutType, false>, dim3(unsigned(grid)), dim3(Traits::kThreads),
+                          Traits::template lds_bytes<OutType>(), stream, A, B, C, M, N, K);
         return launch(&gemm_pipelined<Traits, OutType, true>, dim3(unsigned(grid)), dim3(Traits::kThreads),
                       Traits::template lds_bytes<OutType>(), stream, A, B, C, M, N, K);
     };
-    const auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (tiles(256, 256) >= 128) return go(PipeLarge{});
-    if (tiles(128, 128) >= 64) return go(PipeMid{});
+    const auto cost = [&](int tile, int per_cu, double round_us) {
+        const long tiles = (long)((M + tile - 1) / tile) * ((N + tile - 1) / tile);
+        const long capacity = 256l * per_cu;
+        return double((tiles + capacity - 1) / capacity) * round_us;
+    };
+    const double large = cost(256, 1, 25.5), mid = cost(128, 2, 16.0), small = cost(64, 4, 13.0);
+    if (large <= mid && large <= small) return go(PipeLarge{});
+    if (mid <= small) return go(PipeMid{});
     return go(PipeSmall{});
-}
-
-template <typename OutType>
-int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
-    if (K % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "pipelined GEMM needs K % 64 == 0");
-    const auto tiles = [&](int bm, int bn) { return (long)(M / bm) * (N / bn); };
-    if (M % 256 == 0 && N % 256 == 0 && tiles(256, 256) >= 128)
-        return launch_pipelined<PipeLarge>(A, B, C, M, N, K, stream);
-    if (M % 128 == 0 && N % 128 == 0 && tiles(128, 128) >= 64)
-        return launch_pipelined<PipeMid>(A, B, C, M, N, K, stream);
-    if (M % 64 == 0 && N % 64 == 0) return launch_pipelined<PipeSmall>(A, B, C, M, N, K, stream);
-    return fail(TCU_ERR_UNSUPPORTED_SHAPE, "pipelined GEMM needs M % 64 == 0 and N % 64 == 0");
 }
 
 template <typename OutType>
@@ -275,11 +272,8 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) >= 128 &&
                 (long)K * 512 < (1l << 32))
                 return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
-            // shapes of whole 16 x 16 tiles that are not whole 64 x 64 x 64 tiles: edge tiles, unless the problem is tiny
-            if (M % 16 == 0 && N % 16 == 0 && K % 16 == 0 && (M % 64 != 0 || N % 64 != 0 || K % 64 != 0) &&
-                (long)M * N >= 64 * 64)
-                return gemm_pipelined_edges_dispatch<OutType>(A, B, C, M, N, K, stream);
-            if (M % 64 != 0 || N % 64 != 0 || K % 64 != 0) return gemm_ragged_dispatch<OutType>(A, B, C, M, N, K, stream);
+            // tiny problems: the kernel that takes its operand tiles straight from global memory has the shorter start
+            if ((long)M * N < 64 * 64) return gemm_ragged_dispatch<OutType>(A, B, C, M, N, K, stream);
             [[fallthrough]];
         case TCU_GEMM_PIPELINED:
             return gemm_pipelined_dispatch<OutType>(A, B, C, M, N, K, stream);
