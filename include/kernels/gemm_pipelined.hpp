@@ -41,7 +41,8 @@ struct PipelinedGemmTraits {
     static constexpr int kKS = kBK / 32;  // MFMA k-substeps (32 wide) per LDS tile
 
     static_assert(kBK == 64, "LDS rows are 128 bytes: kBK must be 64 halves");
-    static_assert(kStages == 2, "two LDS stages: a 256 x 256 x 64 stage is 64 KiB of the CU's 160 KiB");
+    static_assert(kStages >= 2 && kStages <= 4, "2 LDS stages (a 256 x 256 x 64 stage is 64 KiB of the CU's 160 KiB) or a "
+                                                "ring of 3 or 4 for the smaller tiles");
     static_assert(kWaveM % 16 == 0 && kWaveN % 16 == 0, "a wavefront owns whole 16x16 MFMA tiles");
 
     static constexpr int kRowBytes = kBK * 2;                    // 128
@@ -93,6 +94,21 @@ DEVICE void load_lds_16B_untracked(const void* gptr, const void* lds_wave_base) 
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off sc1" ::"v"(gptr), "s"(lds_addr) : "m0", "memory");
     else
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "m0", "memory");
+}
+
+/// Untracked direct-to-LDS load of 16 bytes per lane from sbase + voff (a wave-uniform 64-bit base in scalar registers
+/// plus a 32-bit byte offset per lane: no 64-bit address arithmetic per load) to lds_addr + 16 * lane.
+DEVICE void load_lds_16B_sbase(unsigned int voff, const void* sbase, unsigned int lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
+                 : "m0", "memory");
+}
+
+/// Wait until at most kVmcnt of this wavefront's vector-memory operations are outstanding (nothing else).
+template <int kVmcnt>
+DEVICE void wait_vmcnt() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (kVmcnt & 0xF) | ((kVmcnt >> 4) << 14));  // vmcnt(kVmcnt), others at their maximum
+    asm volatile("" ::: "memory");
 }
 
 /// Workgroup barrier that orders LDS accesses only. __syncthreads() also waits for every outstanding global memory
@@ -274,34 +290,102 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int ktiles = kEdges ? (K + kBK - 1) / kBK : K / kBK;
     const bool k_tail = kEdges && K % kBK != 0;
 
-    // prologue: tile 0 -> stage 0
-    issue_stage(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-    if (k_tail && ktiles == 1) zero_k_tail(0, 0);
-    __syncthreads();
-    load_frags(0, 0, 0);
-
-    int stage = 0;
-    for (int kt = 0; kt < ktiles; ++kt) {
-        const int next_stage = stage ^ 1;
+    if constexpr (Traits::kStages > 2) {
+        // ---- ring of kStages stages: kStages - 1 tiles in flight behind the one being multiplied ----------------
+        // The loads are issued as assembly the compiler does not track (it would otherwise make every LDS read wait
+        // for all of them); the kernel's own vmcnt waits before the barrier that hands a stage over are the
+        // synchronisation. A small tile has few MFMAs per k-tile, so its loop is bound by the latency of one tile's
+        // loads divided by the number of tiles in flight.
+        constexpr int S = Traits::kStages;
+        constexpr int L = Traits::kALoads + Traits::kBLoads;  // vector-memory operations per wavefront per tile
+        static_assert((S - 2) * L <= 63, "the vmcnt field counts to 63");
+        const unsigned int lds_base = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds)));
+        auto issue_ring = [&](int stage, int k0) {
+            const unsigned int sa = lds_base + stage * Traits::kStageBytes, sb = sa + Traits::kABytes;
 #pragma unroll
-        for (int kk = 0; kk < kKS - 1; ++kk) {
-            // tile kt+1 goes to the other stage, which everyone left at the barrier of iteration kt-1;
-            // its loads are issued during this iteration's first kKS-1 substeps
-            if (kt + 1 < ktiles) issue_part(next_stage, (kt + 1) * kBK, kk, kKS - 1);
-            load_frags((kk + 1) & 1, stage, kk + 1);
-            mma(kk & 1);
+            for (int q = 0; q < Traits::kALoads; ++q) {
+                if constexpr (kEdges) {
+                    const unsigned int off = a_off[q] + unsigned(k0) * 2u;
+                    detail::load_lds_16B_sbase(off < a_limit ? off : a_limit, a_tile, sa + (wave * Traits::kALoads + q) * 1024);
+                } else {
+                    detail::load_lds_16B_sbase(a_off[q], a_tile + size_t(k0) * 2, sa + (wave * Traits::kALoads + q) * 1024);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < Traits::kBLoads; ++q) {
+                if constexpr (kEdges) {
+                    const unsigned int off = b_off[q] + unsigned(k0) * 2u;
+                    detail::load_lds_16B_sbase(off < b_limit ? off : b_limit, b_tile, sb + (wave * Traits::kBLoads + q) * 1024);
+                } else {
+                    detail::load_lds_16B_sbase(b_off[q], b_tile + size_t(k0) * 2, sb + (wave * Traits::kBLoads + q) * 1024);
+                }
+            }
+        };
+        // wait until this wavefront's loads of a tile have landed, `behind` later tiles' loads still in flight
+        auto wait_tile = [&](int behind) {
+            if (behind >= S - 2) detail::wait_vmcnt<(S - 2) * L>();
+            else if (S > 3 && behind == 1) detail::wait_vmcnt<L>();
+            else detail::wait_vmcnt<0>();
+        };
+#pragma unroll
+        for (int s = 0; s < S; ++s)
+            if (s < ktiles) issue_ring(s, s * kBK);
+        wait_tile(ktiles - 1 < S - 1 ? ktiles - 1 : S - 1);
+        if (k_tail && ktiles == 1) zero_k_tail(0, 0);
+        detail::lds_barrier<63>();
+        load_frags(0, 0, 0);
+
+        int stage = 0;
+        for (int kt = 0; kt < ktiles; ++kt) {
+            const int next_stage = stage + 1 == S ? 0 : stage + 1;
+#pragma unroll
+            for (int kk = 0; kk < kKS - 1; ++kk) {
+                load_frags((kk + 1) & 1, stage, kk + 1);
+                mma(kk & 1);
+            }
+            if (kt + 1 < ktiles) {
+                // tile kt+1 is followed by tiles kt+2 .. min(kt+S-1, ktiles-1) (tile kt+S goes out after the barrier)
+                const int behind = ktiles - 2 - kt;
+                wait_tile(behind < S - 2 ? behind : S - 2);
+                if (k_tail && kt + 2 == ktiles) zero_k_tail(next_stage, (kt + 1) * kBK);
+                // every LDS read of `stage` has been issued; once they have returned everywhere it can be refilled
+                detail::lds_barrier<63>();
+                if (kt + S < ktiles) issue_ring(stage, (kt + S) * kBK);
+                load_frags(kKS & 1, next_stage, 0);
+            }
+            mma((kKS - 1) & 1);
+            stage = next_stage;
         }
-        // Every LDS read of `stage` has been issued; once they return, tile kt+1 has landed and all
-        // wavefronts agree, the other stage can be read (and this one refilled in the next iteration).
-        if (kt + 1 < ktiles) {
-            __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-            if (k_tail && kt + 2 == ktiles) zero_k_tail(next_stage, (kt + 1) * kBK);
-            __syncthreads();
-            load_frags(kKS & 1, next_stage, 0);
+    } else {
+        // prologue: tile 0 -> stage 0
+        issue_stage(0, 0);
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+        if (k_tail && ktiles == 1) zero_k_tail(0, 0);
+        __syncthreads();
+        load_frags(0, 0, 0);
+
+        int stage = 0;
+        for (int kt = 0; kt < ktiles; ++kt) {
+            const int next_stage = stage ^ 1;
+    #pragma unroll
+            for (int kk = 0; kk < kKS - 1; ++kk) {
+                // tile kt+1 goes to the other stage, which everyone left at the barrier of iteration kt-1;
+                // its loads are issued during this iteration's first kKS-1 substeps
+                if (kt + 1 < ktiles) issue_part(next_stage, (kt + 1) * kBK, kk, kKS - 1);
+                load_frags((kk + 1) & 1, stage, kk + 1);
+                mma(kk & 1);
+            }
+            // Every LDS read of `stage` has been issued; once they return, tile kt+1 has landed and all
+            // wavefronts agree, the other stage can be read (and this one refilled in the next iteration).
+            if (kt + 1 < ktiles) {
+                __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+                if (k_tail && kt + 2 == ktiles) zero_k_tail(next_stage, (kt + 1) * kBK);
+                __syncthreads();
+                load_frags(kKS & 1, next_stage, 0);
+            }
+            mma((kKS - 1) & 1);
+            stage = next_stage;
         }
-        mma((kKS - 1) & 1);
-        stage = next_stage;
     }
 
     // ---- epilogue -----------------------------------------------------------------------

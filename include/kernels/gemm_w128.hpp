@@ -73,12 +73,6 @@ DEVICE void mfma_16x16x32_agpr_then_load(f32x4& acc, const f16x8& a, const f16x8
         : "m0", "memory");
 }
 
-/// Direct-to-LDS load, scalar base + 32-bit lane offset (prologue only; inside the loop the fused form is used).
-DEVICE void load_lds_16B_sbase(unsigned int voff, const void* sbase, unsigned int lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
-                 : "m0", "memory");
-}
-
 }  // namespace detail
 
 /// C[i] = sum over z of partial[z][i] (f32 partial sums of a split-K product), 4 elements per lane. n % 4 == 0.

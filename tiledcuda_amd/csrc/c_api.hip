@@ -154,12 +154,15 @@ int launch_all_mem_gemm(const __half* A, const __half* B, OutType* C, hipStream_
 using PipeLarge = PipelinedGemmTraits<256, 256, 64, 4, 2, 2>;  // 8 wavefronts, 2 per SIMD
 using PipeMid = PipelinedGemmTraits<128, 128, 64, 2, 2, 2>;
 using PipeSmall = PipelinedGemmTraits<64, 64, 64, 2, 2, 2>;
+using PipeSmallRing = PipelinedGemmTraits<64, 64, 64, 2, 2, 4>;  // 4-stage ring, 64 KiB of LDS: 2 workgroups per CU
 
 /// The pipelined kernel for M, N, K any multiples of 16. The tile size comes from a cost model: a launch runs
 /// ceil(tiles / capacity) rounds of workgroups, capacity = 256 CUs x the workgroups of that size a CU holds (1, 2, 4),
 /// and a round costs K / 1024 x 25.5, 16 or 13 us for 256 x 256, 128 x 128 and 64 x 64 tiles (measured on full rounds at
-/// K = 1024 .. 4096); the larger tile wins a tie. Edge tiles (rows clamped, stores guarded, the K tail zeroed in LDS)
-/// are compiled in only where the shape is not a whole number of the chosen tiles.
+/// K = 1024 .. 4096); the larger tile wins a tie. With few 64 x 64 tiles per CU there is no neighbour workgroup to hide
+/// the latency of a tile's loads behind: then the same tile with a 4-stage ring (3 tiles in flight, 2 workgroups per
+/// CU, 7 us per round) is the choice. Edge tiles (rows clamped, stores guarded, the K tail zeroed in LDS) are compiled
+/// in only where the shape is not a whole number of the chosen tiles.
 template <typename OutType>
 int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
     if (M % 16 != 0 || N % 16 != 0 || K % 16 != 0)
@@ -181,10 +184,12 @@ int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M,
         const long capacity = 256l * per_cu;
         return double((tiles + capacity - 1) / capacity) * round_us;
     };
-    const double large = cost(256, 1, 25.5), mid = cost(128, 2, 16.0), small = cost(64, 4, 13.0);
-    if (large <= mid && large <= small) return go(PipeLarge{});
-    if (mid <= small) return go(PipeMid{});
-    return go(PipeSmall{});
+    const double large = cost(256, 1, 25.5), mid = cost(128, 2, 16.0), small = cost(64, 4, 13.0), ring = cost(64, 2, 7.0);
+    const double least_small = small < ring ? small : ring;
+    if (large <= mid && large <= least_small) return go(PipeLarge{});
+    if (mid <= least_small) return go(PipeMid{});
+    if (small <= ring) return go(PipeSmall{});
+    return go(PipeSmallRing{});
 }
 
 template <typename OutType>
