@@ -136,7 +136,18 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
         return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +
                                               (wave * T::kLoads + (q & 7)) * 1024);
     };
-    auto load_src = [&](int kt, int q) -> const __half* { return (q < 8 ? a_base : b_base) + kt * T::kBK; };
+    // Rows a multiple of 32 KiB apart put the same k-tile of every row of every panel into the same few memory
+    // channels, and all workgroups walk K in step. Each XCD then starts at a different eighth of K and wraps around
+    // (its workgroups stay in step with each other, which is what makes its L2 work): 7-14 % at K = 16384, nothing at
+    // smaller K. The sum over K is then taken in rotated order: the same value on every run, but not bit for bit the
+    // in-order sum of the other kernels (f32 rounding).
+    const int ktiles = K / T::kBK;
+    const int k_start = __builtin_amdgcn_readfirstlane(
+        ((lda | ldb) & 16383) == 0 && ktiles >= 64 ? int(blockIdx.x & 7) * (ktiles / 8) : 0);
+    auto load_src = [&](int kt, int q) -> const __half* {
+        const int ks = kt + k_start >= ktiles ? kt + k_start - ktiles : kt + k_start;
+        return (q < 8 ? a_base : b_base) + ks * T::kBK;
+    };
 
     // ---- LDS -> registers: fragment r of a substep (r < 8: A rows 16 r.., else B rows 16 (r - 8)..); lane l holds
     // row l % 16, k = 8 (l / 16) .. +7 of the 32-wide substep = logical chunk 4 kk + l / 16 of its row
@@ -150,7 +161,6 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 
     f16x8 fx[16], fy[16];  // fragments of substep 0 / substep 1: [0..7] A, [8..15] B
 
-    const int ktiles = K / T::kBK;
 #pragma unroll
     for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
     if (ktiles > 1) {

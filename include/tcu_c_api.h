@@ -40,7 +40,9 @@ typedef enum {
                                 workgroups a launch takes; edge tiles (rows clamped, stores guarded, k tail zeroed in
                                 LDS) where the shape is not whole tiles */
     TCU_GEMM_WAVE128 = 4,    /* same pipeline, 256 x 256 tile on 4 wavefronts (one per SIMD, 128 x 128 each),
-                                accumulators in AGPRs; results identical to PIPELINED bit for bit */
+                                accumulators in AGPRs; results identical to PIPELINED bit for bit, except where K is a
+                                multiple of 16384 (rows a multiple of 32 KiB apart): there each XCD sums over K in
+                                rotated order, which differs by f32 rounding */
     TCU_GEMM_TILE_PIPELINED = 5, /* the PIPELINED kernel composed from tile-library functors only (direct-to-LDS loader,
                                 two-stage shared ring, ds_read_b128 operand tiles, gemm()); compile-time shapes:
                                 4096^3, 1024^3, 512x768x192, 256x256x64; results identical to PIPELINED bit for bit */
