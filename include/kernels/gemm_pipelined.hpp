@@ -393,6 +393,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
     if constexpr (sizeof(OutType) == 2) {
         __syncthreads();  // everyone is done with the operand stages
         constexpr int kWaveN = Traits::kWaveN, kWaveM = Traits::kWaveM;
+        static_assert((kWaveN & (kWaveN - 1)) == 0 && kWaveN >= 16 && kWaveN <= 512 && kWaveM % (kWaveSize / (kWaveN / 8)) == 0,
+                      "f16 epilogue: a staged row is a power-of-two number of 16-byte pieces, read back by whole wavefronts");
         constexpr int kPitch = kWaveN * 2;  // bytes per staged row
         unsigned char* stg = lds + wave * (kWaveM * kPitch);
         // write: lane owns row i*16 + frow; 4 halves (8 B) at column j*16 + 4*fquad.

@@ -177,6 +177,53 @@ def test_gemm_edge_tiles(tcu, oracle, device, M, N, K, out_dtype):
     assert oracle.max_rel_err(host(out), host(plain)) <= REL_TOL
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (256, 256, 64), (128, 192, 128), (256, 256, 192), (192, 320, 256),
+                                   (256, 320, 320), (512, 512, 384), (1024, 1024, 2048), (80, 112, 48), (208, 400, 112), (144, 272, 1040)])
+@pytest.mark.parametrize("out_dtype", ["f32", "f16"])
+def test_gemm_ring_of_small_tiles(tcu, oracle, device, M, N, K, out_dtype):
+    """Few 64 x 64 tiles per CU: the pipelined kernel runs them with a 4-stage ring (three tiles in flight behind the
+    one being multiplied). Loops of 1 .. 6 and 32 k-tiles (shorter than, equal to and longer than the ring), whole and
+    edge tiles with a k tail; against the oracle and, for the order of the sum, bit for bit against the two-stage kernel
+    of the tile library where that is instantiated."""
+    import torch
+
+    print(f"gemm ring {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    A = oracle.fill_uniform(M * K, 331 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 337 + N).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    guard = torch.full((M + 2, N), -7.0, dtype=dt, device=device)
+    out = guard[1:M + 1]
+    tcu.gemm(dA, dB, out=out, algo="pipelined")
+    torch.cuda.synchronize()
+    assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
+    assert oracle.max_rel_err(host(out), oracle.gemm(A, Bt)) <= REL_TOL
+    if (M, N, K) == (256, 256, 64):
+        assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, algo="tile_pipelined"))
+
+
+def test_gemm_wave128_rotated_k_order(tcu, oracle, device):
+    """K = 16384 (rows 32 KiB apart): each XCD's workgroups start their walk over K at a different eighth and wrap
+    around. 8 tiles = one workgroup on every XCD, so every start is exercised; the oracle on 16 rows of each tile row."""
+    import torch
+
+    M, N, K = 512, 1024, 16384
+    print(f"gemm wave128 rotated k {M}x{N}x{K}", flush=True)
+    A = oracle.fill_uniform(M * K, 401).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 402).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    for dt in (torch.float32, torch.float16):
+        C = tcu.gemm(dA, dB, out_dtype=dt, algo="wave128")
+        torch.cuda.synchronize()
+        got = host(C)
+        for r0 in (0, 240, 256, 496):
+            want = oracle.gemm(A[r0:r0 + 16], Bt)
+            assert oracle.max_rel_err(got[r0:r0 + 16], want) <= REL_TOL
+        # the same sums in the plain order, everywhere
+        assert oracle.max_rel_err(got, host(tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))) <= REL_TOL
+        assert torch.equal(C, tcu.gemm(dA, dB, out_dtype=dt, algo="wave128"))  # the same on every run
+
+
 def test_gemm_wave128_rejects_other_shapes(tcu, device):
     import torch
 
