@@ -156,13 +156,35 @@ using PipeMid = PipelinedGemmTraits<128, 128, 64, 2, 2, 2>;
 using PipeSmall = PipelinedGemmTraits<64, 64, 64, 2, 2, 2>;
 using PipeSmallRing = PipelinedGemmTraits<64, 64, 64, 2, 2, 4>;  // 4-stage ring, 64 KiB of LDS: 2 workgroups per CU
 
-/// The pipelined kernel for M, N, K any multiples of 16. The tile size comes from a cost model: a launch runs
+/// Which tile the pipelined kernel takes for a shape, and what the launch is expected to cost. A launch runs
 /// ceil(tiles / capacity) rounds of workgroups, capacity = 256 CUs x the workgroups of that size a CU holds (1, 2, 4),
 /// and a round costs K / 1024 x 25.5, 16 or 13 us for 256 x 256, 128 x 128 and 64 x 64 tiles (measured on full rounds at
 /// K = 1024 .. 4096); the larger tile wins a tie. With few 64 x 64 tiles per CU there is no neighbour workgroup to hide
 /// the latency of a tile's loads behind: then the same tile with a 4-stage ring (3 tiles in flight, 2 workgroups per
-/// CU, 7 us per round) is the choice. Edge tiles (rows clamped, stores guarded, the K tail zeroed in LDS) are compiled
-/// in only where the shape is not a whole number of the chosen tiles.
+/// CU) is the choice: 3.75 us per K / 1024 with at most one workgroup per CU, 5.8 with two, 7 per round beyond.
+enum PipeConfig { kPipeLarge, kPipeMid, kPipeSmall, kPipeSmallRing };
+struct PipePlan {
+    PipeConfig config;
+    double us;
+};
+PipePlan pipelined_plan(int M, int N, int K) {
+    const auto tiles = [&](int tile) { return (long)((M + tile - 1) / tile) * ((N + tile - 1) / tile); };
+    const auto rounds = [&](int tile, int per_cu) { return double((tiles(tile) + 256l * per_cu - 1) / (256l * per_cu)); };
+    const double large = rounds(256, 1) * 25.5, mid = rounds(128, 2) * 16.0, small = rounds(64, 4) * 13.0;
+    const double ring = tiles(64) <= 256 ? 3.75 : tiles(64) <= 512 ? 5.8 : rounds(64, 2) * 7.0;
+    const double least_small = small < ring ? small : ring;
+    PipePlan plan;
+    if (large <= mid && large <= least_small) plan = {kPipeLarge, large};
+    else if (mid <= least_small) plan = {kPipeMid, mid};
+    else if (small <= ring) plan = {kPipeSmall, small};
+    else plan = {kPipeSmallRing, ring};
+    plan.us = 2.5 + plan.us * K / 1024.0;
+    return plan;
+}
+
+/// The pipelined kernel for M, N, K any multiples of 16, with the tile of pipelined_plan(). Edge tiles (rows clamped,
+/// stores guarded, the K tail zeroed in LDS) are compiled in only where the shape is not a whole number of the chosen
+/// tiles.
 template <typename OutType>
 int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
     if (M % 16 != 0 || N % 16 != 0 || K % 16 != 0)
@@ -179,17 +201,12 @@ int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M,
         return launch(&gemm_pipelined<Traits, OutType, true>, dim3(unsigned(grid)), dim3(Traits::kThreads),
                       Traits::template lds_bytes<OutType>(), stream, A, B, C, M, N, K);
     };
-    const auto cost = [&](int tile, int per_cu, double round_us) {
-        const long tiles = (long)((M + tile - 1) / tile) * ((N + tile - 1) / tile);
-        const long capacity = 256l * per_cu;
-        return double((tiles + capacity - 1) / capacity) * round_us;
-    };
-    const double large = cost(256, 1, 25.5), mid = cost(128, 2, 16.0), small = cost(64, 4, 13.0), ring = cost(64, 2, 7.0);
-    const double least_small = small < ring ? small : ring;
-    if (large <= mid && large <= least_small) return go(PipeLarge{});
-    if (mid <= least_small) return go(PipeMid{});
-    if (small <= ring) return go(PipeSmall{});
-    return go(PipeSmallRing{});
+    switch (pipelined_plan(M, N, K).config) {
+        case kPipeLarge: return go(PipeLarge{});
+        case kPipeMid: return go(PipeMid{});
+        case kPipeSmall: return go(PipeSmall{});
+        default: return go(PipeSmallRing{});
+    }
 }
 
 template <typename OutType>
@@ -227,16 +244,27 @@ int gemm_tile_pipelined_dispatch(const __half* A, const __half* B, OutType* C, i
                                            "and 256x256x64");
 }
 
-/// Number of K-ranges a product is split into when the caller brings a workspace: 1 unless 256 x 256 tiles would
-/// leave most of the chip idle (at most 32 tiles) and K is long enough to give every workgroup at least 512 of it.
+/// Number of K-ranges a product is split into when the caller brings a workspace: 1 unless 256 x 256 tiles would leave
+/// at least half of the chip idle (at most 128 tiles), K gives every workgroup at least 512 of it, and the split is
+/// expected to beat the unsplit launch by 5 %. Expected cost of s ranges (measured, one workgroup per CU at most):
+/// 10 us for the two launches and the epilogues + 1.4 us per k-tile of a range + the partial products written and
+/// read once (2 x s x M x N x 4 bytes at 5.3 TB/s); of the unsplit launch: pipelined_plan().
 int gemm_split_count(int M, int N, int K) {
     using T = GemmW128Traits;
     if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0) return 1;
     const long tiles = (long)(M / T::kBM) * (N / T::kBN);
-    if (tiles > 32) return 1;
-    int s = 1;
-    while (2 * s * tiles <= 256 && K % (2 * s * T::kBK) == 0 && K / (2 * s) >= 512) s *= 2;
-    return s;
+    if (tiles > 128) return 1;
+    const double unsplit_us = pipelined_plan(M, N, K).us;
+    int best = 1;
+    double best_us = 0.95 * unsplit_us;
+    for (int s = 2; s * tiles <= 256 && K % (s * T::kBK) == 0 && K / s >= 512; s *= 2) {
+        const double us = 10.0 + 1.4 * (K / s / T::kBK) + 2.0 * s * double(M) * N * 4 / 5.3e6;
+        if (us < best_us) {
+            best = s;
+            best_us = us;
+        }
+    }
+    return best;
 }
 
 template <typename OutType>
