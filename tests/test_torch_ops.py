@@ -182,6 +182,15 @@ def test_gemm_b2b_lstm_ops(ops, tcu, oracle, device):
     ops.gemm(torch.from_numpy(A).to(device), torch.from_numpy(Bt).to(device), C)
     assert oracle.max_rel_err(C.cpu().numpy(), oracle.gemm(A, Bt)) <= 1e-3
 
+    # few output tiles and a long K: the op splits over K through a workspace it takes from torch's allocator
+    A2 = oracle.fill_uniform(256 * 8192, 1236).reshape(256, 8192)
+    Bt2 = oracle.fill_uniform(256 * 8192, 2236).reshape(256, 8192)
+    assert tcu.gemm_workspace_bytes(256, 256, 8192) > 0
+    C2 = torch.empty(256, 256, dtype=torch.float16, device=device)
+    for _ in range(3):  # the workspace block is reused between calls
+        ops.gemm(torch.from_numpy(A2).to(device), torch.from_numpy(Bt2).to(device), C2)
+    assert oracle.max_rel_err(C2.float().cpu().numpy(), oracle.gemm(A2, Bt2)) <= 1e-3
+
     M, N, K, P = 64, 64, 64, 64
     A3 = oracle.fill_normal(M * K, 1, 0, 0.1).reshape(M, K)
     B3 = oracle.fill_normal(N * K, 2, 0, 0.1).reshape(N, K)

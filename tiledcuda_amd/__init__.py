@@ -141,12 +141,14 @@ def _out_code(dtype: torch.dtype) -> int:
 
 # ------------------------------------------------------------------------------ GEMM
 def gemm(a: torch.Tensor, b_t: torch.Tensor, out: torch.Tensor | None = None,
-         out_dtype: torch.dtype = torch.float16, algo: str = "auto", workspace: torch.Tensor | None = None) -> torch.Tensor:
+         out_dtype: torch.dtype = torch.float16, algo: str = "auto",
+         workspace: torch.Tensor | None | bool = None) -> torch.Tensor:
     """C[M, N] = A[M, K] · B with B column-major, i.e. ``b_t`` is the [N, K] array (``a @ b_t.T``).
 
-    Mirrors the reference's GEMM examples (A row-major, B column-major, f32 accumulate). With ``workspace`` (a
-    contiguous device tensor of at least ``gemm_workspace_bytes(M, N, K)`` bytes; ``algo`` must be "auto") a product
-    with few output tiles and a long K is split over K (``tcu_gemm_f16_ws``).
+    Mirrors the reference's GEMM examples (A row-major, B column-major, f32 accumulate). With ``algo="auto"`` a
+    product with few output tiles and a long K is split over K (``tcu_gemm_f16_ws``) through ``workspace`` (a contiguous
+    device tensor of at least ``gemm_workspace_bytes(M, N, K)`` bytes), or, when none is given, through one taken from
+    torch's caching allocator for the call; ``workspace=False`` never splits.
     """
     M, K = a.shape
     N, K2 = b_t.shape
@@ -156,6 +158,12 @@ def gemm(a: torch.Tensor, b_t: torch.Tensor, out: torch.Tensor | None = None,
         out = torch.empty(M, N, dtype=out_dtype, device=a.device)
     elif tuple(out.shape) != (M, N):
         raise ValueError("out has the wrong shape")
+    if workspace is None and algo == "auto" and a.is_cuda:
+        need = gemm_workspace_bytes(M, N, K)
+        if need > 0:
+            workspace = torch.empty(need, dtype=torch.uint8, device=a.device)
+    if workspace is False:
+        workspace = None
     if workspace is not None:
         if algo != "auto":
             raise ValueError("a workspace goes with algo='auto'")

@@ -88,8 +88,18 @@ void gemm(const at::Tensor& A, const at::Tensor& B, at::Tensor& C) {
     TORCH_CHECK(A.size(1) == B.size(1), "mismatched K dimension");
     TORCH_CHECK(C.size(0) == A.size(0) && C.size(1) == B.size(0), "C must be [M, N]");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(A.device());
-    check_status(tcu_gemm_f16(A.data_ptr(), B.data_ptr(), C.data_ptr(), int(A.size(0)), int(B.size(0)), int(A.size(1)), code,
-                              TCU_GEMM_AUTO, current_stream(A)),
+    const int M = int(A.size(0)), N = int(B.size(0)), K = int(A.size(1));
+    // few output tiles and a long K: split over K through a workspace from torch's caching allocator (stream-ordered:
+    // the block goes back to the allocator when `ws` dies and is reused on this stream only after the work enqueued here)
+    const unsigned long long need = tcu_gemm_workspace_bytes(M, N, K);
+    if (need > 0) {
+        at::Tensor ws = at::empty({static_cast<int64_t>(need)}, A.options().dtype(at::kByte));
+        check_status(tcu_gemm_f16_ws(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, code, ws.data_ptr(), need,
+                                     current_stream(A)),
+                     "gemm");
+        return;
+    }
+    check_status(tcu_gemm_f16(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, code, TCU_GEMM_AUTO, current_stream(A)),
                  "gemm");
 }
 
