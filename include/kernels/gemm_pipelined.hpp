@@ -152,11 +152,11 @@ HOST_DEVICE void xcd_tile_coords(int bid, int tiles_m, int tiles_n, int& tile_m,
 /// ceil(N / kBN) tiles, rows beyond the edge are loaded from the last valid row (their products are computed and
 /// dropped) and the stores are guarded; the loop runs over ceil(K / kBK) tiles, and in the last one every lane loads
 /// the 16-byte pieces that lie beyond K from the start of its row instead and, once they have landed, overwrites them
-/// in LDS with zeros.
+/// in LDS with zeros. ldc: elements between consecutive rows of C (N for a dense C).
 template <typename Traits, typename OutType, bool kEdges = false>
 __global__ void __launch_bounds__(Traits::kThreads)
     gemm_pipelined(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N,
-                   int K) {
+                   int K, int ldc) {
     constexpr int kBM = Traits::kBM, kBN = Traits::kBN, kBK = Traits::kBK;
     constexpr int kMT = Traits::kMT, kNT = Traits::kNT, kKS = Traits::kKS;
 
@@ -420,17 +420,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
         constexpr int kRowsPerIter = kWaveSize / kLanesPerRow;
         const int rr = lane / kLanesPerRow;
         const int cc = lane % kLanesPerRow;  // 16-byte chunk = 8-byte slots 2cc, 2cc+1
-        OutType* cbase = C + size_t(m0 + wave_m * kWaveM) * N + n0 + wave_n * kWaveN;
+        OutType* cbase = C + size_t(m0 + wave_m * kWaveM) * ldc + n0 + wave_n * kWaveN;
 #pragma unroll
         for (int it = 0; it < kWaveM / kRowsPerIter; ++it) {
             const int row = it * kRowsPerIter + rr;
             const int pslot = (2 * cc) ^ (((row & 15) << 1) & kSlotMask);
             const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kPitch + pslot * 8);
             if (kEdges && (m0 + wave_m * kWaveM + row >= M || n0 + wave_n * kWaveN + cc * 8 >= N)) continue;
-            *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(cbase + size_t(row) * N) + cc * 16) = v;
+            *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(cbase + size_t(row) * ldc) + cc * 16) = v;
         }
     } else {
-        OutType* cbase = C + size_t(m0 + wave_m * Traits::kWaveM) * N + n0 + wave_n * Traits::kWaveN;
+        OutType* cbase = C + size_t(m0 + wave_m * Traits::kWaveM) * ldc + n0 + wave_n * Traits::kWaveN;
 #pragma unroll
         for (int i = 0; i < kMT; ++i) {
 #pragma unroll
@@ -438,7 +438,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 if (kEdges && (m0 + wave_m * Traits::kWaveM + i * 16 + frow >= M ||
                                n0 + wave_n * Traits::kWaveN + j * 16 + 4 * fquad >= N))
                     continue;
-                *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * N + j * 16 + 4 * fquad) = acc[i][j];
+                *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * ldc + j * 16 + 4 * fquad) = acc[i][j];
             }
         }
     }

@@ -99,12 +99,13 @@ __global__ void __launch_bounds__(256) splitk_reduce(const float* __restrict__ p
 
 /// grid = ((M / 256) * (N / 256), splits), block = 256, dynamic LDS = GemmW128Traits::kLdsBytes.
 /// lda / ldb: elements between consecutive rows of A / of the stored [N, K] array (K for dense operands; larger when
-/// the operand is a column block of a wider matrix). C is dense. With splits > 1 workgroup row z multiplies the
+/// the operand is a column block of a wider matrix); ldc: elements between consecutive rows of C (N for a dense C;
+/// larger when C is the leading block of a wider matrix). With splits > 1 workgroup row z multiplies the
 /// K-range [z K, (z + 1) K) and writes plane z of C ([splits, M, N]; partial sums for splitk_reduce).
 template <typename OutType>
 __global__ void __launch_bounds__(GemmW128Traits::kThreads)
     gemm_w128(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
-              int lda, int ldb) {
+              int lda, int ldb, int ldc) {
     using T = GemmW128Traits;
     extern __shared__ __align__(1024) unsigned char lds[];
 
@@ -130,7 +131,7 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
     const size_t z = blockIdx.y;
     const __half* a_base = A + size_t(m0) * lda + z * K;
     const __half* b_base = Bt + size_t(n0) * ldb + z * K;
-    C += z * size_t(M) * N;
+    C += z * size_t(M) * ldc;
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
     auto load_dst = [&](int stage, int q) -> unsigned int {
         return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +
@@ -247,7 +248,7 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
         constexpr int kSlotMask = (kPitch / 8 - 1) & ~1;   // 8-byte slots of a row are XOR-ed with 2 * row
         unsigned char* stg = lds + T::kLdsBytesMain + wave * T::kEpilogueBytesPerWave;
         const int rr = lane >> 4, cc = lane & 15;  // read-back: 16 lanes x 16 B per row, 4 rows per instruction
-        OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * N + n0 + wave_n * T::kWaveN;
+        OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * ldc + n0 + wave_n * T::kWaveN;
         // LDS addresses of this lane's 8 staging writes and 4 read-backs of a row group (the same for every group but
         // for the buffer), computed once: with one wavefront per SIMD the epilogue is bound by instruction issue
         unsigned int waddr[8], raddr[4];
@@ -266,7 +267,7 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
         }
         using lds_f16x4_ptr = __attribute__((address_space(3))) f16x4*;
         using lds_u32x4_ptr = __attribute__((address_space(3))) const u32x4*;
-        unsigned char* crow = reinterpret_cast<unsigned char*>(cbase + size_t(rr) * N) + cc * 16;  // row rr of the block
+        unsigned char* crow = reinterpret_cast<unsigned char*>(cbase + size_t(rr) * ldc) + cc * 16;  // row rr of the block
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const unsigned int buf = (i & 1) * (16 * kPitch);
@@ -281,16 +282,16 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const u32x4 v = *reinterpret_cast<lds_u32x4_ptr>(raddr[it] + buf);
-                *reinterpret_cast<u32x4*>(crow + size_t(i * 16 + it * 4) * N * sizeof(OutType)) = v;
+                *reinterpret_cast<u32x4*>(crow + size_t(i * 16 + it * 4) * ldc * sizeof(OutType)) = v;
             }
         }
     } else {
-        OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * N + n0 + wave_n * T::kWaveN;
+        OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * ldc + n0 + wave_n * T::kWaveN;
 #pragma unroll
         for (int i = 0; i < 8; ++i)
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-                *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * N + j * 16 + 4 * fquad) = acc[i][j];
+                *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * ldc + j * 16 + 4 * fquad) = acc[i][j];
     }
 }
 

@@ -225,6 +225,31 @@ def test_gemm_wave128_rotated_k_order(tcu, oracle, device):
         assert torch.equal(C, tcu.gemm(dA, dB, out_dtype=dt, algo="wave128"))  # the same on every run
 
 
+@pytest.mark.parametrize("M,N,K", [(4112, 4112, 1024), (4112, 4096, 512), (4096, 4112, 512), (4144, 4128, 192)])
+@pytest.mark.parametrize("out_dtype", ["f32", "f16"])
+def test_gemm_main_block_and_strips(tcu, oracle, device, M, N, K, out_dtype):
+    """M or N a little above a multiple of 256: AUTO computes the leading block of whole 256 x 256 tiles with the
+    one-wavefront-per-SIMD kernel and the remaining columns / rows with small tiles (three launches on disjoint parts
+    of C) instead of paying a whole extra round of 256 x 256 edge tiles. Against the oracle on the first and last rows
+    (the last ones lie in the bottom strip, every row crosses into the right strip), bit for bit against the
+    single-launch pipelined kernel everywhere, with guard rows around the output."""
+    import torch
+
+    print(f"gemm main block + strips {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    A = oracle.fill_uniform(M * K, 431 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 437 + N).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    guard = torch.full((M + 2, N), -7.0, dtype=dt, device=device)
+    out = guard[1:M + 1]
+    tcu.gemm(dA, dB, out=out, algo="auto")
+    torch.cuda.synchronize()
+    assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
+    rows = list(range(0, 24)) + list(range(M - 24, M))
+    assert oracle.max_rel_err(host(out)[rows], oracle.gemm(A[rows], Bt)) <= REL_TOL
+    assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))
+
+
 def test_gemm_wave128_rejects_other_shapes(tcu, device):
     import torch
 

@@ -186,7 +186,9 @@ PipePlan pipelined_plan(int M, int N, int K) {
 /// stores guarded, the K tail zeroed in LDS) are compiled in only where the shape is not a whole number of the chosen
 /// tiles.
 template <typename OutType>
-int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream,
+                            int ldc = 0) {
+    if (ldc == 0) ldc = N;
     if (M % 16 != 0 || N % 16 != 0 || K % 16 != 0)
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM shapes are whole 16 x 16 tiles: M, N and K must be multiples of 16");
     if ((long)K * 512 >= (1l << 32))
@@ -197,9 +199,9 @@ int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M,
         if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many tiles for one launch");
         if (M % Traits::kBM == 0 && N % Traits::kBN == 0 && K % Traits::kBK == 0)
             return launch(&gemm_pipelined<Traits, OutType, false>, dim3(unsigned(grid)), dim3(Traits::kThreads),
-                          Traits::template lds_bytes<OutType>(), stream, A, B, C, M, N, K);
+                          Traits::template lds_bytes<OutType>(), stream, A, B, C, M, N, K, ldc);
         return launch(&gemm_pipelined<Traits, OutType, true>, dim3(unsigned(grid)), dim3(Traits::kThreads),
-                      Traits::template lds_bytes<OutType>(), stream, A, B, C, M, N, K);
+                      Traits::template lds_bytes<OutType>(), stream, A, B, C, M, N, K, ldc);
     };
     switch (pipelined_plan(M, N, K).config) {
         case kPipeLarge: return go(PipeLarge{});
@@ -211,16 +213,17 @@ int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M,
 
 template <typename OutType>
 int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream,
-                       int lda = 0, int ldb = 0) {
+                       int lda = 0, int ldb = 0, int ldc = 0) {
     using T = GemmW128Traits;
     if (lda == 0) lda = K;
     if (ldb == 0) ldb = K;
+    if (ldc == 0) ldc = N;
     if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0)
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM needs M % 256 == 0, N % 256 == 0, K % 64 == 0");
     if ((long)std::max(lda, ldb) * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
     return launch(&gemm_w128<OutType>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
-                  C, M, N, K, lda, ldb);
+                  C, M, N, K, lda, ldb, ldc);
 }
 
 template <typename OutType, int kM, int kN, int kK, int kTM, int kTN, typename WarpLayout>
@@ -242,6 +245,31 @@ int gemm_tile_pipelined_dispatch(const __half* A, const __half* B, OutType* C, i
     if (M == 256 && N == 256 && K == 64) return launch_tile_pipelined<OutType, 256, 256, 64, 64, 64, W22>(A, B, C, stream);
     return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the tile-API pipelined GEMM is instantiated for 4096^3, 1024^3, 512x768x192 "
                                            "and 256x256x64");
+}
+
+/// M or N a little above a multiple of 256: edge tiles of 256 x 256 cost a whole extra round of workgroups for a
+/// sliver of output. When the cost model says so, the product is computed as three launches on disjoint parts of C:
+/// the leading block of whole 256 x 256 tiles by the one-wavefront-per-SIMD kernel, the columns beyond it (all rows)
+/// and the rows beyond it (the leading columns) by the pipelined kernel with small tiles. Same order of the sum
+/// everywhere, so the result is bit for bit that of one launch. Returns kPlanNotTaken when the plain launch is the
+/// better plan.
+constexpr int kPlanNotTaken = INT_MIN;
+template <typename OutType>
+int gemm_main_and_strips(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    using T = GemmW128Traits;
+    const int Mm = M / T::kBM * T::kBM, Nm = N / T::kBN * T::kBN;
+    if ((Mm == M && Nm == N) || K % T::kBK != 0 || (long)K * 512 >= (1l << 32)) return kPlanNotTaken;
+    const long tiles = (long)(Mm / T::kBM) * (Nm / T::kBN);
+    if (tiles < 128) return kPlanNotTaken;
+    const double main_us = 2.5 + double((tiles + 255) / 256) * 24.0 * K / 1024.0;
+    const double right_us = N > Nm ? 2.0 + pipelined_plan(M, N - Nm, K).us : 0.0;
+    const double bottom_us = M > Mm ? 2.0 + pipelined_plan(M - Mm, Nm, K).us : 0.0;
+    if (main_us + right_us + bottom_us >= pipelined_plan(M, N, K).us) return kPlanNotTaken;
+    int rc = gemm_w128_dispatch<OutType>(A, B, C, Mm, Nm, K, stream, K, K, N);
+    if (rc == TCU_OK && N > Nm) rc = gemm_pipelined_dispatch<OutType>(A, B + size_t(Nm) * K, C + Nm, M, N - Nm, K, stream, N);
+    if (rc == TCU_OK && M > Mm)
+        rc = gemm_pipelined_dispatch<OutType>(A + size_t(Mm) * K, B, C + size_t(Mm) * N, M - Mm, Nm, K, stream, N);
+    return rc;
 }
 
 /// Number of K-ranges a product is split into when the caller brings a workspace: 1 unless 256 x 256 tiles would leave
@@ -275,7 +303,7 @@ int gemm_splitk(const __half* A, const __half* B, OutType* C, int M, int N, int 
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
     const int tiles = (M / T::kBM) * (N / T::kBN);
     int rc = launch(&gemm_w128<float>, dim3(tiles, splits), dim3(T::kThreads), T::kLdsBytes, stream, A, B, partial, M, N,
-                    K / splits, K, K);
+                    K / splits, K, K, N);
     if (rc != TCU_OK) return rc;
     const size_t n = size_t(M) * N;
     return launch(&splitk_reduce<OutType>, dim3(unsigned((n / 4 + 255) / 256)), dim3(256), 0, stream,
@@ -305,6 +333,10 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) >= 128 &&
                 (long)K * 512 < (1l << 32))
                 return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
+            if (M % 16 == 0 && N % 16 == 0) {
+                const int rc = gemm_main_and_strips<OutType>(A, B, C, M, N, K, stream);
+                if (rc != kPlanNotTaken) return rc;
+            }
             // tiny problems: the kernel that takes its operand tiles straight from global memory has the shorter start
             if ((long)M * N < 64 * 64) return gemm_ragged_dispatch<OutType>(A, B, C, M, N, K, stream);
             [[fallthrough]];

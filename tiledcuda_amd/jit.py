@@ -56,7 +56,7 @@ static int launch(const __half* a, const __half* b, float* c, hipStream_t stream
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -3;
         raised = true;
     }}
-    hipLaunchKernelGGL(kernel, dim3(({M} / {TM}) * ({N} / {TN})), dim3(Config::kThreads), lds, stream, a, b, c, {M}, {N}, {K});
+    hipLaunchKernelGGL(kernel, dim3(({M} / {TM}) * ({N} / {TN})), dim3(Config::kThreads), lds, stream, a, b, c, {M}, {N}, {K}, {N});
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }}
 """
