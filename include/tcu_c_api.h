@@ -28,9 +28,11 @@ typedef enum {
 
 typedef enum { TCU_DTYPE_F32 = 0, TCU_DTYPE_F16 = 1 } tcu_dtype;
 
-/* Which GEMM kernel to run. AUTO picks WAVE128 when M and N are multiples of 256 with at least 128 tiles of 256 x 256,
- * else PIPELINED, RAGGED for problems below 64 x 64: every shape made of whole 16 x 16 BaseTiles (M, N, K multiples of
- * 16), the granularity of the reference's tile types, is accepted. */
+/* Which GEMM kernel to run. AUTO picks WAVE128 when M and N are multiples of 256 with at least 128 tiles of 256 x 256;
+ * WAVE128 on the leading block of whole tiles plus PIPELINED on the remaining columns and rows (three launches on
+ * disjoint parts of C, bit for bit the result of one launch) when M or N lie a little above such multiples and that
+ * saves a round of workgroups; else PIPELINED; RAGGED for problems below 64 x 64. Every shape made of whole 16 x 16
+ * BaseTiles (M, N, K multiples of 16), the granularity of the reference's tile types, is accepted. */
 typedef enum {
     TCU_GEMM_AUTO = 0,
     TCU_GEMM_GLOBAL_REG = 1, /* global -> register -> MFMA (README kernel of the reference) */
