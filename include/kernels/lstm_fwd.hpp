@@ -45,6 +45,8 @@ struct LstmFwdTraits {
     static constexpr int kStageBytes = 2 * kTileBytes;             // 32 KiB
     static constexpr int kLoadsPerWave = 4;                        // 32 one-KiB instructions per stage / 8 wavefronts
     static constexpr int kLdsBytes = kStages * kStageBytes;
+    // kI == kH == 0: the sizes are kernel arguments (I % 128 == 0, H % 128 == 0, checked by the launcher)
+    static constexpr bool kRuntimeShape = kI == 0 && kH == 0;
     static_assert(kI % kBK == 0 && kH % kBK == 0 && kH % kTH == 0);
     static_assert((kH / kTH) % 8 == 0, "the workgroup map deals hidden tiles to the 8 XCDs");
     static_assert(kStages >= 2 && (kStages - 2) * kLoadsPerWave <= 63, "vmcnt is a 6-bit counter");
@@ -68,12 +70,15 @@ DEVICE void wait_vmcnt_lgkm0() {
 /// kHoisted: the input half of the gates, x_t · W[:, :I]ᵀ, was computed beforehand for the whole sequence (one large
 /// GEMM) and is passed as pre_t [B, 4H] f32; the step then streams only h_{t-1} and W[:, I:] (half the bytes) and x_t
 /// is not read.
+/// I, H: the sizes, used by LstmFwdTraits<0, 0> (any multiples of 128); the other instantiations have them as constants.
 template <typename Traits, bool kHoisted = false>
 __global__ void __launch_bounds__(Traits::kThreads)
     lstm_cell_fwd(const __half* __restrict__ x_t, const __half* __restrict__ h_in, const __half* __restrict__ W,
                   const __half* __restrict__ bias, const float* c_in, float* c_out, __half* __restrict__ h_out,
-                  int B, const float* __restrict__ pre_t) {
-    constexpr int kI = Traits::kI, kH = Traits::kH, kKK = Traits::kKK, kBK = Traits::kBK;
+                  int B, const float* __restrict__ pre_t, int I, int H) {
+    constexpr int kBK = Traits::kBK;
+    const int kI = Traits::kRuntimeShape ? I : Traits::kI, kH = Traits::kRuntimeShape ? H : Traits::kH;
+    const int kKK = kI + kH;
     constexpr int S = Traits::kStages, L = Traits::kLoadsPerWave;
     extern __shared__ __align__(1024) unsigned char lds[];
 

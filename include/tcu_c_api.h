@@ -87,7 +87,8 @@ typedef enum {
     TCU_LSTM_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, single LDS stage; (I, H) in {(1024,1024),
                                   (128,128), (64,128)}, B % 64 == 0 */
     TCU_LSTM_STREAMING = 2,    /* 32x32x16 MFMA, multi-stage direct-to-LDS ring, k split over two wavefront groups;
-                                  (I, H) in {(1024,1024), (128,128), (256,128)}, B % 64 == 0 */
+                                  I % 128 == 0, H % 128 == 0, B % 64 == 0 (sizes are kernel arguments, except the
+                                  (1024, 1024) instantiation, which has them as constants) */
     TCU_LSTM_RAGGED = 3        /* run-time B, I, H in multiples of 16: MFMA operand tiles filled from global memory */
 } tcu_lstm_algo;
 
@@ -164,9 +165,9 @@ int tcu_flash_attn_fwd_f16_algo(const void* Q, const void* K, const void* V, voi
  * c0 [B, H] f32 or NULL (zeros); h_all [T, B, H] f16 receives every h_t; c_out [B, H] f32
  * receives c_T (it is also the running cell state, so it must not alias c0 unless c0 == c_out).
  * One kernel per step (gate GEMM fused with the cell update). B, I and H must be multiples of 16 (whole tiles) and
- * T * B fit in 31 bits. With B % 64 == 0 the streaming kernel is instantiated for (I, H) = (1024,1024), (128,128),
- * (256,128) and the tile-library kernel for (1024,1024), (128,128), (64,128); AUTO takes the streaming kernel where it
- * exists, else the tile-library one, else the run-time-shape kernel (TCU_LSTM_RAGGED), which takes every shape.
+ * T * B fit in 31 bits. With B % 64 == 0 the streaming kernel takes every I and H in multiples of 128, and the
+ * tile-library kernel is instantiated for (I, H) = (1024,1024), (128,128), (64,128); AUTO takes the streaming kernel
+ * where it applies, else the tile-library one, else the run-time-shape kernel (TCU_LSTM_RAGGED), which takes every shape.
  * The reference snapshot has no LSTM entry (Makefile:3 names a test only).
  */
 int tcu_lstm_f16(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
@@ -182,8 +183,8 @@ int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void
  * of a step, which is what bounds it). Same arguments and results (up to the order of the f32 summation) as
  * tcu_lstm_f16. `workspace` is device memory of at least tcu_lstm_workspace_bytes(T, B, I, H) bytes, 16-byte aligned,
  * owned by the caller and free to reuse once the work enqueued here has run. tcu_lstm_workspace_bytes returns 0 for
- * shapes this path is not instantiated for ((I, H) in {(1024, 1024), (128, 128), (256, 128)}, T * B a multiple of
- * 256); tcu_lstm_f16_ws then fails with TCU_ERR_UNSUPPORTED_SHAPE. No counterpart in the reference (it has no LSTM).
+ * shapes this path does not take (it needs I % 128 == 0, H % 128 == 0, B % 64 == 0 and T * B a multiple of 256);
+ * tcu_lstm_f16_ws then fails with TCU_ERR_UNSUPPORTED_SHAPE. No counterpart in the reference (it has no LSTM).
  */
 unsigned long long tcu_lstm_workspace_bytes(int T, int B, int I, int H);
 int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,

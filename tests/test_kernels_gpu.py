@@ -738,12 +738,13 @@ def test_lstm_small(tcu, oracle, device, T, B, I, H, with_state, algo):
     assert oracle.max_abs_err(host(c_T), c_ref) <= ABS_TOL
 
 
-@pytest.mark.parametrize("T,B,I,H", [(4, 64, 128, 128), (2, 128, 256, 128), (8, 64, 128, 128)])
+@pytest.mark.parametrize("T,B,I,H", [(4, 64, 128, 128), (2, 128, 256, 128), (8, 64, 128, 128), (4, 64, 512, 512),
+                                     (2, 128, 384, 256), (4, 64, 128, 640), (4, 64, 768, 128)])
 @pytest.mark.parametrize("with_state", [False, True])
 def test_lstm_hoisted_input_projection(tcu, oracle, device, T, B, I, H, with_state):
     """tcu_lstm_f16_ws: the input half of the gates from one GEMM over all steps, then steps over h only; against the
     oracle, against the per-step streaming kernel, with a caller-owned workspace larger than needed, and twice in a row
-    on the same workspace."""
+    on the same workspace. Both kernels take any I and H in multiples of 128 (sizes as kernel arguments)."""
     import torch
 
     print(f"lstm hoisted T{T} B{B} I{I} H{H} state={with_state}", flush=True)
@@ -773,7 +774,7 @@ def test_lstm_hoisted_rejects_what_it_cannot_do(tcu, device):
     import torch
 
     assert tcu.lstm_workspace_bytes(3, 64, 128, 128) == 0  # T * B not a multiple of 256
-    assert tcu.lstm_workspace_bytes(4, 64, 64, 64) == 0    # shape not instantiated
+    assert tcu.lstm_workspace_bytes(4, 64, 64, 64) == 0    # I, H not multiples of 128
     x = torch.zeros(4, 64, 128, dtype=torch.float16, device=device)
     W = torch.zeros(512, 256, dtype=torch.float16, device=device)
     b = torch.zeros(512, dtype=torch.float16, device=device)

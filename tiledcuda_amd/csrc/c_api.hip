@@ -536,25 +536,26 @@ int launch_lstm(const __half* x, const __half* W, const __half* bias, const __ha
     return TCU_OK;
 }
 
+/// kI == kH == 0: the run-time-shape instantiation of the streaming kernel (I, H any multiples of 128).
 template <int kI, int kH>
 int launch_lstm_hoisted(const __half* x, const __half* W, const __half* bias, const __half* h0, const float* c0,
-                        __half* h_all, float* c_out, int T, int B, float* pre, hipStream_t stream) {
+                        __half* h_all, float* c_out, int T, int B, int I, int H, float* pre, hipStream_t stream) {
     using Traits = LstmFwdTraits<kI, kH>;
     // pre[T * B, 4H] = x[T * B, I] . W[:, :I]^T: the stored [4H, I] operand is the first I columns of W's rows
     const long rows = long(T) * B;
     if (rows > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_ws: T * B exceeds the 32-bit row count");
-    int rc = gemm_w128_dispatch<float>(x, W, pre, int(rows), 4 * kH, kI, stream, kI, kI + kH);
+    int rc = gemm_w128_dispatch<float>(x, W, pre, int(rows), 4 * H, I, stream, I, I + H);
     if (rc != TCU_OK) return rc;
     auto kernel = &lstm_cell_fwd<Traits, true>;
-    const int grid = (B / Traits::kTM) * (kH / Traits::kTH);
+    const int grid = (B / Traits::kTM) * (H / Traits::kTH);
     for (int t = 0; t < T; ++t) {
-        const __half* x_t = x + size_t(t) * B * kI;
-        const __half* h_in = t == 0 ? h0 : h_all + size_t(t - 1) * B * kH;
+        const __half* x_t = x + size_t(t) * B * I;
+        const __half* h_in = t == 0 ? h0 : h_all + size_t(t - 1) * B * H;
         const float* c_in = t == 0 ? c0 : c_out;
-        __half* h_out = h_all + size_t(t) * B * kH;
-        const float* pre_t = pre + size_t(t) * B * 4 * kH;
+        __half* h_out = h_all + size_t(t) * B * H;
+        const float* pre_t = pre + size_t(t) * B * 4 * H;
         rc = launch(kernel, dim3(grid), dim3(Traits::kThreads), Traits::kLdsBytes, stream, x_t, h_in, W, bias, c_in,
-                    c_out, h_out, B, pre_t);
+                    c_out, h_out, B, pre_t, I, H);
         if (rc != TCU_OK) return lstm_step_failed(rc, t, T);
     }
     return TCU_OK;
@@ -576,19 +577,20 @@ int launch_lstm_ragged(const __half* x, const __half* W, const __half* bias, con
     return TCU_OK;
 }
 
+/// kI == kH == 0: the run-time-shape instantiation (I, H any multiples of 128).
 template <int kI, int kH>
 int launch_lstm_fwd(const __half* x, const __half* W, const __half* bias, const __half* h0, const float* c0,
-                    __half* h_all, float* c_out, int T, int B, hipStream_t stream) {
+                    __half* h_all, float* c_out, int T, int B, int I, int H, hipStream_t stream) {
     using Traits = LstmFwdTraits<kI, kH>;
     auto kernel = &lstm_cell_fwd<Traits>;
-    const int grid = (B / Traits::kTM) * (kH / Traits::kTH);
+    const int grid = (B / Traits::kTM) * (H / Traits::kTH);
     for (int t = 0; t < T; ++t) {
-        const __half* x_t = x + size_t(t) * B * kI;
-        const __half* h_in = t == 0 ? h0 : h_all + size_t(t - 1) * B * kH;
+        const __half* x_t = x + size_t(t) * B * I;
+        const __half* h_in = t == 0 ? h0 : h_all + size_t(t - 1) * B * H;
         const float* c_in = t == 0 ? c0 : c_out;
-        __half* h_out = h_all + size_t(t) * B * kH;
+        __half* h_out = h_all + size_t(t) * B * H;
         int rc = launch(kernel, dim3(grid), dim3(Traits::kThreads), Traits::kLdsBytes, stream, x_t, h_in, W, bias, c_in,
-                        c_out, h_out, B, static_cast<const float*>(nullptr));
+                        c_out, h_out, B, static_cast<const float*>(nullptr), I, H);
         if (rc != TCU_OK) return lstm_step_failed(rc, t, T);
     }
     return TCU_OK;
@@ -707,14 +709,13 @@ int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16: shapes are whole 16 x 16 tiles: B, I and H must be multiples of 16");
     if (algo == TCU_LSTM_RAGGED) return launch_lstm_ragged(xp, wp, bp, h0p, c0p, hp, cp, T, B, I, H, s);
     const bool b64 = B % 64 == 0;
-    if (algo != TCU_LSTM_TILE_LIBRARY && b64) {
-        if (I == 1024 && H == 1024) return launch_lstm_fwd<1024, 1024>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
-        if (I == 128 && H == 128) return launch_lstm_fwd<128, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
-        if (I == 256 && H == 128) return launch_lstm_fwd<256, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
+    if (algo != TCU_LSTM_TILE_LIBRARY && b64 && I % 128 == 0 && H % 128 == 0) {
+        // the benchmark shape with its sizes as constants; every other shape with the sizes as kernel arguments
+        if (I == 1024 && H == 1024) return launch_lstm_fwd<1024, 1024>(xp, wp, bp, h0p, c0p, hp, cp, T, B, I, H, s);
+        return launch_lstm_fwd<0, 0>(xp, wp, bp, h0p, c0p, hp, cp, T, B, I, H, s);
     }
     if (algo == TCU_LSTM_STREAMING)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE,
-                    "the streaming LSTM kernel is instantiated for (I, H) in {(1024,1024), (128,128), (256,128)}, B % 64 == 0");
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the streaming LSTM kernel needs I % 128 == 0, H % 128 == 0 and B % 64 == 0");
     if (b64) {
         if (I == 1024 && H == 1024)
             return launch_lstm<1024, 1024, 64, 16, 64, tl::RowMajor<4, 1>>(xp, wp, bp, h0p, c0p, hp, cp, T, B, s);
@@ -731,7 +732,7 @@ int tcu_lstm_f16_algo(const void* x, const void* W, const void* bias, const void
 }
 
 unsigned long long tcu_lstm_workspace_bytes(int T, int B, int I, int H) {
-    const bool shape_ok = (I == 1024 && H == 1024) || (I == 128 && H == 128) || (I == 256 && H == 128);
+    const bool shape_ok = I > 0 && H > 0 && I % 128 == 0 && H % 128 == 0 && (long)(I + H) * 512 < (1l << 32);
     if (!shape_ok || T <= 0 || B <= 0 || B % 64 != 0 || ((long)T * B) % 256 != 0) return 0;
     return (unsigned long long)T * B * 4 * H * sizeof(float);
 }
@@ -746,8 +747,8 @@ int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* 
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_ws: operands must be 16-byte aligned");
     const unsigned long long need = tcu_lstm_workspace_bytes(T, B, I, H);
     if (need == 0)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_ws: instantiated for (I, H) in {(1024,1024), (128,128), "
-                                               "(256,128)} with B % 64 == 0 and T * B % 256 == 0");
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_ws: needs I % 128 == 0, H % 128 == 0, B % 64 == 0 and "
+                                               "T * B % 256 == 0");
     if (workspace_bytes < need)
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_ws: workspace smaller than tcu_lstm_workspace_bytes()");
     auto s = static_cast<hipStream_t>(stream);
@@ -757,9 +758,8 @@ int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* 
     auto hp = static_cast<__half*>(h_all);
     auto cp = static_cast<float*>(c_out);
     auto pre = static_cast<float*>(workspace);
-    if (I == 1024 && H == 1024) return launch_lstm_hoisted<1024, 1024>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
-    if (I == 128 && H == 128) return launch_lstm_hoisted<128, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
-    return launch_lstm_hoisted<256, 128>(xp, wp, bp, h0p, c0p, hp, cp, T, B, pre, s);
+    if (I == 1024 && H == 1024) return launch_lstm_hoisted<1024, 1024>(xp, wp, bp, h0p, c0p, hp, cp, T, B, I, H, pre, s);
+    return launch_lstm_hoisted<0, 0>(xp, wp, bp, h0p, c0p, hp, cp, T, B, I, H, pre, s);
 }
 
 unsigned long long tcu_lstm_persistent_workspace_bytes(int T, int B, int I, int H) {
@@ -838,8 +838,8 @@ int tcu_lstm_f16_noalloc(const void* x, const void* W, const void* bias, const v
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_noalloc: operands must be 16-byte aligned");
     const unsigned long long need = tcu_lstm_workspace_bytes(T, B, I, H);
     if (need == 0)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_noalloc: instantiated for (I, H) in {(1024,1024), (128,128), "
-                                               "(256,128)} with B % 64 == 0 and T * B % 256 == 0");
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_noalloc: needs I % 128 == 0, H % 128 == 0, B % 64 == 0 and "
+                                               "T * B % 256 == 0");
     if (need > kScratchBytes)
         return fail(TCU_ERR_UNSUPPORTED_SHAPE,
                     "tcu_lstm_f16_noalloc: the gate pre-activations need " + std::to_string(need) +
