@@ -268,7 +268,7 @@ def main():
                "c": torch.empty(Bb, Hh, dtype=torch.float32, device=dev)}
 
         def lstm_step():
-            tcu.lstm(dx, dW, db, out=(out["h"], out["c"]))
+            tcu.lstm(dx, dW, db, out=(out["h"], out["c"]), workspace=False)  # one fused kernel per step
 
         ms = time_kernel(lstm_step, max(5, args.steps // 2), max(2, args.warmup // 2))
         # the 16 dependent step launches of a layer replayed from one HIP graph (the host out of the way)

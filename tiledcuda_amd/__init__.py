@@ -148,7 +148,8 @@ def gemm(a: torch.Tensor, b_t: torch.Tensor, out: torch.Tensor | None = None,
     Mirrors the reference's GEMM examples (A row-major, B column-major, f32 accumulate). With ``algo="auto"`` a
     product with few output tiles and a long K is split over K (``tcu_gemm_f16_ws``) through ``workspace`` (a contiguous
     device tensor of at least ``gemm_workspace_bytes(M, N, K)`` bytes), or, when none is given, through one taken from
-    torch's caching allocator for the call; ``workspace=False`` never splits.
+    torch's caching allocator for the call; ``workspace=False`` never splits (use it, or a workspace of your own, when
+    the call is being captured into a HIP graph: an allocation has no place in a captured stream).
     """
     M, K = a.shape
     N, K2 = b_t.shape
@@ -278,7 +279,7 @@ class TiledFlashAttention:
 
 # ------------------------------------------------------------------------------ LSTM
 def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor | None = None,
-         c0: torch.Tensor | None = None, algo: str = "auto", workspace: torch.Tensor | None = None,
+         c0: torch.Tensor | None = None, algo: str = "auto", workspace: torch.Tensor | None | bool = None,
          out: tuple[torch.Tensor, torch.Tensor] | None = None, check: bool = True
          ) -> tuple[torch.Tensor, torch.Tensor]:
     """Fused LSTM layer. x [T, B, I] f16, W [4H, I+H] f16 (gate rows i,f,g,o), bias [4H] f16,
@@ -286,7 +287,8 @@ def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor 
 
     ``algo="hoisted"`` computes the input half of the gates for all steps in one GEMM first (``tcu_lstm_f16_ws``); it
     needs ``lstm_workspace_bytes(T, B, I, H)`` bytes of device memory, taken from ``workspace`` (any dtype) if given,
-    else allocated here. ``out`` = (h_all, c_T) tensors to write into instead of allocating them.
+    else allocated here. ``algo="auto"`` takes that path where it applies and pays (I >= 512, T >= 4) unless
+    ``workspace=False`` (use that, or a workspace of your own, under HIP graph capture), else one fused kernel per step. ``out`` = (h_all, c_T) tensors to write into instead of allocating them.
 
     ``algo="persistent"`` runs the whole time loop in one weight-stationary launch after the same GEMM
     (``tcu_lstm_f16_persistent``: H = 1024, B <= 256 in multiples of 32; ``lstm_persistent_workspace_bytes``). Its
@@ -323,9 +325,11 @@ def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor 
         if check:
             lstm_persistent_status(workspace)
         return h_all, c_out
+    if algo == "auto" and workspace is not False and x.is_cuda and I >= 512 and T >= 4 and lstm_workspace_bytes(T, B, I, H) > 0:
+        algo = "hoisted"  # a long input size: its half of the gates is cheaper as one GEMM over all steps
     if algo == "hoisted":
         need = lstm_workspace_bytes(T, B, I, H)
-        if workspace is None:
+        if workspace is None or workspace is False:
             workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=x.device)
         if not workspace.is_cuda or not workspace.is_contiguous():
             raise ValueError("workspace must be a contiguous device tensor")

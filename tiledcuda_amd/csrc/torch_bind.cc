@@ -148,6 +148,16 @@ std::tuple<at::Tensor, at::Tensor> lstm(const at::Tensor& x, const at::Tensor& W
     c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
     at::Tensor h_all = at::empty({T, B, H}, x.options());
     at::Tensor c_out = at::empty({B, H}, x.options().dtype(at::kFloat));
+    // with a long input size the input half of the gates is cheaper as one GEMM over all steps; its [T, B, 4H] f32
+    // result lives in a block from torch's caching allocator (stream-ordered, returned when `ws` dies)
+    const unsigned long long need = tcu_lstm_workspace_bytes(int(T), int(B), int(I), int(H));
+    if (need > 0 && I >= 512 && T >= 4) {
+        at::Tensor ws = at::empty({static_cast<int64_t>(need)}, x.options().dtype(at::kByte));
+        check_status(tcu_lstm_f16_ws(x.data_ptr(), W.data_ptr(), bias.data_ptr(), h0p, c0p, h_all.data_ptr(), c_out.data_ptr(),
+                                     int(T), int(B), int(I), int(H), ws.data_ptr(), need, current_stream(x)),
+                     "lstm");
+        return {h_all, c_out};
+    }
     check_status(tcu_lstm_f16(x.data_ptr(), W.data_ptr(), bias.data_ptr(), h0p, c0p, h_all.data_ptr(), c_out.data_ptr(),
                               int(T), int(B), int(I), int(H), current_stream(x)),
                  "lstm");
