@@ -84,17 +84,6 @@ DEVICE void mfma32_score(f32x16& d, const f16x8& a, const f16x8& b) {
 DEVICE void mfma32_out(f32x16& d, const f16x8& a, const u32x4& b) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(d) : "v"(a), "v"(b));
 }
-/// f(integral_constant<int, 0>) ... f(integral_constant<int, kN - 1>): a loop whose index is a constant expression
-/// (wait counts and instruction offsets below are immediates).
-template <int kN, typename F, int... kIs>
-DEVICE void static_for_impl(F&& f, std::integer_sequence<int, kIs...>) {
-    (f(std::integral_constant<int, kIs>{}), ...);
-}
-template <int kN, typename F>
-DEVICE void static_for(F&& f) {
-    static_for_impl<kN>(f, std::make_integer_sequence<int, kN>{});
-}
-
 /// LDS fragment reads issued as inline assembly, so that the waits are the kernel's own: the compiler's waits for LDS
 /// reads it knows about are exact only inside a basic block; for fragments requested in one step of the pipeline
 /// and consumed in the next (across loop back edges and the branch of the rare path) it falls back to waiting for

@@ -23,6 +23,8 @@
 // M % kBM == 0, N % kBN == 0, K % kBK == 0 are required (checked by the host launcher).
 #pragma once
 
+#include <utility>
+
 #include "config.hpp"
 #include "hip_utils.hpp"
 
@@ -70,6 +72,17 @@ struct PipelinedGemmTraits {
 };
 
 namespace detail {
+
+/// f(integral_constant<int, 0>) ... f(integral_constant<int, kN - 1>): a loop whose index is a constant expression
+/// (wait counts and instruction offsets below are immediates).
+template <int kN, typename F, int... kIs>
+DEVICE void static_for_impl(F&& f, std::integer_sequence<int, kIs...>) {
+    (f(std::integral_constant<int, kIs>{}), ...);
+}
+template <int kN, typename F>
+DEVICE void static_for(F&& f) {
+    static_for_impl<kN>(f, std::make_integer_sequence<int, kN>{});
+}
 
 using lds_ptr_t = __attribute__((address_space(3))) void*;
 using glb_ptr_t = const __attribute__((address_space(1))) void*;

@@ -52,12 +52,17 @@ typedef enum {
                                 tiles beyond the edge skipped; the fallback for shapes the tiled kernels do not cover */
 } tcu_gemm_algo;
 
-/* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks RESIDENT where it is instantiated. */
+/* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks ROWS for many rows, else RESIDENT, where
+ * they apply. */
 typedef enum {
     TCU_B2B_AUTO = 0,
     TCU_B2B_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, the reference kernel's structure */
-    TCU_B2B_RESIDENT = 2      /* A tile, 256-column blocks of B and C and the intermediate resident in LDS (K = P = 128,
+    TCU_B2B_RESIDENT = 2,     /* A tile, 256-column blocks of B and C and the intermediate resident in LDS (K = P = 128,
                                  N % 256 == 0, M % 32 == 0); one round of loads per block */
+    TCU_B2B_ROWS = 3          /* for many rows (AUTO from M x batch = 32768): N = 256, K = P = 128, M % 64 == 0; a
+                                 workgroup keeps B and C in LDS and walks over blocks of 256 rows, every wavefront owning
+                                 64 rows (A fragments from global memory, the intermediate stays in registers); agrees
+                                 with RESIDENT up to the order of the f32 sums inside an MFMA */
 } tcu_b2b_algo;
 
 /* Layout of V in tcu_flash_attn_fwd_f16. */

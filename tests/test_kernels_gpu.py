@@ -424,6 +424,49 @@ def test_b2b_gemm_both_kernels_at_256x128x128(tcu, oracle, device, algo, M, batc
         assert torch.equal(D1[0], want)
 
 
+@pytest.mark.parametrize("M,batch,out_dtype", [(64, 1, "f32"), (192, 3, "f16"), (320, 2, "f32"), (8192, 1, "f16"),
+                                               (65536, 1, "f16"), (4096, 40, "f32")])
+def test_b2b_gemm_many_rows_kernel(tcu, oracle, device, M, batch, out_dtype):
+    """(N, K, P) = (256, 128, 128) with the kernel for many rows: workgroups that keep both weight blocks and walk over
+    blocks of 256 rows, a wavefront owning 64 rows (its intermediate never leaves its registers). One wavefront, partly
+    filled blocks, several blocks per workgroup, batches with more items than workgroups per item; against the oracle on
+    rows from the first, a middle and the last block, against the LDS-resident kernel everywhere, a one-hot probe of the
+    index maps; AUTO takes this kernel from 32768 rows."""
+    import torch
+
+    print(f"b2b rows M{M} b{batch} {out_dtype}", flush=True)
+    N, K, P = 256, 128, 128
+    A = oracle.fill_normal(batch * M * K, 171, 0, 0.1).reshape(batch, M, K)
+    Bt = oracle.fill_normal(batch * N * K, 172, 0, 0.1).reshape(batch, N, K)
+    Ct = oracle.fill_normal(batch * P * N, 173, 0, 0.1).reshape(batch, P, N)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    dA, dB, dC = dev(A, device), dev(Bt, device), dev(Ct, device)
+    D = tcu.b2b_gemm(dA, dB, dC, out_dtype=dt, algo="rows")
+    torch.cuda.synchronize()
+    rows = sorted(set(list(range(0, min(M, 64))) + list(range(M // 2, min(M, M // 2 + 32))) + list(range(M - 32, M))))
+    items = sorted({0, batch - 1})
+    ref = oracle.b2b_gemm(np.ascontiguousarray(A[items][:, rows]), Bt[items], Ct[items])
+    assert oracle.max_rel_err(host(D)[items][:, rows], ref, eps=1.0) <= REL_TOL
+    other = tcu.b2b_gemm(dA, dB, dC, out_dtype=dt, algo="resident")
+    assert oracle.max_rel_err(host(D), host(other), eps=1.0) <= REL_TOL
+    if (long_enough := M * batch >= 32768):
+        assert torch.equal(D, tcu.b2b_gemm(dA, dB, dC, out_dtype=dt, algo="auto"))
+    if M == 192:
+        A1 = torch.zeros(1, 192, K, dtype=torch.float16, device=device)
+        B1 = torch.zeros(1, N, K, dtype=torch.float16, device=device)
+        C1 = torch.zeros(1, P, N, dtype=torch.float16, device=device)
+        for i, (m, k, n, p) in enumerate([(0, 0, 0, 0), (191, 127, 255, 127), (37, 5, 200, 66), (64, 77, 13, 1),
+                                          (130, 40, 147, 93)]):
+            A1[0, m, k] = 1.0 + i
+            B1[0, n, k] = 2.0
+            C1[0, p, n] = 0.5
+        D1 = tcu.b2b_gemm(A1, B1, C1, out_dtype=torch.float32, algo="rows")
+        want = (A1[0].float() @ B1[0].float().T) @ C1[0].float().T
+        assert torch.equal(D1[0], want)
+    with pytest.raises(RuntimeError):
+        tcu.b2b_gemm(dA[:, :32].contiguous(), dB, dC, algo="rows")  # M must be a multiple of 64
+
+
 def test_kernels_in_a_hip_graph_replay_like_eager(tcu, oracle, device):
     """Launch-bound callers capture these entry points in HIP graphs: several replays, with eager work and
     synchronisations in between, each give the eager result (operands changed between replays)."""

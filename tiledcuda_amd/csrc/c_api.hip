@@ -381,8 +381,20 @@ int launch_b2b(const __half* A, const __half* B, const __half* C, OutType* D, in
 template <typename OutType>
 int b2b_dispatch(const __half* A, const __half* B, const __half* C, OutType* D, int M, int N, int K, int P, int batch,
                  int algo, hipStream_t stream) {
-    if (algo != TCU_B2B_AUTO && algo != TCU_B2B_TILE_LIBRARY && algo != TCU_B2B_RESIDENT)
+    if (algo != TCU_B2B_AUTO && algo != TCU_B2B_TILE_LIBRARY && algo != TCU_B2B_RESIDENT && algo != TCU_B2B_ROWS)
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: unknown algo");
+    // many rows: workgroups that keep both weight blocks for their whole life and walk over blocks of 256 rows
+    if (algo == TCU_B2B_ROWS || (algo == TCU_B2B_AUTO && (long)M * batch >= 32768)) {
+        if (N == 256 && K == 128 && P == 128 && M % 64 == 0) {
+            using T = B2bRowsTraits;
+            const int blocks = (M + T::kRowsPerBlock - 1) / T::kRowsPerBlock;
+            const int per_item = std::max(1, 256 / batch);  // one workgroup per CU: about 256 in all
+            return launch(&b2b_gemm_rows<OutType>, dim3(std::min(blocks, per_item), batch), dim3(T::kThreads), T::kLdsBytes,
+                          stream, A, B, C, D, M);
+        }
+        if (algo == TCU_B2B_ROWS)
+            return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the many-rows b2b kernel takes N = 256, K = P = 128 and M a multiple of 64");
+    }
     if (algo != TCU_B2B_TILE_LIBRARY) {
         if (N % 256 == 0 && K == 128 && P == 128 && M % 32 == 0)
             return launch(&b2b_gemm_resident<OutType>, dim3(M / B2bResidentTraits::kTM, batch),
