@@ -333,11 +333,12 @@ __global__ void __launch_bounds__(B2bRowsTraits::kThreads)
                         else detail::mfma_16x16x32_agpr(acc1[nt][mt], fb[idx % kRing], fa[mt][s]);
                     }
                 });
-                // MFMA results may be read by other instructions only a number of cycles after issue, and the compiler
-                // does not know the statements above are MFMAs: every accumulator passes through a statement that waits
+                // the compiler does not know the statements above are MFMAs: wait once for the last results, then pass every
+                // accumulator through a statement that comes after the wait
+                detail::mfma_results_wait();
 #pragma unroll
                 for (int nt = 0; nt < 8; ++nt)
-                    asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc1[nt][0]), "+a"(acc1[nt][1]), "+a"(acc1[nt][2]), "+a"(acc1[nt][3]));
+                    asm volatile("" : "+a"(acc1[nt][0]), "+a"(acc1[nt][1]), "+a"(acc1[nt][2]), "+a"(acc1[nt][3]));
 
                 // ---- second product over this half's n: contraction step s2 covers n = 128 half + 32 s2 .. + 31, lane
                 // group g holding n = .. + 4 g .. + 3 and .. + 16 + 4 g .. + 3 (the two halves of its operand); fragment
@@ -375,9 +376,10 @@ __global__ void __launch_bounds__(B2bRowsTraits::kThreads)
                     if constexpr (pt == 2 && s2 + 1 < 4) convert(std::integral_constant<int, s2 + 1>{});
                 });
             });
+            detail::mfma_results_wait();
 #pragma unroll
             for (int pt = 0; pt < 8; ++pt)
-                asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc2[pt][0]), "+a"(acc2[pt][1]), "+a"(acc2[pt][2]), "+a"(acc2[pt][3]));
+                asm volatile("" : "+a"(acc2[pt][0]), "+a"(acc2[pt][1]), "+a"(acc2[pt][2]), "+a"(acc2[pt][3]));
 #pragma unroll
             for (int pt = 0; pt < 8; ++pt)
 #pragma unroll

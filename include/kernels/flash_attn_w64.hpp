@@ -123,8 +123,9 @@ DEVICE unsigned int pack_f16x2(float a, float b) {
 
 /// Wait long enough for every MFMA issued so far to have written its result (32 wait states cover the longest
 /// requirement) before `x` is touched by anything else.
-DEVICE void mfma_settle_v(f32x16& x) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(x)); }
-DEVICE void mfma_settle_a(f32x16& x) { asm volatile("s_nop 15\n\ts_nop 15" : "+a"(x)); }
+/// After detail::mfma_results_wait(): the accumulator is read only behind that wait.
+DEVICE void mfma_settle_v(f32x16& x) { asm volatile("" : "+v"(x)); }
+DEVICE void mfma_settle_a(f32x16& x) { asm volatile("" : "+a"(x)); }
 
 }  // namespace detail
 
@@ -389,6 +390,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
 
     // ---- half 0: exact maximum
     qk_only(0, std::integral_constant<int, 0>{}, q_via_lds ? 1 : 0);
+    detail::mfma_results_wait();
     detail::mfma_settle_v(s_acc[0][0]);
     detail::mfma_settle_v(s_acc[0][1]);
 #pragma unroll
@@ -499,6 +501,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         constexpr float kLimit = 16384.f;
         if (__any(!(fmaxf(lh[0], lh[1]) <= kLimit))) {
             // rare path: move the reference maxima, rescale, re-bias, recompute
+            detail::mfma_results_wait();
             if (kQk) {
                 detail::mfma_settle_v(s_acc[kNxt][0]);
                 detail::mfma_settle_v(s_acc[kNxt][1]);
@@ -608,6 +611,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     }
 
     // ---- epilogue: O[q, d] = Oᵀ[d, q] / l. o_acc[dt][c][r]: d = 32 dt + 8 (r / 4) + 4 h + r % 4, q = 32 c + q32.
+    detail::mfma_results_wait();
 #pragma unroll
     for (int dt = 0; dt < Traits::kDTiles; ++dt)
 #pragma unroll

@@ -124,6 +124,14 @@ DEVICE void wait_vmcnt() {
     asm volatile("" ::: "memory");
 }
 
+/// MFMA results may be read by other instructions only a number of issue slots after the MFMA was issued, and where
+/// the MFMAs are assembly statements the compiler does not know that and would not wait. One call of this after the
+/// last MFMA (20 issue slots of 4 cycles each: the longest requirement, that of a 16-pass instruction, is 19), then
+/// every accumulator passes through an (empty) volatile statement of its own before it is read: volatile statements
+/// keep their order, so all of those come after this one. An s_nop of N + 1 slots costs 4 (N + 1) cycles - a wait per
+/// accumulator, which is how this was first written, cost the GEMM epilogue 1024 cycles instead of 80.
+DEVICE void mfma_results_wait() { asm volatile("s_nop 15\n\ts_nop 3"); }
+
 /// Workgroup barrier that orders LDS accesses only. __syncthreads() also waits for every outstanding global memory
 /// operation of the wavefront (s_waitcnt vmcnt(0): its workgroup fence covers the LDS writes of direct-to-LDS loads),
 /// which would drain a ring of stages at every hand-over: tiles requested ahead must stay in flight across the barrier.

@@ -230,12 +230,12 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
         tile(kt, std::false_type{}, std::false_type{});
     }
 
-    // MFMA results may be read by other instructions only a number of cycles after the MFMA was issued, and the
-    // compiler, not knowing the statements above are MFMAs, would not wait: every accumulator passes through a
-    // statement that waits first (32 wait states cover the longest requirement).
+    // the compiler does not know the statements above are MFMAs: wait once for the last results, then pass every
+    // accumulator through a statement that comes after the wait
+    detail::mfma_results_wait();
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-        asm volatile("s_nop 15\n\ts_nop 15"
+        asm volatile(""
                      : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),
                        "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]));
 

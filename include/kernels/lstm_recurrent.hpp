@@ -272,9 +272,9 @@ __global__ void __launch_bounds__(Traits::kThreads)
             else detail::lds_barrier<0>();
             mfma_piece(fa, fb, 2);
             mfma_piece(fb, fa, 3);
-            // MFMA results may be read by other instructions only a number of cycles after issue, and the compiler
-            // does not know the statements above are MFMAs: wait here (32 wait states cover the longest requirement)
-            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0), "+v"(acc1));
+            // the compiler does not know the statements above are MFMAs: wait for the last results
+            detail::mfma_results_wait();
+            asm volatile("" : "+v"(acc0), "+v"(acc1));
         }
 
         // ---- cell update and this lane's 4 units of h_t
