@@ -199,13 +199,16 @@ __global__ void __launch_bounds__(Traits::kThreads)
         }
         ldst[j] = (is_v ? Traits::kTileBytes : 0) + t * 1024;
     }
-    auto issue_load = [&](int block, int j) {
+    // stage_off: byte offset of the block's ring stage, (block % kStages) * kStageBytes (the loop keeps the offsets it
+    // needs as running values: a remainder by 5 is a dozen scalar instructions, and every instruction of a lone wavefront
+    // takes an issue slot)
+    auto issue_load_at = [&](unsigned int stage_off, int block, int j) {
         const bool is_v = j >= kL / 2;
         const __half* src = (is_v && kVColMajor) ? Vh + size_t(block) * kBN : (is_v ? Vh : Kh) + size_t(block) * kBN * kD;
-        const unsigned int dst =
-            __builtin_amdgcn_readfirstlane(lds_base + (block % kStages) * Traits::kStageBytes + ldst[j]);
+        const unsigned int dst = __builtin_amdgcn_readfirstlane(lds_base + stage_off + ldst[j]);
         detail::load_lds_16B_sbase(goff[j], src, dst);
     };
+    auto issue_load = [&](int block, int j) { issue_load_at((block % kStages) * Traits::kStageBytes, block, j); };
 
     using C0 = std::integral_constant<int, 0>;
     using C1 = std::integral_constant<int, 1>;
@@ -425,14 +428,20 @@ __global__ void __launch_bounds__(Traits::kThreads)
     constexpr int kReadsV = kVColMajor ? 1 : 2, kReadsQk = kReadsV + 1;
     static_assert(8 % kRing == 0 && kAhead <= 3, "ring positions must repeat from one step to the next; the prefetch stays within the first k-step of the next half");
     f16x8 kf[kRing], vf[kRing];
-    auto step = [&](int i, auto cur_c, auto qk_c, auto loads_c, auto next_qk_c, int load_block) {
+    // Step i = 2 J + 1 (kCur = 1) or 2 J + 2 (kCur = 0) touches blocks J, J + 1, J + 2: `ring` holds their stage offsets
+    // and that of the block being loaded.
+    struct RingOffsets {
+        unsigned int a, b, c, load;
+    };
+    auto step = [&](const RingOffsets& ring, auto cur_c, auto qk_c, auto loads_c, auto next_qk_c, int load_block) {
         constexpr int kCur = decltype(cur_c)::value, kNxt = kCur ^ 1;
         constexpr bool kQk = decltype(qk_c)::value, kLoads = decltype(loads_c)::value;
         constexpr bool kNextQk = decltype(next_qk_c)::value;
-        const unsigned int sk = __builtin_amdgcn_readfirstlane(k_half(i + 1));
-        const unsigned int sv = __builtin_amdgcn_readfirstlane(v_block(i - 1));  // key half kNxt of that block
-        const unsigned int sk_next = __builtin_amdgcn_readfirstlane(k_half(i + 2));
-        const unsigned int sv_next = __builtin_amdgcn_readfirstlane(v_block(i));  // key half kCur of that block
+        // K of half i + 1 (block J + 1; its first half for odd i), V of half i - 1 (block J), K of half i + 2, V of half i
+        const unsigned int sk = ring.b + (kCur == 1 ? 0 : Traits::kHalfBytes);
+        const unsigned int sv = ring.a + Traits::kTileBytes;  // key half kNxt of that block
+        const unsigned int sk_next = kCur == 1 ? ring.b + Traits::kHalfBytes : ring.c;
+        const unsigned int sv_next = (kCur == 1 ? ring.a : ring.b) + Traits::kTileBytes;  // key half kCur of that block
         float lh[2] = {0.f, 0.f}, lg[2] = {0.f, 0.f};  // two partial sums per query tile (independent add chains)
         // VALU work of the same wavefront hides under its MFMAs only in small doses: one v_exp_f32 plus one or two
         // plain instructions directly behind each MFMA cost 2-3 cycles per MFMA, the same instructions in groups of
@@ -478,7 +487,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 lh[1] += y0;
                 lg[1] += y1;
             }
-            if (kLoads) issue_load(load_block, s);
+            if (kLoads) issue_load_at(ring.load, load_block, s);
             __builtin_amdgcn_sched_barrier(0);
             // slot C
             detail::mfma32_out(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2]);
@@ -568,30 +577,42 @@ __global__ void __launch_bounds__(Traits::kThreads)
         vf[a] = read_v_untracked(v_block(0), C0{}, C0{}, a & 3);
     }
     // ---- block-iterations: J covers halves 2 J + 1 (odd) and 2 J + 2 (even)
+    constexpr unsigned int kStageB = Traits::kStageBytes, kRingB = kStages * Traits::kStageBytes;
+    auto next_stage = [&](unsigned int off) { return off + kStageB == kRingB ? 0u : off + kStageB; };
     int J = 0;
+    RingOffsets ring{0u, kStageB, 2 * kStageB, 4 * kStageB};  // blocks 0, 1, 2; block J + 4 is loaded
+    auto advance = [&]() {
+        ring.a = ring.b;
+        ring.b = ring.c;
+        ring.c = next_stage(ring.c);
+        ring.load = next_stage(ring.load);
+        ++J;
+    };
     if (q_via_lds) {
         // J = 0: blocks 3 and 4 go to the stages the Q tiles were staged in (everyone has read its Q by now)
         hand_over(std::integral_constant<int, 0>{});
-        step(1, C1{}, Yes{}, Yes{}, Yes{}, 3);
-        step(2, C0{}, Yes{}, Yes{}, Yes{}, 4);
-        J = 1;
+        RingOffsets first = ring;
+        first.load = 3 * kStageB;
+        step(first, C1{}, Yes{}, Yes{}, Yes{}, 3);
+        step(ring, C0{}, Yes{}, Yes{}, Yes{}, 4);
+        advance();
     }
-    for (; J + 4 < nb; ++J) {
+    for (; J + 4 < nb; advance()) {
         hand_over(std::integral_constant<int, kL>{});
-        step(2 * J + 1, C1{}, Yes{}, Yes{}, Yes{}, J + 4);
-        step(2 * J + 2, C0{}, Yes{}, No{}, Yes{}, 0);
+        step(ring, C1{}, Yes{}, Yes{}, Yes{}, J + 4);
+        step(ring, C0{}, Yes{}, No{}, Yes{}, 0);
     }
-    for (; J + 2 < nb; ++J) {
+    for (; J + 2 < nb; advance()) {
         hand_over(std::integral_constant<int, 0>{});
-        step(2 * J + 1, C1{}, Yes{}, No{}, Yes{}, 0);
-        step(2 * J + 2, C0{}, Yes{}, No{}, Yes{}, 0);
+        step(ring, C1{}, Yes{}, No{}, Yes{}, 0);
+        step(ring, C0{}, Yes{}, No{}, Yes{}, 0);
     }
     if (J + 1 < nb) {
-        step(2 * J + 1, C1{}, Yes{}, No{}, Yes{}, 0);
-        step(2 * J + 2, C0{}, Yes{}, No{}, No{}, 0);
-        ++J;
+        step(ring, C1{}, Yes{}, No{}, Yes{}, 0);
+        step(ring, C0{}, Yes{}, No{}, No{}, 0);
+        advance();
     }
-    step(2 * J + 1, C1{}, No{}, No{}, No{}, 0);
+    step(ring, C1{}, No{}, No{}, No{}, 0);
     {
         // the output update with the last half (its first fragments were requested by the step before)
         const unsigned int sv = v_block(2 * J + 1);
