@@ -84,6 +84,18 @@ DEVICE void mfma32_score(f32x16& d, const f16x8& a, const f16x8& b) {
 DEVICE void mfma32_out(f32x16& d, const f16x8& a, const u32x4& b) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(d) : "v"(a), "v"(b));
 }
+/// The same MFMA, then a direct-to-LDS load of 16 bytes per lane from sbase + voff to lds_addr + 16 * lane: m0 is written
+/// before the MFMA, which thereby is the wait state required between the write of m0 and the load (no s_nop).
+DEVICE void mfma32_out_then_load(f32x16& d, const f16x8& a, const u32x4& b, unsigned int voff, const void* sbase,
+                                 unsigned int lds_addr) {
+    asm volatile(
+        "s_mov_b32 m0, %5\n\t"
+        "v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\t"
+        "global_load_lds_dwordx4 %3, %4"
+        : "+a"(d)
+        : "v"(a), "v"(b), "v"(voff), "s"(sbase), "s"(lds_addr)
+        : "m0", "memory");
+}
 /// LDS fragment reads issued as inline assembly, so that the waits are the kernel's own: the compiler's waits for LDS
 /// reads it knows about are exact only inside a basic block; for fragments requested in one step of the pipeline
 /// and consumed in the next (across loop back edges and the branch of the rare path) it falls back to waiting for
@@ -487,10 +499,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 lh[1] += y0;
                 lg[1] += y1;
             }
-            if (kLoads) issue_load_at(ring.load, load_block, s);
             __builtin_amdgcn_sched_barrier(0);
-            // slot C
-            detail::mfma32_out(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2]);
+            // slot C (with this wavefront's load s of the block being fetched riding on the MFMA)
+            if (kLoads) {
+                const bool is_v = s >= kL / 2;
+                const __half* src = (is_v && kVColMajor) ? Vh + size_t(load_block) * kBN
+                                                         : (is_v ? Vh : Kh) + size_t(load_block) * kBN * kD;
+                const unsigned int dst = __builtin_amdgcn_readfirstlane(lds_base + ring.load + ldst[s]);
+                detail::mfma32_out_then_load(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2], goff[s], src, dst);
+            } else {
+                detail::mfma32_out(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2]);
+            }
             y0 = ex(s_acc[kCur][1][2 * s]);
             pack_pair(C0{}, s_c, x0, x1);
             __builtin_amdgcn_sched_barrier(0);
