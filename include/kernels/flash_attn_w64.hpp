@@ -495,7 +495,10 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 else detail::mfma32_score(s_acc[kNxt][1], kf[s % kRing], qf[1][s]);
             }
             x1 = ex(s_acc[kCur][0][2 * s + 1]);
-            if constexpr (s > 0) {
+            if constexpr (s == 1) {  // the first pair starts the sums (no addition to zero: every instruction is a slot)
+                lh[1] = y0;
+                lg[1] = y1;
+            } else if constexpr (s > 1) {
                 lh[1] += y0;
                 lg[1] += y1;
             }
@@ -516,8 +519,13 @@ __global__ void __launch_bounds__(Traits::kThreads)
             // slot D
             detail::mfma32_out(o_acc[s & 3][1], vf[s % kRing], pf[kNxt][1][s >> 2]);
             y1 = ex(s_acc[kCur][1][2 * s + 1]);
-            lh[0] += x0;
-            lg[0] += x1;
+            if constexpr (s == 0) {
+                lh[0] = x0;
+                lg[0] = x1;
+            } else {
+                lh[0] += x0;
+                lg[0] += x1;
+            }
             __builtin_amdgcn_sched_barrier(0);
         });
         lh[1] += y0;
