@@ -14,6 +14,9 @@ Prints ONE JSON line: the driver's contract fields plus
                   is the practical ceiling; the published peak assumes 2.4 GHz)
   cpu_baseline -- the reference's CPU path (fp32 torch.matmul; fp32 softmax(QK^T)V on a sample of heads) and the
                   OpenMP oracle, timed on this host's cores for the same workloads
+  vendor_library_same_run -- hipBLASLt (through torch.matmul) on the headline operands and torch's fused attention on
+                  the C4 operands, timed after the figures above in the same process, with this library re-timed beside
+                  them: boxes of the pool differ by several percent, only a same-run ratio says who is ahead
 """
 from __future__ import annotations
 
@@ -141,6 +144,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--only", default="", help="comma-separated subset of gemm,c1,b2b,attn,lstm,scatter (gemm always runs)")
     ap.add_argument("--no-mfma-probe", action="store_true", help="skip the sustained-MFMA-rate measurement")
+    ap.add_argument("--no-vendor", action="store_true",
+                    help="skip the vendor-library comparison (hipBLASLt through torch.matmul, torch's fused attention)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 128 MiB (read 128 MiB, write 128 MiB) a few times, so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command has a kernel of known traffic to "
@@ -187,6 +192,8 @@ def main():
 
     def gemm_step():
         tcu.gemm(dA, dB, out=dC)
+
+    vendor_attention = None
 
     # ---------------------------------------------------------------- C1: GEMM 128x64x256
     if want("c1"):
@@ -248,6 +255,14 @@ def main():
         err_op = oracle.max_abs_err(do2.reshape(B * H, S, D)[5, 1024:1088].float().cpu().numpy(),
                                     oracle.attention(q[5], k[5], v[5], scale, rows=(1024, 1088))[1024:1088])
         del dvt, do2
+        if not args.no_vendor:
+            sdpa = torch.nn.functional.scaled_dot_product_attention
+            ms_sdpa = time_kernel(lambda: sdpa(dq, dk, dv), 20, 30)
+            ms_again = time_kernel(lambda: tcu.flash_attention(dq, dk, dv, out=do), 20, 30)
+            vendor_attention = {"torch_sdpa_us": ms_sdpa * 1e3, "this_library_us": ms_again * 1e3,
+                                "speed_vs_torch_sdpa": ms_sdpa / ms_again,
+                                "method": "torch.nn.functional.scaled_dot_product_attention on the same tensors, "
+                                          "30 untimed + 20 timed launches each"}
         configs.append({"name": "flash_attn_fwd_b4_h16_s2048_d128", "kernel": "flash_attention_fwd_w64<128>", "ms": ms,
                         "first_launches_us": ms_first * 1e3, "conditioning_launches": 200,
                         "tflops": flops / (ms * 1e-3) / 1e12,
@@ -386,6 +401,37 @@ def main():
                "avg_launch_us": settled_us,
                "achieved": gemm_flops / settled_us / 1e6, "frac": gemm_flops / settled_us / 1e6 / MFMA_F16_PEAK_TFLOPS}
 
+    # the vendor library on the same operands, in the same process and power state (a comparison beside the figure above,
+    # never part of it): hipBLASLt through torch.matmul, and this library again directly after it, 150 untimed + 100
+    # timed launches each, twice; torch's fused attention on the C4 operands when that configuration ran
+    vendor = None
+    if not args.no_vendor:
+        dC2 = torch.empty_like(dC)
+
+        def settled_us_of(fn):
+            for _ in range(150):
+                fn()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(100):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) * 1e3 / 100
+
+        blas_us, ours_us = [], []
+        for _ in range(2):
+            blas_us.append(settled_us_of(lambda: torch.matmul(dA, dB.t(), out=dC2)))
+            ours_us.append(settled_us_of(gemm_step))
+        vendor = {"gemm_4096": {"hipblaslt_torch_matmul_us": min(blas_us), "this_library_us": min(ours_us),
+                                "hipblaslt_tflops": gemm_flops / min(blas_us) / 1e6,
+                                "this_library_tflops": gemm_flops / min(ours_us) / 1e6,
+                                "speed_vs_hipblaslt": min(blas_us) / min(ours_us),
+                                "method": "interleaved, 150 untimed + 100 timed launches each, best of 2"}}
+        del dC2
+        if vendor_attention is not None:
+            vendor["flash_attn_fwd_b4_h16_s2048_d128"] = vendor_attention
+
     rows = (1920, 2048)
     ref = oracle.gemm(A, Bt, rows=rows)
     gemm_err = oracle.max_rel_err(dC[rows[0]:rows[1]].float().cpu().numpy(), ref[rows[0]:rows[1]])
@@ -461,6 +507,7 @@ def main():
                      "sustained_mfma": sustained,
                      "frac_of_sustained_mfma": (gemm_tflops / sustained["tflops"]) if sustained else None},
         "cpu_baseline": cpu,
+        "vendor_library_same_run": vendor,
         "max_rel_err": gemm_err,
         "configs": configs,
         "device": torch.cuda.get_device_name(0),

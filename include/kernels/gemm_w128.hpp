@@ -186,6 +186,9 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 
     // Order of the 16 fragment reads of a phase: row group 0 of the next phase needs A fragment 0 and all B fragments.
     constexpr int kOrder[16] = {0, 8, 9, 10, 11, 12, 13, 14, 15, 1, 2, 3, 4, 5, 6, 7};
+    // MFMA n of row group i works on tile (i, j): odd row groups walk their tiles backwards, so that one operand of
+    // every MFMA, also the first of a row group, is the operand of the MFMA before it
+    auto snake = [](int i, int n) { return (i & 1) ? 7 - n : n; };
 
     // One tile of K. kMore: there is a tile kt+1 (read its substep 0 during phase 2); kMore2: there is a tile kt+2
     // (load it during phase 2). Row group i = MFMA tiles (i, 0..7): the MFMA order is fixed by the asm statements, the
@@ -196,9 +199,10 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int r = 4 * i + (j >> 1);
-                if ((j & 1) == 0 && r < 16) fy[kOrder[r]] = read_frag(stage, 1, kOrder[r]);
+            for (int n = 0; n < 8; ++n) {
+                const int j = snake(i, n);
+                const int r = 4 * i + (n >> 1);
+                if ((n & 1) == 0 && r < 16) fy[kOrder[r]] = read_frag(stage, 1, kOrder[r]);
                 detail::mfma_16x16x32_agpr(acc[i][j], fx[8 + j], fx[i]);
             }
         }
@@ -207,11 +211,12 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int r = 4 * i + (j >> 1);
-                if (kMore && (j & 1) == 0 && r < 16) fx[kOrder[r]] = read_frag(stage ^ 1, 0, kOrder[r]);
-                if (kMore2 && (j & 3) == 1) {
-                    const int q = 2 * i + (j >> 2);
+            for (int n = 0; n < 8; ++n) {
+                const int j = snake(i, n);
+                const int r = 4 * i + (n >> 1);
+                if (kMore && (n & 1) == 0 && r < 16) fx[kOrder[r]] = read_frag(stage ^ 1, 0, kOrder[r]);
+                if (kMore2 && (n & 3) == 1) {
+                    const int q = 2 * i + (n >> 2);
                     detail::mfma_16x16x32_agpr_then_load(acc[i][j], fy[8 + j], fy[i], voff[q], load_src(kt + 2, q),
                                                          load_dst(stage, q));
                 } else {
