@@ -445,9 +445,11 @@ __global__ void __launch_bounds__(Traits::kThreads)
     struct RingOffsets {
         unsigned int a, b, c, load;
     };
+    const __half *warm_a = Kh, *warm_b = Kh;  // two 16 KiB runs that a step with warm-up loads fetches
     auto step = [&](const RingOffsets& ring, auto cur_c, auto qk_c, auto loads_c, auto next_qk_c, int load_block) {
         constexpr int kCur = decltype(cur_c)::value, kNxt = kCur ^ 1;
-        constexpr bool kQk = decltype(qk_c)::value, kLoads = decltype(loads_c)::value;
+        constexpr bool kQk = decltype(qk_c)::value;
+        constexpr int kLoads = decltype(loads_c)::value;  // 0: none, 1: block `load_block` of K and V, 2: warm-up loads
         constexpr bool kNextQk = decltype(next_qk_c)::value;
         // K of half i + 1 (block J + 1; its first half for odd i), V of half i - 1 (block J), K of half i + 2, V of half i
         const unsigned int sk = ring.b + (kCur == 1 ? 0 : Traits::kHalfBytes);
@@ -504,12 +506,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
             }
             __builtin_amdgcn_sched_barrier(0);
             // slot C (with this wavefront's load s of the block being fetched riding on the MFMA)
-            if (kLoads) {
+            if constexpr (kLoads == 1) {
                 const bool is_v = s >= kL / 2;
                 const __half* src = (is_v && kVColMajor) ? Vh + size_t(load_block) * kBN
                                                          : (is_v ? Vh : Kh) + size_t(load_block) * kBN * kD;
                 const unsigned int dst = __builtin_amdgcn_readfirstlane(lds_base + ring.load + ldst[s]);
                 detail::mfma32_out_then_load(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2], goff[s], src, dst);
+            } else if constexpr (kLoads == 2) {
+                // 1 KiB of the 16 KiB run at warm_a (s < 4) or warm_b; the four wavefronts cover both runs
+                const __half* src = (s < kL / 2 ? warm_a : warm_b) + (wave * (kL / 2) + (s & 3)) * 512;
+                const unsigned int dst = __builtin_amdgcn_readfirstlane(lds_base + ring.load + ldst[s]);
+                detail::mfma32_out_then_load(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2], lane * 16u, src, dst);
             } else {
                 detail::mfma32_out(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2]);
             }
@@ -629,6 +636,42 @@ __global__ void __launch_bounds__(Traits::kThreads)
         step(ring, C1{}, Yes{}, Yes{}, Yes{}, J + 4);
         step(ring, C0{}, Yes{}, No{}, Yes{}, 0);
     }
+    // The workgroup that follows this one on the XCD (256 workgroups are resident, ids congruent mod 8 share an XCD:
+    // id + 256) starts with a cold burst: its 256 query rows and the first block of its item's K and V. With no ring
+    // loads left to issue, three of the last steps fetch those 96 KiB instead, into the ring stage that was vacated
+    // last (the data is discarded: the point is that the lines are in this XCD's L2 when the next workgroup asks).
+    {
+        const unsigned int nid = blockIdx.x + 256;
+        if (q_via_lds && nid < gridDim.x && J + 4 == nb) {  // two more block-iterations follow
+            int nhead, nqb;
+            if (batch % 8 == 0) {
+                const int xcd = nid & 7, rest = nid >> 3;
+                nqb = rest % q_blocks;
+                nhead = (rest / q_blocks) * 8 + xcd;
+            } else {
+                nqb = nid % q_blocks;
+                nhead = nid / q_blocks;
+            }
+            const int rows0 = nqb * Traits::kBM;
+            // 64 query rows from row r of that workgroup's block (M % 64 == 0; rows beyond M: the last 64 instead)
+            auto qrows = [&](int r) { return Q + (size_t(nhead) * M + (rows0 + r < M ? rows0 + r : M - 64)) * kD; };
+            using Warm = std::integral_constant<int, 2>;
+            hand_over(std::integral_constant<int, 0>{});
+            warm_a = qrows(0), warm_b = qrows(64);
+            step(ring, C1{}, Yes{}, Warm{}, Yes{}, 0);
+            warm_a = qrows(128), warm_b = qrows(192);
+            step(ring, C0{}, Yes{}, Warm{}, Yes{}, 0);
+            advance();
+            hand_over(std::integral_constant<int, 0>{});
+            // K block 0 is 16 KiB of consecutive rows; so is a row-major V block (a column-major one is 128 pieces of
+            // 128 bytes: K block 1 is fetched in its place)
+            warm_a = K + size_t(nhead) * N * kD;
+            warm_b = kVColMajor ? warm_a + kBN * kD : V + size_t(nhead) * N * kD;
+            step(ring, C1{}, Yes{}, Warm{}, Yes{}, 0);
+            step(ring, C0{}, Yes{}, No{}, Yes{}, 0);
+            advance();
+        }
+    }
     for (; J + 2 < nb; advance()) {
         hand_over(std::integral_constant<int, 0>{});
         step(ring, C1{}, Yes{}, No{}, Yes{}, 0);
@@ -664,6 +707,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     for (int dt = 0; dt < Traits::kDTiles; ++dt)
 #pragma unroll
         for (int c = 0; c < 2; ++c) detail::mfma_settle_a(o_acc[dt][c]);
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);  // vmcnt(0): nothing of this wavefront is still on its way into LDS
     __syncthreads();  // all wavefronts are done with the K/V stages: reuse LDS for staging
     unsigned char* stg = lds + wave * (64 * kRowBytes);
     constexpr int kSlotMask = (kRowBytes / 8 - 1) & ~1;  // 8-byte slots of a staged row are XOR-ed with 2 * (row % 16)
