@@ -14,6 +14,9 @@
 // (operands swapped as above, so the accumulator holds runs of consecutive columns of a row of C).
 #pragma once
 
+#include <type_traits>
+#include <utility>
+
 #include "cell/traits/base.hpp"
 #include "types/layout.hpp"
 #include "types/mfma_tile.hpp"
@@ -154,6 +157,100 @@ struct GemmMfmaTiles {
 };
 
 }  // namespace detail
+
+/// gemm with the instruction stream under the caller's control, for kernels that run ONE wavefront per SIMD (a
+/// wavefront tile so large that its accumulators fill the AGPR half of the SIMD lane's 512 registers: nothing else can
+/// feed the matrix pipe while that wavefront does something else, so where its LDS reads and global loads issue
+/// relative to its matrix instructions decides the kernel's speed):
+///   * the matrix instructions are inline assembly with the accumulator tiles constrained to AGPRs (left alone, the
+///     compiler moves large accumulator sets through VGPRs and spills) and are issued in the order written here:
+///     k-step by k-step, row of A tiles by row, the tiles of a row forwards in even rows and backwards in odd ones, so
+///     that every instruction shares an operand with the one before it;
+///   * before instruction number n = (k * kMs + i) * kNs + position-in-row the caller's hook is called with
+///     std::integral_constant<int, n>: the place for the fragment reads of the next k-step (SharedToRegLoader::load_one)
+///     - they are ordinary LDS reads, the compiler keeps them between the assembly statements they are written between;
+///   * if the hook returns something (a copy::DirectLoad), that direct-to-LDS load is issued in the same assembly
+///     statement as the instruction: m0 is written before the matrix instruction, which thereby is the wait state the
+///     load needs after that write.
+/// The compiler does not know these statements are matrix instructions and inserts none of the wait states their
+/// results need before other instructions read them: call settle_accumulators(c) before c is read by anything else,
+/// and compile the kernel so that c can stay where it is between the calls - __launch_bounds__ of one wavefront per
+/// SIMD (256 threads) when c and the operand tiles need more than 256 registers. A compiler forced to spill or move
+/// an accumulator between two of these statements reads it without the wait, and the result is wrong.
+/// Operands: 16 x 32 / 32 x 16 MFMA tiles of f16, accumulator of 16 x 16 BaseTiles (v_mfma_f32_16x16x32_f16); the sums
+/// are those of gemm(a, b, c) bit for bit.
+template <typename RegTileA, typename RegTileB, typename RegTileC, typename Hook>
+DEVICE void gemm_scheduled(const RegTileA& a, const RegTileB& b, RegTileC& c, Hook&& hook) {
+    using G = detail::GemmMfmaTiles<RegTileA, RegTileB, RegTileC>;
+    static_assert(G::k16, "gemm_scheduled is written for v_mfma_f32_16x16x32_f16 operand tiles");
+    constexpr int kMs = G::kMs, kNs = G::kNs, kKs = G::kKs;
+    [&]<int... kIs>(std::integer_sequence<int, kIs...>) {
+        (
+            [&] {
+                constexpr int n = kIs;
+                constexpr int k = n / (kMs * kNs), i = n / kNs % kMs, pos = n % kNs;
+                constexpr int j = (i & 1) ? kNs - 1 - pos : pos;
+                f16x8 av, bv;
+                f32x4 acc;
+                using HookResult = decltype(hook(std::integral_constant<int, n>{}));
+                if constexpr (std::is_void_v<HookResult>) {
+                    hook(std::integral_constant<int, n>{});
+                    __builtin_memcpy(&av, a(i, k).data(), sizeof(av));
+                    __builtin_memcpy(&bv, b(k, j).data(), sizeof(bv));
+                    __builtin_memcpy(&acc, c(i, j).data(), sizeof(acc));
+                    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(bv), "v"(av));
+                } else {
+                    const HookResult load = hook(std::integral_constant<int, n>{});
+                    __builtin_memcpy(&av, a(i, k).data(), sizeof(av));
+                    __builtin_memcpy(&bv, b(k, j).data(), sizeof(bv));
+                    __builtin_memcpy(&acc, c(i, j).data(), sizeof(acc));
+                    asm volatile(
+                        "s_mov_b32 m0, %5\n\t"
+                        "v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\t"
+                        "global_load_lds_dwordx4 %3, %4"
+                        : "+a"(acc)
+                        : "v"(bv), "v"(av), "v"(load.offset), "s"(load.base), "s"(load.lds_addr)
+                        : "m0", "memory");
+                }
+                __builtin_memcpy(c(i, j).mutable_data(), &acc, sizeof(acc));
+            }(),
+            ...);
+    }(std::make_integer_sequence<int, kMs * kNs * kKs>{});
+}
+
+/// Clear an accumulator tile and place it in AGPRs, where gemm_scheduled keeps it (the statements also keep the
+/// compiler from sinking the clears to the first use, where nothing would hide them).
+template <typename RegTileC>
+DEVICE void clear_pinned(RegTileC& c) {
+    [&]<int... kIs>(std::integer_sequence<int, kIs...>) {
+        (
+            [&] {
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                asm volatile("" : "+a"(acc));
+                __builtin_memcpy(c(kIs / RegTileC::kCols, kIs % RegTileC::kCols).mutable_data(), &acc, sizeof(acc));
+            }(),
+            ...);
+    }(std::make_integer_sequence<int, RegTileC::kRows * RegTileC::kCols>{});
+}
+
+/// After the last gemm_scheduled on c and before anything else reads c: one wait that covers the longest requirement
+/// of a matrix instruction's result (19 issue slots), then every tile passes through a statement of its own (volatile
+/// statements keep their order, so each of those comes after the wait).
+template <typename RegTileC>
+DEVICE void settle_accumulators(RegTileC& c) {
+    asm volatile("s_nop 15\n\ts_nop 3");
+    [&]<int... kIs>(std::integer_sequence<int, kIs...>) {
+        (
+            [&] {
+                auto& tile = c(kIs / RegTileC::kCols, kIs % RegTileC::kCols);
+                f32x4 acc;
+                __builtin_memcpy(&acc, tile.data(), sizeof(acc));
+                asm volatile("" : "+a"(acc));
+                __builtin_memcpy(tile.mutable_data(), &acc, sizeof(acc));
+            }(),
+            ...);
+    }(std::make_integer_sequence<int, RegTileC::kRows * RegTileC::kCols>{});
+}
 
 template <typename RegTileA, typename RegTileB, typename RegTileC>
 DEVICE void gemm(const RegTileA& a, const RegTileB& b, RegTileC& c) {

@@ -79,4 +79,63 @@ struct GlobalToSharedDirectLoader {
     }
 };
 
+/// One direct-to-LDS load instruction, described but not yet issued: every lane fetches 16 bytes from base + offset
+/// (a wave-uniform 64-bit base, which the instruction takes from scalar registers, plus a 32-bit byte offset per
+/// lane: no 64-bit address arithmetic per load) and the 1 KiB lands at lds_addr + 16 * lane.
+struct DirectLoad {
+    unsigned int offset;    // per lane, bytes
+    const void* base;       // wave-uniform
+    unsigned int lds_addr;  // wave-uniform LDS byte address
+};
+
+/// Issue it (untracked by the compiler, like GlobalToSharedDirectLoader's loads). A kernel with one wavefront per SIMD
+/// hands the description to compute::gemm_scheduled instead, which issues it behind a matrix instruction.
+DEVICE void issue(const DirectLoad& load) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(load.offset), "s"(load.base),
+                 "s"(load.lds_addr)
+                 : "m0", "memory");
+}
+
+/// The copy of GlobalToSharedDirectLoader a piece at a time: piece j is the j-th of the kPieces load instructions this
+/// wavefront contributes to a tile. The per-lane offsets (swizzle included) are computed once, at construction, for
+/// global tiles whose lines are kGlobalPitch elements apart; piece(j, src, dst) then only combines them with the
+/// tile's origin `src` (wave-uniform) and the stage `dst`. For kernels that spread the loads of the next tile over the
+/// matrix instructions of the current one instead of issuing them in a burst (the address unit of a CU takes one
+/// vector-memory instruction per ~14 cycles, and a wavefront that waits there issues nothing else).
+template <typename Shared_, typename WarpLayout_, const int kGlobalPitch_>
+struct GlobalToSharedDirectPieces {
+    using Shared = Shared_;
+    using DType = typename Shared::DType;
+    using Loader = GlobalToSharedDirectLoader<Shared_, WarpLayout_>;
+    static constexpr int kPieces = Loader::kLoadsPerWave;
+    static constexpr int kGlobalPitch = kGlobalPitch_;
+    static_assert((long)Shared::kLines * kGlobalPitch * (long)sizeof(DType) < (1l << 32),
+                  "a tile's lines are addressed with 32-bit byte offsets from its origin");
+
+    DEVICE GlobalToSharedDirectPieces() {
+        const int lane = lane_id();
+        wave_ = __builtin_amdgcn_readfirstlane(wave_id());
+        const int line_in_load = lane / Loader::kPiecesPerLine;
+        const int piece = lane % Loader::kPiecesPerLine;  // physical 16-byte piece of the line
+#pragma unroll
+        for (int j = 0; j < kPieces; ++j) {
+            const int line = (wave_ * kPieces + j) * Loader::kLinesPerLoad + line_in_load;
+            const int elem = Shared::kSwizzled ? Shared::Swizzle::apply(line, piece * Loader::kPieceElems)
+                                               : piece * Loader::kPieceElems;
+            offset_[j] = (static_cast<unsigned int>(line) * kGlobalPitch + elem) * static_cast<unsigned int>(sizeof(DType));
+        }
+    }
+
+    /// Piece j of the copy of the global tile whose first element is at `src` into `dst`.
+    DEVICE DirectLoad piece(int j, const DType* src, const Shared& dst) const {
+        const unsigned int lds = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(dst.data())) +
+                                 static_cast<unsigned int>(wave_ * kPieces + j) * 1024u;
+        return DirectLoad{offset_[j], src, static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(lds))};
+    }
+
+  private:
+    unsigned int offset_[kPieces];
+    int wave_;
+};
+
 }  // namespace tiledcuda::cell::copy

@@ -128,6 +128,19 @@ struct SharedToRegLoader : public Base {
             }
         }
     }
+    /// BaseTile (i, j) of this wavefront's share only: for kernels that place each fragment read between particular
+    /// matrix instructions (compute::gemm_scheduled) instead of reading a whole register tile at once.
+    template <typename Shared>
+    DEVICE void load_one(const Shared& src, Reg& dst, int i, int j) {
+        static_assert(std::is_same_v<typename Shared::DType, DType>,
+                      "The data type of Shared and Reg must be the same.");
+        static_assert(Base::template row_exec_count<BaseShape, Shared::kRows>() == Reg::kRows &&
+                          Base::template col_exec_count<BaseShape, Shared::kCols>() == Reg::kCols,
+                      "the register tile must hold exactly this wavefront's share of the shared tile");
+        detail::move_shared_tile<const Shared, BaseTile, true>(
+            src, Base::template warp_row0<Shared::kRows>() + i * BaseShape::kRows,
+            Base::template warp_col0<Shared::kCols>() + j * BaseShape::kCols, dst(i, j));
+    }
 };
 
 /// Store a register tile into this wavefront's share of a shared tile (even split).

@@ -364,4 +364,150 @@ __global__ void __launch_bounds__(Traits::kThreads) gemm_tile_pipelined(const In
     }
 }
 
+/// The one-wavefront-per-SIMD GEMM (kernels/gemm_w128.hpp, the kernel the large shapes run on) written with
+/// tile-library functors only: 256 x 256 x 64 workgroup tile, 2 x 2 wavefronts of 128 x 128, two LDS stages.
+template <typename InType, typename OutType, typename WholeShape>
+struct ScheduledGemmTileTraits {
+    using WarpLayout = tl::RowMajor<2, 2>;
+    static constexpr int kThreads = 4 * kWaveSize;
+    static constexpr int kM = dim_size<0, WholeShape>;
+    static constexpr int kN = dim_size<1, WholeShape>;
+    static constexpr int kK = dim_size<2, WholeShape>;
+    static constexpr int kTM = 256, kTN = 256, kTK = 64, kRK = 32, kStages = 2;
+    static_assert(kM % kTM == 0 && kN % kTN == 0 && kK % kTK == 0);
+
+    using Shape = traits::MfmaTileShape<InType, traits::MfmaShape::k16x16x32>;
+    static constexpr int kMs = kTM / 2 / Shape::kM, kNs = kTN / 2 / Shape::kN;  // 8 x 8 MFMA tiles per wavefront
+
+    using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK, kK>>;
+    using GIteratorA = GTileIterator<GlobalA, TileShape<kTM, kTK>>;
+    using SharedA = SharedTile<InType, tl::RowMajor<kTM, kTK>, true>;
+    using RingA = SharedRing<SharedA, kStages>;
+    using SIteratorA = STileIterator<SharedA, TileShape<kTM, kRK>>;
+    using RegA = RegTile<typename Shape::TileA, tl::RowMajor<kMs, 1>>;
+    using PiecesA = GlobalToSharedDirectPieces<SharedA, WarpLayout, kK>;
+    using S2RLoaderA = SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
+
+    using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kTN, kK>>;
+    using GIteratorB = GTileIterator<GlobalB, TileShape<kTK, kTN>>;
+    using SharedB = SharedTile<InType, tl::ColMajor<kTK, kTN>, true>;
+    using RingB = SharedRing<SharedB, kStages>;
+    using SIteratorB = STileIterator<SharedB, TileShape<kRK, kTN>>;
+    using RegB = RegTile<typename Shape::TileB, tl::ColMajor<1, kNs>>;
+    using PiecesB = GlobalToSharedDirectPieces<SharedB, WarpLayout, kK>;
+    using S2RLoaderB = SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
+
+    using RegAcc = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kMs, kNs>>;
+    using RegC = RegTile<BaseTileRowMajor<OutType>, tl::RowMajor<kMs, kNs>>;
+    using SharedC = SharedTile<OutType, tl::RowMajor<kTM, kTN>, true>;
+    using GlobalC = GlobalTile<OutType, tl::RowMajor<kTM, kTN, kN>>;
+    using R2SStorerC = RegToSharedStorer<RegC, WarpLayout>;
+    using S2GStorerC = SharedToGlobalStorer<SharedC, WarpLayout>;
+
+    static constexpr int kShmInput = RingA::kBytes + RingB::kBytes;
+    static constexpr int kShmOutput = sizeof(OutType) == 2 ? kTM * kTN * int(sizeof(OutType)) : 0;
+    static constexpr int kShmBytes = kShmInput > kShmOutput ? kShmInput : kShmOutput;
+    static_assert(kShmBytes <= kMaxLdsBytes);
+    static_assert(PiecesA::kPieces == 8 && PiecesB::kPieces == 8 && kMs == 8 && kNs == 8,
+                  "the schedule below deals 16 loads and 16 fragment reads over 64 matrix instructions");
+};
+
+/// grid = (kM / 256) * (kN / 256) workgroups (1-D), block = 256, dynamic LDS = Traits::kShmBytes.
+/// A tile of K is two gemm_scheduled calls of 64 matrix instructions (k-steps 0 and 1). The hook of the first reads
+/// the 16 operand fragments of k-step 1, one per two instructions; then one LDS-only barrier (tile k1 + 1 has landed,
+/// everyone has left tile k1's stage); the hook of the second reads the fragments of tile k1 + 1 / k-step 0 and hands
+/// gemm_scheduled this wavefront's 16 loads of tile k1 + 2, one per four instructions, into the stage just vacated.
+/// The schedule, the operand order and therefore the sums are those of gemm_w128 (bit-identical results).
+template <typename InType, typename OutType, typename Traits>
+__global__ void __launch_bounds__(Traits::kThreads) gemm_tile_w128(const InType* dA, const InType* dB, OutType* dC) {
+    constexpr int kM = Traits::kM, kN = Traits::kN, kK = Traits::kK, kTM = Traits::kTM, kTN = Traits::kTN;
+    int tile_m, tile_n;
+    detail::xcd_tile_coords(blockIdx.x, kM / kTM, kN / kTN, tile_m, tile_n);
+
+    extern __shared__ __align__(1024) unsigned char buf[];
+    typename Traits::GIteratorA gAs(dA + size_t(tile_m) * kTM * kK);
+    typename Traits::GIteratorB gBs(dB + size_t(tile_n) * kTN * kK);
+    typename Traits::RingA ringA(reinterpret_cast<InType*>(buf));
+    typename Traits::RingB ringB(reinterpret_cast<InType*>(buf + Traits::RingA::kBytes));
+
+    typename Traits::PiecesA pieces_a;
+    typename Traits::PiecesB pieces_b;
+    typename Traits::S2RLoaderA s2r_a;
+    typename Traits::S2RLoaderB s2r_b;
+
+    typename Traits::RegA rA[2];  // operand tiles of k-step 0 / k-step 1
+    typename Traits::RegB rB[2];
+    typename Traits::RegAcc acc;
+
+    // load q of this wavefront for tile k1 (q < 8: a piece of A, else of B)
+    auto load = [&](int k1, int stage, int q) -> DirectLoad {
+        return q < 8 ? pieces_a.piece(q, gAs(k1).data(), ringA[stage]) : pieces_b.piece(q - 8, gBs(k1).data(), ringB[stage]);
+    };
+    // fragment r of k-step k2 of the tile in `stage`, in the order the next 64 instructions need them: row 0 of A and
+    // all of B first
+    auto read_fragment = [&](int stage, int k2, int which, int r) {
+        typename Traits::SIteratorA sAs(ringA.stage_data(stage));
+        typename Traits::SIteratorB sBs(ringB.stage_data(stage));
+        if (r == 0) s2r_a.load_one(sAs(k2), rA[which], 0, 0);
+        else if (r <= 8) s2r_b.load_one(sBs(k2), rB[which], 0, r - 1);
+        else s2r_a.load_one(sAs(k2), rA[which], r - 8, 0);
+    };
+
+    constexpr int kTiles = Traits::GIteratorA::sc1;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) issue(load(0, 0, q));
+    if constexpr (kTiles > 1) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) issue(load(1, 1, q));
+    }
+    compute::clear_pinned(acc);  // while the first tiles are on their way
+    if constexpr (kTiles > 1) wait_group_and_barrier<16>();  // tile 0 has landed, for everyone
+    else wait_group_and_barrier<0>();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) read_fragment(0, 0, 0, r);
+
+    // kMore: there is a tile k1 + 1; kMore2: there is a tile k1 + 2
+    auto tile = [&](int k1, auto more_c, auto more2_c) {
+        constexpr bool kMore = decltype(more_c)::value, kMore2 = decltype(more2_c)::value;
+        const int stage = k1 & 1;
+        compute::gemm_scheduled(rA[0], rB[0], acc, [&](auto n_c) {
+            constexpr int n = decltype(n_c)::value;
+            if constexpr (n % 2 == 0 && n / 2 < 16) read_fragment(stage, 1, 1, n / 2);
+        });
+        wait_group_and_barrier<0>();
+        compute::gemm_scheduled(rA[1], rB[1], acc, [&](auto n_c) {
+            constexpr int n = decltype(n_c)::value;
+            if constexpr (kMore && n % 2 == 0 && n / 2 < 16) read_fragment(stage ^ 1, 0, 0, n / 2);
+            if constexpr (kMore2 && n % 4 == 1) return load(k1 + 2, stage, n / 4);
+        });
+    };
+    {
+        int k1 = 0;
+        for (; k1 + 2 < kTiles; ++k1) tile(k1, std::true_type{}, std::true_type{});
+        if (k1 + 1 < kTiles) {
+            tile(k1, std::true_type{}, std::false_type{});
+            ++k1;
+        }
+        tile(k1, std::false_type{}, std::false_type{});
+    }
+    compute::settle_accumulators(acc);
+
+    typename Traits::GlobalC gC(dC + size_t(tile_m) * kTM * kN + size_t(tile_n) * kTN);
+    if constexpr (std::is_same_v<OutType, float>) {
+        RegToGlobalStorer<typename Traits::GlobalC, typename Traits::RegAcc, typename Traits::WarpLayout> r2g;
+        r2g(acc, gC);
+    } else {
+        typename Traits::RegC out;
+        compute::RegTileConvert<typename Traits::RegAcc, typename Traits::RegC> convert;
+        convert(acc, out);
+        __syncthreads();  // everyone is done with the operand stages: the space is reused for C
+        typename Traits::SharedC sC(reinterpret_cast<OutType*>(buf));
+        typename Traits::R2SStorerC r2s_c;
+        typename Traits::S2GStorerC s2g_c;
+        r2s_c(out, sC);
+        __syncthreads();
+        s2g_c(sC, gC);
+    }
+}
+
 }  // namespace tiledcuda::kernels

@@ -48,8 +48,12 @@ typedef enum {
     TCU_GEMM_TILE_PIPELINED = 5, /* the PIPELINED kernel composed from tile-library functors only (direct-to-LDS loader,
                                 two-stage shared ring, ds_read_b128 operand tiles, gemm()); compile-time shapes:
                                 4096^3, 1024^3, 512x768x192, 256x256x64; results identical to PIPELINED bit for bit */
-    TCU_GEMM_RAGGED = 6       /* run-time M, N, K in multiples of 16: MFMA operand tiles filled from global memory,
+    TCU_GEMM_RAGGED = 6,      /* run-time M, N, K in multiples of 16: MFMA operand tiles filled from global memory,
                                 tiles beyond the edge skipped; the fallback for shapes the tiled kernels do not cover */
+    TCU_GEMM_TILE_WAVE128 = 7 /* the WAVE128 kernel composed from tile-library functors only (direct-to-LDS loads dealt
+                                a piece at a time, single-fragment LDS reads, gemm_scheduled() with accumulators pinned
+                                in AGPRs); compile-time shapes: 4096^3, 1024^3, 512x768x192, 256x256x64; results
+                                identical to WAVE128 and PIPELINED bit for bit */
 } tcu_gemm_algo;
 
 /* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks ROWS for many rows, else RESIDENT, where

@@ -8,6 +8,8 @@
 // RowMajor<2, 4> / ColMajor<4, 2> mma.sync fragments (register.hpp:108-112).
 #pragma once
 
+#include <utility>
+
 #include "hip_utils.hpp"
 #include "types/layout.hpp"
 #include "util/print.hpp"
@@ -61,7 +63,10 @@ class RegTile {
         if constexpr (kIsBaseTile) return tl::layout_type<Layout>; else return DType::kType;
     }();
 
-    HOST_DEVICE RegTile() { clear(); }
+    /// Every element zero. The elements are initialised one by one in the member initialiser (a pack expansion), not by
+    /// the loop a compiler generates for an array of class-type elements: that loop is not unrolled for large tiles,
+    /// and one dynamic index is enough to keep a whole register tile in scratch memory.
+    HOST_DEVICE RegTile() : RegTile(std::make_integer_sequence<int, kNumel>{}) {}
 
     HOST_DEVICE DType* mutable_data() { return data_; }
 
@@ -94,6 +99,13 @@ class RegTile {
     }
 
   private:
+    template <int... kIs>
+    HOST_DEVICE explicit RegTile(std::integer_sequence<int, kIs...>) : data_{zero_element<kIs>()...} {}
+    template <int>
+    HOST_DEVICE static DType zero_element() {
+        if constexpr (kIsBaseTile) return DType(0.f); else return DType();
+    }
+
     alignas(detail::reg_align(sizeof(DType) * kNumel)) DType data_[kNumel];
 };
 

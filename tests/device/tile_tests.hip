@@ -20,6 +20,7 @@
 #include "types/mod.hpp"
 
 #include <string>
+#include <utility>
 #include <vector>
 
 using namespace tiledcuda;
@@ -223,7 +224,7 @@ __global__ void __launch_bounds__(512) k_tile_gemm(const __half* dA, const __hal
 
 // ------------------------------------------------------------------ CDNA4 data path
 // global -> (direct-to-LDS, stage kStage of a ring of 3) -> global
-template <bool kRowMajor, int kRows, int kCols, typename WarpLayout, bool kSwizzled>
+template <bool kRowMajor, int kRows, int kCols, typename WarpLayout, bool kSwizzled, bool kPieces = false>
 __global__ void __launch_bounds__(512) k_direct_ring_roundtrip(const __half* src, __half* dst) {
     extern __shared__ __align__(1024) unsigned char buf[];
     using Layout = LayoutOf<kRowMajor, kRows, kCols>;
@@ -236,7 +237,14 @@ __global__ void __launch_bounds__(512) k_direct_ring_roundtrip(const __half* src
     GlobalToSharedDirectLoader<Shared, WarpLayout> loader;
     SharedToGlobalStorer<Shared, WarpLayout> storer;
     auto stage = ring[Ring::next(0)];
-    loader(g_src, stage);
+    if constexpr (kPieces) {
+        // the same copy, a load instruction at a time
+        using Pieces = GlobalToSharedDirectPieces<Shared, WarpLayout, kRowMajor ? Global::kRowStride : Global::kColStride>;
+        Pieces pieces;
+        for (int j = Pieces::kPieces - 1; j >= 0; --j) issue(pieces.piece(j, g_src.data(), stage));
+    } else {
+        loader(g_src, stage);
+    }
     wait_group_and_barrier<0>();
     storer(stage, g_dst);
 }
@@ -341,8 +349,9 @@ __global__ void __launch_bounds__(512) k_s2r_transposed(const __half* src, __hal
 
 // C = A · B through direct-to-LDS loads and MFMA-shaped tiles, one workgroup. kShape32: v_mfma_f32_32x32x16_f16,
 // else v_mfma_f32_16x16x32_f16. kBRowMajor: B is stored row-major [kK, kN] and transposed by the loader.
-template <int kM, int kN, int kK, typename WarpLayout, bool kShape32, bool kBRowMajor>
-__global__ void __launch_bounds__(512) k_tile_gemm_mfma(const __half* dA, const __half* dB, float* dC) {
+// (the scheduled form is compiled for one wavefront per SIMD: its accumulators must have room to stay in AGPRs)
+template <int kM, int kN, int kK, typename WarpLayout, bool kShape32, bool kBRowMajor, bool kScheduled = false>
+__global__ void __launch_bounds__(kScheduled ? 256 : 512) k_tile_gemm_mfma(const __half* dA, const __half* dB, float* dC) {
     extern __shared__ __align__(1024) unsigned char buf[];
     auto* sA_ptr = reinterpret_cast<__half*>(buf);
     auto* sB_ptr = sA_ptr + kM * kK;
@@ -383,10 +392,37 @@ __global__ void __launch_bounds__(512) k_tile_gemm_mfma(const __half* dA, const 
     RegA rA;
     RegB rB;
     RegC acc;
-    for (int k = 0; k < SIterA::sc1; ++k) {
-        s2r_a(sAs(k), rA);
-        s2r_b(sBs(k), rB);
-        compute::gemm(rA, rB, acc);
+    if constexpr (kScheduled) {
+        // the one-wavefront-per-SIMD form: accumulators pinned in AGPRs, the fragments of chunk k + 1 read one at a
+        // time from the hook of the matrix instructions of chunk k (the first instructions of a chunk get them)
+        static_assert(!kShape32 && !kBRowMajor);
+        RegA rA2[2];
+        RegB rB2[2];
+        constexpr int kFragsA = RegA::kRows * RegA::kCols, kFragsB = RegB::kRows * RegB::kCols;
+        constexpr int kMfmas = RegA::kRows * RegB::kCols * RegA::kCols;
+        static_assert(kFragsA + kFragsB <= kMfmas);
+        auto read_fragment = [&](int k, int which, int r) {
+            if (r < kFragsA) s2r_a.load_one(sAs(k), rA2[which], r / RegA::kCols, r % RegA::kCols);
+            else s2r_b.load_one(sBs(k), rB2[which], (r - kFragsA) / RegB::kCols, (r - kFragsA) % RegB::kCols);
+        };
+        compute::clear_pinned(acc);
+        for (int r = 0; r < kFragsA + kFragsB; ++r) read_fragment(0, 0, r);
+        [&]<int... kChunks>(std::integer_sequence<int, kChunks...>) {
+            (compute::gemm_scheduled(rA2[kChunks & 1], rB2[kChunks & 1], acc,
+                                     [&](auto n_c) {
+                                         constexpr int n = decltype(n_c)::value;
+                                         if constexpr (kChunks + 1 < SIterA::sc1 && n < kFragsA + kFragsB)
+                                             read_fragment(kChunks + 1, (kChunks + 1) & 1, n);
+                                     }),
+             ...);
+        }(std::make_integer_sequence<int, SIterA::sc1>{});
+        compute::settle_accumulators(acc);
+    } else {
+        for (int k = 0; k < SIterA::sc1; ++k) {
+            s2r_a(sAs(k), rA);
+            s2r_b(sBs(k), rB);
+            compute::gemm(rA, rB, acc);
+        }
     }
     GlobalC gC(dC);
     RegToGlobalStorer<GlobalC, RegC, WarpLayout> r2g;
@@ -652,17 +688,17 @@ void reg_gemm() {
                           &launch_gemm<k_tile_gemm<kM, kN, kK, W, kChunkK, kSwz>>});
 }
 
-template <bool kRowMajor, int kRows, int kCols, int kWR, int kWC, bool kSwz>
+template <bool kRowMajor, int kRows, int kCols, int kWR, int kWC, bool kSwz, bool kPieces = false>
 void reg_direct() {
     using W = tl::RowMajor<kWR, kWC>;
     registry().push_back({"g2s_roundtrip",
-                          std::string("f16_direct_ring") + (kRowMajor ? "_row_" : "_col_") + std::to_string(kRows) + "x" +
+                          std::string(kPieces ? "f16_direct_pieces" : "f16_direct_ring") + (kRowMajor ? "_row_" : "_col_") + std::to_string(kRows) + "x" +
                               std::to_string(kCols) + "_w" + std::to_string(kWR) + "x" + std::to_string(kWC) +
                               (kSwz ? "_swz" : "_plain"),
                           {kRows, kCols, 0, 2, kRowMajor, 0, 0, 0},
                           kWR * kWC * 64,
                           int(3 * kRows * kCols * sizeof(__half)),
-                          &launch2<k_direct_ring_roundtrip<kRowMajor, kRows, kCols, W, kSwz>, __half>});
+                          &launch2<k_direct_ring_roundtrip<kRowMajor, kRows, kCols, W, kSwz, kPieces>, __half>});
 }
 
 template <bool kRowMajor, int kRows, int kCols, int kChunk, int kWR, int kWC, bool kSwz, int kTileMajor>
@@ -693,17 +729,17 @@ void reg_s2r_tr() {
                           &launch2<k_s2r_transposed<kRows, kCols, kChunk, W, kSwz, kTileCols>, __half>});
 }
 
-template <int kM, int kN, int kK, int kWR, int kWC, bool kShape32, bool kBRowMajor>
+template <int kM, int kN, int kK, int kWR, int kWC, bool kShape32, bool kBRowMajor, bool kScheduled = false>
 void reg_gemm_mfma() {
     using W = tl::RowMajor<kWR, kWC>;
     registry().push_back({"tile_gemm",
-                          std::string(kShape32 ? "mfma32x32x16_" : "mfma16x16x32_") + std::to_string(kM) + "x" +
+                          std::string(kScheduled ? "scheduled_" : "") + std::string(kShape32 ? "mfma32x32x16_" : "mfma16x16x32_") + std::to_string(kM) + "x" +
                               std::to_string(kN) + "x" + std::to_string(kK) + "_w" + std::to_string(kWR) + "x" +
                               std::to_string(kWC) + (kBRowMajor ? "_b_row_major" : ""),
                           {kM, kN, kK, 64, kBRowMajor, 0, 0, 0},
                           kWR * kWC * 64,
                           int((kM * kK + kK * kN) * sizeof(__half)),
-                          &launch_gemm<k_tile_gemm_mfma<kM, kN, kK, W, kShape32, kBRowMajor>>});
+                          &launch_gemm<k_tile_gemm_mfma<kM, kN, kK, W, kShape32, kBRowMajor, kScheduled>>});
 }
 
 template <typename E, int kRows, int kCols, int kW, int kOp>
@@ -850,6 +886,12 @@ void build_registry() {
     reg_direct<false, 64, 128, 2, 2, true>();
     reg_direct<false, 64, 256, 4, 2, true>();
     reg_direct<false, 128, 64, 1, 4, false>();
+    // the same copies dealt a piece at a time (GlobalToSharedDirectPieces + issue)
+    reg_direct<true, 64, 64, 2, 2, true, true>();
+    reg_direct<true, 256, 64, 2, 2, true, true>();
+    reg_direct<true, 16, 256, 1, 1, false, true>();
+    reg_direct<false, 64, 256, 2, 2, true, true>();
+    reg_direct<false, 128, 64, 1, 4, false, true>();
     // MFMA-shaped operand tiles out of LDS (ds_read_b128): both instruction shapes, both operands
     reg_s2r_mfma<true, 64, 64, 64, 2, 2, true, 16>();
     reg_s2r_mfma<true, 64, 64, 32, 2, 2, false, 16>();
@@ -878,6 +920,11 @@ void build_registry() {
     reg_gemm_mfma<64, 64, 64, 2, 2, false, true>();
     reg_gemm_mfma<128, 128, 64, 2, 2, false, true>();
     reg_gemm_mfma<64, 64, 128, 2, 2, true, true>();
+    // gemm_scheduled(): AGPR-pinned accumulators, fragment reads placed by the hook (1, 2 and 4 chunks of K)
+    reg_gemm_mfma<64, 64, 64, 2, 2, false, false, true>();
+    reg_gemm_mfma<128, 128, 128, 2, 2, false, false, true>();
+    reg_gemm_mfma<256, 256, 64, 2, 2, false, false, true>();
+    reg_gemm_mfma<128, 64, 256, 1, 1, false, false, true>();
 
     // reductions, broadcasts, softmax (test_reduce.cu / test_broadcast.cu / test_softmax.cu shapes)
     reg_row_op<float, 16, 16, 1, 0>();

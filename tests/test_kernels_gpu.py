@@ -279,6 +279,28 @@ def test_gemm_tile_api_pipelined_is_the_pipelined_kernel(tcu, oracle, device, M,
     assert torch.equal(C, tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 768, 192), (1024, 1024, 1024), (4096, 4096, 4096)])
+@pytest.mark.parametrize("out_dtype", ["f16", "f32"])
+def test_gemm_tile_api_wave128_is_the_wave128_kernel(tcu, oracle, device, M, N, K, out_dtype):
+    """The one-wavefront-per-SIMD kernel written with tile-library functors only (GlobalToSharedDirectPieces,
+    SharedToRegLoader::load_one, gemm_scheduled with AGPR-pinned accumulators) against the oracle and, bit for bit,
+    against the hand-indexed kernel whose schedule it reproduces (1, 3, 16 and 64 k-tiles: every peeled form of the
+    loop over k)."""
+    import torch
+
+    print(f"gemm tile_wave128 {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float16 if out_dtype == "f16" else torch.float32
+    A = oracle.fill_uniform(M * K, 7100 + K).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 8100 + K).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    C = tcu.gemm(dA, dB, out_dtype=dt, algo="tile_wave128")
+    torch.cuda.synchronize()
+    rows = (0, M) if M <= 1024 else (M - 192, M)
+    ref = oracle.gemm(A, Bt, rows=rows)
+    assert oracle.max_rel_err(host(C)[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
+    assert torch.equal(C, tcu.gemm(dA, dB, out_dtype=dt, algo="wave128"))
+
+
 @pytest.mark.parametrize("algo", ["pipelined", "wave128"])
 def test_gemm_one_hot_index_probe(tcu, device, algo):
     """C[m, n] = A[m, k] * Bt[n, k] for one-hot operands: pins rows/cols/transposition exactly."""

@@ -247,6 +247,25 @@ int gemm_tile_pipelined_dispatch(const __half* A, const __half* B, OutType* C, i
                                            "and 256x256x64");
 }
 
+template <typename OutType, int kM, int kN, int kK>
+int launch_tile_w128(const __half* A, const __half* B, OutType* C, hipStream_t stream) {
+    using Traits = ScheduledGemmTileTraits<__half, OutType, GemmShape<kM, kN, kK>>;
+    auto kernel = &gemm_tile_w128<__half, OutType, Traits>;
+    return launch(kernel, dim3((kM / Traits::kTM) * (kN / Traits::kTN)), dim3(Traits::kThreads), Traits::kShmBytes, stream,
+                  A, B, C);
+}
+
+/// The one-wavefront-per-SIMD kernel composed from tile-library functors: compile-time shapes, as above.
+template <typename OutType>
+int gemm_tile_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    if (M == 4096 && N == 4096 && K == 4096) return launch_tile_w128<OutType, 4096, 4096, 4096>(A, B, C, stream);
+    if (M == 1024 && N == 1024 && K == 1024) return launch_tile_w128<OutType, 1024, 1024, 1024>(A, B, C, stream);
+    if (M == 512 && N == 768 && K == 192) return launch_tile_w128<OutType, 512, 768, 192>(A, B, C, stream);
+    if (M == 256 && N == 256 && K == 64) return launch_tile_w128<OutType, 256, 256, 64>(A, B, C, stream);
+    return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the tile-API one-wavefront-per-SIMD GEMM is instantiated for 4096^3, 1024^3, "
+                                           "512x768x192 and 256x256x64");
+}
+
 /// M or N a little above a multiple of 256: edge tiles of 256 x 256 cost a whole extra round of workgroups for a
 /// sliver of output. When the cost model says so, the product is computed as three launches on disjoint parts of C:
 /// the leading block of whole 256 x 256 tiles by the one-wavefront-per-SIMD kernel, the columns beyond it (all rows)
@@ -328,6 +347,8 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             return gemm_tile_pipelined_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_WAVE128:
             return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
+        case TCU_GEMM_TILE_WAVE128:
+            return gemm_tile_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_AUTO:
             // where the 256 x 256 tile is the choice anyway, the one-wavefront-per-SIMD kernel is the faster one
             if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) >= 128 &&
