@@ -17,7 +17,8 @@ def jit(tcu):
 
 
 def test_generated_sources_compile_and_export_kernel_entry(jit, tmp_path):
-    for kind, cfg in (("tile_library", (256, 256, 256, 64, 64, 32, 2, 2)), ("pipelined", (256, 256, 256, 128, 128, 64, 2, 2))):
+    for kind, cfg in (("tile_library", (256, 256, 256, 64, 64, 32, 2, 2)), ("pipelined", (256, 256, 256, 128, 128, 64, 2, 2)),
+                      ("tile_wave128", (512, 256, 192, 256, 256, 64, 2, 2))):
         builder = jit.Compile(file_prefix="t", tmp_dir=str(tmp_path), kernel=kind)
         path = builder.compile(*cfg)
         assert path and os.path.exists(path)
@@ -63,7 +64,8 @@ def test_bad_instantiation_raises(jit, tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kind,cfg", [("tile_library", (64, 64, 32, 2, 2)), ("pipelined", (128, 128, 64, 2, 2))])
+@pytest.mark.parametrize("kind,cfg", [("tile_library", (64, 64, 32, 2, 2)), ("pipelined", (128, 128, 64, 2, 2)),
+                                      ("tile_wave128", (256, 256, 64, 2, 2))])
 def test_jit_gemm_matches_oracle(jit, oracle, device, tmp_path, kind, cfg):
     M = N = K = 256
     A = oracle.fill_uniform(M * K, 41).reshape(M, K)

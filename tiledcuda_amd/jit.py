@@ -5,8 +5,9 @@ fixes the problem and tile shape as template arguments, compiles it to a shared 
 ``extern "C" int kernel_entry(__half*, __half*, float*)`` (entry.py:56-67) and calls it through ctypes;
 ``gemm_func`` (gemm.py:13-42) compiles on first use and launches; ``sweep`` is the tile-shape loop of main.py:90-112
 with the timings returned instead of printed. The compiler is hipcc for gfx950, the kernels are this
-repository's headers (``include/kernels/gemm.hpp`` for the tile-library kernel the reference example builds,
-``include/kernels/gemm_pipelined.hpp`` for the tuned one). A is [M, K] row-major, B is [N, K] (column-major
+repository's headers (``include/kernels/gemm.hpp`` for the tile-library kernel the reference example builds and, as
+``kernel="tile_wave128"``, for the one-wavefront-per-SIMD kernel composed from tile-library functors at any M, N in
+multiples of 256 and K in multiples of 64; ``include/kernels/gemm_pipelined.hpp`` for the hand-indexed one). A is [M, K] row-major, B is [N, K] (column-major
 operand), C is [M, N] fp32.
 """
 from __future__ import annotations
@@ -61,6 +62,27 @@ static int launch(const __half* a, const __half* b, float* c, hipStream_t stream
 }}
 """
 
+_TILE_WAVE128_SOURCE = """#include "kernels/gemm.hpp"
+using namespace tiledcuda;
+using namespace tiledcuda::kernels;
+
+// the one-wavefront-per-SIMD kernel composed from tile-library functors: its tile and wavefront layout are fixed
+static_assert({TM} == 256 && {TN} == 256 && {chunk} == 64 && {wr} == 2 && {wc} == 2,
+              "tile_wave128 is a 256 x 256 x 64 tile on 2 x 2 wavefronts");
+using Config = ScheduledGemmTileTraits<__half, float, GemmShape<{M}, {N}, {K}>>;
+
+static int launch(const __half* a, const __half* b, float* c, hipStream_t stream) {{
+    auto kernel = &gemm_tile_w128<__half, float, Config>;
+    static bool raised = false;
+    if (!raised) {{
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, Config::kShmBytes) != hipSuccess) return -3;
+        raised = true;
+    }}
+    hipLaunchKernelGGL(kernel, dim3(({M} / 256) * ({N} / 256)), dim3(Config::kThreads), Config::kShmBytes, stream, a, b, c);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}}
+"""
+
 _ENTRY = """
 extern "C" int kernel_entry(__half* parameter1, __half* parameter2, float* parameter3) {
     return launch(parameter1, parameter2, parameter3, nullptr);
@@ -70,6 +92,9 @@ extern "C" int kernel_entry_stream(__half* parameter1, __half* parameter2, float
     return launch(parameter1, parameter2, parameter3, static_cast<hipStream_t>(stream));
 }
 """
+
+
+_SOURCES = {"tile_library": _TILE_LIBRARY_SOURCE, "pipelined": _PIPELINED_SOURCE, "tile_wave128": _TILE_WAVE128_SOURCE}
 
 
 def _default_cache_dir() -> str:
@@ -110,8 +135,8 @@ class Compile:
     (cached by file name in ``tmp_dir``), ``apply(lib_path, [A, B, C], device)`` calls its ``kernel_entry``."""
 
     def __init__(self, file_prefix: str = "gemm", tmp_dir: str | None = None, kernel: str = "tile_library"):
-        if kernel not in ("tile_library", "pipelined"):
-            raise ValueError("kernel must be 'tile_library' or 'pipelined'")
+        if kernel not in _SOURCES:
+            raise ValueError("kernel must be one of " + ", ".join(repr(k) for k in _SOURCES))
         self.tmp_dir = tmp_dir or _default_cache_dir()
         self.file_prefix = file_prefix
         self.kernel = kernel
@@ -120,7 +145,7 @@ class Compile:
         self._libs: dict[str, ctypes.CDLL] = {}
 
     def _create_entry_code(self, M, N, K, TM, TN, kChunkK, warp_per_row, warp_per_col) -> str:
-        template = _TILE_LIBRARY_SOURCE if self.kernel == "tile_library" else _PIPELINED_SOURCE
+        template = _SOURCES[self.kernel]
         return template.format(M=M, N=N, K=K, TM=TM, TN=TN, chunk=kChunkK, wr=warp_per_row, wc=warp_per_col) + _ENTRY
 
     def compile(self, M: int, N: int, K: int, TM: int, TN: int, kChunkK: int, warp_per_row: int, warp_per_col: int,
