@@ -1,0 +1,203 @@
+// fp16 GEMM for gfx950 with one wavefront per SIMD and the four wavefronts of a workgroup splitting K: for products
+// with too few 256 x 256 tiles to fill 256 CUs (2048^3 has 64) but enough 128 x 128 tiles. Same contract as
+// kernels/gemm_w128.hpp (C[M, N] = A[M, K] . B, A row-major, B column-major = stored [N, K], f32 accumulate, C
+// row-major f16 or f32; the multi-stage counterpart of the reference's examples/cpp/01_gemm/02_gemm_all_mem/gemm.hpp:103-155).
+//   * With 128 x 128 workgroup tiles split 2 x 2 over wavefronts (64 x 64 each) every 16 matrix instructions need 8
+//     ds_read_b128: four wavefronts then ask for 128 bytes of LDS per cycle at the matrix pipe's peak rate, which is
+//     all the LDS delivers - that tiling is bound by LDS reads. Here every wavefront owns the WHOLE 128 x 128 tile
+//     (16 reads per 64 instructions, half the LDS traffic, the gemm_w128 ratio) over a quarter of K: a tile of K is
+//     128 wide, wavefront w multiplies columns 32 w .. 32 w + 31 of it. The four partial tiles are added through LDS
+//     at the end, after which wavefront w holds rows 32 w .. 32 w + 31 of the result and stores them.
+//   * A stage is 128 + 128 rows of 256 bytes = 64 KiB; two stages. One phase per tile of K: 64 MFMAs, with the 16
+//     fragment reads of the next tile (one per two MFMAs) and this wavefront's 16 direct-to-LDS loads of the tile after
+//     that (one per four MFMAs, each in one statement with its MFMA), then one LDS-only barrier. The loads of a tile
+//     have one phase to land (a third stage does not fit), and a workgroup pulls 64 KiB per 1024 cycles of matrix
+//     work through its CU's load path: the loop runs at the pace of those loads (a phase measures about 1.2 us at
+//     2048^3, the same whether the loads are issued one per four, three or two MFMAs), not of the matrix pipe. That
+//     is still ahead of the LDS-bound tiling: 2048^3 24.4 us against 26.8 us (the vendor library: 24.6-25.8 us).
+//   * Accumulators in AGPRs through inline assembly, scalar-base addressing, XCD-aware tile order: as in gemm_w128.
+// The sum over K is taken in four interleaved parts, so results differ from the other kernels by f32 rounding.
+// M % 128 == 0, N % 128 == 0, K % 128 == 0 (checked by the launcher).
+#pragma once
+
+#include <type_traits>
+
+#include "config.hpp"
+#include "hip_utils.hpp"
+#include "kernels/gemm_w128.hpp"  // detail::mfma_16x16x32_agpr{,_then_load}, load_lds_16B_sbase, lds_barrier
+
+namespace tiledcuda::kernels {
+
+struct GemmW128kTraits {
+    static constexpr int kBM = 128, kBN = 128, kBK = 128;
+    static constexpr int kWaves = 4, kThreads = kWaves * kWaveSize;
+    static constexpr int kRowBytes = kBK * 2;                      // 256
+    static constexpr int kABytes = kBM * kRowBytes, kBBytes = kBN * kRowBytes;
+    static constexpr int kStageBytes = kABytes + kBBytes;          // 64 KiB
+    static constexpr int kLoads = kBM * kRowBytes / 1024 / kWaves;  // 1 KiB load instructions per operand per wavefront
+    static constexpr int kLdsBytes = 2 * kStageBytes;              // 128 KiB; the reduction reuses it
+    static_assert(kLoads == 8, "the phase schedule below is written for 8 + 8 loads per wavefront");
+    static_assert(kLdsBytes <= kMaxLdsBytes);
+};
+
+/// grid = (M / 128) * (N / 128), block = 256, dynamic LDS = GemmW128kTraits::kLdsBytes. lda / ldb / ldc: elements
+/// between consecutive rows of A, of the stored [N, K] array and of C.
+template <typename OutType>
+__global__ void __launch_bounds__(GemmW128kTraits::kThreads)
+    gemm_w128k(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
+               int lda, int ldb, int ldc) {
+    using T = GemmW128kTraits;
+    extern __shared__ __align__(1024) unsigned char lds[];
+
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+    int tile_m, tile_n;
+    detail::xcd_tile_coords(blockIdx.x, M / T::kBM, N / T::kBN, tile_m, tile_n);
+    const int m0 = tile_m * T::kBM, n0 = tile_n * T::kBN;
+
+    // ---- global -> LDS: load instruction q of this wavefront (q < 8: A, else B) fills 4 rows of 256 bytes; lane i
+    // writes physical 16-byte chunk i % 16 of row i / 16, which must hold logical chunk (i % 16) ^ (row % 16)
+    const int lrow = lane >> 4, lchk = lane & 15;
+    unsigned int voff[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+        const int row = (wave * T::kLoads + (q & 7)) * 4 + lrow;
+        voff[q] = static_cast<unsigned int>(row) * static_cast<unsigned int>(q < 8 ? lda : ldb) * 2u + (lchk ^ (row & 15)) * 16;
+    }
+    const __half* a_base = A + size_t(m0) * lda;
+    const __half* b_base = Bt + size_t(n0) * ldb;
+    const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
+    auto load_dst = [&](int stage, int q) -> unsigned int {
+        return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +
+                                              (wave * T::kLoads + (q & 7)) * 1024);
+    };
+    auto load_src = [&](int kt, int q) -> const __half* { return (q < 8 ? a_base : b_base) + kt * T::kBK; };
+
+    // ---- LDS -> registers: fragment r (r < 8: A rows 16 r .., else B rows 16 (r - 8) ..); lane l holds row l % 16,
+    // k = 32 wave + 8 (l / 16) .. + 7 of the tile = logical chunk 4 wave + l / 16 of its row. The 16 rows a 16-lane
+    // group reads have 16 different values of row % 16: 16 different chunks, no bank conflict.
+    const int frow = lane & 15, fquad = lane >> 4;
+    auto read_frag = [&](int stage, int r) -> f16x8 {
+        const int row = (r & 7) * 16 + frow;
+        const int chunk = (4 * wave + fquad) ^ (row & 15);
+        return *reinterpret_cast<const f16x8*>(lds + stage * T::kStageBytes + (r < 8 ? 0 : T::kABytes) + row * T::kRowBytes +
+                                               chunk * 16);
+    };
+
+    f16x8 fx[16], fy[16];  // fragments of the tile being multiplied / of the next one: [0..7] A, [8..15] B
+    const int ktiles = K / T::kBK;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
+#pragma unroll
+    for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(ktiles > 1 ? 1 : 0, q), load_dst(1, q));
+    f32x4 acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        asm volatile(""
+                     : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),
+                       "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]));
+    }
+    detail::lds_barrier<16>();  // tile 0 has landed, for everyone
+#pragma unroll
+    for (int r = 0; r < 16; ++r) fx[r] = read_frag(0, r);
+
+    constexpr int kOrder[16] = {0, 8, 9, 10, 11, 12, 13, 14, 15, 1, 2, 3, 4, 5, 6, 7};
+    auto snake = [](int i, int n) { return (i & 1) ? 7 - n : n; };
+
+    // One tile of K out of `cur`, reading the next tile's fragments into `nxt` and loading the tile after that into
+    // the stage `cur`'s tile came from. Every phase is the same straight-line code: behind the last tile of K the
+    // fragment reads fetch stale data that nobody uses and the loads fetch the last tile once more (clamped index) -
+    // cheaper than peeled copies of the phase, whose control-flow merges made the compiler shuffle and spill
+    // accumulators between the assembly statements, where it knows of no wait states.
+    auto tile = [&](int kt, f16x8 (&cur)[16], f16x8 (&nxt)[16]) {
+        const int stage = kt & 1;
+        const int kload = kt + 2 < ktiles ? kt + 2 : ktiles - 1;
+        // tile kt + 1 has landed and this wavefront's reads of `stage` (issued during the previous phase) have
+        // returned; then everyone's
+        detail::lds_barrier<0>();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int n = 0; n < 8; ++n) {
+                const int j = snake(i, n);
+                const int r = 4 * i + (n >> 1);
+                if ((n & 1) == 0 && r < 16) nxt[kOrder[r]] = read_frag(stage ^ 1, kOrder[r]);
+                if ((n & 3) == 1) {
+                    const int q = 2 * i + (n >> 2);
+                    detail::mfma_16x16x32_agpr_then_load(acc[i][j], cur[8 + j], cur[i], voff[q], load_src(kload, q),
+                                                         load_dst(stage, q));
+                } else {
+                    detail::mfma_16x16x32_agpr(acc[i][j], cur[8 + j], cur[i]);
+                }
+            }
+        }
+    };
+    {
+        int kt = 0;
+        for (; kt + 1 < ktiles; kt += 2) {
+            tile(kt, fx, fy);
+            tile(kt + 1, fy, fx);
+        }
+        if (kt < ktiles) tile(kt, fx, fy);
+    }
+
+    detail::mfma_results_wait();
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        asm volatile(""
+                     : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),
+                       "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]));
+
+    // ---- the four partial tiles are added through LDS, two row groups (32 rows, 16 MFMA tiles) per round. Every
+    // wavefront writes its 16 partial tiles of the round - tile t = 8 (row group % 2) + column tile, 1 KiB each, a
+    // lane's f32x4 at 16 * lane: conflict-free and the same for writer and reader - and then sums the four partials
+    // of tiles 4 w .. 4 w + 3 into registers of its own. Which tiles a wavefront sums is a matter of LDS addresses
+    // only: register indices are the same in all four wavefronts (an index that depended on the wavefront would put
+    // the accumulators into scratch memory). Two buffers of 64 KiB alternate, so one barrier per round is enough: a
+    // buffer is written again two rounds later, after the barrier of the round in between.
+    // Wavefront w ends up with rows 32 r + 16 (w / 2) .. + 15 (r = 0 .. 3), columns 64 (w % 2) .. + 63.
+    detail::lds_barrier<0>();  // nothing is on its way into LDS any more, every wavefront is done with the operand stages
+    using lds_f32x4_ptr = __attribute__((address_space(3))) f32x4*;
+    f32x4 res[4][4];
+#pragma unroll
+    for (int round = 0; round < 4; ++round) {
+        const unsigned int buf = lds_base + (round & 1) * (64 * 1024) + lane * 16;
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+            *reinterpret_cast<lds_f32x4_ptr>(buf + (wave * 16 + t) * 1024) = acc[2 * round + t / 8][t % 8];
+        __syncthreads();
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            f32x4 sum = *reinterpret_cast<lds_f32x4_ptr>(buf + (4 * wave + jj) * 1024);
+#pragma unroll
+            for (int w = 1; w < 4; ++w) {
+                const f32x4 v = *reinterpret_cast<lds_f32x4_ptr>(buf + (w * 16 + 4 * wave + jj) * 1024);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sum[e] += v[e];
+            }
+            res[round][jj] = sum;
+        }
+    }
+
+    // ---- store: res[r][jj][e] = C[32 r + 16 (w / 2) + lane % 16][64 (w % 2) + 16 jj + 4 (lane / 16) + e] of the tile
+    OutType* cbase = C + size_t(m0 + 16 * (wave >> 1) + frow) * ldc + n0 + 64 * (wave & 1) + 4 * fquad;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            OutType* p = cbase + size_t(32 * r) * ldc + 16 * jj;
+            if constexpr (sizeof(OutType) == 4) {
+                *reinterpret_cast<f32x4*>(p) = res[r][jj];
+            } else {
+                f16x4 h;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(res[r][jj][e]);
+                *reinterpret_cast<f16x4*>(p) = h;
+            }
+        }
+    }
+}
+
+}  // namespace tiledcuda::kernels

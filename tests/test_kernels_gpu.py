@@ -301,6 +301,38 @@ def test_gemm_tile_api_wave128_is_the_wave128_kernel(tcu, oracle, device, M, N, 
     assert torch.equal(C, tcu.gemm(dA, dB, out_dtype=dt, algo="wave128"))
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 128, 256), (128, 384, 384), (512, 512, 512), (256, 256, 640),
+                                   (2048, 2048, 2048)])
+@pytest.mark.parametrize("out_dtype", ["f16", "f32"])
+def test_gemm_wave128_ksplit(tcu, oracle, device, M, N, K, out_dtype):
+    """The kernel whose four wavefronts each own the whole 128 x 128 tile over a quarter of K and add their partial
+    tiles through LDS: 1 to 5 tiles of K (odd and even counts: the fragment buffers alternate) against the oracle,
+    guard rows around C; 2048^3 is the shape AUTO sends to it, so AUTO must give the same bits there."""
+    import torch
+
+    print(f"gemm wave128_ksplit {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float16 if out_dtype == "f16" else torch.float32
+    A = oracle.fill_uniform(M * K, 7200 + K).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 8200 + K).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    guard = torch.full((M + 2, N), -7.0, dtype=dt, device=device)
+    out = guard[1:M + 1]
+    tcu.gemm(dA, dB, out=out, algo="wave128_ksplit")
+    torch.cuda.synchronize()
+    assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
+    rows = (0, M) if M <= 1024 else (M - 192, M)
+    ref = oracle.gemm(A, Bt, rows=rows)
+    assert oracle.max_rel_err(host(out)[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
+    if M == 2048:
+        assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt))
+        # every row of the product, through the column sums: C^T 1 = B (A^T 1)
+        col = A.astype(np.float64).sum(axis=0)
+        want = Bt.astype(np.float64) @ col
+        got = host(out).astype(np.float64).sum(axis=0)
+        # entries are ~N(0, 15^2); f16 rounding (<= 2^-11 |c| each) of 2048 of them adds up to about a unit
+        assert np.max(np.abs(got - want)) <= (5.0 if out_dtype == "f16" else 0.1)
+
+
 @pytest.mark.parametrize("algo", ["pipelined", "wave128"])
 def test_gemm_one_hot_index_probe(tcu, device, algo):
     """C[m, n] = A[m, k] * Bt[n, k] for one-hot operands: pins rows/cols/transposition exactly."""
