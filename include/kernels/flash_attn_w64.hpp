@@ -449,7 +449,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     auto step = [&](const RingOffsets& ring, auto cur_c, auto qk_c, auto loads_c, auto next_qk_c, int load_block) {
         constexpr int kCur = decltype(cur_c)::value, kNxt = kCur ^ 1;
         constexpr bool kQk = decltype(qk_c)::value;
-        constexpr int kLoads = decltype(loads_c)::value;  // 0: none, 1: block `load_block` of K and V, 2: warm-up loads
+        constexpr int kLoads = decltype(loads_c)::value;  // 0: none, 1: block `load_block` of K and V, 2 / 3: warm-up loads
         constexpr bool kNextQk = decltype(next_qk_c)::value;
         // K of half i + 1 (block J + 1; its first half for odd i), V of half i - 1 (block J), K of half i + 2, V of half i
         const unsigned int sk = ring.b + (kCur == 1 ? 0 : Traits::kHalfBytes);
@@ -517,6 +517,14 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 const __half* src = (s < kL / 2 ? warm_a : warm_b) + (wave * (kL / 2) + (s & 3)) * 512;
                 const unsigned int dst = __builtin_amdgcn_readfirstlane(lds_base + ring.load + ldst[s]);
                 detail::mfma32_out_then_load(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2], lane * 16u, src, dst);
+            } else if constexpr (kLoads == 3) {
+                // as 2, but warm_b is the first block of a column-major V (128 pieces of 128 bytes, N elements apart):
+                // fetched with the offsets of the ring loads of a V block
+                const bool is_v = s >= kL / 2;
+                const __half* src = is_v ? warm_b : warm_a + (wave * (kL / 2) + (s & 3)) * 512;
+                const unsigned int dst = __builtin_amdgcn_readfirstlane(lds_base + ring.load + ldst[s]);
+                detail::mfma32_out_then_load(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2],
+                                             is_v ? goff[s] : lane * 16u, src, dst);
             } else {
                 detail::mfma32_out(o_acc[s & 3][0], vf[s % kRing], pf[kNxt][0][s >> 2]);
             }
@@ -664,10 +672,10 @@ __global__ void __launch_bounds__(Traits::kThreads)
             advance();
             hand_over(std::integral_constant<int, 0>{});
             // K block 0 is 16 KiB of consecutive rows; so is a row-major V block (a column-major one is 128 pieces of
-            // 128 bytes: K block 1 is fetched in its place)
+            // 128 bytes, which the offsets of the ring loads describe)
             warm_a = K + size_t(nhead) * N * kD;
-            warm_b = kVColMajor ? warm_a + kBN * kD : V + size_t(nhead) * N * kD;
-            step(ring, C1{}, Yes{}, Warm{}, Yes{}, 0);
+            warm_b = V + size_t(nhead) * N * kD;
+            step(ring, C1{}, Yes{}, std::integral_constant<int, kVColMajor ? 3 : 2>{}, Yes{}, 0);
             step(ring, C0{}, Yes{}, No{}, Yes{}, 0);
             advance();
         }
