@@ -50,14 +50,14 @@ typedef enum {
                                 4096^3, 1024^3, 512x768x192, 256x256x64; results identical to PIPELINED bit for bit */
     TCU_GEMM_RAGGED = 6,      /* run-time M, N, K in multiples of 16: MFMA operand tiles filled from global memory,
                                 tiles beyond the edge skipped; the fallback for shapes the tiled kernels do not cover */
-    TCU_GEMM_WAVE128_KSPLIT = 8, /* 128 x 128 tile on 4 wavefronts (one per SIMD) that each own the whole tile over a
-                                quarter of every 128-wide step of K, partial tiles added through LDS: for products with
-                                too few 256 x 256 tiles to fill the GPU (2048^3); M, N, K multiples of 128; the sum over
-                                K is taken in four interleaved parts (differs from the other kernels by f32 rounding) */
-    TCU_GEMM_TILE_WAVE128 = 7 /* the WAVE128 kernel composed from tile-library functors only (direct-to-LDS loads dealt
+    TCU_GEMM_TILE_WAVE128 = 7, /* the WAVE128 kernel composed from tile-library functors only (direct-to-LDS loads dealt
                                 a piece at a time, single-fragment LDS reads, gemm_scheduled() with accumulators pinned
                                 in AGPRs); compile-time shapes: 4096^3, 1024^3, 512x768x192, 256x256x64; results
                                 identical to WAVE128 and PIPELINED bit for bit */
+    TCU_GEMM_WAVE128_KSPLIT = 8 /* 128 x 128 tile on 4 wavefronts (one per SIMD) that each own the whole tile over a
+                                quarter of every 128-wide step of K, partial tiles added through LDS: for products with
+                                too few 256 x 256 tiles to fill the GPU (2048^3); M, N, K multiples of 128; the sum over
+                                K is taken in four interleaved parts (differs from the other kernels by f32 rounding) */
 } tcu_gemm_algo;
 
 /* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks ROWS for many rows, else RESIDENT, where
