@@ -126,6 +126,10 @@ def test_unsupported_shapes_are_reported_not_launched(tcu):
     assert l.tcu_gemm_f16(p, p, p, 64, 64, 40, 0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_gemm_f16(p, p, p, 256, 256, 256, 0, 1, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_gemm_f16(p, p, p, 128, 256, 64, 0, 4, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
+    assert l.tcu_gemm_f16(p, p, p, 512, 512, 512, 0, 7, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # tile-API kernels: fixed shapes
+    assert l.tcu_gemm_f16(p, p, p, 256, 256, 192, 0, 8, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # K-splitting kernel: K % 128
+    assert l.tcu_gemm_f16(p, p, p, 192, 256, 256, 0, 8, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # ... and M, N % 128
+    assert l.tcu_gemm_f16(p, p, p, 256, 256, 256, 0, 9, 0) == tcu.TCU_ERR_INVALID_ARGUMENT
     assert l.tcu_b2b_gemm_f16(p, p, p, p, 64, 96, 64, 64, 1, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 64, 128, 64, 1.0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_flash_attn_fwd_f16(p, p, p, p, 1, 64, 100, 128, 128, 1.0, 1, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
