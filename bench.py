@@ -429,6 +429,20 @@ def main():
                                 "speed_vs_hipblaslt": min(blas_us) / min(ours_us),
                                 "method": "interleaved, 150 untimed + 100 timed launches each, best of 2"}}
         del dC2
+        # the other GEMM shapes of the comparison table (random operands of the same distribution; both libraries through
+        # their default dispatch, 60 untimed + 40 timed launches each, the better of two passes)
+        shapes = []
+        for (m_, n_, k_) in [(8192, 8192, 8192), (8192, 4096, 4096), (2048, 8192, 8192), (3072, 4096, 4096),
+                             (16384, 16384, 1024), (4096, 4096, 16384), (2048, 2048, 2048), (1024, 1024, 8192)]:
+            a_ = (torch.rand(m_, k_, device=dev) * 2 - 1).half()
+            b_ = (torch.rand(n_, k_, device=dev) * 2 - 1).half()
+            c_ = torch.empty(m_, n_, dtype=torch.float16, device=dev)
+            ours = min(time_kernel(lambda: tcu.gemm(a_, b_, out=c_), 40, 60) for _ in range(2)) * 1e3
+            blas = min(time_kernel(lambda: torch.matmul(a_, b_.t(), out=c_), 40, 60) for _ in range(2)) * 1e3
+            shapes.append({"shape": [m_, n_, k_], "this_library_us": ours, "hipblaslt_us": blas,
+                           "this_library_tflops": 2.0 * m_ * n_ * k_ / ours / 1e6, "speed_vs_hipblaslt": blas / ours})
+            del a_, b_, c_
+        vendor["gemm_other_shapes"] = shapes
         if vendor_attention is not None:
             vendor["flash_attn_fwd_b4_h16_s2048_d128"] = vendor_attention
 
