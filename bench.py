@@ -12,8 +12,9 @@ Prints ONE JSON line: the driver's contract fields plus
                   "sustained_mfma" entry is the rate and core clock the GPU holds on a loop of nothing but
                   MFMAs fed with the same operand distribution (the matrix pipe is power-managed, so this
                   is the practical ceiling; the published peak assumes 2.4 GHz)
-  cpu_baseline -- the reference's CPU path (fp32 torch.matmul; fp32 softmax(QK^T)V on a sample of heads) and the
-                  OpenMP oracle, timed on this host's cores for the same workloads
+  cpu_baseline -- the reference's CPU path (fp32 torch.matmul; fp32 softmax(QK^T)V on a sample of heads; the LSTM
+                  layer as an explicit fp32 loop; the back-to-back GEMM as two fp32 matmuls) and the OpenMP oracle,
+                  timed on this host's cores for the same workloads
   vendor_library_same_run -- hipBLASLt (through torch.matmul) on the headline operands and torch's fused attention on
                   the C4 operands, timed after the figures above in the same process, with this library re-timed beside
                   them: boxes of the pool differ by several percent, only a same-run ratio says who is ahead
@@ -484,6 +485,42 @@ def main():
             cpu["attention_f32"] = {"value": reps * heads * 4.0 * S * S * D / dta / 1e12, "unit": "TFLOP/s", "cores": cores,
                                     "sample": f"{reps} x {heads} of the 64 (batch, head) items of B4 H16 S2048 D128, explicit "
                                               f"softmax(QK^T/sqrt(d))V in fp32 with torch, {dta:.1f} s"}
+        # (2b) the fused LSTM layer as an explicit fp32 loop (gates = [x_t, h] W^T + b; i, f, g, o; c and h updates) with
+        # torch on the full C5 shape, and the back-to-back GEMM of C3 as two fp32 matmuls
+        if want("lstm"):
+            xf, Wf, bf = torch.from_numpy(x).float(), torch.from_numpy(W).float(), torch.from_numpy(b).float()
+            Wt = Wf.t().contiguous()
+            reps, t0 = 0, time.perf_counter()
+            while True:
+                h_ = torch.zeros(Bb, Hh)
+                c_ = torch.zeros(Bb, Hh)
+                for t_ in range(T):
+                    gates = torch.addmm(bf, torch.cat((xf[t_], h_), dim=1), Wt)
+                    gi, gf, gg, go = gates.split(Hh, dim=1)
+                    c_ = torch.sigmoid(gf) * c_ + torch.sigmoid(gi) * torch.tanh(gg)
+                    h_ = torch.sigmoid(go) * torch.tanh(c_)
+                reps += 1
+                dtl = time.perf_counter() - t0
+                if dtl >= 3.0 or reps >= 64:
+                    break
+            lstm_bytes = (2.0 * (4 * Hh * (I + Hh) + 4 * Hh + Bb * I + 2 * Bb * Hh) + 4.0 * 2 * Bb * Hh) * T
+            cpu["lstm_f32"] = {"value": reps * lstm_bytes / dtl / 1e9, "unit": "GB/s", "us_per_step": dtl / reps / T * 1e6,
+                               "tflops": reps * 2.0 * Bb * (I + Hh) * 4 * Hh * T / dtl / 1e12, "cores": cores,
+                               "sample": f"{reps} x the full layer (B256 I1024 H1024 T16) as an explicit fp32 loop with torch "
+                                         f"in {dtl:.1f} s; GB/s counts the algorithmic fp16/fp32 bytes of the GPU path"}
+            del xf, Wf, bf, Wt
+        if want("b2b"):
+            a3, b3, c3 = torch.from_numpy(A3).float(), torch.from_numpy(B3).float(), torch.from_numpy(C3).float()
+            reps, t0 = 0, time.perf_counter()
+            while True:
+                torch.matmul(torch.matmul(a3, b3.t()), c3.t())
+                reps += 1
+                dtb = time.perf_counter() - t0
+                if dtb >= 1.0 or reps >= 256:
+                    break
+            cpu["b2b_gemm_f32"] = {"value": reps * (2.0 * 8192 * 128 * 256 * 2) / dtb / 1e12, "unit": "TFLOP/s", "cores": cores,
+                                   "sample": f"{reps} x (A B) C for 8192x256x128x128 as two fp32 torch.matmul calls in {dtb:.1f} s"}
+            del a3, b3, c3
         # (3) the OpenMP f32-accumulate oracle on the same GEMM (what the parity tests check against)
         oracle.gemm(A, Bt, rows=(0, 64))  # warm the thread pool
         reps, t0 = 0, time.perf_counter()
