@@ -268,6 +268,20 @@ def main():
                         "first_launches_us": ms_first * 1e3, "conditioning_launches": 200,
                         "tflops": flops / (ms * 1e-3) / 1e12,
                         "frac_mfma_peak": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, "max_abs_err": err})
+        # a longer sequence on the same kernel (not a BASELINE configuration): the fixed cost per 256-query item is
+        # amortised over four times the keys
+        Sl, Hl = 8192, 32  # 1024 workgroups: a grid no other launch of this kernel in the run has
+        ql, kl, vl = (oracle.fill_normal(Hl * Sl * D, seed).reshape(Hl, Sl, D) for seed in (1241, 2241, 3241))
+        dql, dkl, dvl = (to_dev(t.reshape(1, Hl, Sl, D)) for t in (ql, kl, vl))
+        dol = torch.empty(1, Hl, Sl, D, dtype=torch.float16, device=dev)
+        ms_long = time_kernel(lambda: tcu.flash_attention(dql, dkl, dvl, out=dol), 15, 20)
+        err_long = oracle.max_abs_err(dol.reshape(Hl, Sl, D)[3, 4096:4160].float().cpu().numpy(),
+                                      oracle.attention(ql[3], kl[3], vl[3], scale, rows=(4096, 4160))[4096:4160])
+        flops_long = 4.0 * Hl * Sl * Sl * D
+        configs.append({"name": "flash_attn_fwd_b1_h32_s8192_d128_longer_sequence", "kernel": "flash_attention_fwd_w64<128>",
+                        "ms": ms_long, "tflops": flops_long / (ms_long * 1e-3) / 1e12,
+                        "frac_mfma_peak": flops_long / (ms_long * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, "max_abs_err": err_long})
+        del dql, dkl, dvl, dol
         configs.append({"name": "flash_attention_fwd_op_convention_b64_s2048_d128_v_col_major",
                         "kernel": "flash_attention_fwd_w64<128, column-major V>", "ms": ms_op,
                         "tflops": flops / (ms_op * 1e-3) / 1e12,
