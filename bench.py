@@ -115,7 +115,7 @@ def probe_mfma(torch, operands, shape, waves=8, iters=20000):
     """Sustained MFMA rate on `operands` (fp16 device tensor, >= 256*waves*4096 halves): TFLOP/s and core MHz."""
     import ctypes
 
-    lib = ctypes.CDLL(os.path.join(ROOT, "tiledcuda_amd", "lib", "libtcu_probe.so"))
+    lib = ctypes.CDLL(os.path.join(ROOT, "bench_support", "_build", "libtcu_probe.so"))
     lib.tcu_probe_mfma_f16.restype = ctypes.c_int
     lib.tcu_probe_mfma_f16.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4 + [ctypes.c_void_p]
     wgs = 256

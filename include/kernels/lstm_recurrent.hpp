@@ -27,7 +27,7 @@
 //     `spin_ticks` (100 MHz ticks): when it expires, or when a group is spread over several XCDs, the workgroup
 //     raises the error word and exits, and so does, in turn, every workgroup that waits for it. The outputs are then
 //     invalid; the host reads the word.
-// sync: 1 KiB-aligned device words, all zero at launch: [g] the XCDs group g runs on (one bit each), [8] error,
+// sync: 128-byte aligned device words, all zero at launch: [g] the XCDs group g runs on (one bit each), [8] error,
 // [32 (g + 1)] the step counter of group g (128 bytes apart). Requirements: H == 1024 (the register budget), B % 32 == 0,
 // B <= 256 (8 XCDs), grid == 256 workgroups of 256 threads.
 #pragma once

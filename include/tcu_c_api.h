@@ -80,7 +80,8 @@ typedef enum {
 } tcu_v_layout;
 
 /* Which attention kernel to run (tcu_flash_attn_fwd_f16_algo). For a row-major V, AUTO picks WAVE64 for long sequences
- * (head size 128, M % 256 == 0, N >= 1024, at least 128 blocks of 256 queries) and MFMA32_FUSED otherwise. */
+ * (head size 128, M % 256 == 0, N >= 1024, at least 128 blocks of 256 queries) and MFMA32_FUSED otherwise; for a
+ * column-major V (head size 128) AUTO always picks WAVE64, which takes every M % 64 == 0 and N % 64 == 0. */
 typedef enum {
     TCU_ATTN_AUTO = 0,
     TCU_ATTN_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, like the reference kernel */
@@ -90,7 +91,8 @@ typedef enum {
                                   when they keep growing along the keys; same results up to rounding */
     TCU_ATTN_WAVE64 = 4        /* 4 wavefronts x 64 queries, one per SIMD: half the LDS traffic per MFMA, all matrix
                                   instructions placed by hand, softmax of 32 keys interleaved with the MFMAs of the
-                                  neighbouring 32; row-major V, head size 128, M % 256 == 0 */
+                                  neighbouring 32; either V layout, head size 128, M % 64 == 0 (wavefronts of the
+                                  last workgroup whose 64 queries lie beyond M idle), N % 64 == 0, N * 256 < 2^32 */
 } tcu_attn_algo;
 
 /* Which LSTM step kernel to run (tcu_lstm_f16_algo). AUTO picks STREAMING where it is instantiated, else
@@ -211,8 +213,9 @@ int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* 
  * one GEMM into the workspace; the recurrence then runs weight-stationary: every XCD keeps a copy of W[:, I:] in the
  * registers of its 32 CUs and owns 32 batch rows, and h_t is exchanged between those CUs through the XCD's L2 only.
  * Same arguments and results (up to the order of the f32 summation) as tcu_lstm_f16_ws. `workspace`: device memory of
- * at least tcu_lstm_persistent_workspace_bytes(T, B, I, H) bytes (0 = shape not supported), 1 KiB-aligned, owned by
- * the caller; its first 4 KiB are synchronisation words, cleared by the call.
+ * at least tcu_lstm_persistent_workspace_bytes(T, B, I, H) bytes (0 = shape not supported), 128-byte aligned (the step
+ * counters sit in cache lines of their own), owned by the caller; its first 4 KiB are synchronisation words, cleared by
+ * the call.
  * The launch needs all of its 256 workgroups resident at the same time, i.e. a GPU that is not occupied by another
  * kernel for long; its waits are bounded (2 s; TCU_LSTM_PERSISTENT_SPIN_US in the environment overrides, in
  * microseconds), and every workgroup exits normally when a wait expires. The call itself is asynchronous like all

@@ -1020,6 +1020,30 @@ def test_lstm_persistent_bounded_wait(tcu, device, monkeypatch):
     assert torch.equal(good[0], again[0]) and torch.equal(good[1], again[1])
 
 
+def test_lstm_persistent_workspace_at_allocator_granularity(tcu, device):
+    """torch's caching allocator hands out blocks in multiples of 512 bytes: a workspace that starts at an odd multiple
+    of 512 is a valid argument (the step counters need 128-byte alignment only) and gives the same result."""
+    import torch
+
+    T, B, I, H = 4, 64, 64, 1024
+    g = torch.Generator(device="cpu").manual_seed(7)
+    x = (torch.randn(T, B, I, generator=g) * 0.5).half().to(device)
+    W = (torch.randn(4 * H, I + H, generator=g) * 0.03).half().to(device)
+    b = (torch.randn(4 * H, generator=g) * 0.1).half().to(device)
+    need = tcu.lstm_persistent_workspace_bytes(T, B, I, H)
+    buf = torch.empty(need + 2048, dtype=torch.uint8, device=device)
+    base = (-buf.data_ptr()) % 1024  # offset of the first 1 KiB boundary inside buf
+    print("lstm persistent: workspace at 1 KiB + 512", flush=True)
+    aligned = tcu.lstm(x, W, b, algo="persistent", workspace=buf[base:base + need])
+    odd = buf[base + 512:base + 512 + need]
+    assert odd.data_ptr() % 1024 == 512
+    shifted = tcu.lstm(x, W, b, algo="persistent", workspace=odd)
+    torch.cuda.synchronize()
+    assert torch.equal(aligned[0], shifted[0]) and torch.equal(aligned[1], shifted[1])
+    with pytest.raises(RuntimeError, match="aligned"):
+        tcu.lstm(x, W, b, algo="persistent", workspace=buf[base + 64:base + 64 + need])
+
+
 def test_lstm_persistent_rejects_what_it_cannot_do(tcu, device):
     import torch
 

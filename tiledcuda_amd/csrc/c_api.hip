@@ -22,6 +22,8 @@
 #include <set>
 #include <algorithm>
 #include <string>
+#include <tuple>
+#include <type_traits>
 #include <utility>
 
 using namespace tiledcuda;
@@ -45,9 +47,13 @@ int hip_fail(hipError_t e, const char* what) {
     return fail(TCU_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
 }
 
-/// Launch with dynamic LDS; raises the limit when the kernel needs more than the default.
-template <typename Kernel, typename... Args>
-int launch(Kernel kernel, dim3 grid, dim3 block, int lds_bytes, hipStream_t stream, Args... args) {
+/// Launch with dynamic LDS; raises the limit when the kernel needs more than the default. The kernel's parameter types
+/// are taken from the kernel pointer and every argument is converted to its parameter's type before its address goes
+/// into the argument array: an argument of another width or a wrong count is a compile error, not a garbled launch.
+template <typename... Params, typename... Args>
+int launch(void (*kernel)(Params...), dim3 grid, dim3 block, int lds_bytes, hipStream_t stream, Args&&... args) {
+    static_assert(sizeof...(Params) == sizeof...(Args), "launch: argument count differs from the kernel's parameter count");
+    static_assert((std::is_convertible_v<Args&&, Params> && ...), "launch: an argument does not convert to its parameter's type");
     if (lds_bytes > kMaxLdsBytes) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "kernel needs more LDS than a CU has");
     if (lds_bytes > 48 * 1024) {
         // once per kernel function (and per device: the attribute is per device)
@@ -71,7 +77,11 @@ int launch(Kernel kernel, dim3 grid, dim3 block, int lds_bytes, hipStream_t stre
     }
     // the launch's own return value: an error left behind earlier by unrelated code of the calling thread is neither
     // reported as this launch's nor cleared
-    void* argv[] = {static_cast<void*>(&args)...};
+    std::tuple<std::remove_cv_t<Params>...> params(std::forward<Args>(args)...);
+    void* argv[sizeof...(Params) + 1];
+    [&]<size_t... kIs>(std::index_sequence<kIs...>) {
+        ((argv[kIs] = static_cast<void*>(&std::get<kIs>(params))), ...);
+    }(std::index_sequence_for<Params...>{});
     hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, size_t(lds_bytes), stream);
     if (e != hipSuccess) return hip_fail(e, "kernel launch");
     return TCU_OK;
@@ -834,8 +844,8 @@ int tcu_lstm_f16_persistent(const void* x, const void* W, const void* bias, cons
     if (!x || !W || !bias || !h_all || !c_out || !workspace)
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: null pointer");
     if (!positive({T, B, I, H})) return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: sizes must be positive");
-    if (!aligned16({x, W, bias, h0, c0, h_all, c_out}) || reinterpret_cast<uintptr_t>(workspace) % 1024 != 0)
-        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: operands must be 16-byte aligned, the workspace 1 KiB-aligned");
+    if (!aligned16({x, W, bias, h0, c0, h_all, c_out}) || reinterpret_cast<uintptr_t>(workspace) % 128 != 0)
+        return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: operands must be 16-byte aligned, the workspace 128-byte aligned");
     const unsigned long long need = tcu_lstm_persistent_workspace_bytes(T, B, I, H);
     if (need == 0)
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_persistent: needs H == 1024, I % 64 == 0, B % 32 == 0, B <= 256 "
