@@ -158,64 +158,163 @@ struct GemmMfmaTiles {
 
 }  // namespace detail
 
-/// gemm with the instruction stream under the caller's control, for kernels that run ONE wavefront per SIMD (a
-/// wavefront tile so large that its accumulators fill the AGPR half of the SIMD lane's 512 registers: nothing else can
-/// feed the matrix pipe while that wavefront does something else, so where its LDS reads and global loads issue
-/// relative to its matrix instructions decides the kernel's speed):
-///   * the matrix instructions are inline assembly with the accumulator tiles constrained to AGPRs (left alone, the
-///     compiler moves large accumulator sets through VGPRs and spills) and are issued in the order written here:
-///     k-step by k-step, row of A tiles by row, the tiles of a row forwards in even rows and backwards in odd ones, so
-///     that every instruction shares an operand with the one before it;
+/// Which register file an accumulator or operand of a scheduled product is pinned in. A wavefront that runs alone on
+/// its SIMD has 256 VGPRs and 256 AGPRs; the matrix instructions take their accumulator and either operand from both.
+enum class RegFile { kVgpr = 0, kAgpr = 1 };
+
+/// The matrix instructions of a tile product c += a b, one at a time, for kernels that place every instruction
+/// themselves (one wavefront per SIMD: nothing else feeds the matrix pipe while that wavefront does something else,
+/// so where its LDS reads, global loads and vector-ALU work sit relative to its matrix instructions decides the
+/// kernel's speed). at<i, j, k>(a, b, c) issues c(i, j) += a(i, k) b(k, j) as inline assembly, with the accumulator
+/// tile constrained to kAccFile and the A tile to kAFile (left alone, the compiler moves large accumulator sets through
+/// VGPRs and spills); the statements are volatile, so they stay in the order written. Operand tiles: 16 x 32 / 32 x 16
+/// (v_mfma_f32_16x16x32_f16, accumulator of 16 x 16 BaseTiles) or 32 x 16 / 16 x 32 (v_mfma_f32_32x32x16_f16,
+/// 32 x 32 accumulator tiles) of f16; the sums are those of gemm(a, b, c) bit for bit.
+/// The compiler does not know these statements are matrix instructions and inserts none of the wait states their
+/// results need before other instructions read them: keep every such read at least two matrix instructions behind the
+/// write, or call settle_accumulators(c) first; and compile the kernel so that c can stay where it is between the
+/// calls (__launch_bounds__ of one wavefront per SIMD when the pinned tiles need more than 256 registers).
+template <typename RegTileA, typename RegTileB, typename RegTileC, const RegFile kAccFile = RegFile::kAgpr,
+          const RegFile kAFile = RegFile::kVgpr>
+struct ScheduledGemm {
+    using G = detail::GemmMfmaTiles<RegTileA, RegTileB, RegTileC>;
+    static constexpr int kMs = G::kMs, kNs = G::kNs, kKs = G::kKs;
+    static constexpr int kCount = kMs * kNs * kKs;
+    using Acc = std::conditional_t<G::k16, f32x4, f32x16>;
+
+#define TCU_SCHEDULED_MFMA(ACC, AOP)                                                                              \
+    if constexpr (G::k16)                                                                                         \
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+" ACC(acc) : "v"(bv), AOP(av));               \
+    else                                                                                                          \
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+" ACC(acc) : "v"(bv), AOP(av))
+#define TCU_SCHEDULED_MFMA_LOAD(ACC, AOP)                                                                         \
+    if constexpr (G::k16)                                                                                         \
+        asm volatile("s_mov_b32 m0, %5\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %3, %4" \
+                     : "+" ACC(acc)                                                                               \
+                     : "v"(bv), AOP(av), "v"(load.offset), "s"(load.base), "s"(load.lds_addr)                    \
+                     : "m0", "memory");                                                                           \
+    else                                                                                                          \
+        asm volatile("s_mov_b32 m0, %5\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %3, %4" \
+                     : "+" ACC(acc)                                                                               \
+                     : "v"(bv), AOP(av), "v"(load.offset), "s"(load.base), "s"(load.lds_addr)                    \
+                     : "m0", "memory")
+#define TCU_SCHEDULED_MFMA_FROM(ACC, AOP)                                                                         \
+    if constexpr (G::k16)                                                                                         \
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %3" : "=&" ACC(acc) : "v"(bv), AOP(av), "v"(from));   \
+    else                                                                                                          \
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&" ACC(acc) : "v"(bv), AOP(av), "v"(from))
+#define TCU_SCHEDULED_DISPATCH(MACRO)                                                 \
+    if constexpr (kAccFile == RegFile::kAgpr && kAFile == RegFile::kVgpr) {           \
+        MACRO("a", "v");                                                              \
+    } else if constexpr (kAccFile == RegFile::kAgpr && kAFile == RegFile::kAgpr) {    \
+        MACRO("a", "a");                                                              \
+    } else if constexpr (kAccFile == RegFile::kVgpr && kAFile == RegFile::kVgpr) {    \
+        MACRO("v", "v");                                                              \
+    } else {                                                                          \
+        MACRO("v", "a");                                                              \
+    }
+
+    /// c(kI, kJ) += a(kI, kK) b(kK, kJ).
+    template <int kI, int kJ, int kK>
+    DEVICE static void at(const RegTileA& a, const RegTileB& b, RegTileC& c) {
+        f16x8 av, bv;
+        Acc acc;
+        __builtin_memcpy(&av, a(kI, kK).data(), sizeof(av));
+        __builtin_memcpy(&bv, b(kK, kJ).data(), sizeof(bv));
+        __builtin_memcpy(&acc, c(kI, kJ).data(), sizeof(acc));
+        TCU_SCHEDULED_DISPATCH(TCU_SCHEDULED_MFMA)
+        __builtin_memcpy(c(kI, kJ).mutable_data(), &acc, sizeof(acc));
+    }
+
+    /// The same, followed in the same statement by a direct-to-LDS load (a copy::DirectLoad): m0 is written before the
+    /// matrix instruction, which thereby is the wait state the load needs after that write.
+    template <int kI, int kJ, int kK, typename Load>
+    DEVICE static void at(const RegTileA& a, const RegTileB& b, RegTileC& c, const Load& load) {
+        f16x8 av, bv;
+        Acc acc;
+        __builtin_memcpy(&av, a(kI, kK).data(), sizeof(av));
+        __builtin_memcpy(&bv, b(kK, kJ).data(), sizeof(bv));
+        __builtin_memcpy(&acc, c(kI, kJ).data(), sizeof(acc));
+        TCU_SCHEDULED_DISPATCH(TCU_SCHEDULED_MFMA_LOAD)
+        __builtin_memcpy(c(kI, kJ).mutable_data(), &acc, sizeof(acc));
+    }
+
+    /// c(kI, kJ) = a(kI, kK) b(kK, kJ) + init: the first instruction of a product whose sums start from another tile
+    /// (held in VGPRs) instead of from c's old contents, e.g. scores accumulated from minus the row maximum.
+    template <int kI, int kJ, int kK, typename TileInit>
+    DEVICE static void at_from(const RegTileA& a, const RegTileB& b, RegTileC& c, const TileInit& init) {
+        f16x8 av, bv;
+        Acc acc, from;
+        static_assert(sizeof(TileInit) == sizeof(Acc), "the initial tile must have the accumulator tile's shape");
+        __builtin_memcpy(&av, a(kI, kK).data(), sizeof(av));
+        __builtin_memcpy(&bv, b(kK, kJ).data(), sizeof(bv));
+        __builtin_memcpy(&from, init.data(), sizeof(from));
+        TCU_SCHEDULED_DISPATCH(TCU_SCHEDULED_MFMA_FROM)
+        __builtin_memcpy(c(kI, kJ).mutable_data(), &acc, sizeof(acc));
+    }
+#undef TCU_SCHEDULED_DISPATCH
+#undef TCU_SCHEDULED_MFMA_FROM
+#undef TCU_SCHEDULED_MFMA_LOAD
+#undef TCU_SCHEDULED_MFMA
+};
+
+/// The whole product c += a b through ScheduledGemm, in a fixed order, with a hook per instruction:
+///   * the instructions go k-step by k-step, row of A tiles by row, the tiles of a row forwards in even rows and
+///     backwards in odd ones, so that every instruction shares an operand with the one before it;
 ///   * before instruction number n = (k * kMs + i) * kNs + position-in-row the caller's hook is called with
 ///     std::integral_constant<int, n>: the place for the fragment reads of the next k-step (SharedToRegLoader::load_one)
 ///     - they are ordinary LDS reads, the compiler keeps them between the assembly statements they are written between;
 ///   * if the hook returns something (a copy::DirectLoad), that direct-to-LDS load is issued in the same assembly
-///     statement as the instruction: m0 is written before the matrix instruction, which thereby is the wait state the
-///     load needs after that write.
-/// The compiler does not know these statements are matrix instructions and inserts none of the wait states their
-/// results need before other instructions read them: call settle_accumulators(c) before c is read by anything else,
-/// and compile the kernel so that c can stay where it is between the calls - __launch_bounds__ of one wavefront per
-/// SIMD (256 threads) when c and the operand tiles need more than 256 registers. A compiler forced to spill or move
-/// an accumulator between two of these statements reads it without the wait, and the result is wrong.
-/// Operands: 16 x 32 / 32 x 16 MFMA tiles of f16, accumulator of 16 x 16 BaseTiles (v_mfma_f32_16x16x32_f16); the sums
-/// are those of gemm(a, b, c) bit for bit.
+///     statement as the instruction;
+///   * if the hook has a member after(std::integral_constant<int, n>), it is called behind instruction n: the place
+///     for small doses of vector-ALU work (one transcendental plus one or two plain instructions hide under a matrix
+///     instruction of the same wavefront; larger groups cost their full issue time), e.g. a slice of a softmax.
+/// Accumulators in AGPRs, operands in VGPRs. See ScheduledGemm for what the caller owes the accumulators
+/// (settle_accumulators before any other read, __launch_bounds__ of one wavefront per SIMD).
 template <typename RegTileA, typename RegTileB, typename RegTileC, typename Hook>
 DEVICE void gemm_scheduled(const RegTileA& a, const RegTileB& b, RegTileC& c, Hook&& hook) {
-    using G = detail::GemmMfmaTiles<RegTileA, RegTileB, RegTileC>;
-    static_assert(G::k16, "gemm_scheduled is written for v_mfma_f32_16x16x32_f16 operand tiles");
-    constexpr int kMs = G::kMs, kNs = G::kNs, kKs = G::kKs;
+    using S = ScheduledGemm<RegTileA, RegTileB, RegTileC>;
+    constexpr int kMs = S::kMs, kNs = S::kNs;
     [&]<int... kIs>(std::integer_sequence<int, kIs...>) {
         (
             [&] {
                 constexpr int n = kIs;
                 constexpr int k = n / (kMs * kNs), i = n / kNs % kMs, pos = n % kNs;
                 constexpr int j = (i & 1) ? kNs - 1 - pos : pos;
-                f16x8 av, bv;
-                f32x4 acc;
-                using HookResult = decltype(hook(std::integral_constant<int, n>{}));
+                using N = std::integral_constant<int, n>;
+                using HookResult = decltype(hook(N{}));
                 if constexpr (std::is_void_v<HookResult>) {
-                    hook(std::integral_constant<int, n>{});
-                    __builtin_memcpy(&av, a(i, k).data(), sizeof(av));
-                    __builtin_memcpy(&bv, b(k, j).data(), sizeof(bv));
-                    __builtin_memcpy(&acc, c(i, j).data(), sizeof(acc));
-                    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(bv), "v"(av));
+                    hook(N{});
+                    S::template at<i, j, k>(a, b, c);
                 } else {
-                    const HookResult load = hook(std::integral_constant<int, n>{});
-                    __builtin_memcpy(&av, a(i, k).data(), sizeof(av));
-                    __builtin_memcpy(&bv, b(k, j).data(), sizeof(bv));
-                    __builtin_memcpy(&acc, c(i, j).data(), sizeof(acc));
-                    asm volatile(
-                        "s_mov_b32 m0, %5\n\t"
-                        "v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\t"
-                        "global_load_lds_dwordx4 %3, %4"
-                        : "+a"(acc)
-                        : "v"(bv), "v"(av), "v"(load.offset), "s"(load.base), "s"(load.lds_addr)
-                        : "m0", "memory");
+                    const HookResult load = hook(N{});
+                    S::template at<i, j, k>(a, b, c, load);
                 }
-                __builtin_memcpy(c(i, j).mutable_data(), &acc, sizeof(acc));
+                if constexpr (requires { hook.after(N{}); }) hook.after(N{});
             }(),
             ...);
-    }(std::make_integer_sequence<int, kMs * kNs * kKs>{});
+    }(std::make_integer_sequence<int, S::kCount>{});
+}
+
+/// Pin every tile of a register tile in the given register file as of here (an empty statement the compiler must
+/// satisfy): operand tiles that a ScheduledGemm takes from AGPRs, or values that must not be rematerialised later.
+template <const RegFile kFile, typename Reg>
+DEVICE void pin_tiles(Reg& t) {
+    [&]<int... kIs>(std::integer_sequence<int, kIs...>) {
+        (
+            [&] {
+                using Tile = typename Reg::DType;
+                using Vec = std::conditional_t<sizeof(Tile) == 16, u32x4, u32x16>;
+                static_assert(sizeof(Tile) == sizeof(Vec), "tiles of 4 or 16 registers per lane");
+                auto& tile = t(kIs / Reg::kCols, kIs % Reg::kCols);
+                Vec v;
+                __builtin_memcpy(&v, tile.data(), sizeof(v));
+                if constexpr (kFile == RegFile::kAgpr) asm volatile("" : "+a"(v));
+                else asm volatile("" : "+v"(v));
+                __builtin_memcpy(tile.mutable_data(), &v, sizeof(v));
+            }(),
+            ...);
+    }(std::make_integer_sequence<int, Reg::kRows * Reg::kCols>{});
 }
 
 /// Clear an accumulator tile and place it in AGPRs, where gemm_scheduled keeps it (the statements also keep the
@@ -225,7 +324,10 @@ DEVICE void clear_pinned(RegTileC& c) {
     [&]<int... kIs>(std::integer_sequence<int, kIs...>) {
         (
             [&] {
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                using Acc = std::conditional_t<sizeof(typename RegTileC::DType) == sizeof(f32x4), f32x4, f32x16>;
+                Acc acc;
+#pragma unroll
+                for (int e = 0; e < int(sizeof(Acc) / sizeof(float)); ++e) acc[e] = 0.f;
                 asm volatile("" : "+a"(acc));
                 __builtin_memcpy(c(kIs / RegTileC::kCols, kIs % RegTileC::kCols).mutable_data(), &acc, sizeof(acc));
             }(),
@@ -243,7 +345,8 @@ DEVICE void settle_accumulators(RegTileC& c) {
         (
             [&] {
                 auto& tile = c(kIs / RegTileC::kCols, kIs % RegTileC::kCols);
-                f32x4 acc;
+                using Acc = std::conditional_t<sizeof(typename RegTileC::DType) == sizeof(f32x4), f32x4, f32x16>;
+                Acc acc;
                 __builtin_memcpy(&acc, tile.data(), sizeof(acc));
                 asm volatile("" : "+a"(acc));
                 __builtin_memcpy(tile.mutable_data(), &acc, sizeof(acc));

@@ -128,7 +128,8 @@ struct GlobalToSharedDirectPieces {
 
     /// Piece j of the copy of the global tile whose first element is at `src` into `dst`.
     DEVICE DirectLoad piece(int j, const DType* src, const Shared& dst) const {
-        const unsigned int lds = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(dst.data())) +
+        using lds_cptr = __attribute__((address_space(3))) const void*;
+        const unsigned int lds = static_cast<unsigned int>(reinterpret_cast<uintptr_t>((lds_cptr)(dst.data()))) +
                                  static_cast<unsigned int>(wave_ * kPieces + j) * 1024u;
         return DirectLoad{offset_[j], src, static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(lds))};
     }

@@ -231,4 +231,149 @@ struct SharedToRegLoaderTr : public Base {
     }
 };
 
+/// Wait until at most kOutstanding of this wavefront's LDS reads are still in flight (they return in order): the
+/// companion of SharedToRegPieces / SharedToRegTrPieces, whose reads the compiler does not track.
+template <int kOutstanding>
+DEVICE void wait_shared_reads() {
+    static_assert(kOutstanding >= 0 && kOutstanding < 16);
+    __builtin_amdgcn_s_waitcnt(0xC07F | (kOutstanding << 8));  // lgkmcnt(kOutstanding), nothing else
+}
+
+namespace detail {
+/// Wave-uniform LDS byte address of logical line 0, element 0 of a (sub-)tile whose origin lies a multiple of the
+/// swizzle's line period into its allocation (the permutation then looks the same from the view as from the tile).
+template <typename Shared>
+DEVICE unsigned int shared_view_address(const Shared& tile) {
+    // (through an LDS-qualified pointer: the cast back from the generic address space then folds away, where the
+    // truncation of a generic address would keep a null check per use)
+    using lds_cptr = __attribute__((address_space(3))) const void*;
+    const unsigned int base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>((lds_cptr)(tile.data())));
+    return base + static_cast<unsigned int>(tile.line0() * Shared::kPitch + tile.elem0()) *
+                      static_cast<unsigned int>(sizeof(typename Shared::DType));
+}
+}  // namespace detail
+
+/// SharedToRegLoader a fragment at a time with the waits in the caller's hands, for kernels that run one wavefront
+/// per SIMD and request each operand fragment a fixed number of matrix instructions before its use, also across loop
+/// back-edges and between stages of a SharedRing. The compiler's own waits for LDS reads are exact only inside a basic
+/// block; across a back-edge it waits for every read in flight, including those just requested for later
+/// instructions. So the reads here are assembly the compiler does not track: read<i, j>() requests fragment (i, j) of
+/// the register tile (one ds_read_b128 for an MFMA operand tile of 2-byte elements), and the caller places
+/// wait_shared_reads<N>() before the first use. The per-lane byte offset of every fragment inside the tile (swizzle
+/// included) is computed once, at construction, and kept in a register; a read adds the wave-uniform address of the
+/// (sub-)tile it is pointed at: one vector addition per read.
+/// Shared_ is the tile type the offsets are computed for (a whole stage of a ring, or the sub-tile a wavefront's
+/// operand comes from); read() takes any view of that type whose origin is a multiple of the swizzle's line period.
+template <typename Reg_, typename Shared_, typename WarpLayout_, const WarpReuse kMode_,
+          typename Base = warp::CopyBase<WarpLayout_, kMode_>>
+struct SharedToRegPieces : public Base {
+    using Reg = Reg_;
+    using Shared = Shared_;
+    using BaseTile = typename Reg::DType;
+    using DType = typename BaseTile::DType;
+    using G = TileGeometry<BaseTile>;
+    using BaseShape = TileExtent<BaseTile>;
+    static_assert(std::is_same_v<typename Shared::DType, DType> && sizeof(DType) == 2 && G::kRuns == 1 && G::kRunLen == 8 &&
+                      G::kRowMajor == Shared::kIsRowMajor,
+                  "one ds_read_b128 per fragment: MFMA operand tiles of 2-byte elements whose runs lie along the lines");
+    static_assert(Base::template row_exec_count<BaseShape, Shared::kRows>() == Reg::kRows &&
+                      Base::template col_exec_count<BaseShape, Shared::kCols>() == Reg::kCols,
+                  "the register tile must hold exactly this wavefront's share of the shared tile");
+
+    DEVICE SharedToRegPieces() {
+        const int lane = lane_id();
+        const int major = lane % G::kLaneMajor, minor = (lane / G::kLaneMajor) * G::kRunLen;
+        const int row0 = Base::template warp_row0<Shared::kRows>();
+        const int col0 = Base::template warp_col0<Shared::kCols>();
+        const Shared whole(nullptr);
+#pragma unroll
+        for (int i = 0; i < Reg::kRows; ++i)
+#pragma unroll
+            for (int j = 0; j < Reg::kCols; ++j) {
+                const int row = row0 + i * BaseShape::kRows + (G::kRowMajor ? major : minor);
+                const int col = col0 + j * BaseShape::kCols + (G::kRowMajor ? minor : major);
+                offset_[i][j] = static_cast<unsigned int>(whole.offset(row, col)) * static_cast<unsigned int>(sizeof(DType));
+                asm volatile("" : "+v"(offset_[i][j]));  // computed once, not again at every use
+            }
+    }
+
+    /// Request fragment (kI, kJ) of this wavefront's share of `src` into dst(kI, kJ); not waited for.
+    template <int kI, int kJ>
+    DEVICE void read(const Shared& src, Reg& dst) const {
+        f16x8 r;
+        asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(offset_[kI][kJ] + detail::shared_view_address(src)));
+        __builtin_memcpy(dst(kI, kJ).mutable_data(), &r, sizeof(r));
+    }
+
+  private:
+    unsigned int offset_[Reg::kRows][Reg::kCols];
+};
+
+/// The same for the transposing read (SharedToRegLoaderTr: a column-major operand out of a row-major shared tile):
+/// read<i, j>() requests the two ds_read_b64_tr_b16 of operand tile (i, j). One per-lane offset per COLUMN of operand
+/// tiles is kept; the contraction index (the tile's row i) is an immediate of the instruction, which requires a
+/// swizzle whose line period divides 4 (tl::LdsSwizzleTr).
+/// kAccumulatorOrder: which contraction indices a lane receives. false: the standard operand order (lane group
+/// g = lane / 32 or lane / 16 / ... holds indices 8 g .. 8 g + 7 of the tile's 16). true, for 16 x 32 tiles: the order
+/// in which the 32 x 32 accumulator of a preceding product holds its columns - slot e of lane half h is index
+/// 8 (e / 4) + 4 h + e % 4 - so that accumulator values converted to 2-byte elements ARE the A operand of the next
+/// product without leaving the lane (the contraction index of a matrix instruction may be permuted as long as both
+/// operands agree).
+template <typename Reg_, typename Shared_, typename WarpLayout_, const WarpReuse kMode_, const bool kAccumulatorOrder = false,
+          typename Base = warp::CopyBase<WarpLayout_, kMode_>>
+struct SharedToRegTrPieces : public Base {
+    using Reg = Reg_;
+    using Shared = Shared_;
+    using BaseTile = typename Reg::DType;
+    using DType = typename BaseTile::DType;
+    using G = TileGeometry<BaseTile>;
+    using BaseShape = TileExtent<BaseTile>;
+    static_assert(std::is_same_v<typename Shared::DType, DType> && sizeof(DType) == 2 && Shared::kIsRowMajor &&
+                      !G::kRowMajor && G::kRunLen == 8 && G::kRuns == 1,
+                  "the transposing read serves column-major operand tiles of 2-byte elements out of a row-major tile");
+    static_assert(!Shared::kSwizzled || 4 % Shared::Swizzle::kLinePeriod == 0,
+                  "the tile's row is an immediate of the read: the swizzle must repeat every 4 lines (tl::LdsSwizzleTr)");
+    static_assert(!kAccumulatorOrder || G::kLaneMajor == 32, "the accumulator order is that of the 32 x 32 accumulator");
+    static_assert(Base::template row_exec_count<BaseShape, Shared::kRows>() == Reg::kRows &&
+                      Base::template col_exec_count<BaseShape, Shared::kCols>() == Reg::kCols,
+                  "the register tile must hold exactly this wavefront's share of the shared tile");
+    static constexpr int kLineBytes = Shared::kPitch * int(sizeof(DType));
+    // rows between the two reads of an operand tile, and how many rows a lane group's index moves the first one
+    static constexpr int kPartRows = kAccumulatorOrder ? 8 : 4;
+    static constexpr int kGroupRows = kAccumulatorOrder ? 4 : 8;
+
+    DEVICE SharedToRegTrPieces() {
+        const int lane = lane_id();
+        const int L = lane & 15;
+        const int col_grp = ((lane >> 4) % (G::kLaneMajor / 16)) * 16;
+        const int line = Base::template warp_row0<Shared::kRows>() + (lane / G::kLaneMajor) * kGroupRows + (L >> 2);
+        const int col0 = Base::template warp_col0<Shared::kCols>();
+        const Shared whole(nullptr);
+#pragma unroll
+        for (int j = 0; j < Reg::kCols; ++j) {
+            const int col = col0 + j * BaseShape::kCols + col_grp + 4 * (L & 3);
+            offset_[j] = static_cast<unsigned int>(whole.offset(line, col)) * static_cast<unsigned int>(sizeof(DType));
+            asm volatile("" : "+v"(offset_[j]));
+        }
+    }
+
+    /// Request operand tile (kI, kJ) of this wavefront's share of the view `src` shifted down by kLine0 lines (a
+    /// multiple of 4, folded into the instruction's immediate together with the tile's own row); not waited for.
+    template <int kI, int kJ, int kLine0 = 0>
+    DEVICE void read(const Shared& src, Reg& dst) const {
+        static_assert(kLine0 % 4 == 0);
+        constexpr int kOff0 = (kLine0 + kI * BaseShape::kRows) * kLineBytes, kOff1 = kOff0 + kPartRows * kLineBytes;
+        static_assert(kOff1 < 65536, "the immediate offset of an LDS read has 16 bits");
+        f16x4 lo, hi;
+        asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                     : "=&v"(lo), "=&v"(hi)
+                     : "v"(offset_[kJ] + detail::shared_view_address(src)), "n"(kOff0), "n"(kOff1));
+        const f16x8 r = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        __builtin_memcpy(dst(kI, kJ).mutable_data(), &r, sizeof(r));
+    }
+
+  private:
+    unsigned int offset_[Reg::kCols];
+};
+
 }  // namespace tiledcuda::cell::copy

@@ -37,4 +37,16 @@ DEVICE void wait_group_and_barrier() {
     asm volatile("" ::: "memory");
 }
 
+/// wait_group_and_barrier for a kernel that keeps LDS fragment reads in flight across the hand-over (requested with
+/// copy::SharedToRegPieces for the matrix instructions that follow the barrier): only the vector-memory counter is
+/// waited for. Correct when the reads in flight address stages that are not being handed over - the caller's
+/// business, like the reads' own waits (copy::wait_shared_reads).
+template <int N = 0>
+DEVICE void wait_group_and_barrier_keep_reads() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00 | (N & 0xF) | ((N >> 4) << 14));  // vmcnt(N) only
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 }  // namespace tiledcuda::cell

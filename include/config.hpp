@@ -24,6 +24,7 @@ using f32x4 = float __attribute__((ext_vector_type(4)));
 using f32x16 = float __attribute__((ext_vector_type(16)));
 using u32x2 = unsigned __attribute__((ext_vector_type(2)));
 using u32x4 = unsigned __attribute__((ext_vector_type(4)));
+using u32x16 = unsigned __attribute__((ext_vector_type(16)));
 
 DEVICE int lane_id() { return static_cast<int>(threadIdx.x) & (kWaveSize - 1); }
 DEVICE int wave_id() { return static_cast<int>(threadIdx.x) >> 6; }

@@ -89,10 +89,15 @@ typedef enum {
     TCU_ATTN_MFMA32_FUSED = 3, /* MFMA32 with the softmax of block j+1 computed speculatively under the MFMAs of
                                   block j: faster when row maxima settle early, up to ~10 % slower than MFMA32
                                   when they keep growing along the keys; same results up to rounding */
-    TCU_ATTN_WAVE64 = 4        /* 4 wavefronts x 64 queries, one per SIMD: half the LDS traffic per MFMA, all matrix
+    TCU_ATTN_WAVE64 = 4,       /* 4 wavefronts x 64 queries, one per SIMD: half the LDS traffic per MFMA, all matrix
                                   instructions placed by hand, softmax of 32 keys interleaved with the MFMAs of the
                                   neighbouring 32; either V layout, head size 128, M % 64 == 0 (wavefronts of the
                                   last workgroup whose 64 queries lie beyond M idle), N % 64 == 0, N * 256 < 2^32 */
+    TCU_ATTN_TILE_WAVE64 = 5   /* the WAVE64 kernel composed from tile-library functors only (matrix instructions placed
+                                  one by one with ScheduledGemm, interleaved 5-stage shared rings, fragment reads issued
+                                  ahead with SharedToRegPieces / SharedToRegTrPieces); compile-time sequence lengths:
+                                  (M, N) in {(2048, 2048), (512, 1024), (256, 640), (256, 320)}, head size 128, row-major
+                                  V; results identical to WAVE64 bit for bit */
 } tcu_attn_algo;
 
 /* Which LSTM step kernel to run (tcu_lstm_f16_algo). AUTO picks STREAMING where it is instantiated, else

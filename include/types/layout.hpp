@@ -110,12 +110,34 @@ struct LdsSwizzle {
         detail::cmax(1, detail::cmin(16 / kLinesPerWindow, detail::pow2_divisor(kChunksPerLine) >> kShift));
 
     static_assert(kPitch % kChunk == 0, "the pitch of a shared tile must be a multiple of 4 elements");
+    /// apply(line + kLinePeriod, elem) == apply(line, elem): a view that starts a multiple of this many lines into
+    /// the tile sees the same permutation (so its line offset is purely additive).
+    static constexpr int kLinePeriod = kLinesPerWindow * kNumSwz;
 
     /// Position, within its line, of logical element `elem` of line `line`.
     HOST_DEVICE static constexpr int apply(int line, int elem) {
         const int chunk = elem >> 2;
         const int s = ((line / kLinesPerWindow) & (kNumSwz - 1)) << kShift;
         return ((chunk ^ s) << 2) | (elem & 3);
+    }
+};
+
+/// XOR permutation for tiles of 2-byte elements that are read ACROSS their lines with the transposing LDS read
+/// (ds_read_b64_tr_b16: the B operand of a matrix instruction out of a row-major tile, e.g. V [keys, head_dim] of an
+/// attention layer). One pass of such a read serves two 16-lane groups, each of which fetches 4 consecutive lines x 32
+/// bytes; the two groups sit on adjacent 32-byte units. Lines of 256 bytes all start on bank 0, so the 4 lines are spread
+/// with unit ^= 2 * (line % 4); lines of 128 bytes alternate between the two halves of the banks, so only lines 2 apart
+/// collide: unit ^= line & 2. 32-byte units (and with them the 16-byte pieces of direct-to-LDS loads) stay contiguous.
+template <const int kPitch, const int kElemBytes>
+struct LdsSwizzleTr {
+    static_assert(kElemBytes == 2 && (kPitch == 128 || kPitch == 64),
+                  "written for lines of 128 or 256 bytes of 2-byte elements");
+    static constexpr int kUnit = 16;  // elements per 32-byte unit
+    static constexpr int kLinePeriod = 4;
+
+    HOST_DEVICE static constexpr int apply(int line, int elem) {
+        const int s = kPitch == 128 ? ((line & 3) << 1) : (line & 2);
+        return (((elem / kUnit) ^ s) * kUnit) | (elem % kUnit);
     }
 };
 

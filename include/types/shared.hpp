@@ -4,17 +4,23 @@
 // function of absolute coordinates within the pitched allocation.
 #pragma once
 
+#include <type_traits>
+
 #include "types/layout.hpp"
 #include "util/print.hpp"
 
 namespace tiledcuda::cell {
 namespace tl = tile_layout;
 
-template <typename Element_, typename Layout_, const bool kSwizzled_ = false>
+/// SwizzlePolicy_: which XOR permutation a swizzled tile uses (void = tl::LdsSwizzle, the one for plain vector reads
+/// along a line; tl::LdsSwizzleTr for tiles read across lines with the transposing LDS read). Sub-tiles cut by
+/// STileIterator keep their tile's policy.
+template <typename Element_, typename Layout_, const bool kSwizzled_ = false, typename SwizzlePolicy_ = void>
 class SharedTile {
   public:
     using DType = Element_;
     using Layout = Layout_;
+    using SwizzlePolicy = SwizzlePolicy_;
 
     static constexpr int kNumel = tl::get_numel<Layout>;
 
@@ -34,7 +40,7 @@ class SharedTile {
     static constexpr int kLines = kIsRowMajor ? kRows : kCols;
     static constexpr int kLineLen = kIsRowMajor ? kCols : kRows;
 
-    using Swizzle = tl::LdsSwizzle<kPitch, sizeof(DType)>;
+    using Swizzle = std::conditional_t<std::is_void_v<SwizzlePolicy_>, tl::LdsSwizzle<kPitch, sizeof(DType)>, SwizzlePolicy_>;
 
     HOST_DEVICE SharedTile(DType* data) : data_(data), line0_(0), elem0_(0) {}
 
@@ -84,15 +90,21 @@ class SharedTile {
 
 /// kStages copies of a shared tile laid out back to back: the LDS side of a multi-stage global -> LDS pipeline
 /// (the reference's kernels have one stage and wait for every load, examples/cpp/01_gemm/02_gemm_all_mem/gemm.hpp:139-143).
-/// ring[s] is a whole-tile view of stage s; stages advance modulo kStages.
-template <typename Shared_, const int kStages_>
+/// ring[s] is a whole-tile view of stage s; stages advance modulo kStages. kStrideNumel_: elements from one stage to
+/// the next (0 = the tile's own size: stages back to back); larger when the stages of two rings are interleaved, e.g.
+/// the K and V blocks of an attention kernel as [K0 V0 K1 V1 ...].
+template <typename Shared_, const int kStages_, const int kStrideNumel_ = 0>
 class SharedRing {
   public:
     using Shared = Shared_;
     using DType = typename Shared::DType;
     static constexpr int kStages = kStages_;
-    static constexpr int kStageNumel = Shared::kLines * Shared::kPitch;
-    static constexpr int kBytes = kStages * kStageNumel * int(sizeof(DType));
+    static constexpr int kTileNumel = Shared::kLines * Shared::kPitch;
+    static constexpr int kStageNumel = kStrideNumel_ == 0 ? kTileNumel : kStrideNumel_;
+    static_assert(kStageNumel >= kTileNumel, "stages must not overlap");
+    static constexpr int kStageBytes = kStageNumel * int(sizeof(DType));
+    // bytes from the first stage's start to the last stage's end
+    static constexpr int kBytes = ((kStages - 1) * kStageNumel + kTileNumel) * int(sizeof(DType));
 
     HOST_DEVICE explicit SharedRing(DType* base) : base_(base) {}
 

@@ -47,7 +47,7 @@ class STileIterator {
 
     HOST_DEVICE auto operator()(int x, int y) const {
         using SubLayout = tl::MatrixLayout<kChunkRow, kChunkCol, Tile::kRowStride, Tile::kColStride>;
-        using NewTile = SharedTile<DType, SubLayout, Tile::kSwizzled>;
+        using NewTile = SharedTile<DType, SubLayout, Tile::kSwizzled, typename Tile::SwizzlePolicy>;
         const int row = x * kChunkRow, col = y * kChunkCol;
         return Tile::kIsRowMajor ? NewTile(data_, line0_ + row, elem0_ + col)
                                  : NewTile(data_, line0_ + col, elem0_ + row);
@@ -55,14 +55,14 @@ class STileIterator {
 
     HOST_DEVICE auto operator()(int x, const Underscore&) const {
         using SubLayout = tl::MatrixLayout<kChunkRow, Tile::kCols, Tile::kRowStride, Tile::kColStride>;
-        using Iter = STileIterator<SharedTile<DType, SubLayout, Tile::kSwizzled>, ChunkShape>;
+        using Iter = STileIterator<SharedTile<DType, SubLayout, Tile::kSwizzled, typename Tile::SwizzlePolicy>, ChunkShape>;
         const int row = x * kChunkRow;
         return Tile::kIsRowMajor ? Iter(data_, line0_ + row, elem0_) : Iter(data_, line0_, elem0_ + row);
     }
 
     HOST_DEVICE auto operator()(const Underscore&, int y) const {
         using SubLayout = tl::MatrixLayout<Tile::kRows, kChunkCol, Tile::kRowStride, Tile::kColStride>;
-        using Iter = STileIterator<SharedTile<DType, SubLayout, Tile::kSwizzled>, ChunkShape>;
+        using Iter = STileIterator<SharedTile<DType, SubLayout, Tile::kSwizzled, typename Tile::SwizzlePolicy>, ChunkShape>;
         const int col = y * kChunkCol;
         return Tile::kIsRowMajor ? Iter(data_, line0_, elem0_ + col) : Iter(data_, line0_ + col, elem0_);
     }

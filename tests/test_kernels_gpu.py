@@ -747,6 +747,35 @@ def test_flash_attention_wave64_maximum_jumps_late(tcu, oracle, device):
     assert oracle.max_abs_err(host(O), ref) <= 2e-2  # logits of several hundred: see test_flash_attention_growing_maxima
 
 
+@pytest.mark.parametrize("batch,M,N", [(3, 256, 320), (8, 256, 640), (2, 512, 1024), (64, 2048, 2048)])
+def test_flash_attention_tile_wave64_is_wave64(tcu, oracle, device, batch, M, N):
+    """The one-wavefront-per-SIMD kernel composed from tile-library functors (tile_wave64) does the arithmetic of the
+    hand-indexed one in the same order: bit-identical outputs, at 5 key blocks (the minimum), at sizes with one and two
+    rounds of workgroups, and with keys that force the rare re-basing path; and within tolerance of the oracle."""
+    import torch
+
+    D = 128
+    print(f"attention tile_wave64 b{batch} {M}x{N}", flush=True)
+    q = oracle.fill_normal(batch * M * D, 81).reshape(batch, M, D).astype(np.float32)
+    k = oracle.fill_normal(batch * N * D, 82).reshape(batch, N, D).astype(np.float32)
+    v = oracle.fill_normal(batch * N * D, 83).reshape(batch, N, D)
+    if N == 640:
+        qdir = q / np.linalg.norm(q, axis=-1, keepdims=True)
+        for pos, gain in ((0, 30.0), (200, 60.0), (225, 120.0), (300, 200.0), (639, 400.0)):
+            k[:, pos] = qdir[:, pos % M] * gain
+    q, k = q.astype(np.float16), k.astype(np.float16)
+    dq, dk, dv = dev(q, device), dev(k, device), dev(v, device)
+    ref_kernel = tcu.flash_attention(dq, dk, dv, algo="wave64")
+    out = torch.full_like(ref_kernel, float("nan"))
+    tcu.flash_attention(dq, dk, dv, out=out, algo="tile_wave64")
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref_kernel)
+    heads = [0, batch - 1]
+    ref = oracle.attention(np.ascontiguousarray(q[heads, :64]), np.ascontiguousarray(k[heads]), np.ascontiguousarray(v[heads]),
+                           1.0 / math.sqrt(D))
+    assert oracle.max_abs_err(host(out)[heads, :64], ref) <= (2e-2 if N == 640 else ABS_TOL)
+
+
 def test_flash_attention_properties(tcu, oracle, device):
     """Size-independent properties: constant V, zero scale, joint permutation of keys/values."""
     import torch

@@ -6,6 +6,7 @@
 
 #include "kernels/b2b_gemm_fwd.hpp"
 #include "kernels/flash_attn_fwd.hpp"
+#include "kernels/flash_attn_tile_w64.hpp"
 #include "kernels/flash_attn_w64.hpp"
 #include "kernels/gemm_pipelined.hpp"
 #include "kernels/gemm_ragged.hpp"
@@ -526,6 +527,28 @@ int launch_fa_w64(const __half* Q, const __half* K, const __half* V, __half* O, 
                   dim3(Traits::kThreads), Traits::kLdsBytes, stream, Q, K, V, O, batch, M, N, scale);
 }
 
+template <int kM, int kN>
+int launch_fa_tile_w64(const __half* Q, const __half* K, const __half* V, __half* O, int batch, float scale,
+                       hipStream_t stream) {
+    using Traits = FlashW64TileTraits<__half, kM, kN, 128>;
+    return launch(&flash_attention_tile_w64<__half, Traits>, dim3((kM / Traits::kTM) * batch), dim3(Traits::kThreads),
+                  Traits::kShmBytes, stream, Q, K, V, O, batch, scale);
+}
+
+/// The one-wavefront-per-SIMD kernel composed from tile-library functors: compile-time sequence lengths, like every
+/// kernel written against the tile API (the benchmark shape and the shapes its tests use).
+int fa_tile_w64_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, int Kd,
+                         float scale, int v_layout, hipStream_t stream) {
+    if (Kd != 128 || v_layout != TCU_V_ROW_MAJOR)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the tile-API one-wavefront-per-SIMD attention kernel takes head size 128 and a row-major V");
+    if (M == 2048 && N == 2048) return launch_fa_tile_w64<2048, 2048>(Q, K, V, O, batch, scale, stream);
+    if (M == 512 && N == 1024) return launch_fa_tile_w64<512, 1024>(Q, K, V, O, batch, scale, stream);
+    if (M == 256 && N == 640) return launch_fa_tile_w64<256, 640>(Q, K, V, O, batch, scale, stream);
+    if (M == 256 && N == 320) return launch_fa_tile_w64<256, 320>(Q, K, V, O, batch, scale, stream);
+    return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the tile-API one-wavefront-per-SIMD attention kernel is instantiated for "
+                                           "(M, N) in {(2048, 2048), (512, 1024), (256, 640), (256, 320)}");
+}
+
 template <int kD, bool kFused>
 int fa_fwd_by_rows(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
                    hipStream_t stream) {
@@ -540,9 +563,10 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     if (Kd != P) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs the query and value head sizes equal");
     if (M % 64 != 0 || N % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs M % 64 == 0 and N % 64 == 0");
     if (algo != TCU_ATTN_AUTO && algo != TCU_ATTN_TILE_LIBRARY && algo != TCU_ATTN_MFMA32 &&
-        algo != TCU_ATTN_MFMA32_FUSED && algo != TCU_ATTN_WAVE64)
+        algo != TCU_ATTN_MFMA32_FUSED && algo != TCU_ATTN_WAVE64 && algo != TCU_ATTN_TILE_WAVE64)
         return fail(TCU_ERR_INVALID_ARGUMENT, "unknown attention algo");
     if (v_layout != TCU_V_ROW_MAJOR && v_layout != TCU_V_COL_MAJOR) return fail(TCU_ERR_INVALID_ARGUMENT, "unknown v_layout");
+    if (algo == TCU_ATTN_TILE_WAVE64) return fa_tile_w64_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
     if (algo == TCU_ATTN_WAVE64) {
         if (Kd != 128)
             return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel is instantiated for head size 128");
