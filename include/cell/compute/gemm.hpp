@@ -174,6 +174,10 @@ enum class RegFile { kVgpr = 0, kAgpr = 1 };
 /// results need before other instructions read them: keep every such read at least two matrix instructions behind the
 /// write, or call settle_accumulators(c) first; and compile the kernel so that c can stay where it is between the
 /// calls (__launch_bounds__ of one wavefront per SIMD when the pinned tiles need more than 256 registers).
+/// The same holds in the other direction: a vector-ALU write to a register (clearing an accumulator, converting an
+/// operand) DIRECTLY in front of the matrix instruction that reads it is not waited for either - observed on gfx950: the
+/// instruction took the register's previous contents as its C operand. Write such registers a few instructions ahead
+/// (clear_pinned / pin_tiles at the point where the tile is set up, not in front of the product).
 template <typename RegTileA, typename RegTileB, typename RegTileC, const RegFile kAccFile = RegFile::kAgpr,
           const RegFile kAFile = RegFile::kVgpr>
 struct ScheduledGemm {

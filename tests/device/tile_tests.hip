@@ -18,6 +18,7 @@
 // CPU oracle or against the identity.
 #include "cell/mod.hpp"
 #include "types/mod.hpp"
+#include "util/static_for.hpp"
 
 #include <string>
 #include <utility>
@@ -429,6 +430,152 @@ __global__ void __launch_bounds__(kScheduled ? 256 : 512) k_tile_gemm_mfma(const
     r2g(acc, gC);
 }
 
+/// A gemm_scheduled hook that does nothing before an instruction and counts the calls behind them.
+struct CountingHook {
+    int issued = 0;
+    template <typename N>
+    DEVICE void operator()(N) {}
+    template <typename N>
+    DEVICE void after(N) {
+        ++issued;
+    }
+};
+
+// C = A · B with the fragment-at-a-time readers of a one-wavefront-per-SIMD kernel: A through SharedToRegPieces (one
+// untracked ds_read_b128 per operand tile), B stored ROW-major [kK, kN] in a tile with the transposing-read swizzle
+// (tl::LdsSwizzleTr) through SharedToRegTrPieces (standard contraction order), both waited for with
+// wait_shared_reads; the matrix instructions through gemm_scheduled on v_mfma_f32_32x32x16_f16 tiles (accumulators
+// pinned in AGPRs), whose after() hook runs behind every instruction (here it counts them into C's padding check).
+template <int kM, int kN, int kK, typename WarpLayout>
+__global__ void __launch_bounds__(256) k_tile_gemm_pieces(const __half* dA, const __half* dB, float* dC) {
+    extern __shared__ __align__(1024) unsigned char buf[];
+    auto* sA_ptr = reinterpret_cast<__half*>(buf);
+    auto* sB_ptr = sA_ptr + kM * kK;
+    constexpr int kWR = tl::num_rows<WarpLayout>, kWC = tl::num_cols<WarpLayout>;
+    using Shape = traits::MfmaTileShape<__half, traits::MfmaShape::k32x32x16>;
+    using GlobalA = GlobalTile<__half, tl::RowMajor<kM, kK>>;
+    using SharedA = SharedTile<__half, tl::RowMajor<kM, kK>, true>;
+    using RegA = RegTile<typename Shape::TileA, tl::RowMajor<kM / kWR / 32, kK / 16>>;
+    using GlobalB = GlobalTile<__half, tl::RowMajor<kK, kN>>;
+    using SharedB = SharedTile<__half, tl::RowMajor<kK, kN>, true, tl::LdsSwizzleTr<kN, 2>>;
+    using RegB = RegTile<typename Shape::TileB, tl::ColMajor<kK / 16, kN / kWC / 32>>;
+    using GlobalC = GlobalTile<float, tl::RowMajor<kM, kN>>;
+    using RegC = RegTile<typename Shape::TileC, tl::RowMajor<kM / kWR / 32, kN / kWC / 32>>;
+
+    GlobalA gA(dA);
+    GlobalB gB(dB);
+    SharedA sA(sA_ptr);
+    SharedB sB(sB_ptr);
+    GlobalToSharedDirectLoader<SharedA, WarpLayout> g2s_a;
+    GlobalToSharedDirectLoader<SharedB, WarpLayout> g2s_b;
+    g2s_a(gA, sA);
+    g2s_b(gB, sB);
+    wait_group_and_barrier<0>();
+
+    SharedToRegPieces<RegA, SharedA, WarpLayout, WarpReuse::kRowReuseCont> read_a;
+    SharedToRegTrPieces<RegB, SharedB, WarpLayout, WarpReuse::kColReuseCont> read_b;
+    RegA rA;
+    RegB rB;
+    RegC acc;
+    compute::clear_pinned(acc);
+    static_for<RegA::kRows>([&](auto i_c) {
+        static_for<RegA::kCols>([&](auto k_c) { read_a.template read<decltype(i_c)::value, decltype(k_c)::value>(sA, rA); });
+    });
+    static_for<RegB::kRows>([&](auto k_c) {
+        static_for<RegB::kCols>([&](auto j_c) { read_b.template read<decltype(k_c)::value, decltype(j_c)::value>(sB, rB); });
+    });
+    wait_shared_reads<0>();
+    CountingHook hook;
+    compute::gemm_scheduled(rA, rB, acc, hook);
+    compute::settle_accumulators(acc);
+    if (hook.issued != RegA::kRows * RegA::kCols * RegB::kCols) return;  // C stays NaN: the case fails
+    GlobalC gC(dC);
+    RegToGlobalStorer<GlobalC, RegC, WarpLayout> r2g;
+    r2g(acc, gC);
+}
+
+// D = f16(A · B) · V on wavefronts that own 32 rows each: the 32 x 32 accumulator tiles of the first product, converted
+// to f16 in place, ARE the A operand of the second one, because V (row-major [kN, kP], transposing-read swizzle) is
+// fetched in the accumulator's own contraction order (SharedToRegTrPieces<..., kAccumulatorOrder = true>); every
+// matrix instruction placed with ScheduledGemm::at. b = B column-major (stored [kN, kK]) followed by V.
+template <int kM, int kN, int kK, int kP, typename WarpLayout>
+__global__ void __launch_bounds__(256) k_tile_b2b_accumulator_order(const __half* dA, const __half* dBV, float* dD) {
+    extern __shared__ __align__(1024) unsigned char buf[];
+    auto* sA_ptr = reinterpret_cast<__half*>(buf);
+    auto* sB_ptr = sA_ptr + kM * kK;
+    auto* sV_ptr = sB_ptr + kN * kK;
+    constexpr int kWR = tl::num_rows<WarpLayout>;
+    static_assert(tl::num_cols<WarpLayout> == 1 && kM == 32 * kWR);
+    using Shape = traits::MfmaTileShape<__half, traits::MfmaShape::k32x32x16>;
+    using SharedA = SharedTile<__half, tl::RowMajor<kM, kK>, true>;
+    using SharedB = SharedTile<__half, tl::ColMajor<kK, kN>, true>;
+    using SharedV = SharedTile<__half, tl::RowMajor<kN, kP>, true, tl::LdsSwizzleTr<kP, 2>>;
+    using RegA = RegTile<typename Shape::TileA, tl::RowMajor<1, kK / 16>>;
+    using RegB = RegTile<typename Shape::TileB, tl::ColMajor<kK / 16, kN / 32>>;
+    using RegS = RegTile<typename Shape::TileC, tl::RowMajor<1, kN / 32>>;
+    using RegP = RegTile<typename Shape::TileA, tl::RowMajor<1, kN / 16>>;
+    using RegV = RegTile<typename Shape::TileB, tl::ColMajor<kN / 16, kP / 32>>;
+    using RegD = RegTile<typename Shape::TileC, tl::RowMajor<1, kP / 32>>;
+    using GlobalD = GlobalTile<float, tl::RowMajor<kM, kP>>;
+
+    GlobalTile<__half, tl::RowMajor<kM, kK>> gA(dA);
+    GlobalTile<__half, tl::ColMajor<kK, kN>> gB(dBV);
+    GlobalTile<__half, tl::RowMajor<kN, kP>> gV(dBV + kN * kK);
+    SharedA sA(sA_ptr);
+    SharedB sB(sB_ptr);
+    SharedV sV(sV_ptr);
+    GlobalToSharedDirectLoader<SharedA, WarpLayout>{}(gA, sA);
+    GlobalToSharedDirectLoader<SharedB, WarpLayout>{}(gB, sB);
+    GlobalToSharedDirectLoader<SharedV, WarpLayout>{}(gV, sV);
+    wait_group_and_barrier<0>();
+
+    RegA rA;
+    RegB rB;
+    RegV rV;
+    // the accumulators of the first product are cleared (vector-ALU writes) HERE, well ahead of its first matrix
+    // instruction: see ScheduledGemm on vector-ALU writes directly in front of an instruction that reads them
+    RegS rS;
+    compute::pin_tiles<compute::RegFile::kVgpr>(rS);
+    SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>{}(sA, rA);
+    SharedToRegPieces<RegB, SharedB, WarpLayout, WarpReuse::kColReuseCont> read_b;
+    SharedToRegTrPieces<RegV, SharedV, WarpLayout, WarpReuse::kColReuseCont, true> read_v;
+    static_for<RegB::kRows * RegB::kCols>([&](auto n_c) {
+        constexpr int n = decltype(n_c)::value;
+        read_b.template read<n / RegB::kCols, n % RegB::kCols>(sB, rB);
+    });
+    static_for<RegV::kRows * RegV::kCols>([&](auto n_c) {
+        constexpr int n = decltype(n_c)::value;
+        read_v.template read<n / RegV::kCols, n % RegV::kCols>(sV, rV);
+    });
+    wait_shared_reads<0>();
+
+    // first product, accumulators in VGPRs (they are read by the vector ALU next)
+    using First = compute::ScheduledGemm<RegA, RegB, RegS, compute::RegFile::kVgpr, compute::RegFile::kVgpr>;
+    static_for<RegB::kCols>([&](auto j_c) {
+        static_for<RegA::kCols>([&](auto k_c) { First::template at<0, decltype(j_c)::value, decltype(k_c)::value>(rA, rB, rS); });
+    });
+    asm volatile("s_nop 15\n\ts_nop 3");
+    compute::pin_tiles<compute::RegFile::kVgpr>(rS);
+    // accumulator tile j, elements 8 s2 + e  ->  A operand tile 2 j + s2, element e
+    RegP rP;
+    static_for<RegS::kCols>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+#pragma unroll
+        for (int e = 0; e < 16; e += 2)
+            compute::convert_pair_here(rS(0, j)(e), rS(0, j)(e + 1), rP(0, 2 * j + e / 8).mutable_data() + e % 8);
+    });
+    RegD rD;
+    compute::clear_pinned(rD);
+    using Second = compute::ScheduledGemm<RegP, RegV, RegD>;
+    static_for<RegV::kRows>([&](auto k_c) {
+        static_for<RegV::kCols>([&](auto j_c) { Second::template at<0, decltype(j_c)::value, decltype(k_c)::value>(rP, rV, rD); });
+    });
+    compute::settle_accumulators(rD);
+    GlobalD gD(dD);
+    RegToGlobalStorer<GlobalD, RegD, WarpLayout> r2g;
+    r2g(rD, gD);
+}
+
 // ------------------------------------------------------------------ reduce / broadcast / softmax
 // src [kRows, kCols] f32 row-major, one wavefront per 16... rows split over kW wavefronts.
 // out_vec[kRows]: op 0 = row sum, 1 = row max; out_tile: op 2 = broadcast of row sums,
@@ -611,6 +758,30 @@ template <auto Kernel, typename E>
 void launch_ops(const void* a, const void*, void* c, void* d, int threads, int lds, hipStream_t s) {
     hipLaunchKernelGGL(Kernel, dim3(1), dim3(threads), lds, s, static_cast<const E*>(a), static_cast<E*>(c),
                        static_cast<E*>(d));
+}
+
+template <int kM, int kN, int kK, int kWR, int kWC>
+void reg_gemm_pieces() {
+    using W = tl::RowMajor<kWR, kWC>;
+    registry().push_back({"tile_gemm",
+                          "pieces_scheduled_mfma32x32x16_" + std::to_string(kM) + "x" + std::to_string(kN) + "x" +
+                              std::to_string(kK) + "_w" + std::to_string(kWR) + "x" + std::to_string(kWC) + "_b_row_major",
+                          {kM, kN, kK, 2, 1, 0, 0, 0},
+                          kWR * kWC * 64,
+                          (kM + kN) * kK * 2,
+                          &launch_gemm<k_tile_gemm_pieces<kM, kN, kK, W>>});
+}
+
+template <int kM, int kN, int kK, int kP, int kWR>
+void reg_b2b_acc_order() {
+    using W = tl::RowMajor<kWR, 1>;
+    registry().push_back({"tile_b2b",
+                          "accumulator_order_" + std::to_string(kM) + "x" + std::to_string(kN) + "x" + std::to_string(kK) +
+                              "x" + std::to_string(kP) + "_w" + std::to_string(kWR) + "x1",
+                          {kM, kN, kK, kP, 0, 0, 0, 0},
+                          kWR * 64,
+                          (kM * kK + kN * kK + kN * kP) * 2,
+                          &launch_gemm<k_tile_b2b_accumulator_order<kM, kN, kK, kP, W>>});
 }
 
 template <typename E>
@@ -977,6 +1148,17 @@ void build_registry() {
     reg_elementwise<__half, true, 32, 32, 1, 6>();
     reg_elementwise<__half, false, 32, 32, 1, 7>();
     reg_elementwise<__half, false, 32, 32, 1, 8>();
+
+    // (new cases go last: the host side seeds its inputs with the case number)
+    // fragment-at-a-time readers + gemm_scheduled on 32x32x16 tiles with an after() hook; B row-major
+    reg_gemm_pieces<64, 64, 64, 2, 2>();
+    reg_gemm_pieces<128, 128, 64, 2, 2>();
+    reg_gemm_pieces<128, 64, 128, 4, 1>();
+    reg_gemm_pieces<32, 128, 32, 1, 1>();
+    // two chained products with the accumulator of the first as the A operand of the second
+    reg_b2b_acc_order<32, 64, 64, 64, 1>();
+    reg_b2b_acc_order<64, 128, 32, 64, 2>();
+    reg_b2b_acc_order<128, 64, 128, 64, 4>();
 }
 
 thread_local std::string g_err;

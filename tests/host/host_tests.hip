@@ -174,6 +174,62 @@ static void test_swizzle(bool expect_conflict_free) {
     }
 }
 
+// The swizzle for tiles read with the transposing LDS read: a bijection per line that keeps 32-byte units whole and
+// repeats every 4 lines; one pass of ds_read_b64_tr_b16 (32 lanes = two 16-lane groups on adjacent 32-byte units, each
+// group fetching 4 consecutive lines x 4 x 8 bytes) must touch 64 distinct banks.
+template <int kPitch>
+static void test_swizzle_tr() {
+    using Swz = tl::LdsSwizzleTr<kPitch, 2>;
+    CHECK(Swz::kLinePeriod == 4);
+    for (int line = 0; line < 64; ++line) {
+        std::set<int> seen;
+        for (int e = 0; e < kPitch; ++e) {
+            const int p = Swz::apply(line, e);
+            CHECK(p >= 0 && p < kPitch);
+            seen.insert(p);
+            if (e % 16 == 0)
+                for (int t = 1; t < 16; ++t) CHECK(Swz::apply(line, e + t) == p + t);
+            CHECK(Swz::apply(line + 4, e) == p);
+        }
+        CHECK(int(seen.size()) == kPitch);
+    }
+    for (int line0 = 0; line0 < 64; line0 += 4) {
+        for (int col0 = 0; col0 < kPitch; col0 += 32) {
+            std::set<int> banks;
+            for (int lane = 0; lane < 32; ++lane) {
+                const int L = lane & 15, grp = lane >> 4;
+                const int line = line0 + (L >> 2), col = col0 + 16 * grp + 4 * (L & 3);
+                const int byte = (line * kPitch + Swz::apply(line, col)) * 2;
+                for (int b = 0; b < 8; b += 4) banks.insert(((byte + b) / 4) % 64);
+            }
+            CHECK(int(banks.size()) == 64);
+        }
+    }
+}
+
+// A ring whose stages are further apart than a tile (two rings interleaved in one allocation).
+static void test_strided_ring() {
+    using Shared = SharedTile<__half, tl::RowMajor<64, 128>, true>;
+    using Packed = SharedRing<Shared, 5>;
+    using Strided = SharedRing<Shared, 5, 2 * 64 * 128>;
+    CHECK(Packed::kStageNumel == 64 * 128 && Packed::kBytes == 5 * 64 * 128 * 2);
+    CHECK(Strided::kStageNumel == 2 * 64 * 128 && Strided::kStageBytes == 32768);
+    CHECK(Strided::kBytes == (4 * 2 + 1) * 64 * 128 * 2);
+    __half* base = nullptr;
+    Strided ring(base);
+    CHECK(ring.stage_data(3) == base + 3 * 2 * 64 * 128);
+    CHECK(ring[2].data() == base + 2 * 2 * 64 * 128);
+    CHECK(Strided::next(4) == 0 && Strided::next(1) == 2);
+    // a tile with the transposing-read policy keeps it in the sub-tiles its iterator cuts
+    using SharedV = SharedTile<__half, tl::RowMajor<64, 128>, true, tl::LdsSwizzleTr<128, 2>>;
+    using Halves = STileIterator<SharedV, TileShape<32, 128>>;
+    Halves halves(base);
+    auto second = halves(1);
+    CHECK(second.line0() == 32 && second.elem0() == 0);
+    CHECK((std::is_same_v<typename decltype(second)::Swizzle, tl::LdsSwizzleTr<128, 2>>));
+    CHECK(second.offset(1, 0) == 33 * 128 + tl::LdsSwizzleTr<128, 2>::apply(33, 0));
+}
+
 static void test_shared_tile_views() {
     using Shared = SharedTile<__half, tl::RowMajor<64, 128>, true>;
     using SIter = STileIterator<Shared, TileShape<64, 32>>;
@@ -260,6 +316,9 @@ int main() {
     test_swizzle<256, 2>(true);
     test_swizzle<48, 2>(false);
     test_swizzle<80, 2>(false);
+    test_swizzle_tr<128>();
+    test_swizzle_tr<64>();
+    test_strided_ring();
     test_swizzle<16, 4>(true);
     test_swizzle<32, 4>(true);
     test_swizzle<64, 4>(true);

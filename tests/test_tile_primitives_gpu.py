@@ -46,8 +46,8 @@ CASES = _cases()
 def test_registry_is_populated():
     assert os.path.exists(LIB), "device test library missing: run __graft_entry__.build()"
     kinds = {c[1] for c in CASES}
-    assert kinds == {"g2s_roundtrip", "s2r_identity", "store_roundtrip", "g2r_roundtrip", "tile_gemm", "row_ops",
-                     "col_ops", "elementwise"}
+    assert kinds == {"g2s_roundtrip", "s2r_identity", "store_roundtrip", "g2r_roundtrip", "tile_gemm", "tile_b2b",
+                     "row_ops", "col_ops", "elementwise"}
 
 
 def _np_dtype(nbytes):
@@ -89,6 +89,19 @@ def test_tile_case(case, device, oracle):
         run(a, b, c, None)
         err = oracle.max_rel_err(c.cpu().numpy(), oracle.gemm(A, Bt))
         assert err <= 1e-3, f"max rel err {err}"
+    elif kind == "tile_b2b":
+        # D = f16(A B) V: B column-major (stored [N, K]) followed by V row-major [N, P] in one buffer
+        M, N, K, P = dims[:4]
+        A = oracle.fill_normal(M * K, 300 + idx, 0, 0.5).reshape(M, K)
+        Bt = oracle.fill_normal(N * K, 400 + idx, 0, 0.5).reshape(N, K)
+        V = oracle.fill_normal(N * P, 500 + idx, 0, 0.5).reshape(N, P)
+        a = torch.from_numpy(A).to(device)
+        b = torch.from_numpy(np.concatenate([Bt.reshape(-1), V.reshape(-1)])).to(device)
+        c = torch.full((M, P), float("nan"), dtype=torch.float32, device=device)
+        run(a, b, c, None)
+        ref = oracle.b2b_gemm(A[None], Bt[None], np.ascontiguousarray(V.T)[None])[0]
+        err = oracle.max_rel_err(c.cpu().numpy(), ref, eps=1.0)
+        assert err <= 1e-3, f"max err relative to rms {err}"
     elif kind in ("row_ops", "col_ops"):
         rows, cols, op, nbytes = dims[:4]
         dt = _np_dtype(nbytes)
