@@ -168,4 +168,134 @@ __global__ void __launch_bounds__(Traits::kThreads) KeFusedGemm(const InType* dA
     storer_d(rD_out, gD);
 }
 
+/// The LDS-resident back-to-back GEMM (kernels/b2b_gemm_fwd.hpp, what K = P = 128 runs on) written with tile-library
+/// types and functors only. Against KeFusedGemm above: every operand goes global -> LDS directly
+/// (GlobalToSharedDirectLoader), all of a block's loads in flight at once and handed over with
+/// wait_group_and_barrier<N>(); the products run on v_mfma_f32_16x16x32_f16 operand tiles (one ds_read_b128 per tile);
+/// the 8 wavefronts split the first product by n and the second by p, so the f16-rounded intermediate crosses
+/// wavefronts through a shared tile (RegToSharedStorer / SharedToRegLoader) instead of staying in one wavefront's
+/// registers - which is what lets 32 rows keep a whole CU busy. N is walked in blocks of 256 through the same shared
+/// tiles: B is refilled under the second product of the current block, C under the first product of the next.
+/// The sums are those of b2b_gemm_resident in the same order: bit-identical results.
+template <typename InType, typename OutType, const int kN_>
+struct ResidentFusedGemmTraits {
+    static constexpr int kN = kN_, kK = 128, kP = 128;
+    static constexpr int kTM = 32, kTN = 256;
+    static_assert(kN % kTN == 0);
+    using WarpLayout = tl::RowMajor<1, 8>;
+    static constexpr int kWaves = 8, kThreads = kWaves * kWaveSize;
+    using Shape = traits::MfmaTileShape<InType, traits::MfmaShape::k16x16x32>;
+
+    using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK>>;
+    using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kTN>>;       // 256 columns of B: 256 rows of the stored [N, K]
+    using GlobalC = GlobalTile<InType, tl::ColMajor<kTN, kP, kN>>;   // 256 rows of C: columns of the stored [P, N]
+    using GlobalD = GlobalTile<OutType, tl::RowMajor<kTM, kP>>;
+    using SharedA = SharedTile<InType, tl::RowMajor<kTM, kK>, true>;
+    using SharedB = SharedTile<InType, tl::ColMajor<kK, kTN>, true>;
+    using SharedC = SharedTile<InType, tl::ColMajor<kTN, kP>, true>;
+    using SharedS = SharedTile<InType, tl::RowMajor<kTM, kTN>, true>;  // the intermediate of one block
+    static constexpr int kShmBytes =
+        (SharedA::kNumel + SharedB::kNumel + SharedC::kNumel + SharedS::kNumel) * int(sizeof(InType));  // 152 KiB
+    static_assert(kShmBytes <= kMaxLdsBytes);
+
+    using LoadA = GlobalToSharedDirectLoader<SharedA, WarpLayout>;
+    using LoadB = GlobalToSharedDirectLoader<SharedB, WarpLayout>;
+    using LoadC = GlobalToSharedDirectLoader<SharedC, WarpLayout>;
+    static constexpr int kLoadsC = LoadC::kLoadsPerWave;  // the youngest loads of a block: still in flight at its first hand-over
+
+    // first product: a wavefront owns 32 values of n
+    using RegA = RegTile<typename Shape::TileA, tl::RowMajor<kTM / 16, kK / 32>>;
+    using RegB = RegTile<typename Shape::TileB, tl::ColMajor<kK / 32, kTN / kWaves / 16>>;
+    using RegAcc = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kTM / 16, kTN / kWaves / 16>>;
+    using RegAccCast = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kTM / 16, kTN / kWaves / 16>>;
+    using ReadA = SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
+    using ReadB = SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
+    using ConvertAcc = compute::RegTileConvert<RegAcc, RegAccCast>;
+    using StoreS = RegToSharedStorer<RegAccCast, WarpLayout>;
+    // second product: a wavefront owns 16 values of p
+    using RegS = RegTile<typename Shape::TileA, tl::RowMajor<kTM / 16, kTN / 32>>;
+    using RegC = RegTile<typename Shape::TileB, tl::ColMajor<kTN / 32, kP / kWaves / 16>>;
+    using RegD = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kTM / 16, kP / kWaves / 16>>;
+    using RegDCast = RegTile<BaseTileRowMajor<OutType>, tl::RowMajor<kTM / 16, kP / kWaves / 16>>;
+    using ReadS = SharedToRegLoader<RegS, WarpLayout, WarpReuse::kRowReuseCont>;
+    using ReadC = SharedToRegLoader<RegC, WarpLayout, WarpReuse::kColReuseCont>;
+    using ConvertD = compute::RegTileConvert<RegD, RegDCast>;
+    using StoreD = RegToGlobalStorer<GlobalD, RegDCast, WarpLayout>;
+};
+
+/// grid = (M / 32, batch), block = 512, dynamic LDS = Traits::kShmBytes.
+template <typename InType, typename OutType, typename Traits>
+__global__ void __launch_bounds__(Traits::kThreads)
+    b2b_gemm_tile_resident(const InType* dA, const InType* dB, const InType* dC, OutType* dD, int kM) {
+    constexpr int kN = Traits::kN, kK = Traits::kK, kP = Traits::kP, kTM = Traits::kTM, kTN = Traits::kTN;
+    constexpr int kBlocks = kN / kTN;
+    const size_t batch = blockIdx.y;
+    const InType* A = dA + (batch * kM + size_t(blockIdx.x) * kTM) * kK;
+    const InType* B = dB + batch * size_t(kN) * kK;
+    const InType* C = dC + batch * size_t(kP) * kN;
+    OutType* D = dD + (batch * kM + size_t(blockIdx.x) * kTM) * kP;
+
+    extern __shared__ __align__(1024) unsigned char shared_buf[];
+    auto* shm = reinterpret_cast<InType*>(shared_buf);
+    typename Traits::SharedA sA(shm);
+    typename Traits::SharedB sB(shm + Traits::SharedA::kNumel);
+    typename Traits::SharedC sC(shm + Traits::SharedA::kNumel + Traits::SharedB::kNumel);
+    typename Traits::SharedS sS(shm + Traits::SharedA::kNumel + Traits::SharedB::kNumel + Traits::SharedC::kNumel);
+
+    typename Traits::LoadA load_a;
+    typename Traits::LoadB load_b;
+    typename Traits::LoadC load_c;
+    auto block_b = [&](int nb) { return typename Traits::GlobalB(B + size_t(nb) * kTN * kK); };
+    auto block_c = [&](int nb) { return typename Traits::GlobalC(C + size_t(nb) * kTN); };
+
+    // everything of the first block in flight at once: one memory round trip when N is a single block
+    load_a(typename Traits::GlobalA(A), sA);
+    load_b(block_b(0), sB);
+    load_c(block_c(0), sC);
+
+    typename Traits::ReadA read_a;
+    typename Traits::ReadB read_b;
+    typename Traits::ReadS read_s;
+    typename Traits::ReadC read_c;
+    typename Traits::ConvertAcc cast_acc;
+    typename Traits::StoreS store_s;
+
+    typename Traits::RegA rA;
+    typename Traits::RegB rB;
+    typename Traits::RegS rS;
+    typename Traits::RegC rC;
+    typename Traits::RegAcc acc;
+    typename Traits::RegAccCast acc_half;
+    typename Traits::RegD rD;
+
+    for (int nb = 0; nb < kBlocks; ++nb) {
+        // A and this block of B have landed (the younger loads, of C, may still be on their way), for everyone; and
+        // everyone is done with the previous block's C and intermediate
+        wait_group_and_barrier<Traits::kLoadsC>();
+        if (nb == 0) read_a(sA, rA);
+        read_b(sB, rB);
+        acc.clear();
+        compute::gemm(rA, rB, acc);
+        cast_acc(acc, acc_half);  // the intermediate is rounded to f16: part of the operation's specification
+        store_s(acc_half, sS);
+        wait_group_and_barrier<0>();  // C has landed, the intermediate is written, B is free; for everyone
+        if (nb + 1 < kBlocks) load_b(block_b(nb + 1), sB);  // under the second product
+        read_s(sS, rS);
+        read_c(sC, rC);
+        compute::gemm(rS, rC, rD);
+        if (nb + 1 < kBlocks) {
+            // everyone's reads of C and of the intermediate have returned: C is refilled under the next first product
+            __syncthreads();
+            load_c(block_c(nb + 1), sC);
+        }
+    }
+
+    typename Traits::RegDCast rD_out;
+    typename Traits::ConvertD cast_d;
+    cast_d(rD, rD_out);
+    typename Traits::GlobalD gD(D);
+    typename Traits::StoreD store_d;
+    store_d(rD_out, gD);
+}
+
 }  // namespace tiledcuda::kernels

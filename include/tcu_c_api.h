@@ -67,6 +67,9 @@ typedef enum {
     TCU_B2B_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, the reference kernel's structure */
     TCU_B2B_RESIDENT = 2,     /* A tile, 256-column blocks of B and C and the intermediate resident in LDS (K = P = 128,
                                  N % 256 == 0, M % 32 == 0); one round of loads per block */
+    TCU_B2B_TILE_RESIDENT = 4, /* the RESIDENT kernel composed from tile-library functors only (direct-to-LDS loaders,
+                                 16x16x32 operand tiles, the intermediate through a shared tile); compile-time N in
+                                 {256, 1024, 2048}, K = P = 128, M % 32 == 0; results identical to RESIDENT bit for bit */
     TCU_B2B_ROWS = 3          /* for many rows (AUTO from M x batch = 32768): N = 256, K = P = 128, M % 64 == 0; a
                                  workgroup keeps B and C in LDS and walks over blocks of 256 rows, every wavefront owning
                                  64 rows (A fragments from global memory, the intermediate stays in registers); agrees

@@ -446,6 +446,31 @@ def test_b2b_gemm_reference_shape_list(tcu, oracle, device, M, N, K, P, batch, a
         assert oracle.max_rel_err(got[b], oracle.b2b_gemm(A[b], Bt[b], Ct[b]), eps=1.0) <= REL_TOL
 
 
+@pytest.mark.parametrize("M,N,batch,out_dtype", [(32, 256, 1, "f32"), (96, 256, 3, "f16"), (8192, 256, 1, "f16"),
+                                                 (64, 1024, 2, "f16"), (2048, 2048, 1, "f32")])
+def test_b2b_gemm_tile_resident_is_resident(tcu, oracle, device, M, N, batch, out_dtype):
+    """The LDS-resident kernel composed from tile-library functors (tile_resident) sums in the order of the
+    hand-indexed one: bit-identical outputs, for one block of N and for several (B and C refilled under the products),
+    and within tolerance of the oracle."""
+    import torch
+
+    print(f"b2b tile_resident M{M} N{N} b{batch} {out_dtype}", flush=True)
+    K, P = 128, 128
+    A = oracle.fill_normal(batch * M * K, 171, 0, 0.1).reshape(batch, M, K)
+    Bt = oracle.fill_normal(batch * N * K, 172, 0, 0.1).reshape(batch, N, K)
+    Ct = oracle.fill_normal(batch * P * N, 173, 0, 0.1).reshape(batch, P, N)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    dA, dB, dC = dev(A, device), dev(Bt, device), dev(Ct, device)
+    want = tcu.b2b_gemm(dA, dB, dC, out_dtype=dt, algo="resident")
+    got = torch.full_like(want, float("nan"))
+    tcu.b2b_gemm(dA, dB, dC, out=got, out_dtype=dt, algo="tile_resident")
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    rows = slice(0, min(M, 64))
+    ref = oracle.b2b_gemm(np.ascontiguousarray(A[:, rows]), Bt, Ct)
+    assert oracle.max_rel_err(host(got)[:, rows], ref, eps=1.0) <= REL_TOL
+
+
 @pytest.mark.parametrize("algo", ["tile_library", "resident"])
 @pytest.mark.parametrize("M,batch,out_dtype", [(32, 1, "f32"), (96, 3, "f16"), (8192, 1, "f16"), (16384, 2, "f32")])
 def test_b2b_gemm_both_kernels_at_256x128x128(tcu, oracle, device, algo, M, batch, out_dtype):

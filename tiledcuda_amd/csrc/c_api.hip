@@ -434,11 +434,29 @@ int launch_b2b(const __half* A, const __half* B, const __half* C, OutType* D, in
     return launch(kernel, dim3(M / kTM, 1, batch), dim3(Traits::kThreads), Traits::kShmBytes, stream, A, B, C, D, M);
 }
 
+template <typename OutType, int kN>
+int launch_b2b_tile_resident(const __half* A, const __half* B, const __half* C, OutType* D, int M, int batch, hipStream_t stream) {
+    using Traits = ResidentFusedGemmTraits<__half, OutType, kN>;
+    return launch(&b2b_gemm_tile_resident<__half, OutType, Traits>, dim3(M / Traits::kTM, batch), dim3(Traits::kThreads),
+                  Traits::kShmBytes, stream, A, B, C, D, M);
+}
+
 template <typename OutType>
 int b2b_dispatch(const __half* A, const __half* B, const __half* C, OutType* D, int M, int N, int K, int P, int batch,
                  int algo, hipStream_t stream) {
-    if (algo != TCU_B2B_AUTO && algo != TCU_B2B_TILE_LIBRARY && algo != TCU_B2B_RESIDENT && algo != TCU_B2B_ROWS)
+    if (algo != TCU_B2B_AUTO && algo != TCU_B2B_TILE_LIBRARY && algo != TCU_B2B_RESIDENT && algo != TCU_B2B_ROWS &&
+        algo != TCU_B2B_TILE_RESIDENT)
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_b2b_gemm_f16: unknown algo");
+    if (algo == TCU_B2B_TILE_RESIDENT) {
+        // the LDS-resident kernel composed from tile-library functors: compile-time N, like every tile-API kernel
+        if (K == 128 && P == 128 && M % 32 == 0) {
+            if (N == 256) return launch_b2b_tile_resident<OutType, 256>(A, B, C, D, M, batch, stream);
+            if (N == 1024) return launch_b2b_tile_resident<OutType, 1024>(A, B, C, D, M, batch, stream);
+            if (N == 2048) return launch_b2b_tile_resident<OutType, 2048>(A, B, C, D, M, batch, stream);
+        }
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the tile-API LDS-resident b2b kernel is instantiated for K = P = 128, N in "
+                                               "{256, 1024, 2048}, M a multiple of 32");
+    }
     // many rows: workgroups that keep both weight blocks for their whole life and walk over blocks of 256 rows
     if (algo == TCU_B2B_ROWS || (algo == TCU_B2B_AUTO && (long)M * batch >= 32768)) {
         if (N == 256 && K == 128 && P == 128 && M % 64 == 0) {
