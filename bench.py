@@ -137,6 +137,34 @@ def probe_mfma(torch, operands, shape, waves=8, iters=20000):
             "wavefronts_per_cu": waves}
 
 
+def probe_mfma_reuse(torch, operands, shape, iters=4000):
+    """Sustained MFMA rate of the one-wavefront-per-SIMD register pattern (4 wavefronts per CU, a grid of accumulator
+    tiles filling the AGPRs, every operand fragment feeding 8 or 4 instructions) on `operands`: TFLOP/s and core MHz."""
+    import ctypes
+
+    lib = ctypes.CDLL(os.path.join(ROOT, "bench_support", "_build", "libtcu_probe.so"))
+    lib.tcu_probe_mfma_f16_reuse.restype = ctypes.c_int
+    lib.tcu_probe_mfma_f16_reuse.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_void_p]
+    wgs = 256
+    assert operands.numel() >= wgs * 256 * 128
+    clocks = torch.zeros(2 * wgs, dtype=torch.int64, device=operands.device)
+    sink = torch.zeros(1, dtype=torch.float32, device=operands.device)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = lib.tcu_probe_mfma_f16_reuse(operands.data_ptr(), clocks.data_ptr(), sink.data_ptr(), shape, wgs, iters, stream)
+        if rc != 0:
+            raise RuntimeError(f"tcu_probe_mfma_f16_reuse failed with hipError {rc}")
+
+    ms = time_kernel(launch, 3, 1)
+    ticks = clocks.cpu().numpy().reshape(wgs, 2).astype("float64")
+    flops = wgs * 4 * iters * float(1 << 20 if shape == 1 else 1 << 19)
+    return {"tflops": flops / (ms * 1e-3) / 1e12, "core_clock_mhz": 100.0 * ticks[:, 0].sum() / ticks[:, 1].sum(),
+            "instruction": "v_mfma_f32_16x16x32_f16" if shape == 1 else "v_mfma_f32_32x32x16_f16",
+            "wavefronts_per_cu": 4, "pattern": "8 x 8 accumulator tiles, each operand fragment feeds 8 instructions"
+            if shape == 1 else "4 x 4 accumulator tiles, each operand fragment feeds 4 instructions"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -147,6 +175,11 @@ def main():
     ap.add_argument("--no-mfma-probe", action="store_true", help="skip the sustained-MFMA-rate measurement")
     ap.add_argument("--no-vendor", action="store_true",
                     help="skip the vendor-library comparison (hipBLASLt through torch.matmul, torch's fused attention)")
+    ap.add_argument("--extra-kernels", action="store_true",
+                    help="also run the kernels AUTO dispatches off the benchmark shapes (K-splitting GEMM at 2048^3, the "
+                         "many-rows back-to-back GEMM at M = 65536, the split-K pair at 1024 x 1024 x 16384) and the "
+                         "tile-API compositions of the tuned kernels, 60 launches each: the command the rocprofv3 "
+                         "summaries of those kernels under profiles/ are made with")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 128 MiB (read 128 MiB, write 128 MiB) a few times, so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command has a kernel of known traffic to "
@@ -238,7 +271,7 @@ def main():
         v = oracle.fill_normal(cnt, 3238).reshape(B * H, S, D)
         dq, dk, dv = (to_dev(t.reshape(B, H, S, D)) for t in (q, k, v))
         do = torch.empty(B, H, S, D, dtype=torch.float16, device=dev)
-        flops = 4.0 * B * H * S * S * D
+        flops = flops_attn = 4.0 * B * H * S * S * D
         # the first launches after the light configurations above run at clocks that have not come up yet (about 150-160 us
         # each); that figure is kept as "first_launches_us", the configuration's own figure is taken after 200 untimed
         # conditioning launches of the same kernel (as for the headline GEMM)
@@ -367,6 +400,50 @@ def main():
                         "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "round_trip_exact": ok})
         del upd, data
 
+    # ---------------------------------------------------------------- kernels AUTO dispatches off the benchmark shapes,
+    # and the tile-API compositions beside their hand-indexed counterparts (--extra-kernels)
+    if args.extra_kernels:
+        def rand16(*shape):
+            return (torch.rand(*shape, device=dev) * 2 - 1).half()
+
+        a_, b_ = rand16(2048, 2048), rand16(2048, 2048)
+        c_ = torch.empty(2048, 2048, dtype=torch.float16, device=dev)
+        ms = time_kernel(lambda: tcu.gemm(a_, b_, out=c_), 40, 20)
+        configs.append({"name": "gemm_2048_cubed_auto", "kernel": "gemm_w128k<__half>", "ms": ms,
+                        "tflops": 2.0 * 2048 ** 3 / (ms * 1e-3) / 1e12})
+        a_, b_ = rand16(1024, 16384), rand16(1024, 16384)
+        c_ = torch.empty(1024, 1024, dtype=torch.float16, device=dev)
+        ws_ = torch.empty(max(16, tcu.gemm_workspace_bytes(1024, 1024, 16384)), dtype=torch.uint8, device=dev)
+        ms = time_kernel(lambda: tcu.gemm(a_, b_, out=c_, workspace=ws_), 40, 20)
+        configs.append({"name": "gemm_1024x1024x16384_split_k", "kernel": "gemm_w128<float> over K-ranges + splitk_reduce<__half>",
+                        "ms": ms, "workspace_bytes": int(ws_.numel()), "tflops": 2.0 * 1024 * 1024 * 16384 / (ms * 1e-3) / 1e12})
+        Mr = 65536
+        a_ = (torch.randn(Mr, 128, device=dev) * 0.1).half()
+        b_ = (torch.randn(256, 128, device=dev) * 0.1).half()
+        c_ = (torch.randn(128, 256, device=dev) * 0.1).half()
+        d_ = torch.empty(1, Mr, 128, dtype=torch.float16, device=dev)
+        ms = time_kernel(lambda: tcu.b2b_gemm(a_, b_, c_, out=d_), 40, 20)
+        nbytes = 2.0 * (2 * Mr * 128 + 2 * 256 * 128)
+        configs.append({"name": "b2b_65536x256x128x128_auto", "kernel": "b2b_gemm_rows<__half>", "ms": ms,
+                        "gbs": nbytes / (ms * 1e-3) / 1e9, "tflops": 4.0 * Mr * 256 * 128 / (ms * 1e-3) / 1e12})
+        if want("b2b"):
+            ms_t = time_graph(lambda: tcu.b2b_gemm(d3a, d3b, d3c, out=d3d, algo="tile_resident"), 10 * args.steps, args.warmup)
+            ms_r = time_graph(lambda: tcu.b2b_gemm(d3a, d3b, d3c, out=d3d, algo="resident"), 10 * args.steps, args.warmup)
+            configs.append({"name": "b2b_8192x256x128x128_tile_api_composition", "kernel": "b2b_gemm_tile_resident",
+                            "us_in_hip_graph": None if ms_t is None else ms_t * 1e3,
+                            "hand_indexed_us_in_hip_graph": None if ms_r is None else ms_r * 1e3})
+        if want("attn"):
+            ms_t = time_kernel(lambda: tcu.flash_attention(dq, dk, dv, out=do, algo="tile_wave64"), 40, 100)
+            ms_r = time_kernel(lambda: tcu.flash_attention(dq, dk, dv, out=do, algo="wave64"), 40, 100)
+            configs.append({"name": "flash_attn_fwd_b4_h16_s2048_d128_tile_api_composition", "kernel": "flash_attention_tile_w64",
+                            "ms": ms_t, "tflops": flops_attn / (ms_t * 1e-3) / 1e12, "hand_indexed_ms": ms_r})
+        dCt = torch.empty_like(dC)
+        ms_t = time_kernel(lambda: tcu.gemm(dA, dB, out=dCt, algo="tile_wave128"), 40, 100)
+        ms_r = time_kernel(lambda: tcu.gemm(dA, dB, out=dCt, algo="wave128"), 40, 100)
+        configs.append({"name": "gemm_4096_tile_api_composition", "kernel": "gemm_tile_w128", "ms": ms_t,
+                        "tflops": gemm_flops / (ms_t * 1e-3) / 1e12, "hand_indexed_ms": ms_r})
+        del a_, b_, c_, d_, ws_, dCt
+
     # sustained MFMA rate on the same operand distribution (U[-1,1] fp16), the kernel's MFMA shape, 8 wavefronts per CU
     sustained = None
     if not args.no_mfma_probe:
@@ -375,6 +452,12 @@ def main():
         sustained["operands"] = "the GEMM's A matrix (U[-1,1] fp16)"
         sustained["tflops_on_zero_operands"] = zeros["tflops"]
         sustained["core_clock_mhz_on_zero_operands"] = zeros["core_clock_mhz"]
+        # both instruction shapes, as independent instructions at 8 wavefronts per CU and in the register pattern of the
+        # one-wavefront-per-SIMD kernels (4 wavefronts per CU, operand reuse, all AGPRs as accumulators), same operands:
+        # what "the ceiling" is depends on the pattern, so the headline's fraction is taken against its own pattern
+        sustained["by_pattern"] = [probe_mfma(torch, dA, shape=0), probe_mfma_reuse(torch, dA, shape=1),
+                                   probe_mfma_reuse(torch, dA, shape=0)]
+        sustained["kernel_pattern_tflops"] = sustained["by_pattern"][1]["tflops"]
 
     # ---------------------------------------------------------------- C2 timed (after the other configurations: the
     # headline measurement then starts from a GPU that has been busy for a while, like a step of a long job, not
@@ -570,7 +653,9 @@ def main():
                      "kernel": GEMM_4096_KERNEL + " (256x256x64 tile, 2x2 wavefronts, one per SIMD)",
                      "flops_per_launch": gemm_flops, "avg_launch_us": gemm_ms * 1e3, "settled": settled,
                      "sustained_mfma": sustained,
-                     "frac_of_sustained_mfma": (gemm_tflops / sustained["tflops"]) if sustained else None},
+                     "frac_of_sustained_mfma": (gemm_tflops / sustained["tflops"]) if sustained else None,
+                     "frac_of_sustained_mfma_kernel_pattern":
+                         (gemm_tflops / sustained["kernel_pattern_tflops"]) if sustained else None},
         "cpu_baseline": cpu,
         "vendor_library_same_run": vendor,
         "max_rel_err": gemm_err,

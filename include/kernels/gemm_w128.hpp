@@ -102,16 +102,21 @@ __global__ void __launch_bounds__(256) splitk_reduce(const float* __restrict__ p
 /// the operand is a column block of a wider matrix); ldc: elements between consecutive rows of C (N for a dense C;
 /// larger when C is the leading block of a wider matrix). With splits > 1 workgroup row z multiplies the
 /// K-range [z K, (z + 1) K) and writes plane z of C ([splits, M, N]; partial sums for splitk_reduce).
+/// zero_words / zero_count: device words that the first workgroup sets to zero on the side (null / 0: none) - the
+/// synchronisation words of a kernel that follows this one on the stream, cleared without a launch of their own.
 template <typename OutType>
 __global__ void __launch_bounds__(GemmW128Traits::kThreads)
     gemm_w128(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
-              int lda, int ldb, int ldc) {
+              int lda, int ldb, int ldc, unsigned int* __restrict__ zero_words, int zero_count) {
     using T = GemmW128Traits;
     extern __shared__ __align__(1024) unsigned char lds[];
 
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(wave_id());
     const int wave_m = wave >> 1, wave_n = wave & 1;
+    if (zero_count > 0 && blockIdx.x == 0 && blockIdx.y == 0) {
+        for (int i = threadIdx.x; i < zero_count; i += T::kThreads) zero_words[i] = 0u;
+    }
     int tile_m, tile_n;
     detail::xcd_tile_coords(blockIdx.x, M / T::kBM, N / T::kBN, tile_m, tile_n);
     const int m0 = tile_m * T::kBM, n0 = tile_n * T::kBN;

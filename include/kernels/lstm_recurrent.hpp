@@ -32,6 +32,8 @@
 // B <= 256 (8 XCDs), grid == 256 workgroups of 256 threads.
 #pragma once
 
+#include <type_traits>
+
 #include "config.hpp"
 #include "hip_utils.hpp"
 #include "kernels/gemm_pipelined.hpp"  // detail::lds_barrier
@@ -77,12 +79,12 @@ DEVICE void mfma32_weights_in_agprs_zero(f32x16& acc, const f16x8& w, const f16x
 }
 }  // namespace detail
 
-/// pre: [T, B, 4H] f32 (gate-major columns, as W's rows); W: [4H, ldw] f16, the recurrent block starts at column
+/// pre: [T, B, 4H] f32 or f16 (PreType; gate-major columns, as W's rows); W: [4H, ldw] f16, the recurrent block starts at column
 /// w_col0; bias [4H] f16; h0 [B, H] f16 or null (zeros); c0 [B, H] f32 or null; h_all [T, B, H] f16; c_out [B, H] f32.
 /// peers: workgroups per XCD to wait for (kCusPerXcd; anything else only to exercise the bounded wait).
-template <typename Traits>
+template <typename Traits, typename PreType = float>
 __global__ void __launch_bounds__(Traits::kThreads)
-    lstm_recurrent_xcd(const float* __restrict__ pre, const __half* __restrict__ W, int ldw, int w_col0,
+    lstm_recurrent_xcd(const PreType* __restrict__ pre, const __half* __restrict__ W, int ldw, int w_col0,
                        const __half* __restrict__ bias, const __half* __restrict__ h0, const float* __restrict__ c0,
                        __half* h_all, float* __restrict__ c_out, int T, int B, unsigned int* sync,
                        unsigned long long spin_ticks, unsigned int peers) {
@@ -161,13 +163,23 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int hid = unit0 + 4 * fhalf;
     f32x4 c_state = {0.f, 0.f, 0.f, 0.f};
     if (c0) c_state = *reinterpret_cast<const f32x4*>(c0 + size_t(b) * kH + hid);
+    // four consecutive pre-activations of one gate: one 16-byte or 8-byte load; widened to f32 only where the values
+    // are used (a conversion next to the load would make the compiler wait for the load, and with it for every older
+    // load of the wavefront, right there)
+    using PreRaw = std::conditional_t<sizeof(PreType) == 4, f32x4, f16x4>;
+    auto load_pre = [&](size_t row, int g) -> PreRaw {
+        return *reinterpret_cast<const PreRaw*>(pre + row * (4 * kH) + g * kH + hid);
+    };
+    auto widen_pre = [](const PreRaw& v) -> f32x4 {
+        return f32x4{static_cast<float>(v[0]), static_cast<float>(v[1]), static_cast<float>(v[2]), static_cast<float>(v[3])};
+    };
     f32x4 bias_v[4], pre_v[4];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         const f16x4 bv = *reinterpret_cast<const f16x4*>(bias + g * kH + hid);
 #pragma unroll
         for (int e = 0; e < 4; ++e) bias_v[g][e] = static_cast<float>(bv[e]);
-        pre_v[g] = *reinterpret_cast<const f32x4*>(pre + size_t(b) * (4 * kH) + g * kH + hid);
+        pre_v[g] = widen_pre(load_pre(size_t(b), g));
     }
 
     // ---- global -> LDS: load instruction j (0..15) of wavefront w brings rows 8 w .. 8 w + 7, logical 16-byte chunks
@@ -248,11 +260,10 @@ __global__ void __launch_bounds__(Traits::kThreads)
             issue_h(h_prev + size_t(row0) * kH);
         }
         // pre-activations of the next step, a step ahead (independent of h)
-        f32x4 pre_next[4];
+        PreRaw pre_next[4];
         if (t + 1 < T) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g)
-                pre_next[g] = *reinterpret_cast<const f32x4*>(pre + (size_t(t + 1) * B + b) * (4 * kH) + g * kH + hid);
+            for (int g = 0; g < 4; ++g) pre_next[g] = load_pre(size_t(t + 1) * B + b, g);
         }
         if (h_prev) {
             // Piece p (this wavefront's loads 4 p .. 4 p + 3) has landed when at most the loads issued after it are
@@ -292,7 +303,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         *reinterpret_cast<f16x4*>(h_all + (size_t(t) * B + b) * kH + hid) = h_new;
         if (t + 1 < T) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) pre_v[g] = pre_next[g];
+            for (int g = 0; g < 4; ++g) pre_v[g] = widen_pre(pre_next[g]);
             // arrival: every wavefront's stores of h_t have been acknowledged by the L2, then one lane counts
             detail::lds_barrier<0>();
             if (threadIdx.x == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -302,7 +313,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
 }
 
 /// Zeroes the synchronisation words before a launch of lstm_recurrent_xcd (a kernel, not a memset: it may be recorded
-/// into a HIP graph). One workgroup of kSyncWords threads.
+/// into a HIP graph). One workgroup of kSyncWords threads. (The layer entry point lets the projection GEMM that precedes
+/// the recurrence do this instead; the kernel is for callers that launch the recurrence on its own.)
 __global__ void lstm_recurrent_clear_sync(unsigned int* sync) { sync[threadIdx.x] = 0u; }
 
 }  // namespace tiledcuda::kernels

@@ -218,9 +218,11 @@ int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* 
  * The LSTM layer with the whole time loop in ONE launch, for the large-hidden-size case where a step is bound by
  * streaming the recurrent weights and by the cost of a dependent launch (H == 1024, I % 64 == 0, B % 32 == 0, B <= 256,
  * T * B % 256 == 0; a device of 256 CUs in 8 XCDs). As in tcu_lstm_f16_ws the input half of the gates of all steps is
- * one GEMM into the workspace; the recurrence then runs weight-stationary: every XCD keeps a copy of W[:, I:] in the
- * registers of its 32 CUs and owns 32 batch rows, and h_t is exchanged between those CUs through the XCD's L2 only.
- * Same arguments and results (up to the order of the f32 summation) as tcu_lstm_f16_ws. `workspace`: device memory of
+ * one GEMM into the workspace - here with its f32 sums rounded once to f16 (half the bytes to write and read back; the
+ * gates' pre-activations then carry a relative error of 2^-11 on that half, far inside the layer's 1e-2 tolerance) -;
+ * the recurrence then runs weight-stationary: every XCD keeps a copy of W[:, I:] in the registers of its 32 CUs and owns
+ * 32 batch rows, and h_t is exchanged between those CUs through the XCD's L2 only.
+ * Same arguments as tcu_lstm_f16_ws; results equal to its up to that rounding and the order of the f32 summation. `workspace`: device memory of
  * at least tcu_lstm_persistent_workspace_bytes(T, B, I, H) bytes (0 = shape not supported), 128-byte aligned (the step
  * counters sit in cache lines of their own), owned by the caller; its first 4 KiB are synchronisation words, cleared by
  * the call.

@@ -225,7 +225,7 @@ int gemm_pipelined_dispatch(const __half* A, const __half* B, OutType* C, int M,
 
 template <typename OutType>
 int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream,
-                       int lda = 0, int ldb = 0, int ldc = 0) {
+                       int lda = 0, int ldb = 0, int ldc = 0, unsigned int* zero_words = nullptr, int zero_count = 0) {
     using T = GemmW128Traits;
     if (lda == 0) lda = K;
     if (ldb == 0) ldb = K;
@@ -235,7 +235,7 @@ int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int 
     if ((long)std::max(lda, ldb) * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
     return launch(&gemm_w128<OutType>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
-                  C, M, N, K, lda, ldb, ldc);
+                  C, M, N, K, lda, ldb, ldc, zero_words, zero_count);
 }
 
 template <typename OutType>
@@ -347,7 +347,7 @@ int gemm_splitk(const __half* A, const __half* B, OutType* C, int M, int N, int 
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
     const int tiles = (M / T::kBM) * (N / T::kBN);
     int rc = launch(&gemm_w128<float>, dim3(tiles, splits), dim3(T::kThreads), T::kLdsBytes, stream, A, B, partial, M, N,
-                    K / splits, K, K, N);
+                    K / splits, K, K, N, static_cast<unsigned int*>(nullptr), 0);
     if (rc != TCU_OK) return rc;
     const size_t n = size_t(M) * N;
     return launch(&splitk_reduce<OutType>, dim3(unsigned((n / 4 + 255) / 256)), dim3(256), 0, stream,
@@ -876,7 +876,8 @@ unsigned long long tcu_lstm_persistent_workspace_bytes(int T, int B, int I, int 
     if (T <= 0 || B <= 0 || I <= 0 || H != Traits::kH) return 0;
     if (B % Traits::kRows != 0 || B > Traits::kRows * Traits::kXcds || I % 64 != 0) return 0;
     if ((long)T * B % 256 != 0 || (long)T * B > INT_MAX) return 0;
-    return kPersistentSyncBytes + (unsigned long long)T * B * 4 * H * sizeof(float);
+    // the pre-activations of all steps in f16: [T, B, 4H]
+    return kPersistentSyncBytes + (unsigned long long)T * B * 4 * H * sizeof(__half);
 }
 
 int tcu_lstm_f16_persistent(const void* x, const void* W, const void* bias, const void* h0, const void* c0, void* h_all,
@@ -908,14 +909,15 @@ int tcu_lstm_f16_persistent(const void* x, const void* W, const void* bias, cons
     if (const char* e = std::getenv("TCU_LSTM_PERSISTENT_PEERS")) peers = unsigned(std::strtoul(e, nullptr, 10));
     auto s = static_cast<hipStream_t>(stream);
     auto sync = static_cast<unsigned int*>(workspace);
-    auto pre = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + kPersistentSyncBytes);
+    auto pre = reinterpret_cast<__half*>(static_cast<unsigned char*>(workspace) + kPersistentSyncBytes);
     auto xp = static_cast<const __half*>(x), wp = static_cast<const __half*>(W);
-    int rc = launch(&lstm_recurrent_clear_sync, dim3(1), dim3(Traits::kSyncWords), 0, s, sync);
+    // The projection GEMM writes the pre-activations as f16 (f32 sums rounded once: half the bytes written here and read
+    // by the recurrence, where the f32 form of tcu_lstm_f16_ws is bound by the volume of that write) and clears the
+    // synchronisation words on the side (its first workgroup): no launch of its own.
+    int rc = gemm_w128_dispatch<__half>(xp, wp, pre, T * B, 4 * H, I, s, I, I + H, 0, sync, Traits::kSyncWords);
     if (rc != TCU_OK) return rc;
-    rc = gemm_w128_dispatch<float>(xp, wp, pre, T * B, 4 * H, I, s, I, I + H);
-    if (rc != TCU_OK) return rc;
-    return launch(&lstm_recurrent_xcd<Traits>, dim3(Traits::kGrid), dim3(Traits::kThreads), Traits::kLdsBytes, s,
-                  static_cast<const float*>(pre), wp, I + H, I, static_cast<const __half*>(bias),
+    return launch(&lstm_recurrent_xcd<Traits, __half>, dim3(Traits::kGrid), dim3(Traits::kThreads), Traits::kLdsBytes, s,
+                  static_cast<const __half*>(pre), wp, I + H, I, static_cast<const __half*>(bias),
                   static_cast<const __half*>(h0), static_cast<const float*>(c0), static_cast<__half*>(h_all),
                   static_cast<float*>(c_out), T, B, sync, spin_us * 100ull, peers);
 }
