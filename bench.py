@@ -499,6 +499,23 @@ def main():
                "avg_launch_us": settled_us,
                "achieved": gemm_flops / settled_us / 1e6, "frac": gemm_flops / settled_us / 1e6 / MFMA_F16_PEAK_TFLOPS}
 
+    # The same kernel, the same launch, on all-zero operands (no bit of the matrix pipe's inputs toggles): the core clock
+    # then stays at its maximum, and the time shows what the kernel's instruction stream sustains when the power
+    # management does not hold the clock down. Beside the headline, never part of it.
+    zero_operands = None
+    if not args.no_mfma_probe:
+        dZ = torch.zeros(n, n, dtype=torch.float16, device=dev)
+        dCz = torch.empty_like(dC)
+        for _ in range(200):
+            tcu.gemm(dZ, dZ, out=dCz)
+        z_us = time_kernel(lambda: tcu.gemm(dZ, dZ, out=dCz), 100, 50) * 1e3
+        zero_operands = {"avg_launch_us": z_us, "achieved": gemm_flops / z_us / 1e6,
+                         "frac": gemm_flops / z_us / 1e6 / MFMA_F16_PEAK_TFLOPS,
+                         "note": "gemm_w128 at 4096^3 on all-zero A and B: same instructions, no operand toggling, full clock"}
+        del dZ, dCz
+        for _ in range(150):  # back to the workload's own power state before the vendor comparison
+            gemm_step()
+
     # the vendor library on the same operands, in the same process and power state (a comparison beside the figure above,
     # never part of it): hipBLASLt through torch.matmul, and this library again directly after it, 150 untimed + 100
     # timed launches each, twice; torch's fused attention on the C4 operands when that configuration ran
@@ -652,7 +669,7 @@ def main():
                      "traffic": traffic_from_profile(GEMM_4096_PROFILE, GEMM_4096_KERNEL),
                      "kernel": GEMM_4096_KERNEL + " (256x256x64 tile, 2x2 wavefronts, one per SIMD)",
                      "flops_per_launch": gemm_flops, "avg_launch_us": gemm_ms * 1e3, "settled": settled,
-                     "sustained_mfma": sustained,
+                     "sustained_mfma": sustained, "same_kernel_on_zero_operands": zero_operands,
                      "frac_of_sustained_mfma": (gemm_tflops / sustained["tflops"]) if sustained else None,
                      "frac_of_sustained_mfma_kernel_pattern":
                          (gemm_tflops / sustained["kernel_pattern_tflops"]) if sustained else None},

@@ -177,13 +177,18 @@ __global__ void __launch_bounds__(Traits::kThreads) KeFusedGemm(const InType* dA
 /// registers - which is what lets 32 rows keep a whole CU busy. N is walked in blocks of 256 through the same shared
 /// tiles: B is refilled under the second product of the current block, C under the first product of the next.
 /// The sums are those of b2b_gemm_resident in the same order: bit-identical results.
-template <typename InType, typename OutType, const int kN_>
+/// kK_, kP_: the inner sizes (whole, resident); kTN_: columns of B / rows of C per block; kWaves_: wavefronts, each of
+/// which owns kTN / kWaves values of n in the first product and kP / kWaves values of p in the second (multiples of
+/// 16). The defaults are the K = P = 128 configuration; <N, 64, 64, 128, 4> serves K = P = 64.
+template <typename InType, typename OutType, const int kN_, const int kK_ = 128, const int kP_ = 128, const int kTN_ = 256,
+          const int kWaves_ = 8>
 struct ResidentFusedGemmTraits {
-    static constexpr int kN = kN_, kK = 128, kP = 128;
-    static constexpr int kTM = 32, kTN = 256;
-    static_assert(kN % kTN == 0);
-    using WarpLayout = tl::RowMajor<1, 8>;
-    static constexpr int kWaves = 8, kThreads = kWaves * kWaveSize;
+    static constexpr int kN = kN_, kK = kK_, kP = kP_;
+    static constexpr int kTM = 32, kTN = kTN_;
+    static_assert(kN % kTN == 0 && kK % 32 == 0 && kTN % 32 == 0);
+    static constexpr int kWaves = kWaves_, kThreads = kWaves * kWaveSize;
+    static_assert(kTN % (16 * kWaves) == 0 && kP % (16 * kWaves) == 0, "every wavefront owns whole 16-wide tiles of n and of p");
+    using WarpLayout = tl::RowMajor<1, kWaves>;
     using Shape = traits::MfmaTileShape<InType, traits::MfmaShape::k16x16x32>;
 
     using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK>>;
@@ -195,7 +200,7 @@ struct ResidentFusedGemmTraits {
     using SharedC = SharedTile<InType, tl::ColMajor<kTN, kP>, true>;
     using SharedS = SharedTile<InType, tl::RowMajor<kTM, kTN>, true>;  // the intermediate of one block
     static constexpr int kShmBytes =
-        (SharedA::kNumel + SharedB::kNumel + SharedC::kNumel + SharedS::kNumel) * int(sizeof(InType));  // 152 KiB
+        (SharedA::kNumel + SharedB::kNumel + SharedC::kNumel + SharedS::kNumel) * int(sizeof(InType));  // 152 KiB by default
     static_assert(kShmBytes <= kMaxLdsBytes);
 
     using LoadA = GlobalToSharedDirectLoader<SharedA, WarpLayout>;

@@ -61,15 +61,16 @@ typedef enum {
 } tcu_gemm_algo;
 
 /* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks ROWS for many rows, else RESIDENT, where
- * they apply. */
+ * they apply; TILE_RESIDENT for K = P = 64 with N in {128, 256}; else TILE_LIBRARY. */
 typedef enum {
     TCU_B2B_AUTO = 0,
     TCU_B2B_TILE_LIBRARY = 1, /* composed from the 16x16 tile primitives, the reference kernel's structure */
     TCU_B2B_RESIDENT = 2,     /* A tile, 256-column blocks of B and C and the intermediate resident in LDS (K = P = 128,
                                  N % 256 == 0, M % 32 == 0); one round of loads per block */
     TCU_B2B_TILE_RESIDENT = 4, /* the RESIDENT kernel composed from tile-library functors only (direct-to-LDS loaders,
-                                 16x16x32 operand tiles, the intermediate through a shared tile); compile-time N in
-                                 {256, 1024, 2048}, K = P = 128, M % 32 == 0; results identical to RESIDENT bit for bit */
+                                 16x16x32 operand tiles, the intermediate through a shared tile); compile-time sizes:
+                                 K = P = 128 with N in {256, 1024, 2048} (results identical to RESIDENT bit for bit) and
+                                 K = P = 64 with N in {128, 256}; M % 32 == 0 */
     TCU_B2B_ROWS = 3          /* for many rows (AUTO from M x batch = 32768): N = 256, K = P = 128, M % 64 == 0; a
                                  workgroup keeps B and C in LDS and walks over blocks of 256 rows, every wavefront owning
                                  64 rows (A fragments from global memory, the intermediate stays in registers); agrees

@@ -471,6 +471,32 @@ def test_b2b_gemm_tile_resident_is_resident(tcu, oracle, device, M, N, batch, ou
     assert oracle.max_rel_err(host(got)[:, rows], ref, eps=1.0) <= REL_TOL
 
 
+@pytest.mark.parametrize("M,N,batch,out_dtype", [(256, 128, 1, "f32"), (96, 256, 3, "f16"), (8192, 128, 2, "f16")])
+def test_b2b_gemm_inner_size_64(tcu, oracle, device, M, N, batch, out_dtype):
+    """K = P = 64 (the reference driver's (256, 128, 64, 64), examples/cpp/02_fused_two_gemms/fused_gemm.cu:212-259, and
+    larger M / N): the LDS-resident composition from tile-library functors, which is what AUTO runs there, against the
+    oracle; AUTO gives the same bits."""
+    import torch
+
+    print(f"b2b K=P=64 M{M} N{N} b{batch} {out_dtype}", flush=True)
+    K, P = 64, 64
+    A = oracle.fill_normal(batch * M * K, 271, 0, 0.1).reshape(batch, M, K)
+    Bt = oracle.fill_normal(batch * N * K, 272, 0, 0.1).reshape(batch, N, K)
+    Ct = oracle.fill_normal(batch * P * N, 273, 0, 0.1).reshape(batch, P, N)
+    dt = torch.float32 if out_dtype == "f32" else torch.float16
+    dA, dB, dC = dev(A, device), dev(Bt, device), dev(Ct, device)
+    got = tcu.b2b_gemm(dA, dB, dC, out_dtype=dt, algo="tile_resident")
+    auto = tcu.b2b_gemm(dA, dB, dC, out_dtype=dt)
+    torch.cuda.synchronize()
+    assert torch.equal(got, auto)
+    rows = slice(0, min(M, 128))
+    ref = oracle.b2b_gemm(np.ascontiguousarray(A[:, rows]), Bt, Ct)
+    assert oracle.max_rel_err(host(got)[:, rows], ref, eps=1.0) <= REL_TOL
+    if N == 128:
+        tile = tcu.b2b_gemm(dA, dB, dC, out_dtype=dt, algo="tile_library")
+        assert oracle.max_rel_err(host(tile)[:, rows], ref, eps=1.0) <= REL_TOL
+
+
 @pytest.mark.parametrize("algo", ["tile_library", "resident"])
 @pytest.mark.parametrize("M,batch,out_dtype", [(32, 1, "f32"), (96, 3, "f16"), (8192, 1, "f16"), (16384, 2, "f32")])
 def test_b2b_gemm_both_kernels_at_256x128x128(tcu, oracle, device, algo, M, batch, out_dtype):
