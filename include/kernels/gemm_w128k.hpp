@@ -17,7 +17,9 @@
 //     is still ahead of the LDS-bound tiling: 2048^3 24.4 us against 26.8 us (the vendor library: 24.6-25.8 us).
 //   * Accumulators in AGPRs through inline assembly, scalar-base addressing, XCD-aware tile order: as in gemm_w128.
 // The sum over K is taken in four interleaved parts, so results differ from the other kernels by f32 rounding.
-// M % 128 == 0, N % 128 == 0, K % 128 == 0 (checked by the launcher).
+// K % 128 == 0; M % 128 == 0 and N % 128 == 0, or with kEdges any M, N in multiples of 16: the grid then covers
+// ceil(M / 128) x ceil(N / 128) tiles, rows beyond the edge are loaded from the last valid row (their products are
+// computed and dropped) and the stores are guarded per 16 x 16 block (checked by the launcher).
 #pragma once
 
 #include <type_traits>
@@ -41,8 +43,8 @@ struct GemmW128kTraits {
 };
 
 /// grid = (M / 128) * (N / 128), block = 256, dynamic LDS = GemmW128kTraits::kLdsBytes. lda / ldb / ldc: elements
-/// between consecutive rows of A, of the stored [N, K] array and of C.
-template <typename OutType>
+/// between consecutive rows of A, of the stored [N, K] array and of C. kEdges: grid = ceil(M / 128) * ceil(N / 128).
+template <typename OutType, bool kEdges = false>
 __global__ void __launch_bounds__(GemmW128kTraits::kThreads)
     gemm_w128k(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
                int lda, int ldb, int ldc) {
@@ -52,17 +54,23 @@ __global__ void __launch_bounds__(GemmW128kTraits::kThreads)
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(wave_id());
     int tile_m, tile_n;
-    detail::xcd_tile_coords(blockIdx.x, M / T::kBM, N / T::kBN, tile_m, tile_n);
+    detail::xcd_tile_coords(blockIdx.x, (M + T::kBM - 1) / T::kBM, (N + T::kBN - 1) / T::kBN, tile_m, tile_n);
     const int m0 = tile_m * T::kBM, n0 = tile_n * T::kBN;
 
     // ---- global -> LDS: load instruction q of this wavefront (q < 8: A, else B) fills 4 rows of 256 bytes; lane i
-    // writes physical 16-byte chunk i % 16 of row i / 16, which must hold logical chunk (i % 16) ^ (row % 16)
+    // writes physical 16-byte chunk i % 16 of row i / 16, which must hold logical chunk (i % 16) ^ (row % 16).
+    // kEdges: a row beyond the matrix is fetched from the last valid row instead (its LDS place and swizzle are its own)
     const int lrow = lane >> 4, lchk = lane & 15;
     unsigned int voff[16];
 #pragma unroll
     for (int q = 0; q < 16; ++q) {
         const int row = (wave * T::kLoads + (q & 7)) * 4 + lrow;
-        voff[q] = static_cast<unsigned int>(row) * static_cast<unsigned int>(q < 8 ? lda : ldb) * 2u + (lchk ^ (row & 15)) * 16;
+        int src_row = row;
+        if constexpr (kEdges) {
+            const int last = (q < 8 ? M - m0 : N - n0) - 1;
+            src_row = row < last ? row : last;
+        }
+        voff[q] = static_cast<unsigned int>(src_row) * static_cast<unsigned int>(q < 8 ? lda : ldb) * 2u + (lchk ^ (row & 15)) * 16;
     }
     const __half* a_base = A + size_t(m0) * lda;
     const __half* b_base = Bt + size_t(n0) * ldb;
@@ -188,6 +196,10 @@ __global__ void __launch_bounds__(GemmW128kTraits::kThreads)
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
             OutType* p = cbase + size_t(32 * r) * ldc + 16 * jj;
+            if constexpr (kEdges) {
+                // M and N are multiples of 16: a 16 x 16 block lies inside the matrix or outside it as a whole
+                if (m0 + 32 * r + 16 * (wave >> 1) >= M || n0 + 64 * (wave & 1) + 16 * jj >= N) continue;
+            }
             if constexpr (sizeof(OutType) == 4) {
                 *reinterpret_cast<f32x4*>(p) = res[r][jj];
             } else {

@@ -56,8 +56,9 @@ typedef enum {
                                 identical to WAVE128 and PIPELINED bit for bit */
     TCU_GEMM_WAVE128_KSPLIT = 8 /* 128 x 128 tile on 4 wavefronts (one per SIMD) that each own the whole tile over a
                                 quarter of every 128-wide step of K, partial tiles added through LDS: for products with
-                                too few 256 x 256 tiles to fill the GPU (2048^3); M, N, K multiples of 128; the sum over
-                                K is taken in four interleaved parts (differs from the other kernels by f32 rounding) */
+                                too few 256 x 256 tiles to fill the GPU (2048^3, 1552 x 1552 x 4096); K a multiple of 128,
+                                M and N multiples of 16 (edge tiles: rows clamped, stores guarded); the sum over K is
+                                taken in four interleaved parts (differs from the other kernels by f32 rounding) */
 } tcu_gemm_algo;
 
 /* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks ROWS for many rows, else RESIDENT, where

@@ -333,6 +333,40 @@ def test_gemm_wave128_ksplit(tcu, oracle, device, M, N, K, out_dtype):
         assert np.max(np.abs(got - want)) <= (5.0 if out_dtype == "f16" else 0.1)
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 16, 128), (144, 112, 256), (272, 400, 384), (1552, 1552, 4096), (1536, 1616, 2048)])
+@pytest.mark.parametrize("out_dtype", ["f16", "f32"])
+def test_gemm_wave128_ksplit_edge_tiles(tcu, oracle, device, M, N, K, out_dtype):
+    """The K-splitting kernel on shapes that are not whole 128 x 128 tiles (M, N in multiples of 16): rows beyond the
+    edge are fetched from the last valid row and their results dropped, the stores are guarded - nothing outside C is
+    written (guard rows and guard columns around it) and every element of C matches the oracle. 1552 x 1552 x 4096
+    (169 tiles) is a shape AUTO sends to it."""
+    import torch
+
+    print(f"gemm wave128_ksplit edges {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float16 if out_dtype == "f16" else torch.float32
+    A = oracle.fill_uniform(M * K, 9200 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 9300 + N).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    guard = torch.full((M + 2, N), -7.0, dtype=dt, device=device)
+    out = guard[1:M + 1]
+    tcu.gemm(dA, dB, out=out, algo="wave128_ksplit")
+    torch.cuda.synchronize()
+    assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
+    got = host(out)
+    assert np.isfinite(got).all()
+    rows = (0, M) if M <= 512 else (M - 160, M)  # the last rows include the edge tiles
+    ref = oracle.gemm(A, Bt, rows=rows)
+    assert oracle.max_rel_err(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
+    if M > 512:
+        # every element, through row and column sums in float64
+        a64, b64 = A.astype(np.float64), Bt.astype(np.float64)
+        tol = 5.0 if out_dtype == "f16" else 0.2
+        assert np.max(np.abs(got.astype(np.float64).sum(axis=0) - b64 @ a64.sum(axis=0))) <= tol
+        assert np.max(np.abs(got.astype(np.float64).sum(axis=1) - a64 @ b64.sum(axis=0))) <= tol
+    if (M, N, K) == (1552, 1552, 4096):
+        assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, workspace=False))  # AUTO takes this kernel here
+
+
 @pytest.mark.parametrize("algo", ["pipelined", "wave128"])
 def test_gemm_one_hot_index_probe(tcu, device, algo):
     """C[m, n] = A[m, k] * Bt[n, k] for one-hot operands: pins rows/cols/transposition exactly."""

@@ -241,14 +241,19 @@ int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int 
 template <typename OutType>
 int gemm_w128k_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
     using T = GemmW128kTraits;
-    if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the K-splitting one-wavefront-per-SIMD GEMM needs M, N and K in multiples of 128");
+    if (M % 16 != 0 || N % 16 != 0 || K % T::kBK != 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the K-splitting one-wavefront-per-SIMD GEMM needs M and N in multiples of 16 "
+                                               "and K in multiples of 128");
     if ((long)K * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the K-splitting GEMM addresses a 128-row panel with 32-bit offsets");
-    const long grid = (long)(M / T::kBM) * (N / T::kBN);
+    const long grid = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
     if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many tiles for one launch");
-    return launch(&gemm_w128k<OutType>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M, N, K, K,
-                  K, N);
+    if (M % T::kBM == 0 && N % T::kBN == 0)
+        return launch(&gemm_w128k<OutType, false>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M,
+                      N, K, K, K, N);
+    // edge tiles: rows beyond M or N loaded from the last valid row, stores guarded per 16 x 16 block
+    return launch(&gemm_w128k<OutType, true>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M, N,
+                  K, K, K, N);
 }
 
 template <typename OutType, int kM, int kN, int kK, int kTM, int kTN, typename WarpLayout>
@@ -385,8 +390,8 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             // kernel whose wavefronts split K (each owns the whole 128 x 128 tile) beats the LDS-bound 64 x 64-per-
             // wavefront tilings (2048^3: 24.4 against 26.8 us, 1536 x 1536 x 4096: 35.7 against 39.8 us); with a
             // short K its reduction through LDS costs more than it saves (1792 x 1792 x 1024: 16.0 against 13.1 us)
-            if (M % 128 == 0 && N % 128 == 0 && K % 128 == 0 && K >= 2048 && (long)K * 256 < (1l << 32)) {
-                const long tiles = (long)(M / 128) * (N / 128);
+            if (M % 16 == 0 && N % 16 == 0 && K % 128 == 0 && K >= 2048 && (long)K * 256 < (1l << 32)) {
+                const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
                 if (tiles >= 128 && tiles <= 256) return gemm_w128k_dispatch<OutType>(A, B, C, M, N, K, stream);
             }
             if (M % 16 == 0 && N % 16 == 0) {
