@@ -314,11 +314,12 @@ struct SharedToRegPieces : public Base {
 /// tiles is kept; the contraction index (the tile's row i) is an immediate of the instruction, which requires a
 /// swizzle whose line period divides 4 (tl::LdsSwizzleTr).
 /// kAccumulatorOrder: which contraction indices a lane receives. false: the standard operand order (lane group
-/// g = lane / 32 or lane / 16 / ... holds indices 8 g .. 8 g + 7 of the tile's 16). true, for 16 x 32 tiles: the order
-/// in which the 32 x 32 accumulator of a preceding product holds its columns - slot e of lane half h is index
-/// 8 (e / 4) + 4 h + e % 4 - so that accumulator values converted to 2-byte elements ARE the A operand of the next
-/// product without leaving the lane (the contraction index of a matrix instruction may be permuted as long as both
-/// operands agree).
+/// g = lane / 32 or lane / 16 holds indices 8 g .. 8 g + 7 of the tile). true: the order in which the accumulators of
+/// a preceding product hold their columns, so that accumulator values converted to 2-byte elements ARE the A operand
+/// of the next product without leaving the lane (the contraction index of a matrix instruction may be permuted as long
+/// as both operands agree). For 16 x 32 tiles (B of v_mfma_f32_32x32x16_f16) that is one 32 x 32 accumulator: slot e of
+/// lane half h is index 8 (e / 4) + 4 h + e % 4. For 32 x 16 tiles (B of v_mfma_f32_16x16x32_f16) it is two 16 x 16
+/// accumulators side by side: slot e of lane group g is index 16 (e / 4) + 4 g + e % 4.
 template <typename Reg_, typename Shared_, typename WarpLayout_, const WarpReuse kMode_, const bool kAccumulatorOrder = false,
           typename Base = warp::CopyBase<WarpLayout_, kMode_>>
 struct SharedToRegTrPieces : public Base {
@@ -331,16 +332,17 @@ struct SharedToRegTrPieces : public Base {
     static_assert(std::is_same_v<typename Shared::DType, DType> && sizeof(DType) == 2 && Shared::kIsRowMajor &&
                       !G::kRowMajor && G::kRunLen == 8 && G::kRuns == 1,
                   "the transposing read serves column-major operand tiles of 2-byte elements out of a row-major tile");
-    static_assert(!Shared::kSwizzled || 4 % Shared::Swizzle::kLinePeriod == 0,
-                  "the tile's row is an immediate of the read: the swizzle must repeat every 4 lines (tl::LdsSwizzleTr)");
-    static_assert(!kAccumulatorOrder || G::kLaneMajor == 32, "the accumulator order is that of the 32 x 32 accumulator");
+    static constexpr int kPeriod = Shared::kSwizzled ? Shared::Swizzle::kLinePeriod : 1;
     static_assert(Base::template row_exec_count<BaseShape, Shared::kRows>() == Reg::kRows &&
                       Base::template col_exec_count<BaseShape, Shared::kCols>() == Reg::kCols,
                   "the register tile must hold exactly this wavefront's share of the shared tile");
     static constexpr int kLineBytes = Shared::kPitch * int(sizeof(DType));
     // rows between the two reads of an operand tile, and how many rows a lane group's index moves the first one
-    static constexpr int kPartRows = kAccumulatorOrder ? 8 : 4;
+    static constexpr int kPartRows = kAccumulatorOrder ? 4 * (kWaveSize / G::kLaneMajor) : 4;
     static constexpr int kGroupRows = kAccumulatorOrder ? 4 : 8;
+    static_assert(kPartRows % kPeriod == 0 && BaseShape::kRows % kPeriod == 0,
+                  "the tile's row is an immediate of the read: the swizzle must repeat with the rows between the two reads "
+                  "and with the tile height (tl::LdsSwizzleTr)");
 
     DEVICE SharedToRegTrPieces() {
         const int lane = lane_id();
@@ -361,7 +363,7 @@ struct SharedToRegTrPieces : public Base {
     /// multiple of 4, folded into the instruction's immediate together with the tile's own row); not waited for.
     template <int kI, int kJ, int kLine0 = 0>
     DEVICE void read(const Shared& src, Reg& dst) const {
-        static_assert(kLine0 % 4 == 0);
+        static_assert(kLine0 % 4 == 0 && kLine0 % kPeriod == 0);
         constexpr int kOff0 = (kLine0 + kI * BaseShape::kRows) * kLineBytes, kOff1 = kOff0 + kPartRows * kLineBytes;
         static_assert(kOff1 < 65536, "the immediate offset of an LDS read has 16 bits");
         f16x4 lo, hi;

@@ -365,13 +365,6 @@ __global__ void __launch_bounds__(Traits::kThreads)
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    // first fragments of step 1: K of half 2 (block 1), V of half 0
-    static_for<kAhead>([&](auto a_c) {
-        constexpr int a = decltype(a_c)::value;
-        k_frag.template read<a, 0>(k_half(1, 0), rK);
-        v_frag.template read<0, a & 3>(v_half(0, 0), rV);
-    });
-
     // ---- block-iterations: J covers halves 2 J + 1 and 2 J + 2
     using Yes = std::true_type;
     using No = std::false_type;
@@ -389,6 +382,13 @@ __global__ void __launch_bounds__(Traits::kThreads)
     {
         // J = 0: blocks 3 and 4 go to the stages Q passed through (everyone has read its Q by now)
         wait_group_and_barrier_keep_reads<0>();
+        // first fragments of step 1: K of half 2 (block 1), V of half 0 - behind the barrier: block 1 is complete only
+        // when every wavefront's pieces of it have landed
+        static_for<kAhead>([&](auto a_c) {
+            constexpr int a = decltype(a_c)::value;
+            k_frag.template read<a, 0>(k_half(1, 0), rK);
+            v_frag.template read<0, a & 3>(v_half(0, 0), rV);
+        });
         Stages first = ring;
         first.load = 3;
         step(first, I1{}, Yes{}, I1{}, Yes{}, 3);

@@ -612,12 +612,18 @@ __global__ void __launch_bounds__(Traits::kThreads)
         asm volatile("" ::: "memory");
     };
 
-    // first fragments of step 1
+    // first fragments of step 1: K of half 2 (block 1), V of half 0. With Q staged through LDS, block 1 was requested
+    // only under the scores of half 0 and every wavefront fetched a quarter of it: the reads then go behind the first
+    // hand-over (before it, another wavefront's quarter may still be on its way - seen as rare wrong rows when the
+    // block missed the L2).
+    auto first_fragments = [&]() {
 #pragma unroll
-    for (int a = 0; a < kAhead; ++a) {
-        if (nb > 1) kf[a] = read_k_untracked(k_half(2), a);
-        vf[a] = read_v_untracked(v_block(0), C0{}, C0{}, a & 3);
-    }
+        for (int a = 0; a < kAhead; ++a) {
+            if (nb > 1) kf[a] = read_k_untracked(k_half(2), a);
+            vf[a] = read_v_untracked(v_block(0), C0{}, C0{}, a & 3);
+        }
+    };
+    if (!q_via_lds) first_fragments();
     // ---- block-iterations: J covers halves 2 J + 1 (odd) and 2 J + 2 (even)
     constexpr unsigned int kStageB = Traits::kStageBytes, kRingB = kStages * Traits::kStageBytes;
     auto next_stage = [&](unsigned int off) { return off + kStageB == kRingB ? 0u : off + kStageB; };
@@ -633,6 +639,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     if (q_via_lds) {
         // J = 0: blocks 3 and 4 go to the stages the Q tiles were staged in (everyone has read its Q by now)
         hand_over(std::integral_constant<int, 0>{});
+        first_fragments();
         RingOffsets first = ring;
         first.load = 3 * kStageB;
         step(first, C1{}, Yes{}, Yes{}, Yes{}, 3);

@@ -1,0 +1,482 @@
+// FlashAttention-2 forward, one wavefront per SIMD, on v_mfma_f32_16x16x32_f16 - the f16 matrix instruction that
+// contracts 32 indices per issue. Same design as kernels/flash_attn_tile_w64.hpp (which uses v_mfma_f32_32x32x16_f16)
+// and written with the same tile-library functors, the way the reference composes its attention kernel from its L2
+// functors (src/kernels/flash_attn.cu:134-312; traits :18-131):
+//   a workgroup of 4 wavefronts owns 256 queries, a wavefront 64 (four 16-row tiles); K and V blocks of 64 keys pass
+//   through two interleaved 5-stage SharedRings filled by GlobalToSharedDirectPieces (one direct-to-LDS load riding on a
+//   matrix instruction at a time); S = Q Kᵀ and O += P V are tile products whose every instruction is placed by
+//   compute::ScheduledGemm::at<i, j, k>() (O and the Q operand pinned in AGPRs, the scores in VGPRs); operand fragments
+//   are requested three groups of instructions ahead with SharedToRegPieces (ds_read_b128, K) and SharedToRegTrPieces
+//   (ds_read_b64_tr_b16, V, in the order in which two 16 x 16 score accumulators hold their keys, so that the converted
+//   scores ARE the A operand of the second product) and awaited with wait_shared_reads<N>(); the softmax of 32 keys is
+//   sliced over the 64 matrix instructions of the neighbouring 32 - a v_exp_f32 behind every second one, the sums
+//   and conversions behind the others (compute::Exp2Raw, convert_pair_here); stages are handed over with
+//   wait_group_and_barrier_keep_reads<N>(); the output leaves through RegToSharedStorer / SharedToGlobalStorer.
+// Why a second instruction shape: under the chip's power limit the core clock follows the work, and a stream of
+// 16x16x32 instructions sustains a clock about an eighth higher than the same arithmetic in 32x32x16 instructions
+// (half the accumulator traffic per multiply-add). A wavefront alone on its SIMD has issue slots to spare for twice the
+// number of instructions as long as the vector work between them stays in doses of one transcendental or two plain
+// operations.
+// Numerics: as flash_attention_fwd_w64 (Q pre-multiplied by scale * log2 e in f16, scores relative to a reference
+// maximum that moves only when a partial sum could leave f16 range, f32 sums and output); the sums inside a matrix
+// instruction cover 32 instead of 16 indices, so results differ from that kernel in the last bits.
+// Requirements: head size 128, row-major V, M % 256 == 0, N % 64 == 0, N >= 320 (Q passes through two ring stages
+// before the fifth block needs them). M, N and the batch count are run-time values.
+#pragma once
+
+#include <type_traits>
+#include <utility>
+
+#include "cell/mod.hpp"
+#include "types/mod.hpp"
+#include "util/static_for.hpp"
+
+namespace tiledcuda::kernels {
+
+using namespace tiledcuda::cell;
+using namespace tiledcuda::cell::copy;
+namespace tl = tiledcuda::cell::tile_layout;
+
+template <typename InType, const int kD_>
+struct FlashW64K32Traits {
+    static constexpr int kD = kD_;
+    using WarpLayout = tl::RowMajor<4, 1>;
+    static constexpr int kWaves = 4, kThreads = kWaves * kWaveSize;
+    static constexpr int kTM = 64 * kWaves, kTN = 64, kHalf = 32, kStages = 5;
+    static_assert(kD == 128, "the step schedule is written for head size 128");
+
+    using Shape = traits::MfmaTileShape<InType, traits::MfmaShape::k16x16x32>;
+    static constexpr int kQTiles = 64 / 16;     // 16-row query tiles of a wavefront
+    static constexpr int kKeyTiles = kHalf / 16;  // 16-key tiles of a half
+    static constexpr int kDSteps = kD / 32;     // contraction steps of S = Q Kᵀ
+    static constexpr int kDTiles = kD / 16;     // 16-column tiles of O
+
+    // global views of one query block / key block
+    using GlobalQ = GlobalTile<InType, tl::RowMajor<kTM, kD>>;
+    using GlobalO = GlobalTile<InType, tl::RowMajor<kTM, kD>>;
+
+    // LDS: a ring stage is a K block followed by a V block; Q passes once through stages 3 and 4
+    using SharedK = SharedTile<InType, tl::ColMajor<kD, kTN>, true>;  // Kᵀ [d, keys], stored [keys, d]
+    using SharedV = SharedTile<InType, tl::RowMajor<kTN, kD>, true, tl::LdsSwizzleTr<kD, sizeof(InType), 8>>;
+    static constexpr int kBlockNumel = kTN * kD;
+    using RingK = SharedRing<SharedK, kStages, 2 * kBlockNumel>;
+    using RingV = SharedRing<SharedV, kStages, 2 * kBlockNumel>;
+    using SharedQ = SharedTile<InType, tl::RowMajor<kTM, kD>, true>;
+    using SharedO = SharedTile<InType, tl::RowMajor<kTM, kD>, true>;
+    static constexpr int kShmBytes = kStages * 2 * kBlockNumel * int(sizeof(InType));  // 160 KiB
+    static_assert(kShmBytes <= kMaxLdsBytes && 2 * 2 * kBlockNumel == kTM * kD, "Q fills exactly two stages");
+
+    // the 32-key halves a step works on
+    using KHalves = STileIterator<SharedK, TileShape<kD, kHalf>>;
+    using VHalves = STileIterator<SharedV, TileShape<kHalf, kD>>;
+    using SharedKHalf = decltype(std::declval<KHalves>()(0));
+    using SharedVHalf = decltype(std::declval<VHalves>()(0));
+
+    // register tiles of one wavefront (64 queries)
+    using RegQ = RegTile<typename Shape::TileA, tl::RowMajor<kQTiles, kDSteps>>;     // A of S = Q Kᵀ, in AGPRs
+    using RegK = RegTile<typename Shape::TileB, tl::ColMajor<kDSteps, kKeyTiles>>;   // B of S: the 8 fragments of a half
+    using RegS = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, kKeyTiles>>; // scores of 32 keys
+    using RegM = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, 1>>;         // where the score sums start
+    using RegP = RegTile<typename Shape::TileA, tl::RowMajor<kQTiles, 1>>;           // probabilities: A of O += P V
+    using RegV = RegTile<typename Shape::TileB, tl::ColMajor<1, kDTiles>>;           // B of O += P V
+    using RegO = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, kDTiles>>;   // in AGPRs
+    using RegOut = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kQTiles, kDTiles>>;
+
+    using QLoader = GlobalToSharedDirectLoader<SharedQ, WarpLayout>;
+    using QFragments = SharedToRegLoader<RegQ, WarpLayout, WarpReuse::kRowReuseCont>;
+    using PiecesK = GlobalToSharedDirectPieces<SharedK, WarpLayout, kD>;
+    using PiecesV = GlobalToSharedDirectPieces<SharedV, WarpLayout, kD>;
+    using KFragmentsNow = SharedToRegLoader<RegK, WarpLayout, WarpReuse::kColReuseCont>;
+    using KFragments = SharedToRegPieces<RegK, SharedKHalf, WarpLayout, WarpReuse::kColReuseCont>;
+    using VFragments = SharedToRegTrPieces<RegV, SharedVHalf, WarpLayout, WarpReuse::kColReuseCont, true>;
+    using Scores = compute::ScheduledGemm<RegQ, RegK, RegS, compute::RegFile::kVgpr, compute::RegFile::kAgpr>;
+    using Output = compute::ScheduledGemm<RegP, RegV, RegO, compute::RegFile::kAgpr, compute::RegFile::kVgpr>;
+    using OutToShared = RegToSharedStorer<RegOut, WarpLayout>;
+    using OutToGlobal = SharedToGlobalStorer<SharedO, WarpLayout>;
+    static_assert(PiecesK::kPieces == 4 && PiecesV::kPieces == 4, "a wavefront issues 8 loads per block, one per group");
+    static_assert(kDSteps * kKeyTiles == 8 && kDTiles == 8, "a step has 8 groups: a K fragment and a V fragment each");
+};
+
+/// grid = (M / 256) * batch workgroups (1-D), block = 256, dynamic LDS = Traits::kShmBytes.
+template <typename InType, typename Traits>
+__global__ void __launch_bounds__(Traits::kThreads)
+    flash_attention_w64_k32(const InType* dQ, const InType* dK, const InType* dV, InType* dO, int batch, int kM, int kN,
+                            float scale) {
+    constexpr int kD = Traits::kD, kTN = Traits::kTN;
+    constexpr int kQT = Traits::kQTiles, kDT = Traits::kDTiles;
+    using RegQ = typename Traits::RegQ;
+    using RegK = typename Traits::RegK;
+    using RegS = typename Traits::RegS;
+    using RegM = typename Traits::RegM;
+    using RegP = typename Traits::RegP;
+    using RegV = typename Traits::RegV;
+    using RegO = typename Traits::RegO;
+    using Scores = typename Traits::Scores;
+    using Output = typename Traits::Output;
+    extern __shared__ __align__(1024) unsigned char buf[];
+    const int nb = kN / kTN;
+
+    // query blocks of one (batch, head) item get workgroup ids congruent modulo 8: one XCD, K and V fetched once
+    const int q_blocks = kM / Traits::kTM;
+    int head_i, q_block;
+    if (batch % 8 == 0) {
+        const int xcd = blockIdx.x & 7, rest = blockIdx.x >> 3;
+        q_block = rest % q_blocks;
+        head_i = (rest / q_blocks) * 8 + xcd;
+    } else {
+        q_block = blockIdx.x % q_blocks;
+        head_i = blockIdx.x / q_blocks;
+    }
+    const size_t head = head_i;
+    const InType* Qb = dQ + (head * kM + size_t(q_block) * Traits::kTM) * kD;
+    const InType* Kh = dK + head * size_t(kN) * kD;
+    const InType* Vh = dV + head * size_t(kN) * kD;
+    InType* Ob = dO + (head * kM + size_t(q_block) * Traits::kTM) * kD;
+
+    InType* shm = reinterpret_cast<InType*>(buf);
+    typename Traits::RingK ringK(shm);
+    typename Traits::RingV ringV(shm + Traits::kBlockNumel);
+    typename Traits::SharedQ sQ(shm + 3 * 2 * Traits::kBlockNumel);  // stages 3 and 4
+
+    typename Traits::PiecesK pieces_k;
+    typename Traits::PiecesV pieces_v;
+    typename Traits::KFragments k_frag;
+    typename Traits::VFragments v_frag;
+
+    // load s of this wavefront for key block `block` into ring stage `stage`: 4 pieces of K, then 4 of V
+    auto block_load = [&](int stage, int block, int s) -> DirectLoad {
+        return s < 4 ? pieces_k.piece(s, Kh + size_t(block) * kTN * kD, ringK[stage])
+                     : pieces_v.piece(s - 4, Vh + size_t(block) * kTN * kD, ringV[stage]);
+    };
+    auto k_half = [&](int stage, int t) { return typename Traits::KHalves(ringK.stage_data(stage))(t); };
+    auto v_half = [&](int stage, int t) { return typename Traits::VHalves(ringV.stage_data(stage))(t); };
+
+    // ---- prologue: Q and block 0 are requested together (the cold latencies overlap); blocks 1 and 2 under the
+    // first two score computations, blocks 3 and 4 (into the stages Q passed through) in the first block-iteration
+    {
+        typename Traits::QLoader load_q;
+        typename Traits::GlobalQ gQ(Qb);
+        load_q(gQ, sQ);
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) issue(block_load(0, 0, s));
+    wait_group_and_barrier<0>();
+
+    RegQ rQ;
+    {
+        typename Traits::QFragments read_q;
+        read_q(sQ, rQ);
+        // pre-multiplied by scale * log2(e): the scores come out of the matrix instruction in the log2 domain
+        const float cscale = scale * 1.4426950408889634f;
+#pragma unroll
+        for (int c = 0; c < kQT; ++c)
+#pragma unroll
+            for (int s = 0; s < Traits::kDSteps; ++s) {
+                _Float16* q = reinterpret_cast<_Float16*>(rQ(c, s).mutable_data());
+#pragma unroll
+                for (int e = 0; e < 8; ++e) q[e] = static_cast<_Float16>(static_cast<float>(q[e]) * cscale);
+            }
+        compute::pin_tiles<compute::RegFile::kAgpr>(rQ);
+    }
+
+    RegO rO;
+    compute::clear_pinned(rO);
+
+    RegS rS[2];     // score tiles of two consecutive halves, relative to the reference maximum
+    RegP rP[2];     // their probabilities
+    RegM neg_max;   // minus the reference maximum of this lane's query of each tile, in all 4 slots
+    float m_run[kQT], l_run[kQT];
+    RegK rK;        // fragments in flight / in use: (d-step, key tile)
+    RegV rV;        // (0, d tile)
+
+    compute::Exp2Raw<float> exp2;
+    using f16x2 = _Float16 __attribute__((ext_vector_type(2)));
+    // maximum over the 4 lane groups that share a query row
+    auto row_max = [](float v) {
+        v = fmaxf(v, __shfl_xor(v, 16, 64));
+        return fmaxf(v, __shfl_xor(v, 32, 64));
+    };
+
+    // scores of half `t` of the block in `stage` into rS[kBuf] (before the pipeline runs: plain reads), issuing this
+    // wavefront's loads of block `load_block` behind the groups
+    auto scores_only = [&](int stage, int t, auto buf_c, int load_block) {
+        constexpr int kBuf = decltype(buf_c)::value;
+        typename Traits::KFragmentsNow read_k;
+        const auto sk = k_half(stage, t);
+        RegK kf;
+        read_k.load_one(sk, kf, 0, 0);
+        static_for<8>([&](auto g_c) {
+            constexpr int g = decltype(g_c)::value, ds = g % 4, kt = g / 4;
+            if constexpr (g + 1 < 8) read_k.load_one(sk, kf, (g + 1) % 4, (g + 1) / 4);
+            static_for<kQT>([&](auto c_c) {
+                constexpr int c = decltype(c_c)::value;
+                if constexpr (ds == 0) Scores::template at_from<c, kt, 0>(rQ, kf, rS[kBuf], neg_max(c, 0));
+                else Scores::template at<c, kt, ds>(rQ, kf, rS[kBuf]);
+            });
+            issue(block_load(load_block, load_block, g));
+        });
+    };
+
+    // probabilities of one score tile's 4 keys: to f16, into slots 4 kt .. 4 kt + 3 of the A operand, and their sum
+    auto tile_softmax_now = [&](const BaseTileRowMajor<float>& sc, float shift, _Float16* dst) {
+        const float p0 = exp2(sc(0, 0) - shift), p1 = exp2(sc(0, 1) - shift);
+        const float p2 = exp2(sc(0, 2) - shift), p3 = exp2(sc(0, 3) - shift);
+        const f16x2 lo = {static_cast<_Float16>(p0), static_cast<_Float16>(p1)};
+        const f16x2 hi = {static_cast<_Float16>(p2), static_cast<_Float16>(p3)};
+        __builtin_memcpy(dst, &lo, sizeof(lo));
+        __builtin_memcpy(dst + 2, &hi, sizeof(hi));
+        return (p0 + p1) + (p2 + p3);
+    };
+
+    // ---- half 0: exact maxima
+#pragma unroll
+    for (int c = 0; c < kQT; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) neg_max(c, 0)(0, e) = 0.f;
+    compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
+    scores_only(0, 0, std::integral_constant<int, 0>{}, 1);
+    asm volatile("s_nop 15\n\ts_nop 3");
+    compute::pin_tiles<compute::RegFile::kVgpr>(rS[0]);
+#pragma unroll
+    for (int c = 0; c < kQT; ++c) {
+        float mx = rS[0](c, 0)(0, 0);
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, rS[0](c, kt)(0, e));
+        mx = row_max(mx);
+        m_run[c] = mx;
+        _Float16* p = reinterpret_cast<_Float16*>(rP[0](c, 0).mutable_data());
+        l_run[c] = tile_softmax_now(rS[0](c, 0), mx, p) + tile_softmax_now(rS[0](c, 1), mx, p + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) neg_max(c, 0)(0, e) = -mx;
+    }
+    compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
+    scores_only(0, 1, std::integral_constant<int, 1>{}, 2);
+
+    // ---- one pipelined step on half i: softmax of half i (rS[kCur] -> rP[kCur]), scores of half i + 1 into rS[kNxt]
+    // (if kQk), O += P V with half i - 1 (rP[kNxt]). ring: stages of blocks J, J + 1, J + 2 and of the block being
+    // loaded. kLoads: 0 none, 1 block `load_block`.
+    // A step is 8 groups of 8 matrix instructions: group g multiplies K fragment g (d-step g % 4 of key tile g / 4) with
+    // the 4 query tiles, then V fragment g (d tile g) with the 4 probability tiles, and takes score tile
+    // (g / 2, g % 2) of half i through the softmax. Fragments are requested kAhead groups before their instructions,
+    // across step boundaries.
+    struct Stages {
+        int a, b, c, load;
+    };
+    constexpr int kAhead = 3;
+    constexpr int kReadsV = 2, kReadsQk = 3;  // LDS read instructions per group
+
+    auto step = [&](const Stages& ring, auto cur_c, auto qk_c, auto loads_c, auto next_qk_c, int load_block) {
+        constexpr int kCur = decltype(cur_c)::value, kNxt = kCur ^ 1;
+        constexpr bool kQk = decltype(qk_c)::value, kNextQk = decltype(next_qk_c)::value;
+        constexpr int kLoads = decltype(loads_c)::value;
+        // K of half i + 1, V of half i - 1, K of half i + 2, V of half i
+        const auto sk = kCur == 1 ? k_half(ring.b, 0) : k_half(ring.b, 1);
+        const auto sv = v_half(ring.a, kNxt);
+        const auto sk_next = kCur == 1 ? k_half(ring.b, 1) : k_half(ring.c, 0);
+        const auto sv_next = v_half(kCur == 1 ? ring.a : ring.b, kCur);
+        float lh[kQT] = {0.f, 0.f, 0.f, 0.f};
+        float x0 = 0.f, x1 = 0.f, x2 = 0.f, x3 = 0.f;
+        static_for<8>([&](auto g_c) {
+            constexpr int g = decltype(g_c)::value;
+            constexpr int gp = g + kAhead;
+            if constexpr (gp < 8) {
+                if constexpr (kQk) k_frag.template read<gp % 4, gp / 4>(sk, rK);
+                v_frag.template read<0, gp>(sv, rV);
+                wait_shared_reads<kAhead * (kQk ? kReadsQk : kReadsV)>();
+            } else {
+                if constexpr (kNextQk) k_frag.template read<(gp - 8) % 4, (gp - 8) / 4>(sk_next, rK);
+                v_frag.template read<0, gp - 8>(sv_next, rV);
+                wait_shared_reads<(7 - g) * (kQk ? kReadsQk : kReadsV) + (gp - 7) * (kNextQk ? kReadsQk : kReadsV)>();
+            }
+            constexpr int ds = g % 4, kt = g / 4;   // the K fragment of this group
+            constexpr int sc = g / 2, st = g % 2;   // the score tile of half i this group takes through the softmax
+            const auto& sv4 = rS[kCur](sc, st);
+            _Float16* pdst = reinterpret_cast<_Float16*>(rP[kCur](sc, 0).mutable_data()) + 4 * st;
+            _Float16* pprev = reinterpret_cast<_Float16*>(rP[kCur]((g + 7) % 8 / 2, 0).mutable_data()) + 4 * ((g + 7) % 2);
+            auto score = [&](auto c_c) {
+                constexpr int c = decltype(c_c)::value;
+                if constexpr (kQk) {
+                    if constexpr (ds == 0) Scores::template at_from<c, kt, 0>(rQ, rK, rS[kNxt], neg_max(c, 0));
+                    else Scores::template at<c, kt, ds>(rQ, rK, rS[kNxt]);
+                }
+            };
+            using I0 = std::integral_constant<int, 0>;
+            using I1 = std::integral_constant<int, 1>;
+            using I2 = std::integral_constant<int, 2>;
+            using I3 = std::integral_constant<int, 3>;
+            // slot 0
+            score(I0{});
+            x0 = exp2(sv4(0, 0));
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 1: the second pair of the group before
+            score(I1{});
+            if constexpr (g > 0) {
+                compute::convert_pair_here(x2, x3, reinterpret_cast<__half*>(pprev) + 2);
+                lh[(g - 1) / 2] += x3;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 2
+            score(I2{});
+            x1 = exp2(sv4(0, 1));
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 3
+            score(I3{});
+            lh[sc] += x0;
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 4 (with this wavefront's load g riding on the matrix instruction)
+            if constexpr (kLoads == 1) {
+                Output::template at<0, g, 0>(rP[kNxt], rV, rO, block_load(ring.load, load_block, g));
+            } else {
+                Output::template at<0, g, 0>(rP[kNxt], rV, rO);
+            }
+            x2 = exp2(sv4(0, 2));
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 5
+            Output::template at<1, g, 0>(rP[kNxt], rV, rO);
+            compute::convert_pair_here(x0, x1, reinterpret_cast<__half*>(pdst));
+            lh[sc] += x1;
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 6
+            Output::template at<2, g, 0>(rP[kNxt], rV, rO);
+            x3 = exp2(sv4(0, 3));
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 7
+            Output::template at<3, g, 0>(rP[kNxt], rV, rO);
+            lh[sc] += x2;
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        lh[kQT - 1] += x3;
+        compute::convert_pair_here(x2, x3, reinterpret_cast<__half*>(rP[kCur](kQT - 1, 0).mutable_data()) + 6);
+        // no probability of this half can have left f16 range while its sum stays below 2^14
+        constexpr float kLimit = 16384.f;
+        if (__any(!(fmaxf(fmaxf(lh[0], lh[1]), fmaxf(lh[2], lh[3])) <= kLimit))) {
+            // rare path: move the reference maxima, rescale, re-bias the scores already computed, recompute
+            asm volatile("s_nop 15\n\ts_nop 3");
+            if constexpr (kQk) compute::pin_tiles<compute::RegFile::kVgpr>(rS[kNxt]);
+            compute::pin_tiles<compute::RegFile::kAgpr>(rO);
+#pragma unroll
+            for (int c = 0; c < kQT; ++c) {
+                float mx = rS[kCur](c, 0)(0, 0);
+#pragma unroll
+                for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) mx = fmaxf(mx, rS[kCur](c, kt2)(0, e));
+                mx = row_max(mx);
+                const float shift = mx > 8.0f ? mx : 0.f;
+                const float alpha = exp2(-shift);
+                m_run[c] += shift;
+                l_run[c] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < kDT; ++dt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) rO(c, dt)(0, e) *= alpha;
+                if constexpr (kQk) {
+#pragma unroll
+                    for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) rS[kNxt](c, kt2)(0, e) -= shift;
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) neg_max(c, 0)(0, e) = -m_run[c];
+                _Float16* p = reinterpret_cast<_Float16*>(rP[kCur](c, 0).mutable_data());
+                lh[c] = tile_softmax_now(rS[kCur](c, 0), shift, p) + tile_softmax_now(rS[kCur](c, 1), shift, p + 4);
+            }
+            compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
+            compute::pin_tiles<compute::RegFile::kAgpr>(rO);
+        }
+#pragma unroll
+        for (int c = 0; c < kQT; ++c) l_run[c] += lh[c];
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // ---- block-iterations: J covers halves 2 J + 1 and 2 J + 2
+    using Yes = std::true_type;
+    using No = std::false_type;
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    int J = 0;
+    Stages ring{0, 1, 2, 4};
+    auto advance = [&]() {
+        ring.a = ring.b;
+        ring.b = ring.c;
+        ring.c = Traits::RingK::next(ring.c);
+        ring.load = Traits::RingK::next(ring.load);
+        ++J;
+    };
+    {
+        // J = 0: blocks 3 and 4 go to the stages Q passed through (everyone has read its Q by now)
+        wait_group_and_barrier_keep_reads<0>();
+        // first fragments of step 1: K of half 2 (block 1), V of half 0 - behind the barrier: block 1 is complete only
+        // when every wavefront's pieces of it have landed
+        static_for<kAhead>([&](auto a_c) {
+            constexpr int a = decltype(a_c)::value;
+            k_frag.template read<a % 4, a / 4>(k_half(1, 0), rK);
+            v_frag.template read<0, a>(v_half(0, 0), rV);
+        });
+        Stages first = ring;
+        first.load = 3;
+        step(first, I1{}, Yes{}, I1{}, Yes{}, 3);
+        step(ring, I0{}, Yes{}, I1{}, Yes{}, 4);
+        advance();
+    }
+#pragma unroll 1
+    for (; J + 4 < nb; advance()) {
+        wait_group_and_barrier_keep_reads<8>();
+        step(ring, I1{}, Yes{}, I1{}, Yes{}, J + 4);
+        step(ring, I0{}, Yes{}, I0{}, Yes{}, 0);
+    }
+#pragma unroll 1
+    for (; J + 2 < nb; advance()) {
+        wait_group_and_barrier_keep_reads<0>();
+        step(ring, I1{}, Yes{}, I0{}, Yes{}, 0);
+        step(ring, I0{}, Yes{}, I0{}, Yes{}, 0);
+    }
+    if (J + 1 < nb) {
+        step(ring, I1{}, Yes{}, I0{}, Yes{}, 0);
+        step(ring, I0{}, Yes{}, I0{}, No{}, 0);
+        advance();
+    }
+    step(ring, I1{}, No{}, I0{}, No{}, 0);
+    {
+        // O += P V with the last half (its first fragments were requested by the step before)
+        const auto sv = v_half(ring.a, 1);
+        static_for<8>([&](auto g_c) {
+            constexpr int g = decltype(g_c)::value;
+            constexpr int gp = g + kAhead;
+            if constexpr (gp < 8) {
+                v_frag.template read<0, gp>(sv, rV);
+                wait_shared_reads<kAhead * kReadsV>();
+            } else {
+                wait_shared_reads<(7 - g) * kReadsV>();
+            }
+            static_for<kQT>([&](auto c_c) { Output::template at<decltype(c_c)::value, g, 0>(rP[1], rV, rO); });
+        });
+    }
+
+    // ---- epilogue: O = O / l, to f16, through LDS for row-contiguous 16-byte stores
+    compute::settle_accumulators(rO);
+    typename Traits::RegOut out;
+#pragma unroll
+    for (int c = 0; c < kQT; ++c) {
+        float l_tot = l_run[c] + __shfl_xor(l_run[c], 16, 64);
+        l_tot += __shfl_xor(l_tot, 32, 64);
+        const float inv_l = 1.0f / l_tot;
+#pragma unroll
+        for (int dt = 0; dt < kDT; ++dt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) out(c, dt)(0, e) = __float2half(rO(c, dt)(0, e) * inv_l);
+    }
+    wait_group<0>();
+    __syncthreads();  // every wavefront is done with the K/V stages: the space is reused for O
+    typename Traits::SharedO sO(shm);
+    typename Traits::OutToShared to_shared;
+    typename Traits::OutToGlobal to_global;
+    typename Traits::GlobalO gO(Ob);
+    to_shared(out, sO);
+    __syncthreads();
+    to_global(sO, gO);
+}
+
+}  // namespace tiledcuda::kernels

@@ -98,11 +98,15 @@ typedef enum {
                                   instructions placed by hand, softmax of 32 keys interleaved with the MFMAs of the
                                   neighbouring 32; either V layout, head size 128, M % 64 == 0 (wavefronts of the
                                   last workgroup whose 64 queries lie beyond M idle), N % 64 == 0, N * 256 < 2^32 */
-    TCU_ATTN_TILE_WAVE64 = 5   /* the WAVE64 kernel composed from tile-library functors only (matrix instructions placed
+    TCU_ATTN_TILE_WAVE64 = 5,  /* the WAVE64 kernel composed from tile-library functors only (matrix instructions placed
                                   one by one with ScheduledGemm, interleaved 5-stage shared rings, fragment reads issued
                                   ahead with SharedToRegPieces / SharedToRegTrPieces); compile-time sequence lengths:
                                   (M, N) in {(2048, 2048), (512, 1024), (256, 640), (256, 320)}, head size 128, row-major
                                   V; results identical to WAVE64 bit for bit */
+    TCU_ATTN_WAVE64_K32 = 6    /* the WAVE64 design on v_mfma_f32_16x16x32_f16 (tile-library functors; twice the matrix
+                                  instructions, each contracting 32 indices: the chip sustains a higher clock on them);
+                                  row-major V, head size 128, M % 256 == 0, N % 64 == 0, N >= 320; results equal to
+                                  WAVE64 up to the summation order inside a matrix instruction */
 } tcu_attn_algo;
 
 /* Which LSTM step kernel to run (tcu_lstm_f16_algo). AUTO picks STREAMING where it is instantiated, else

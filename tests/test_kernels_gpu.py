@@ -861,6 +861,65 @@ def test_flash_attention_tile_wave64_is_wave64(tcu, oracle, device, batch, M, N)
     assert oracle.max_abs_err(host(out)[heads, :64], ref) <= (2e-2 if N == 640 else ABS_TOL)
 
 
+@pytest.mark.parametrize("batch,M,N", [(3, 256, 320), (8, 256, 640), (2, 512, 1024), (5, 768, 448), (64, 2048, 2048)])
+def test_flash_attention_wave64_k32(tcu, oracle, device, batch, M, N):
+    """The one-wavefront-per-SIMD design on the 16x16x32 matrix instruction (wave64_k32): against the oracle on whole
+    heads at small sizes and on a sample of rows at the benchmark size, and against the 32x32x16 kernel everywhere (same
+    arithmetic up to the order of the sums inside a matrix instruction); at 5 key blocks (the minimum), an odd number of
+    blocks, one and two rounds of workgroups, and with keys that force the rare re-basing path."""
+    import torch
+
+    D = 128
+    print(f"attention wave64_k32 b{batch} {M}x{N}", flush=True)
+    q = oracle.fill_normal(batch * M * D, 91).reshape(batch, M, D).astype(np.float32)
+    k = oracle.fill_normal(batch * N * D, 92).reshape(batch, N, D).astype(np.float32)
+    v = oracle.fill_normal(batch * N * D, 93).reshape(batch, N, D)
+    if N == 640:
+        qdir = q / np.linalg.norm(q, axis=-1, keepdims=True)
+        for pos, gain in ((0, 30.0), (200, 60.0), (225, 120.0), (300, 200.0), (639, 400.0)):
+            k[:, pos] = qdir[:, pos % M] * gain
+    q, k = q.astype(np.float16), k.astype(np.float16)
+    dq, dk, dv = dev(q, device), dev(k, device), dev(v, device)
+    ref_kernel = tcu.flash_attention(dq, dk, dv, algo="wave64")
+    out = torch.full_like(ref_kernel, float("nan"))
+    tcu.flash_attention(dq, dk, dv, out=out, algo="wave64_k32")
+    torch.cuda.synchronize()
+    tol = 2e-2 if N == 640 else ABS_TOL
+    assert torch.isfinite(out).all()
+    assert (out.float() - ref_kernel.float()).abs().max().item() <= tol
+    heads = [0, batch - 1]
+    rows = M if batch * M * N <= (1 << 21) else 64
+    ref = oracle.attention(np.ascontiguousarray(q[heads, :rows]), np.ascontiguousarray(k[heads]), np.ascontiguousarray(v[heads]),
+                           1.0 / math.sqrt(D))
+    assert oracle.max_abs_err(host(out)[heads, :rows], ref) <= tol
+    ref_tail = oracle.attention(np.ascontiguousarray(q[heads, M - 64:]), np.ascontiguousarray(k[heads]),
+                                np.ascontiguousarray(v[heads]), 1.0 / math.sqrt(D))
+    assert oracle.max_abs_err(host(out)[heads, M - 64:], ref_tail) <= tol
+
+
+@pytest.mark.parametrize("algo", ["wave64", "tile_wave64", "wave64_k32"])
+def test_flash_attention_wave64_with_cold_caches(tcu, oracle, device, algo):
+    """The one-wavefront-per-SIMD kernels request their first operand fragments of key block 1 only behind the barrier
+    that says every wavefront's quarter of the block has landed. (They once did so before it: right whenever the block
+    came from the L2 in time, wrong rows in a few heads when it did not.) Every launch here starts with the caches
+    evicted and is compared with the 8-wavefront kernel, which shares none of that code."""
+    import torch
+
+    B, S, D = 64, 2048, 128
+    print(f"attention {algo} with cold caches", flush=True)
+    g = torch.Generator(device="cpu").manual_seed(7)
+    q, k, v = (torch.randn(B, S, D, generator=g).half().to(device) for _ in range(3))
+    ref = tcu.flash_attention(q, k, v, algo="mfma32")
+    evict = torch.zeros(256 << 20, device=device)  # 1 GiB: larger than every cache level
+    for _ in range(12):
+        evict.add_(1.0)
+        out = torch.full_like(ref, float("nan"))
+        tcu.flash_attention(q, k, v, out=out, algo=algo)
+        torch.cuda.synchronize()
+        assert torch.isfinite(out).all()
+        assert (out.float() - ref.float()).abs().max().item() <= 1e-3
+
+
 def test_flash_attention_properties(tcu, oracle, device):
     """Size-independent properties: constant V, zero scale, joint permutation of keys/values."""
     import torch

@@ -40,7 +40,7 @@ GEMM_ALGOS = {"auto": 0, "global_reg": 1, "all_mem": 2, "pipelined": 3, "wave128
 TCU_V_COL_MAJOR = 0
 TCU_V_ROW_MAJOR = 1
 
-ATTN_ALGOS = {"auto": 0, "tile_library": 1, "mfma32": 2, "mfma32_fused": 3, "wave64": 4, "tile_wave64": 5}
+ATTN_ALGOS = {"auto": 0, "tile_library": 1, "mfma32": 2, "mfma32_fused": 3, "wave64": 4, "tile_wave64": 5, "wave64_k32": 6}
 LSTM_ALGOS = {"auto": 0, "tile_library": 1, "streaming": 2, "ragged": 3}
 B2B_ALGOS = {"auto": 0, "tile_library": 1, "resident": 2, "rows": 3, "tile_resident": 4}
 SCATTER_MODES = {"assign": 0, "add": 1}

@@ -7,6 +7,7 @@
 #include "kernels/b2b_gemm_fwd.hpp"
 #include "kernels/flash_attn_fwd.hpp"
 #include "kernels/flash_attn_tile_w64.hpp"
+#include "kernels/flash_attn_w64_k32.hpp"
 #include "kernels/flash_attn_w64.hpp"
 #include "kernels/gemm_pipelined.hpp"
 #include "kernels/gemm_ragged.hpp"
@@ -582,6 +583,20 @@ int fa_tile_w64_dispatch(const __half* Q, const __half* K, const __half* V, __ha
                                            "(M, N) in {(2048, 2048), (512, 1024), (256, 640), (256, 320)}");
 }
 
+/// The one-wavefront-per-SIMD kernel on the 16x16x32 instruction (tile-library functors, run-time M and N).
+int fa_w64_k32_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, int Kd,
+                        float scale, int v_layout, hipStream_t stream) {
+    using Traits = FlashW64K32Traits<__half, 128>;
+    if (Kd != 128 || v_layout != TCU_V_ROW_MAJOR)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel takes head size 128 and a row-major V");
+    if (M % Traits::kTM != 0 || N < Traits::kStages * Traits::kTN)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel needs M % 256 == 0 and N >= 320");
+    if ((long)N * 256 >= (1l << 32))
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel addresses a V block with 32-bit offsets");
+    return launch(&flash_attention_w64_k32<__half, Traits>, dim3((M / Traits::kTM) * batch), dim3(Traits::kThreads),
+                  Traits::kShmBytes, stream, Q, K, V, O, batch, M, N, scale);
+}
+
 template <int kD, bool kFused>
 int fa_fwd_by_rows(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
                    hipStream_t stream) {
@@ -596,10 +611,12 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     if (Kd != P) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs the query and value head sizes equal");
     if (M % 64 != 0 || N % 64 != 0) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention needs M % 64 == 0 and N % 64 == 0");
     if (algo != TCU_ATTN_AUTO && algo != TCU_ATTN_TILE_LIBRARY && algo != TCU_ATTN_MFMA32 &&
-        algo != TCU_ATTN_MFMA32_FUSED && algo != TCU_ATTN_WAVE64 && algo != TCU_ATTN_TILE_WAVE64)
+        algo != TCU_ATTN_MFMA32_FUSED && algo != TCU_ATTN_WAVE64 && algo != TCU_ATTN_TILE_WAVE64 &&
+        algo != TCU_ATTN_WAVE64_K32)
         return fail(TCU_ERR_INVALID_ARGUMENT, "unknown attention algo");
     if (v_layout != TCU_V_ROW_MAJOR && v_layout != TCU_V_COL_MAJOR) return fail(TCU_ERR_INVALID_ARGUMENT, "unknown v_layout");
     if (algo == TCU_ATTN_TILE_WAVE64) return fa_tile_w64_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
+    if (algo == TCU_ATTN_WAVE64_K32) return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
     if (algo == TCU_ATTN_WAVE64) {
         if (Kd != 128)
             return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel is instantiated for head size 128");
