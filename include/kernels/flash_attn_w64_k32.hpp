@@ -306,12 +306,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
             using I1 = std::integral_constant<int, 1>;
             using I2 = std::integral_constant<int, 2>;
             using I3 = std::integral_constant<int, 3>;
+            // Every matrix instruction is followed by its dose of vector work, in this order: the barriers between the
+            // two keep the compiler from pairing the matrix instructions up (two in a row leave the second waiting for
+            // the pipe with nothing else to issue, and the vector work behind them then runs with the pipe idle).
             // slot 0
             score(I0{});
+            __builtin_amdgcn_sched_barrier(0);
             x0 = exp2(sv4(0, 0));
             __builtin_amdgcn_sched_barrier(0);
             // slot 1: the second pair of the group before
             score(I1{});
+            __builtin_amdgcn_sched_barrier(0);
             if constexpr (g > 0) {
                 compute::convert_pair_here(x2, x3, reinterpret_cast<__half*>(pprev) + 2);
                 lh[(g - 1) / 2] += x3;
@@ -319,10 +324,12 @@ __global__ void __launch_bounds__(Traits::kThreads)
             __builtin_amdgcn_sched_barrier(0);
             // slot 2
             score(I2{});
+            __builtin_amdgcn_sched_barrier(0);
             x1 = exp2(sv4(0, 1));
             __builtin_amdgcn_sched_barrier(0);
             // slot 3
             score(I3{});
+            __builtin_amdgcn_sched_barrier(0);
             lh[sc] += x0;
             __builtin_amdgcn_sched_barrier(0);
             // slot 4 (with this wavefront's load g riding on the matrix instruction)
@@ -331,19 +338,23 @@ __global__ void __launch_bounds__(Traits::kThreads)
             } else {
                 Output::template at<0, g, 0>(rP[kNxt], rV, rO);
             }
+            __builtin_amdgcn_sched_barrier(0);
             x2 = exp2(sv4(0, 2));
             __builtin_amdgcn_sched_barrier(0);
             // slot 5
             Output::template at<1, g, 0>(rP[kNxt], rV, rO);
+            __builtin_amdgcn_sched_barrier(0);
             compute::convert_pair_here(x0, x1, reinterpret_cast<__half*>(pdst));
             lh[sc] += x1;
             __builtin_amdgcn_sched_barrier(0);
             // slot 6
             Output::template at<2, g, 0>(rP[kNxt], rV, rO);
+            __builtin_amdgcn_sched_barrier(0);
             x3 = exp2(sv4(0, 3));
             __builtin_amdgcn_sched_barrier(0);
             // slot 7
             Output::template at<3, g, 0>(rP[kNxt], rV, rO);
+            __builtin_amdgcn_sched_barrier(0);
             lh[sc] += x2;
             __builtin_amdgcn_sched_barrier(0);
         });
