@@ -305,6 +305,43 @@ struct SharedToRegPieces : public Base {
         __builtin_memcpy(dst(kI, kJ).mutable_data(), &r, sizeof(r));
     }
 
+    /// The same without an addition in front of every read (a vector addition directly in front of the LDS read that
+    /// takes its result stalls the wavefront for several cycles, and every instruction between two matrix
+    /// instructions costs issue time): bind() makes the kept offsets absolute addresses inside the view `src`, once;
+    /// read_bound<i, j, kBytes>() then reads fragment (i, j) of the view that lies kBytes further on (an immediate of the
+    /// instruction: a multiple of the swizzle's period in lines, below 64 KiB), and shift<i, j>(bytes) moves one
+    /// fragment's address on to another view (another stage of a ring) - one addition per fragment and move, placed
+    /// by the caller well ahead of the fragment's next read.
+    DEVICE void bind(const Shared& src) {
+        const unsigned int base = detail::shared_view_address(src);
+#pragma unroll
+        for (int i = 0; i < Reg::kRows; ++i)
+#pragma unroll
+            for (int j = 0; j < Reg::kCols; ++j) {
+                offset_[i][j] += base;
+                asm volatile("" : "+v"(offset_[i][j]));
+            }
+    }
+    template <int kI, int kJ, int kBytes = 0>
+    DEVICE void read_bound(Reg& dst) const {
+        read_bound_to<kI, kJ, kBytes>(dst(kI, kJ));
+    }
+    /// ... into any operand tile (a kernel that keeps only the fragments in flight, as a ring of a few tiles).
+    template <int kI, int kJ, int kBytes = 0>
+    DEVICE void read_bound_to(BaseTile& dst) const {
+        static_assert(kBytes >= 0 && kBytes < 65536 &&
+                          kBytes % ((Shared::kSwizzled ? Shared::Swizzle::kLinePeriod : 1) * Shared::kPitch * int(sizeof(DType))) == 0,
+                      "the immediate moves the view by whole periods of the swizzle");
+        f16x8 r;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(offset_[kI][kJ]), "n"(kBytes));
+        __builtin_memcpy(dst.mutable_data(), &r, sizeof(r));
+    }
+    template <int kI, int kJ>
+    DEVICE void shift(int bytes) {
+        offset_[kI][kJ] += static_cast<unsigned int>(bytes);
+        asm volatile("" : "+v"(offset_[kI][kJ]));
+    }
+
   private:
     unsigned int offset_[Reg::kRows][Reg::kCols];
 };
@@ -372,6 +409,38 @@ struct SharedToRegTrPieces : public Base {
                      : "v"(offset_[kJ] + detail::shared_view_address(src)), "n"(kOff0), "n"(kOff1));
         const f16x8 r = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         __builtin_memcpy(dst(kI, kJ).mutable_data(), &r, sizeof(r));
+    }
+
+    /// Absolute addresses, as in SharedToRegPieces: bind() once to a view, read_bound<i, j, kBytes>() reads operand tile
+    /// (i, j) of the view kBytes further on, shift<j>(bytes) moves the address kept for column j of operand tiles.
+    DEVICE void bind(const Shared& src) {
+        const unsigned int base = detail::shared_view_address(src);
+#pragma unroll
+        for (int j = 0; j < Reg::kCols; ++j) {
+            offset_[j] += base;
+            asm volatile("" : "+v"(offset_[j]));
+        }
+    }
+    template <int kI, int kJ, int kBytes = 0>
+    DEVICE void read_bound(Reg& dst) const {
+        read_bound_to<kI, kJ, kBytes>(dst(kI, kJ));
+    }
+    template <int kI, int kJ, int kBytes = 0>
+    DEVICE void read_bound_to(BaseTile& dst) const {
+        static_assert(kBytes >= 0 && kBytes % (kPeriod * kLineBytes) == 0, "the immediate moves the view by whole periods of the swizzle");
+        constexpr int kOff0 = kBytes + kI * BaseShape::kRows * kLineBytes, kOff1 = kOff0 + kPartRows * kLineBytes;
+        static_assert(kOff1 < 65536, "the immediate offset of an LDS read has 16 bits");
+        f16x4 lo, hi;
+        asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                     : "=&v"(lo), "=&v"(hi)
+                     : "v"(offset_[kJ]), "n"(kOff0), "n"(kOff1));
+        const f16x8 r = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        __builtin_memcpy(dst.mutable_data(), &r, sizeof(r));
+    }
+    template <int kJ>
+    DEVICE void shift(int bytes) {
+        offset_[kJ] += static_cast<unsigned int>(bytes);
+        asm volatile("" : "+v"(offset_[kJ]));
     }
 
   private:

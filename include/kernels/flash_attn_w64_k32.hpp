@@ -6,20 +6,23 @@
 //   through two interleaved 5-stage SharedRings filled by GlobalToSharedDirectPieces (one direct-to-LDS load riding on a
 //   matrix instruction at a time); S = Q Kᵀ and O += P V are tile products whose every instruction is placed by
 //   compute::ScheduledGemm::at<i, j, k>() (O and the Q operand pinned in AGPRs, the scores in VGPRs); operand fragments
-//   are requested three groups of instructions ahead with SharedToRegPieces (ds_read_b128, K) and SharedToRegTrPieces
-//   (ds_read_b64_tr_b16, V, in the order in which two 16 x 16 score accumulators hold their keys, so that the converted
-//   scores ARE the A operand of the second product) and awaited with wait_shared_reads<N>(); the softmax of 32 keys is
-//   sliced over the 64 matrix instructions of the neighbouring 32 - a v_exp_f32 behind every second one, the sums
-//   and conversions behind the others (compute::Exp2Raw, convert_pair_here); stages are handed over with
-//   wait_group_and_barrier_keep_reads<N>(); the output leaves through RegToSharedStorer / SharedToGlobalStorer.
+//   live in rings of four tiles and are requested three groups of instructions ahead through SharedToRegPieces
+//   (ds_read_b128, K) and SharedToRegTrPieces (ds_read_b64_tr_b16, V, in the order in which two 16 x 16 score
+//   accumulators hold their keys, so that the converted scores ARE the A operand of the second product) with addresses
+//   bound to the ring stage (bind / read_bound_to / shift: no addition in front of a read), awaited with
+//   wait_shared_reads<N>(); the softmax of 32 keys is sliced over the 64 matrix instructions of the neighbouring 32 -
+//   a v_exp_f32 behind every second one, the sums and conversions behind the others (compute::Exp2Raw,
+//   convert_pair_here); stages are handed over with wait_group_and_barrier_keep_reads<N>(); the last three steps fetch
+//   what the next workgroup on the XCD will ask for first; the output leaves through RegToSharedStorer /
+//   SharedToGlobalStorer.
 // Why a second instruction shape: under the chip's power limit the core clock follows the work, and a stream of
 // 16x16x32 instructions sustains a clock about an eighth higher than the same arithmetic in 32x32x16 instructions
-// (half the accumulator traffic per multiply-add). A wavefront alone on its SIMD has issue slots to spare for twice the
-// number of instructions as long as the vector work between them stays in doses of one transcendental or two plain
-// operations.
+// (half the accumulator traffic per multiply-add). The price is issue time: what a wavefront alone on its SIMD places
+// between two 16-cycle matrix instructions is not free (see the comment at `step`), so the schedule counts slots.
 // Numerics: as flash_attention_fwd_w64 (Q pre-multiplied by scale * log2 e in f16, scores relative to a reference
 // maximum that moves only when a partial sum could leave f16 range, f32 sums and output); the sums inside a matrix
-// instruction cover 32 instead of 16 indices, so results differ from that kernel in the last bits.
+// instruction cover 32 instead of 16 indices and the final division is a reciprocal and a product, so results differ
+// from that kernel in the last bits.
 // Requirements: head size 128, row-major V, M % 256 == 0, N % 64 == 0, N >= 320 (Q passes through two ring stages
 // before the fifth block needs them). M, N and the batch count are run-time values.
 #pragma once
@@ -74,21 +77,23 @@ struct FlashW64K32Traits {
 
     // register tiles of one wavefront (64 queries)
     using RegQ = RegTile<typename Shape::TileA, tl::RowMajor<kQTiles, kDSteps>>;     // A of S = Q Kᵀ, in AGPRs
-    using RegK = RegTile<typename Shape::TileB, tl::ColMajor<kDSteps, kKeyTiles>>;   // B of S: the 8 fragments of a half
-    using RegS = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, kKeyTiles>>; // scores of 32 keys
+    using RegK = RegTile<typename Shape::TileB, tl::ColMajor<kDSteps, 1>>;           // B of S: a ring of 4 fragments
+    using RegKAll = RegTile<typename Shape::TileB, tl::ColMajor<kDSteps, kKeyTiles>>; // what the fragment loader addresses
+    using RegS = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, 1>>;         // scores of 16 keys
     using RegM = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, 1>>;         // where the score sums start
     using RegP = RegTile<typename Shape::TileA, tl::RowMajor<kQTiles, 1>>;           // probabilities: A of O += P V
-    using RegV = RegTile<typename Shape::TileB, tl::ColMajor<1, kDTiles>>;           // B of O += P V
-    using RegO = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, kDTiles>>;   // in AGPRs
+    using RegV = RegTile<typename Shape::TileB, tl::ColMajor<1, 4>>;                 // B of O += P V: a ring of 4 fragments
+    using RegVAll = RegTile<typename Shape::TileB, tl::ColMajor<1, kDTiles>>;
+    using RegO = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, 4>>;         // half of the head size; in AGPRs
     using RegOut = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kQTiles, kDTiles>>;
 
     using QLoader = GlobalToSharedDirectLoader<SharedQ, WarpLayout>;
     using QFragments = SharedToRegLoader<RegQ, WarpLayout, WarpReuse::kRowReuseCont>;
     using PiecesK = GlobalToSharedDirectPieces<SharedK, WarpLayout, kD>;
     using PiecesV = GlobalToSharedDirectPieces<SharedV, WarpLayout, kD>;
-    using KFragmentsNow = SharedToRegLoader<RegK, WarpLayout, WarpReuse::kColReuseCont>;
-    using KFragments = SharedToRegPieces<RegK, SharedKHalf, WarpLayout, WarpReuse::kColReuseCont>;
-    using VFragments = SharedToRegTrPieces<RegV, SharedVHalf, WarpLayout, WarpReuse::kColReuseCont, true>;
+    using KFragmentsNow = SharedToRegLoader<RegKAll, WarpLayout, WarpReuse::kColReuseCont>;
+    using KFragments = SharedToRegPieces<RegKAll, SharedKHalf, WarpLayout, WarpReuse::kColReuseCont>;
+    using VFragments = SharedToRegTrPieces<RegVAll, SharedVHalf, WarpLayout, WarpReuse::kColReuseCont, true>;
     using Scores = compute::ScheduledGemm<RegQ, RegK, RegS, compute::RegFile::kVgpr, compute::RegFile::kAgpr>;
     using Output = compute::ScheduledGemm<RegP, RegV, RegO, compute::RegFile::kAgpr, compute::RegFile::kVgpr>;
     using OutToShared = RegToSharedStorer<RegOut, WarpLayout>;
@@ -179,15 +184,16 @@ __global__ void __launch_bounds__(Traits::kThreads)
         compute::pin_tiles<compute::RegFile::kAgpr>(rQ);
     }
 
-    RegO rO;
-    compute::clear_pinned(rO);
+    RegO rO[2];     // d tiles 0..3 and 4..7
+    compute::clear_pinned(rO[0]);
+    compute::clear_pinned(rO[1]);
 
-    RegS rS[2];     // score tiles of two consecutive halves, relative to the reference maximum
+    RegS rS[2][2];  // [half buffer][key tile]: score tiles of two consecutive halves, relative to the reference maximum
     RegP rP[2];     // their probabilities
     RegM neg_max;   // minus the reference maximum of this lane's query of each tile, in all 4 slots
     float m_run[kQT], l_run[kQT];
-    RegK rK;        // fragments in flight / in use: (d-step, key tile)
-    RegV rV;        // (0, d tile)
+    RegK rK;        // ring of the fragments in flight / in use: fragment g lives in tile g % 4
+    RegV rV;
 
     compute::Exp2Raw<float> exp2;
     using f16x2 = _Float16 __attribute__((ext_vector_type(2)));
@@ -203,21 +209,23 @@ __global__ void __launch_bounds__(Traits::kThreads)
         constexpr int kBuf = decltype(buf_c)::value;
         typename Traits::KFragmentsNow read_k;
         const auto sk = k_half(stage, t);
-        RegK kf;
+        typename Traits::RegKAll kf;
         read_k.load_one(sk, kf, 0, 0);
         static_for<8>([&](auto g_c) {
             constexpr int g = decltype(g_c)::value, ds = g % 4, kt = g / 4;
             if constexpr (g + 1 < 8) read_k.load_one(sk, kf, (g + 1) % 4, (g + 1) / 4);
+            RegK one;
+            one(ds, 0) = kf(ds, kt);
             static_for<kQT>([&](auto c_c) {
                 constexpr int c = decltype(c_c)::value;
-                if constexpr (ds == 0) Scores::template at_from<c, kt, 0>(rQ, kf, rS[kBuf], neg_max(c, 0));
-                else Scores::template at<c, kt, ds>(rQ, kf, rS[kBuf]);
+                if constexpr (ds == 0) Scores::template at_from<c, 0, 0>(rQ, one, rS[kBuf][kt], neg_max(c, 0));
+                else Scores::template at<c, 0, ds>(rQ, one, rS[kBuf][kt]);
             });
             issue(block_load(load_block, load_block, g));
         });
     };
 
-    // probabilities of one score tile's 4 keys: to f16, into slots 4 kt .. 4 kt + 3 of the A operand, and their sum
+    // probabilities of one score tile's 4 keys: to f16, into 4 slots of the A operand, and their sum
     auto tile_softmax_now = [&](const BaseTileRowMajor<float>& sc, float shift, _Float16* dst) {
         const float p0 = exp2(sc(0, 0) - shift), p1 = exp2(sc(0, 1) - shift);
         const float p2 = exp2(sc(0, 2) - shift), p3 = exp2(sc(0, 3) - shift);
@@ -236,169 +244,220 @@ __global__ void __launch_bounds__(Traits::kThreads)
     compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
     scores_only(0, 0, std::integral_constant<int, 0>{}, 1);
     asm volatile("s_nop 15\n\ts_nop 3");
-    compute::pin_tiles<compute::RegFile::kVgpr>(rS[0]);
+    compute::pin_tiles<compute::RegFile::kVgpr>(rS[0][0]);
+    compute::pin_tiles<compute::RegFile::kVgpr>(rS[0][1]);
 #pragma unroll
     for (int c = 0; c < kQT; ++c) {
-        float mx = rS[0](c, 0)(0, 0);
+        float mx = rS[0][0](c, 0)(0, 0);
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, rS[0](c, kt)(0, e));
+            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, rS[0][kt](c, 0)(0, e));
         mx = row_max(mx);
         m_run[c] = mx;
         _Float16* p = reinterpret_cast<_Float16*>(rP[0](c, 0).mutable_data());
-        l_run[c] = tile_softmax_now(rS[0](c, 0), mx, p) + tile_softmax_now(rS[0](c, 1), mx, p + 4);
+        l_run[c] = tile_softmax_now(rS[0][0](c, 0), mx, p) + tile_softmax_now(rS[0][1](c, 0), mx, p + 4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) neg_max(c, 0)(0, e) = -mx;
     }
     compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
     scores_only(0, 1, std::integral_constant<int, 1>{}, 2);
 
-    // ---- one pipelined step on half i: softmax of half i (rS[kCur] -> rP[kCur]), scores of half i + 1 into rS[kNxt]
-    // (if kQk), O += P V with half i - 1 (rP[kNxt]). ring: stages of blocks J, J + 1, J + 2 and of the block being
-    // loaded. kLoads: 0 none, 1 block `load_block`.
-    // A step is 8 groups of 8 matrix instructions: group g multiplies K fragment g (d-step g % 4 of key tile g / 4) with
-    // the 4 query tiles, then V fragment g (d tile g) with the 4 probability tiles, and takes score tile
-    // (g / 2, g % 2) of half i through the softmax. Fragments are requested kAhead groups before their instructions,
-    // across step boundaries.
     struct Stages {
         int a, b, c, load;
     };
     constexpr int kAhead = 3;
     constexpr int kReadsV = 2, kReadsQk = 3;  // LDS read instructions per group
+    constexpr int kHalfBytes = Traits::kHalf * kD * int(sizeof(InType));  // between the halves of a K or V block
+    constexpr int kStageBytes = 2 * Traits::kBlockNumel * int(sizeof(InType));
 
+    // The workgroup that follows this one on the XCD (ids congruent mod 8 share an XCD: id + 256) starts with a cold
+    // burst: its 256 query rows and the first block of its item's K and V, 96 KiB of consecutive memory. The last three
+    // steps of this workgroup have no ring loads left to issue and fetch those instead (kLoads == 2, 3), into a ring
+    // stage that is vacant (the data is discarded: the point is that the lines are in this XCD's L2 when the next
+    // workgroup asks). Without a successor the workgroup fetches its own again.
+    const char *warm_src = nullptr, *warm_src_v = nullptr;  // 8 KiB of consecutive memory per step and wavefront
+    unsigned int warm_lds = 0;
+    const unsigned int lane_off16 = lane_id() * 16u;
+    int nhead = head_i, nqb = q_block;
+    {
+        const unsigned int nid = blockIdx.x + 256;
+        if (nid < gridDim.x) {
+            if (batch % 8 == 0) {
+                const int xcd = nid & 7, rest = nid >> 3;
+                nqb = rest % q_blocks;
+                nhead = (rest / q_blocks) * 8 + xcd;
+            } else {
+                nqb = nid % q_blocks;
+                nhead = nid / q_blocks;
+            }
+        }
+    }
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave_id());
+
+    // A fragment's address moves on to the next ring stage between its read of half 1 of a block and its read of half 0
+    // of the next: fragments 0..2 (requested at the end of a step for the next one) behind the first step of a
+    // block-iteration, fragments 3..7 behind the second.
+    auto shift_fragments = [&](const Stages& ring, auto first_c, auto last_c) {
+        const int dK = (ring.c - ring.b) * kStageBytes, dV = (ring.b - ring.a) * kStageBytes;
+        static_for<decltype(last_c)::value - decltype(first_c)::value>([&](auto i_c) {
+            constexpr int f = decltype(first_c)::value + decltype(i_c)::value;
+            k_frag.template shift<f % 4, f / 4>(dK);
+            v_frag.template shift<f>(dV);
+        });
+    };
+
+    // ---- one pipelined step on half i: softmax of half i (rS[kCur] -> rP[kCur]), scores of half i + 1 into rS[kNxt]
+    // (if kQk), O += P V with half i - 1 (rP[kNxt]). ring: stages of blocks J, J + 1, J + 2 and of the block being
+    // loaded. kLoads: 0 none, 1 block `load_block`, 2 / 3 the warm-up loads.
+    // A step is 8 groups of 8 matrix instructions: group g multiplies K fragment g (d-step g % 4 of key tile g / 4) with
+    // the 4 query tiles, then V fragment g (d tile g) with the 4 probability tiles, and takes score tile (g / 2, g % 2)
+    // of half i through the softmax. The fragments of group g + kAhead are requested inside group g (K behind the
+    // fourth, V behind the eighth matrix instruction), through addresses bound to the ring stage (no addition per
+    // read). What goes between two matrix instructions is measured, not guessed: every matrix instruction is followed
+    // by its dose in this order (the barriers keep the compiler from pairing the matrix instructions up), and the doses
+    // come in pairs of issue slots - a v_exp_f32 counts as two, everything else as one; a pair costs 4 cycles on top of
+    // the matrix instruction's 16, a single slot costs as much, three or four cost 8.
     auto step = [&](const Stages& ring, auto cur_c, auto qk_c, auto loads_c, auto next_qk_c, int load_block) {
         constexpr int kCur = decltype(cur_c)::value, kNxt = kCur ^ 1;
         constexpr bool kQk = decltype(qk_c)::value, kNextQk = decltype(next_qk_c)::value;
         constexpr int kLoads = decltype(loads_c)::value;
-        // K of half i + 1, V of half i - 1, K of half i + 2, V of half i
-        const auto sk = kCur == 1 ? k_half(ring.b, 0) : k_half(ring.b, 1);
-        const auto sv = v_half(ring.a, kNxt);
-        const auto sk_next = kCur == 1 ? k_half(ring.b, 1) : k_half(ring.c, 0);
-        const auto sv_next = v_half(kCur == 1 ? ring.a : ring.b, kCur);
         float lh[kQT] = {0.f, 0.f, 0.f, 0.f};
         float x0 = 0.f, x1 = 0.f, x2 = 0.f, x3 = 0.f;
         static_for<8>([&](auto g_c) {
             constexpr int g = decltype(g_c)::value;
-            constexpr int gp = g + kAhead;
-            if constexpr (gp < 8) {
-                if constexpr (kQk) k_frag.template read<gp % 4, gp / 4>(sk, rK);
-                v_frag.template read<0, gp>(sv, rV);
-                wait_shared_reads<kAhead * (kQk ? kReadsQk : kReadsV)>();
-            } else {
-                if constexpr (kNextQk) k_frag.template read<(gp - 8) % 4, (gp - 8) / 4>(sk_next, rK);
-                v_frag.template read<0, gp - 8>(sv_next, rV);
-                wait_shared_reads<(7 - g) * (kQk ? kReadsQk : kReadsV) + (gp - 7) * (kNextQk ? kReadsQk : kReadsV)>();
-            }
+            constexpr int gp = g + kAhead, f = gp % 8;
+            // the fragments of group g + kAhead: halves 0 of the blocks in the first step of a block-iteration
+            // (kCur == 1) until the step's end, halves 1 afterwards
+            constexpr int kImm = ((gp < 8) == (kCur == 1)) ? 0 : kHalfBytes;
+            constexpr bool kReadK = gp < 8 ? kQk : kNextQk;
+            // reads in flight that are younger than the fragments of this group and the next, at the top of the group
+            // (the requests of this group are not yet issued): one wait per two groups
+            constexpr int kPerGroup = kQk ? kReadsQk : kReadsV, kPerGroupNext = kNextQk ? kReadsQk : kReadsV;
+            constexpr int kYounger = gp < 8 ? (kAhead - 1) * kPerGroup : (7 - g) * kPerGroup + (gp - 8) * kPerGroupNext;
+            if constexpr (g % 2 == 0) wait_shared_reads<kYounger - kPerGroup>();
             constexpr int ds = g % 4, kt = g / 4;   // the K fragment of this group
             constexpr int sc = g / 2, st = g % 2;   // the score tile of half i this group takes through the softmax
-            const auto& sv4 = rS[kCur](sc, st);
+            const auto& sv4 = rS[kCur][st](sc, 0);
             _Float16* pdst = reinterpret_cast<_Float16*>(rP[kCur](sc, 0).mutable_data()) + 4 * st;
             _Float16* pprev = reinterpret_cast<_Float16*>(rP[kCur]((g + 7) % 8 / 2, 0).mutable_data()) + 4 * ((g + 7) % 2);
             auto score = [&](auto c_c) {
                 constexpr int c = decltype(c_c)::value;
                 if constexpr (kQk) {
-                    if constexpr (ds == 0) Scores::template at_from<c, kt, 0>(rQ, rK, rS[kNxt], neg_max(c, 0));
-                    else Scores::template at<c, kt, ds>(rQ, rK, rS[kNxt]);
+                    if constexpr (ds == 0) Scores::template at_from<c, 0, 0>(rQ, rK, rS[kNxt][kt], neg_max(c, 0));
+                    else Scores::template at<c, 0, ds>(rQ, rK, rS[kNxt][kt]);
                 }
             };
             using I0 = std::integral_constant<int, 0>;
             using I1 = std::integral_constant<int, 1>;
             using I2 = std::integral_constant<int, 2>;
             using I3 = std::integral_constant<int, 3>;
-            // Every matrix instruction is followed by its dose of vector work, in this order: the barriers between the
-            // two keep the compiler from pairing the matrix instructions up (two in a row leave the second waiting for
-            // the pipe with nothing else to issue, and the vector work behind them then runs with the pipe idle).
-            // slot 0
             score(I0{});
             __builtin_amdgcn_sched_barrier(0);
             x0 = exp2(sv4(0, 0));
             __builtin_amdgcn_sched_barrier(0);
-            // slot 1: the second pair of the group before
             score(I1{});
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (g > 0) {
+            if constexpr (g > 0) {  // the second pair of the group before
                 compute::convert_pair_here(x2, x3, reinterpret_cast<__half*>(pprev) + 2);
                 lh[(g - 1) / 2] += x3;
             }
             __builtin_amdgcn_sched_barrier(0);
-            // slot 2
             score(I2{});
             __builtin_amdgcn_sched_barrier(0);
             x1 = exp2(sv4(0, 1));
             __builtin_amdgcn_sched_barrier(0);
-            // slot 3
             score(I3{});
             __builtin_amdgcn_sched_barrier(0);
             lh[sc] += x0;
+            if constexpr (kReadK) k_frag.template read_bound_to<f % 4, f / 4, kImm>(rK(f % 4, 0));
             __builtin_amdgcn_sched_barrier(0);
-            // slot 4 (with this wavefront's load g riding on the matrix instruction)
             if constexpr (kLoads == 1) {
-                Output::template at<0, g, 0>(rP[kNxt], rV, rO, block_load(ring.load, load_block, g));
+                Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4], block_load(ring.load, load_block, g));
+            } else if constexpr (kLoads == 2 || kLoads == 3) {
+                Output::template at<0, g % 4, 0>(
+                    rP[kNxt], rV, rO[g / 4],
+                    DirectLoad{lane_off16, (kLoads == 3 && g >= 4 ? warm_src_v : warm_src) + g * 1024, warm_lds});
             } else {
-                Output::template at<0, g, 0>(rP[kNxt], rV, rO);
+                Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
             }
             __builtin_amdgcn_sched_barrier(0);
             x2 = exp2(sv4(0, 2));
             __builtin_amdgcn_sched_barrier(0);
-            // slot 5
-            Output::template at<1, g, 0>(rP[kNxt], rV, rO);
+            Output::template at<1, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
             __builtin_amdgcn_sched_barrier(0);
             compute::convert_pair_here(x0, x1, reinterpret_cast<__half*>(pdst));
             lh[sc] += x1;
             __builtin_amdgcn_sched_barrier(0);
-            // slot 6
-            Output::template at<2, g, 0>(rP[kNxt], rV, rO);
+            Output::template at<2, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
             __builtin_amdgcn_sched_barrier(0);
             x3 = exp2(sv4(0, 3));
             __builtin_amdgcn_sched_barrier(0);
-            // slot 7
-            Output::template at<3, g, 0>(rP[kNxt], rV, rO);
+            Output::template at<3, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
             __builtin_amdgcn_sched_barrier(0);
             lh[sc] += x2;
+            v_frag.template read_bound_to<0, f, kImm>(rV(0, f % 4));
             __builtin_amdgcn_sched_barrier(0);
         });
         lh[kQT - 1] += x3;
         compute::convert_pair_here(x2, x3, reinterpret_cast<__half*>(rP[kCur](kQT - 1, 0).mutable_data()) + 6);
-        // no probability of this half can have left f16 range while its sum stays below 2^14
+        // No probability of this half can have left f16 range while its sum stays below 2^14. The comparison first, then
+        // work that does not depend on it, then the branch: the scalar unit sees the result of a vector comparison only
+        // some 20 cycles after it was issued.
         constexpr float kLimit = 16384.f;
-        if (__any(!(fmaxf(fmaxf(lh[0], lh[1]), fmaxf(lh[2], lh[3])) <= kLimit))) {
+        unsigned long long over = __ballot(!(fmaxf(fmaxf(lh[0], lh[1]), fmaxf(lh[2], lh[3])) <= kLimit));
+        asm volatile("" : "+s"(over));
+        float l_before[kQT];  // (the half's sums may be infinite when the branch is taken: kept apart)
+#pragma unroll
+        for (int c = 0; c < kQT; ++c) {
+            l_before[c] = l_run[c];
+            l_run[c] += lh[c];
+        }
+        if constexpr (kCur == 1) shift_fragments(ring, std::integral_constant<int, 0>{}, std::integral_constant<int, 3>{});
+        else shift_fragments(ring, std::integral_constant<int, 3>{}, std::integral_constant<int, 8>{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (__builtin_expect(over != 0, 0)) {
             // rare path: move the reference maxima, rescale, re-bias the scores already computed, recompute
             asm volatile("s_nop 15\n\ts_nop 3");
-            if constexpr (kQk) compute::pin_tiles<compute::RegFile::kVgpr>(rS[kNxt]);
-            compute::pin_tiles<compute::RegFile::kAgpr>(rO);
+            if constexpr (kQk) {
+                compute::pin_tiles<compute::RegFile::kVgpr>(rS[kNxt][0]);
+                compute::pin_tiles<compute::RegFile::kVgpr>(rS[kNxt][1]);
+            }
+            compute::pin_tiles<compute::RegFile::kAgpr>(rO[0]);
+            compute::pin_tiles<compute::RegFile::kAgpr>(rO[1]);
 #pragma unroll
             for (int c = 0; c < kQT; ++c) {
-                float mx = rS[kCur](c, 0)(0, 0);
+                float mx = rS[kCur][0](c, 0)(0, 0);
 #pragma unroll
                 for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) mx = fmaxf(mx, rS[kCur](c, kt2)(0, e));
+                    for (int e = 0; e < 4; ++e) mx = fmaxf(mx, rS[kCur][kt2](c, 0)(0, e));
                 mx = row_max(mx);
                 const float shift = mx > 8.0f ? mx : 0.f;
                 const float alpha = exp2(-shift);
                 m_run[c] += shift;
-                l_run[c] *= alpha;
 #pragma unroll
-                for (int dt = 0; dt < kDT; ++dt)
+                for (int h = 0; h < 2; ++h)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) rO(c, dt)(0, e) *= alpha;
+                    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) rO[h](c, dt)(0, e) *= alpha;
                 if constexpr (kQk) {
 #pragma unroll
                     for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) rS[kNxt](c, kt2)(0, e) -= shift;
+                        for (int e = 0; e < 4; ++e) rS[kNxt][kt2](c, 0)(0, e) -= shift;
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) neg_max(c, 0)(0, e) = -m_run[c];
                 _Float16* p = reinterpret_cast<_Float16*>(rP[kCur](c, 0).mutable_data());
-                lh[c] = tile_softmax_now(rS[kCur](c, 0), shift, p) + tile_softmax_now(rS[kCur](c, 1), shift, p + 4);
+                const float lsum = tile_softmax_now(rS[kCur][0](c, 0), shift, p) + tile_softmax_now(rS[kCur][1](c, 0), shift, p + 4);
+                l_run[c] = l_before[c] * alpha + lsum;
             }
             compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
-            compute::pin_tiles<compute::RegFile::kAgpr>(rO);
+            compute::pin_tiles<compute::RegFile::kAgpr>(rO[0]);
+            compute::pin_tiles<compute::RegFile::kAgpr>(rO[1]);
         }
-#pragma unroll
-        for (int c = 0; c < kQT; ++c) l_run[c] += lh[c];
         __builtin_amdgcn_sched_barrier(0);
     };
 
@@ -421,10 +480,12 @@ __global__ void __launch_bounds__(Traits::kThreads)
         wait_group_and_barrier_keep_reads<0>();
         // first fragments of step 1: K of half 2 (block 1), V of half 0 - behind the barrier: block 1 is complete only
         // when every wavefront's pieces of it have landed
+        k_frag.bind(k_half(1, 0));
+        v_frag.bind(v_half(0, 0));
         static_for<kAhead>([&](auto a_c) {
             constexpr int a = decltype(a_c)::value;
-            k_frag.template read<a % 4, a / 4>(k_half(1, 0), rK);
-            v_frag.template read<0, a>(v_half(0, 0), rV);
+            k_frag.template read_bound_to<a % 4, a / 4>(rK(a % 4, 0));
+            v_frag.template read_bound_to<0, a>(rV(0, a % 4));
         });
         Stages first = ring;
         first.load = 3;
@@ -432,6 +493,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         step(ring, I0{}, Yes{}, I1{}, Yes{}, 4);
         advance();
     }
+    // (left alone, the compiler unrolls these loops and the longer live ranges cost registers the kernel does not have)
 #pragma unroll 1
     for (; J + 4 < nb; advance()) {
         wait_group_and_barrier_keep_reads<8>();
@@ -444,43 +506,60 @@ __global__ void __launch_bounds__(Traits::kThreads)
         step(ring, I1{}, Yes{}, I0{}, Yes{}, 0);
         step(ring, I0{}, Yes{}, I0{}, Yes{}, 0);
     }
+    // the last three steps carry the warm-up loads: 16 KiB of the successor's query rows per wavefront in two steps, then
+    // 4 KiB each of its first K and V block
+    {
+        using lds_cptr = __attribute__((address_space(3))) const void*;
+        warm_lds = static_cast<unsigned int>(reinterpret_cast<uintptr_t>((lds_cptr)(ringK[ring.c].data()))) + wave_u * 1024u;
+    }
+    const char* next_q = reinterpret_cast<const char*>(dQ + (size_t(nhead) * kM + size_t(nqb) * Traits::kTM) * kD) + wave_u * 16384;
+    using Warm = std::integral_constant<int, 2>;
+    using WarmKV = std::integral_constant<int, 3>;
     if (J + 1 < nb) {
-        step(ring, I1{}, Yes{}, I0{}, Yes{}, 0);
-        step(ring, I0{}, Yes{}, I0{}, No{}, 0);
+        warm_src = next_q;
+        step(ring, I1{}, Yes{}, Warm{}, Yes{}, 0);
+        warm_src = next_q + 8192;
+        step(ring, I0{}, Yes{}, Warm{}, No{}, 0);
         advance();
     }
-    step(ring, I1{}, No{}, I0{}, No{}, 0);
+    warm_src = reinterpret_cast<const char*>(dK + size_t(nhead) * kN * kD) + wave_u * 4096;
+    warm_src_v = reinterpret_cast<const char*>(dV + size_t(nhead) * kN * kD) + wave_u * 4096 - 4096;  // its loads are 4..7
+    step(ring, I1{}, No{}, WarmKV{}, No{}, 0);
     {
         // O += P V with the last half (its first fragments were requested by the step before)
-        const auto sv = v_half(ring.a, 1);
         static_for<8>([&](auto g_c) {
             constexpr int g = decltype(g_c)::value;
             constexpr int gp = g + kAhead;
             if constexpr (gp < 8) {
-                v_frag.template read<0, gp>(sv, rV);
+                v_frag.template read_bound_to<0, gp, kHalfBytes>(rV(0, gp % 4));
                 wait_shared_reads<kAhead * kReadsV>();
             } else {
                 wait_shared_reads<(7 - g) * kReadsV>();
             }
-            static_for<kQT>([&](auto c_c) { Output::template at<decltype(c_c)::value, g, 0>(rP[1], rV, rO); });
+            static_for<kQT>([&](auto c_c) { Output::template at<decltype(c_c)::value, g % 4, 0>(rP[1], rV, rO[g / 4]); });
         });
     }
 
-    // ---- epilogue: O = O / l, to f16, through LDS for row-contiguous 16-byte stores
-    compute::settle_accumulators(rO);
+    // ---- epilogue: O = O / l, to f16, through LDS for row-contiguous 16-byte stores (8-byte stores straight from the
+    // accumulator layout were measured: three times slower)
+    compute::settle_accumulators(rO[0]);
+    compute::settle_accumulators(rO[1]);
     typename Traits::RegOut out;
 #pragma unroll
     for (int c = 0; c < kQT; ++c) {
         float l_tot = l_run[c] + __shfl_xor(l_run[c], 16, 64);
         l_tot += __shfl_xor(l_tot, 32, 64);
-        const float inv_l = 1.0f / l_tot;
+        const float inv_l = __builtin_amdgcn_rcpf(l_tot);
 #pragma unroll
-        for (int dt = 0; dt < kDT; ++dt)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) out(c, dt)(0, e) = __float2half(rO(c, dt)(0, e) * inv_l);
+        for (int dt = 0; dt < kDT; ++dt) {
+            const auto& o = rO[dt / 4](c, dt % 4);
+            __half* dst = reinterpret_cast<__half*>(out(c, dt).mutable_data());
+            compute::convert_pair_here(o(0, 0) * inv_l, o(0, 1) * inv_l, dst);
+            compute::convert_pair_here(o(0, 2) * inv_l, o(0, 3) * inv_l, dst + 2);
+        }
     }
     wait_group<0>();
-    __syncthreads();  // every wavefront is done with the K/V stages: the space is reused for O
+    __syncthreads();  // every wavefront is done with the K/V stages (and its warm-up loads have landed): reused for O
     typename Traits::SharedO sO(shm);
     typename Traits::OutToShared to_shared;
     typename Traits::OutToGlobal to_global;

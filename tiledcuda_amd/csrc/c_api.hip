@@ -627,7 +627,7 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
         if (Kd != 128 && Kd != 64) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
         // long sequences with enough query blocks to fill the chip: the kernel with 64 queries per wavefront
         if (algo == TCU_ATTN_AUTO && Kd == 128 && M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 128)
-            return launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream);
+            return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
         if (algo == TCU_ATTN_MFMA32)
             return Kd == 128 ? fa_fwd_by_rows<128, false>(Q, K, V, O, batch, M, N, scale, stream)
                              : fa_fwd_by_rows<64, false>(Q, K, V, O, batch, M, N, scale, stream);
