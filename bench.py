@@ -297,7 +297,7 @@ def main():
                                 "speed_vs_torch_sdpa": ms_sdpa / ms_again,
                                 "method": "torch.nn.functional.scaled_dot_product_attention on the same tensors, "
                                           "30 untimed + 20 timed launches each"}
-        configs.append({"name": "flash_attn_fwd_b4_h16_s2048_d128", "kernel": "flash_attention_fwd_w64<128>", "ms": ms,
+        configs.append({"name": "flash_attn_fwd_b4_h16_s2048_d128", "kernel": "flash_attention_w64_k32<128>", "ms": ms,
                         "first_launches_us": ms_first * 1e3, "conditioning_launches": 200,
                         "tflops": flops / (ms * 1e-3) / 1e12,
                         "frac_mfma_peak": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, "max_abs_err": err})
@@ -311,7 +311,7 @@ def main():
         err_long = oracle.max_abs_err(dol.reshape(Hl, Sl, D)[3, 4096:4160].float().cpu().numpy(),
                                       oracle.attention(ql[3], kl[3], vl[3], scale, rows=(4096, 4160))[4096:4160])
         flops_long = 4.0 * Hl * Sl * Sl * D
-        configs.append({"name": "flash_attn_fwd_b1_h32_s8192_d128_longer_sequence", "kernel": "flash_attention_fwd_w64<128>",
+        configs.append({"name": "flash_attn_fwd_b1_h32_s8192_d128_longer_sequence", "kernel": "flash_attention_w64_k32<128>",
                         "ms": ms_long, "tflops": flops_long / (ms_long * 1e-3) / 1e12,
                         "frac_mfma_peak": flops_long / (ms_long * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, "max_abs_err": err_long})
         del dql, dkl, dvl, dol
@@ -447,6 +447,11 @@ def main():
             configs.append({"name": "flash_attn_fwd_b4_h16_s2048_d128_tile_api_composition", "kernel": "flash_attention_tile_w64",
                             "ms": ms_t, "tflops": flops_attn / (ms_t * 1e-3) / 1e12, "hand_indexed_ms": ms_r,
                             "speed_vs_hand_indexed": ms_r / ms_t})
+            # the same design on the two f16 matrix instructions, interleaved: 32x32x16 (hand-indexed) against 16x16x32
+            ms_32, ms_16 = pair(lambda: tcu.flash_attention(dq, dk, dv, out=do, algo="wave64"),
+                                lambda: tcu.flash_attention(dq, dk, dv, out=do, algo="wave64_k32"), 40, 100)
+            configs.append({"name": "flash_attn_fwd_b4_h16_s2048_d128_by_matrix_instruction", "kernel": "flash_attention_w64_k32 / flash_attention_fwd_w64",
+                            "ms_16x16x32": ms_16, "ms_32x32x16": ms_32, "speed_16x16x32_vs_32x32x16": ms_32 / ms_16})
         dCt = torch.empty_like(dC)
         ms_r, ms_t = pair(lambda: tcu.gemm(dA, dB, out=dCt, algo="wave128"), lambda: tcu.gemm(dA, dB, out=dCt, algo="tile_wave128"), 40, 100)
         configs.append({"name": "gemm_4096_tile_api_composition", "kernel": "gemm_tile_w128", "ms": ms_t,
