@@ -165,6 +165,38 @@ def probe_mfma_reuse(torch, operands, shape, iters=4000):
             if shape == 1 else "4 x 4 accumulator tiles, each operand fragment feeds 4 instructions"}
 
 
+def probe_mfma_gaps(torch, operands, iters=4000):
+    """Shader-clock cycles per matrix instruction when a wavefront alone on its SIMD places the same filler behind every
+    matrix instruction (8 independent ones per loop pass): what the one-wavefront-per-SIMD kernels' schedules are built
+    on. Per instruction shape: {filler: cycles per matrix instruction}."""
+    import ctypes
+
+    lib = ctypes.CDLL(os.path.join(ROOT, "bench_support", "_build", "libtcu_probe.so"))
+    lib.tcu_probe_mfma_gap.restype = ctypes.c_int
+    lib.tcu_probe_mfma_gap.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4 + [ctypes.c_void_p]
+    fillers = ["nothing", "1 v_add_f32", "2 v_add_f32", "3 v_add_f32", "4 v_add_f32", "v_exp_f32", "v_exp_f32 + v_add_f32",
+               "v_exp_f32 + 2 v_add_f32", "ds_read_b128", "v_add_u32 feeding a ds_read_b128", "2 ds_read_b64_tr_b16",
+               "v_cvt_pk_f16_f32 + v_add_f32", "ds_read_b128 behind every second one"]
+    wgs = 256
+    clocks = torch.zeros(wgs, dtype=torch.int64, device=operands.device)
+    sink = torch.zeros(1, dtype=torch.float32, device=operands.device)
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for shape, name in ((1, "v_mfma_f32_16x16x32_f16"), (0, "v_mfma_f32_32x32x16_f16")):
+        res = {}
+        for fill, label in enumerate(fillers):
+            for _ in range(2):
+                rc = lib.tcu_probe_mfma_gap(operands.data_ptr(), clocks.data_ptr(), sink.data_ptr(), shape, fill, wgs, iters, stream)
+                if rc != 0:
+                    raise RuntimeError(f"tcu_probe_mfma_gap failed with hipError {rc}")
+            torch.cuda.synchronize()
+            res[label] = round(float(clocks.double().mean()) / iters / 8, 2)
+        out[name] = res
+    out["note"] = ("cycles per matrix instruction, loop overhead of 8 instructions per pass included (about 2.5 cycles per "
+                   "instruction for the 16-cycle shape)")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -472,6 +504,8 @@ def main():
         sustained["by_pattern"] = [probe_mfma(torch, dA, shape=0), probe_mfma_reuse(torch, dA, shape=1),
                                    probe_mfma_reuse(torch, dA, shape=0)]
         sustained["kernel_pattern_tflops"] = sustained["by_pattern"][1]["tflops"]
+        if args.extra_kernels:
+            sustained["issue_cost_between_matrix_instructions"] = probe_mfma_gaps(torch, dA)
 
     # ---------------------------------------------------------------- C2 timed (after the other configurations: the
     # headline measurement then starts from a GPU that has been busy for a while, like a step of a long job, not

@@ -84,7 +84,7 @@ typedef enum {
     TCU_V_ROW_MAJOR = 1  /* V stored [N, P] per batch item: the usual [seq, head_dim] */
 } tcu_v_layout;
 
-/* Which attention kernel to run (tcu_flash_attn_fwd_f16_algo). For a row-major V, AUTO picks WAVE64 for long sequences
+/* Which attention kernel to run (tcu_flash_attn_fwd_f16_algo). For a row-major V, AUTO picks WAVE64_K32 for long sequences
  * (head size 128, M % 256 == 0, N >= 1024, at least 128 blocks of 256 queries) and MFMA32_FUSED otherwise; for a
  * column-major V (head size 128) AUTO always picks WAVE64, which takes every M % 64 == 0 and N % 64 == 0. */
 typedef enum {

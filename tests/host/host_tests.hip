@@ -207,6 +207,39 @@ static void test_swizzle_tr() {
     }
 }
 
+// The 8-line form (operand tiles 16 wide: the two 16-lane groups of a pass sit on the same 32-byte unit of 8 consecutive
+// lines, lane group g four lines below group g - 1): a bijection per line that keeps 32-byte units whole, repeats every 8
+// lines, and makes every pass of the read touch 64 distinct banks.
+static void test_swizzle_tr8() {
+    constexpr int kPitch = 128;
+    using Swz = tl::LdsSwizzleTr<kPitch, 2, 8>;
+    CHECK(Swz::kLinePeriod == 8);
+    for (int line = 0; line < 64; ++line) {
+        std::set<int> seen;
+        for (int e = 0; e < kPitch; ++e) {
+            const int p = Swz::apply(line, e);
+            CHECK(p >= 0 && p < kPitch);
+            seen.insert(p);
+            if (e % 16 == 0)
+                for (int t = 1; t < 16; ++t) CHECK(Swz::apply(line, e + t) == p + t);
+            CHECK(Swz::apply(line + 8, e) == p);
+        }
+        CHECK(int(seen.size()) == kPitch);
+    }
+    for (int line0 = 0; line0 < 64; line0 += 8) {
+        for (int col0 = 0; col0 < kPitch; col0 += 16) {
+            std::set<int> banks;
+            for (int lane = 0; lane < 32; ++lane) {
+                const int L = lane & 15, grp = lane >> 4;
+                const int line = line0 + 4 * grp + (L >> 2), col = col0 + 4 * (L & 3);
+                const int byte = (line * kPitch + Swz::apply(line, col)) * 2;
+                for (int b = 0; b < 8; b += 4) banks.insert(((byte + b) / 4) % 64);
+            }
+            CHECK(int(banks.size()) == 64);
+        }
+    }
+}
+
 // A ring whose stages are further apart than a tile (two rings interleaved in one allocation).
 static void test_strided_ring() {
     using Shared = SharedTile<__half, tl::RowMajor<64, 128>, true>;
@@ -318,6 +351,7 @@ int main() {
     test_swizzle<80, 2>(false);
     test_swizzle_tr<128>();
     test_swizzle_tr<64>();
+    test_swizzle_tr8();
     test_strided_ring();
     test_swizzle<16, 4>(true);
     test_swizzle<32, 4>(true);
