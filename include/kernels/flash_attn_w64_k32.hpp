@@ -88,6 +88,7 @@ struct FlashW64K32Traits {
     using RegOut = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kQTiles, kDTiles>>;
 
     using QLoader = GlobalToSharedDirectLoader<SharedQ, WarpLayout>;
+    using PiecesQ = GlobalToSharedDirectPieces<SharedQ, WarpLayout, kD>;  // the same copy a load at a time (the next item's Q)
     using QFragments = SharedToRegLoader<RegQ, WarpLayout, WarpReuse::kRowReuseCont>;
     using PiecesK = GlobalToSharedDirectPieces<SharedK, WarpLayout, kD>;
     using PiecesV = GlobalToSharedDirectPieces<SharedV, WarpLayout, kD>;
@@ -99,16 +100,19 @@ struct FlashW64K32Traits {
     using OutToShared = RegToSharedStorer<RegOut, WarpLayout>;
     using OutToGlobal = SharedToGlobalStorer<SharedO, WarpLayout>;
     static_assert(PiecesK::kPieces == 4 && PiecesV::kPieces == 4, "a wavefront issues 8 loads per block, one per group");
+    static_assert(PiecesQ::kPieces == 16, "a wavefront fetches its 64 query rows with 16 loads: two steps' worth");
     static_assert(kDSteps * kKeyTiles == 8 && kDTiles == 8, "a step has 8 groups: a K fragment and a V fragment each");
 };
 
-/// grid = (M / 256) * batch workgroups (1-D), block = 256, dynamic LDS = Traits::kShmBytes.
+/// grid = min((M / 256) * batch, number of CUs) workgroups (1-D), block = 256, dynamic LDS = Traits::kShmBytes. A workgroup
+/// takes the items (blocks of 256 queries of one batch item) blockIdx.x, blockIdx.x + gridDim.x, ... one after the
+/// other: gridDim.x must be a multiple of 8 (or hold every item), so that a workgroup's items stay on its XCD's mapping.
 template <typename InType, typename Traits>
 __global__ void __launch_bounds__(Traits::kThreads)
     flash_attention_w64_k32(const InType* dQ, const InType* dK, const InType* dV, InType* dO, int batch, int kM, int kN,
                             float scale) {
     constexpr int kD = Traits::kD, kTN = Traits::kTN;
-    constexpr int kQT = Traits::kQTiles, kDT = Traits::kDTiles;
+    constexpr int kQT = Traits::kQTiles, kDT = Traits::kDTiles, kStages = Traits::kStages;
     using RegQ = typename Traits::RegQ;
     using RegK = typename Traits::RegK;
     using RegS = typename Traits::RegS;
@@ -121,27 +125,60 @@ __global__ void __launch_bounds__(Traits::kThreads)
     extern __shared__ __align__(1024) unsigned char buf[];
     const int nb = kN / kTN;
 
-    // query blocks of one (batch, head) item get workgroup ids congruent modulo 8: one XCD, K and V fetched once
+    // query blocks of one (batch, head) item get item numbers congruent modulo 8: one XCD, K and V fetched once
     const int q_blocks = kM / Traits::kTM;
-    int head_i, q_block;
-    if (batch % 8 == 0) {
-        const int xcd = blockIdx.x & 7, rest = blockIdx.x >> 3;
-        q_block = rest % q_blocks;
-        head_i = (rest / q_blocks) * 8 + xcd;
-    } else {
-        q_block = blockIdx.x % q_blocks;
-        head_i = blockIdx.x / q_blocks;
-    }
-    const size_t head = head_i;
+    const int items = q_blocks * batch;
+    auto locate = [&](int w, size_t& head, int& q_block) {
+        if (batch % 8 == 0) {
+            const int xcd = w & 7, rest = w >> 3;
+            q_block = rest % q_blocks;
+            head = size_t(rest / q_blocks) * 8 + xcd;
+        } else {
+            q_block = w % q_blocks;
+            head = size_t(w / q_blocks);
+        }
+    };
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave_id());
+    // The ring stage of key block 0 of the current item, and whether the item's Q and first block are in LDS already
+    // (the workgroup's previous item fetched them under its last steps).
+    int s0 = 0;
+    bool fetched = false;
+#pragma unroll 1
+    for (int w = blockIdx.x; w < items; w += gridDim.x) {
+    size_t head;
+    int q_block;
+    locate(w, head, q_block);
     const InType* Qb = dQ + (head * kM + size_t(q_block) * Traits::kTM) * kD;
     const InType* Kh = dK + head * size_t(kN) * kD;
     const InType* Vh = dV + head * size_t(kN) * kD;
     InType* Ob = dO + (head * kM + size_t(q_block) * Traits::kTM) * kD;
+    // the workgroup's next item (without one: this item again, so that the schedule has one form)
+    const InType *Qnext, *Knext, *Vnext;
+    {
+        size_t nhead;
+        int nqb;
+        locate(w + int(gridDim.x) < items ? w + int(gridDim.x) : w, nhead, nqb);
+        Qnext = dQ + (nhead * kM + size_t(nqb) * Traits::kTM) * kD;
+        Knext = dK + nhead * size_t(kN) * kD;
+        Vnext = dV + nhead * size_t(kN) * kD;
+    }
+    auto st = [&](int i) {  // ring stage of key block i < 5 of this item
+        const int t = s0 + i;
+        return t >= kStages ? t - kStages : t;
+    };
 
     InType* shm = reinterpret_cast<InType*>(buf);
     typename Traits::RingK ringK(shm);
     typename Traits::RingV ringV(shm + Traits::kBlockNumel);
-    typename Traits::SharedQ sQ(shm + 3 * 2 * Traits::kBlockNumel);  // stages 3 and 4
+    // Q and O pass through LDS a wavefront at a time: each wavefront writes and reads only its own 64 rows (16 KiB, a
+    // quarter of the tile). A 256-row tile laid over two ring stages that need not be neighbours in memory (the ring
+    // wraps): wavefronts 0, 1 use stage `sa`, wavefronts 2, 3 stage `sb`; the pointer is where row 0 would be for this
+    // wavefront's rows to land there.
+    constexpr int kStageNumel = 2 * Traits::kBlockNumel, kWaveRowsNumel = 64 * kD;
+    auto rows_over_two_stages = [&](int sa, int sb) -> InType* {
+        return shm + (wave_u < 2 ? sa : sb) * kStageNumel + (wave_u & 1) * kWaveRowsNumel - wave_u * kWaveRowsNumel;
+    };
+    typename Traits::SharedQ sQ(rows_over_two_stages(st(3), st(4)));
 
     typename Traits::PiecesK pieces_k;
     typename Traits::PiecesV pieces_v;
@@ -158,14 +195,14 @@ __global__ void __launch_bounds__(Traits::kThreads)
 
     // ---- prologue: Q and block 0 are requested together (the cold latencies overlap); blocks 1 and 2 under the
     // first two score computations, blocks 3 and 4 (into the stages Q passed through) in the first block-iteration
-    {
+    if (!fetched) {
         typename Traits::QLoader load_q;
         typename Traits::GlobalQ gQ(Qb);
         load_q(gQ, sQ);
-    }
 #pragma unroll
-    for (int s = 0; s < 8; ++s) issue(block_load(0, 0, s));
-    wait_group_and_barrier<0>();
+        for (int s = 0; s < 8; ++s) issue(block_load(st(0), 0, s));
+        wait_group_and_barrier<0>();
+    }
 
     RegQ rQ;
     {
@@ -221,7 +258,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
                 if constexpr (ds == 0) Scores::template at_from<c, 0, 0>(rQ, one, rS[kBuf][kt], neg_max(c, 0));
                 else Scores::template at<c, 0, ds>(rQ, one, rS[kBuf][kt]);
             });
-            issue(block_load(load_block, load_block, g));
+            issue(block_load(st(load_block), load_block, g));
         });
     };
 
@@ -242,7 +279,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
 #pragma unroll
         for (int e = 0; e < 4; ++e) neg_max(c, 0)(0, e) = 0.f;
     compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
-    scores_only(0, 0, std::integral_constant<int, 0>{}, 1);
+    scores_only(st(0), 0, std::integral_constant<int, 0>{}, 1);
     asm volatile("s_nop 15\n\ts_nop 3");
     compute::pin_tiles<compute::RegFile::kVgpr>(rS[0][0]);
     compute::pin_tiles<compute::RegFile::kVgpr>(rS[0][1]);
@@ -261,7 +298,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         for (int e = 0; e < 4; ++e) neg_max(c, 0)(0, e) = -mx;
     }
     compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
-    scores_only(0, 1, std::integral_constant<int, 1>{}, 2);
+    scores_only(st(0), 1, std::integral_constant<int, 1>{}, 2);
 
     struct Stages {
         int a, b, c, load;
@@ -271,29 +308,12 @@ __global__ void __launch_bounds__(Traits::kThreads)
     constexpr int kHalfBytes = Traits::kHalf * kD * int(sizeof(InType));  // between the halves of a K or V block
     constexpr int kStageBytes = 2 * Traits::kBlockNumel * int(sizeof(InType));
 
-    // The workgroup that follows this one on the XCD (ids congruent mod 8 share an XCD: id + 256) starts with a cold
-    // burst: its 256 query rows and the first block of its item's K and V, 96 KiB of consecutive memory. The last three
-    // steps of this workgroup have no ring loads left to issue and fetch those instead (kLoads == 2, 3), into a ring
-    // stage that is vacant (the data is discarded: the point is that the lines are in this XCD's L2 when the next
-    // workgroup asks). Without a successor the workgroup fetches its own again.
-    const char *warm_src = nullptr, *warm_src_v = nullptr;  // 8 KiB of consecutive memory per step and wavefront
-    unsigned int warm_lds = 0;
-    const unsigned int lane_off16 = lane_id() * 16u;
-    int nhead = head_i, nqb = q_block;
-    {
-        const unsigned int nid = blockIdx.x + 256;
-        if (nid < gridDim.x) {
-            if (batch % 8 == 0) {
-                const int xcd = nid & 7, rest = nid >> 3;
-                nqb = rest % q_blocks;
-                nhead = (rest / q_blocks) * 8 + xcd;
-            } else {
-                nqb = nid % q_blocks;
-                nhead = nid / q_blocks;
-            }
-        }
-    }
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave_id());
+    // The last three steps of an item have no ring loads left to issue and fetch what the workgroup's next item starts
+    // with instead - its 256 query rows (kLoads == 2, 4: 8 of a wavefront's 16 loads each) and its first K / V block
+    // (kLoads == 3) - into the three ring stages this item has left for good. The next item then starts computing at once.
+    typename Traits::PiecesQ pieces_q;
+    int next_s0 = 0;                                    // the stage of the next item's block 0
+    typename Traits::SharedQ sQnext(shm);               // (set when the fetch begins)
 
     // A fragment's address moves on to the next ring stage between its read of half 1 of a block and its read of half 0
     // of the next: fragments 0..2 (requested at the end of a step for the next one) behind the first step of a
@@ -309,7 +329,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
 
     // ---- one pipelined step on half i: softmax of half i (rS[kCur] -> rP[kCur]), scores of half i + 1 into rS[kNxt]
     // (if kQk), O += P V with half i - 1 (rP[kNxt]). ring: stages of blocks J, J + 1, J + 2 and of the block being
-    // loaded. kLoads: 0 none, 1 block `load_block`, 2 / 3 the warm-up loads.
+    // loaded. kLoads: 0 none, 1 block `load_block`, 2 / 4 / 3 the next item's Q (first, second half) / first block.
     // A step is 8 groups of 8 matrix instructions: group g multiplies K fragment g (d-step g % 4 of key tile g / 4) with
     // the 4 query tiles, then V fragment g (d tile g) with the 4 probability tiles, and takes score tile (g / 2, g % 2)
     // of half i through the softmax. The fragments of group g + kAhead are requested inside group g (K behind the
@@ -374,10 +394,12 @@ __global__ void __launch_bounds__(Traits::kThreads)
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (kLoads == 1) {
                 Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4], block_load(ring.load, load_block, g));
-            } else if constexpr (kLoads == 2 || kLoads == 3) {
+            } else if constexpr (kLoads == 2 || kLoads == 4) {
+                Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4], pieces_q.piece(kLoads == 2 ? g : 8 + g, Qnext, sQnext));
+            } else if constexpr (kLoads == 3) {
                 Output::template at<0, g % 4, 0>(
                     rP[kNxt], rV, rO[g / 4],
-                    DirectLoad{lane_off16, (kLoads == 3 && g >= 4 ? warm_src_v : warm_src) + g * 1024, warm_lds});
+                    g < 4 ? pieces_k.piece(g, Knext, ringK[next_s0]) : pieces_v.piece(g - 4, Vnext, ringV[next_s0]));
             } else {
                 Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
             }
@@ -467,7 +489,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     int J = 0;
-    Stages ring{0, 1, 2, 4};
+    Stages ring{st(0), st(1), st(2), st(4)};
     auto advance = [&]() {
         ring.a = ring.b;
         ring.b = ring.c;
@@ -480,15 +502,15 @@ __global__ void __launch_bounds__(Traits::kThreads)
         wait_group_and_barrier_keep_reads<0>();
         // first fragments of step 1: K of half 2 (block 1), V of half 0 - behind the barrier: block 1 is complete only
         // when every wavefront's pieces of it have landed
-        k_frag.bind(k_half(1, 0));
-        v_frag.bind(v_half(0, 0));
+        k_frag.bind(k_half(st(1), 0));
+        v_frag.bind(v_half(st(0), 0));
         static_for<kAhead>([&](auto a_c) {
             constexpr int a = decltype(a_c)::value;
             k_frag.template read_bound_to<a % 4, a / 4>(rK(a % 4, 0));
             v_frag.template read_bound_to<0, a>(rV(0, a % 4));
         });
         Stages first = ring;
-        first.load = 3;
+        first.load = st(3);
         step(first, I1{}, Yes{}, I1{}, Yes{}, 3);
         step(ring, I0{}, Yes{}, I1{}, Yes{}, 4);
         advance();
@@ -506,25 +528,26 @@ __global__ void __launch_bounds__(Traits::kThreads)
         step(ring, I1{}, Yes{}, I0{}, Yes{}, 0);
         step(ring, I0{}, Yes{}, I0{}, Yes{}, 0);
     }
-    // the last three steps carry the warm-up loads: 16 KiB of the successor's query rows per wavefront in two steps, then
-    // 4 KiB each of its first K and V block
+    // The last three steps carry the next item's first loads. The stages they go to: this item's last two blocks sit
+    // in ring.a and ring.b; the other three are free once every wavefront has left block nb - 3 (the barrier). Q goes to
+    // the first two of them, the first K / V block to the third, which makes that one stage 0 of the next item's ring
+    // (its Q then lies in its stages 3 and 4, where this item's did).
+    const int last_a = ring.a, last_b = ring.b;
     {
-        using lds_cptr = __attribute__((address_space(3))) const void*;
-        warm_lds = static_cast<unsigned int>(reinterpret_cast<uintptr_t>((lds_cptr)(ringK[ring.c].data()))) + wave_u * 1024u;
+        const int f0 = ring.c, f1 = Traits::RingK::next(f0);
+        next_s0 = Traits::RingK::next(f1);
+        wait_group_and_barrier_keep_reads<0>();
+        sQnext = typename Traits::SharedQ(rows_over_two_stages(f0, f1));
     }
-    const char* next_q = reinterpret_cast<const char*>(dQ + (size_t(nhead) * kM + size_t(nqb) * Traits::kTM) * kD) + wave_u * 16384;
-    using Warm = std::integral_constant<int, 2>;
-    using WarmKV = std::integral_constant<int, 3>;
+    using FetchQ0 = std::integral_constant<int, 2>;
+    using FetchQ1 = std::integral_constant<int, 4>;
+    using FetchKV = std::integral_constant<int, 3>;
     if (J + 1 < nb) {
-        warm_src = next_q;
-        step(ring, I1{}, Yes{}, Warm{}, Yes{}, 0);
-        warm_src = next_q + 8192;
-        step(ring, I0{}, Yes{}, Warm{}, No{}, 0);
+        step(ring, I1{}, Yes{}, FetchQ0{}, Yes{}, 0);
+        step(ring, I0{}, Yes{}, FetchQ1{}, No{}, 0);
         advance();
     }
-    warm_src = reinterpret_cast<const char*>(dK + size_t(nhead) * kN * kD) + wave_u * 4096;
-    warm_src_v = reinterpret_cast<const char*>(dV + size_t(nhead) * kN * kD) + wave_u * 4096 - 4096;  // its loads are 4..7
-    step(ring, I1{}, No{}, WarmKV{}, No{}, 0);
+    step(ring, I1{}, No{}, FetchKV{}, No{}, 0);
     {
         // O += P V with the last half (its first fragments were requested by the step before)
         static_for<8>([&](auto g_c) {
@@ -558,15 +581,22 @@ __global__ void __launch_bounds__(Traits::kThreads)
             compute::convert_pair_here(o(0, 2) * inv_l, o(0, 3) * inv_l, dst + 2);
         }
     }
+    // this wavefront's pieces of the next item's Q and first block have landed, then everyone's; and every wavefront is
+    // done with the stages of the last two blocks, which take the output now (a wavefront's own rows only: nothing to
+    // wait for between writing and reading them)
     wait_group<0>();
-    __syncthreads();  // every wavefront is done with the K/V stages (and its warm-up loads have landed): reused for O
-    typename Traits::SharedO sO(shm);
+    __syncthreads();
+    typename Traits::SharedO sO(rows_over_two_stages(last_a, last_b));
     typename Traits::OutToShared to_shared;
     typename Traits::OutToGlobal to_global;
     typename Traits::GlobalO gO(Ob);
     to_shared(out, sO);
-    __syncthreads();
     to_global(sO, gO);
+    // the next item loads its blocks 1 and 2 into these two stages: not before everyone has read its rows back
+    __builtin_amdgcn_s_barrier();
+    s0 = next_s0;
+    fetched = true;
+    }  // items of this workgroup
 }
 
 }  // namespace tiledcuda::kernels

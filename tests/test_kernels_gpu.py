@@ -861,12 +861,15 @@ def test_flash_attention_tile_wave64_is_wave64(tcu, oracle, device, batch, M, N)
     assert oracle.max_abs_err(host(out)[heads, :64], ref) <= (2e-2 if N == 640 else ABS_TOL)
 
 
-@pytest.mark.parametrize("batch,M,N", [(3, 256, 320), (8, 256, 640), (2, 512, 1024), (5, 768, 448), (64, 2048, 2048)])
+@pytest.mark.parametrize("batch,M,N", [(3, 256, 320), (8, 256, 640), (2, 512, 1024), (5, 768, 448), (64, 2048, 2048),
+                                       (203, 1024, 448), (96, 2048, 384), (330, 256, 640)])
 def test_flash_attention_wave64_k32(tcu, oracle, device, batch, M, N):
     """The one-wavefront-per-SIMD design on the 16x16x32 matrix instruction (wave64_k32): against the oracle on whole
     heads at small sizes and on a sample of rows at the benchmark size, and against the 32x32x16 kernel everywhere (same
     arithmetic up to the order of the sums inside a matrix instruction); at 5 key blocks (the minimum), an odd number of
-    blocks, one and two rounds of workgroups, and with keys that force the rare re-basing path."""
+    blocks, with keys that force the rare re-basing path, and with one, two, three and a ragged number of items per
+    workgroup (a workgroup takes its items one after the other and fetches the next one's first operands under the last
+    steps of the current one: 5 ring positions x the two-stage regions that wrap around the ring)."""
     import torch
 
     D = 128

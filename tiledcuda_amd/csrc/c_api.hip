@@ -593,7 +593,15 @@ int fa_w64_k32_dispatch(const __half* Q, const __half* K, const __half* V, __hal
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel needs M % 256 == 0 and N >= 320");
     if ((long)N * 256 >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel addresses a V block with 32-bit offsets");
-    return launch(&flash_attention_w64_k32<__half, Traits>, dim3((M / Traits::kTM) * batch), dim3(Traits::kThreads),
+    // one workgroup per CU; a workgroup with more than one item fetches the next one's first operands under the last
+    // steps of the current one. Items keep their XCD (item number modulo 8) only if the grid is a multiple of 8.
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus < 8)
+        return fail(TCU_ERR_HIP, "attention: cannot read the number of compute units");
+    const long items = (long)(M / Traits::kTM) * batch;
+    const long grid = std::min<long>(items, cus - cus % 8);
+    return launch(&flash_attention_w64_k32<__half, Traits>, dim3(unsigned(grid)), dim3(Traits::kThreads),
                   Traits::kShmBytes, stream, Q, K, V, O, batch, M, N, scale);
 }
 
