@@ -104,7 +104,9 @@ typedef enum {
                                   (M, N) in {(2048, 2048), (512, 1024), (256, 640), (256, 320)}, head size 128, row-major
                                   V; results identical to WAVE64 bit for bit */
     TCU_ATTN_WAVE64_K32 = 6    /* the WAVE64 design on v_mfma_f32_16x16x32_f16 (tile-library functors; twice the matrix
-                                  instructions, each contracting 32 indices: the chip sustains a higher clock on them);
+                                  instructions, each contracting 32 indices: the chip sustains a higher clock on them),
+                                  launched as one workgroup per CU that takes its blocks of 256 queries one after the
+                                  other and fetches the next one's first operands under the last steps of the current;
                                   row-major V, head size 128, M % 256 == 0, N % 64 == 0, N >= 320; results equal to
                                   WAVE64 up to the summation order inside a matrix instruction */
 } tcu_attn_algo;
