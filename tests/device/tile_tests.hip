@@ -494,6 +494,95 @@ __global__ void __launch_bounds__(256) k_tile_gemm_pieces(const __half* dA, cons
     r2g(acc, gC);
 }
 
+// The same chain on v_mfma_f32_16x16x32_f16: two 16 x 16 score accumulators side by side, converted, are the 16 x 32 A
+// operand of the second product when V is fetched in their contraction order (SharedToRegTrPieces<..., true> on 32 x 16
+// operand tiles, a shared tile with the 8-line form of LdsSwizzleTr). The fragment readers run in their bound form:
+// bind() once, read_bound() / read_bound_to() with immediates, shift() to another allocation and back.
+template <int kM, int kN, int kK, int kP, typename WarpLayout>
+__global__ void __launch_bounds__(256) k_tile_b2b_accumulator_order_k32(const __half* dA, const __half* dBV, float* dD) {
+    extern __shared__ __align__(1024) unsigned char buf[];
+    auto* sA_ptr = reinterpret_cast<__half*>(buf) + 2048;  // (4 KiB in front: the bound views below start there)
+    auto* sB_ptr = sA_ptr + kM * kK;
+    auto* sV_ptr = sB_ptr + kN * kK;
+    constexpr int kWR = tl::num_rows<WarpLayout>;
+    static_assert(tl::num_cols<WarpLayout> == 1 && kM == 16 * kWR && kN % 32 == 0 && kK % 32 == 0 && kP == 128);
+    using Shape = traits::MfmaTileShape<__half, traits::MfmaShape::k16x16x32>;
+    using SharedA = SharedTile<__half, tl::RowMajor<kM, kK>, true>;
+    using SharedB = SharedTile<__half, tl::ColMajor<kK, kN>, true>;
+    using SharedV = SharedTile<__half, tl::RowMajor<kN, kP>, true, tl::LdsSwizzleTr<kP, 2, 8>>;
+    using RegA = RegTile<typename Shape::TileA, tl::RowMajor<1, kK / 32>>;
+    using RegB = RegTile<typename Shape::TileB, tl::ColMajor<kK / 32, kN / 16>>;
+    using RegS = RegTile<typename Shape::TileC, tl::RowMajor<1, kN / 16>>;
+    using RegP = RegTile<typename Shape::TileA, tl::RowMajor<1, kN / 32>>;
+    using RegV = RegTile<typename Shape::TileB, tl::ColMajor<kN / 32, kP / 16>>;
+    using RegD = RegTile<typename Shape::TileC, tl::RowMajor<1, kP / 16>>;
+    using GlobalD = GlobalTile<float, tl::RowMajor<kM, kP>>;
+
+    GlobalTile<__half, tl::RowMajor<kM, kK>> gA(dA);
+    GlobalTile<__half, tl::ColMajor<kK, kN>> gB(dBV);
+    GlobalTile<__half, tl::RowMajor<kN, kP>> gV(dBV + kN * kK);
+    SharedA sA(sA_ptr);
+    SharedB sB(sB_ptr);
+    SharedV sV(sV_ptr);
+    GlobalToSharedDirectLoader<SharedA, WarpLayout>{}(gA, sA);
+    GlobalToSharedDirectLoader<SharedB, WarpLayout>{}(gB, sB);
+    GlobalToSharedDirectLoader<SharedV, WarpLayout>{}(gV, sV);
+    wait_group_and_barrier<0>();
+
+    RegA rA;
+    RegB rB;
+    RegV rV;
+    RegS rS;
+    compute::pin_tiles<compute::RegFile::kVgpr>(rS);
+    SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>{}(sA, rA);
+    SharedToRegPieces<RegB, SharedB, WarpLayout, WarpReuse::kColReuseCont> read_b;
+    SharedToRegTrPieces<RegV, SharedV, WarpLayout, WarpReuse::kColReuseCont, true> read_v;
+    // bound to a view 4 KiB in front of the tile, every read with the immediate that brings it back; one fragment's
+    // address moved away and back with shift()
+    read_b.bind(SharedB(sB_ptr - 2048));
+    read_v.bind(SharedV(sV_ptr - 2048));
+    read_b.template shift<0, 0>(8192);
+    read_v.template shift<0>(-4096);
+    read_b.template shift<0, 0>(-8192);
+    read_v.template shift<0>(4096);
+    static_for<RegB::kRows * RegB::kCols>([&](auto n_c) {
+        constexpr int n = decltype(n_c)::value;
+        read_b.template read_bound<n / RegB::kCols, n % RegB::kCols, 4096>(rB);
+    });
+    static_for<RegV::kRows * RegV::kCols>([&](auto n_c) {
+        constexpr int n = decltype(n_c)::value;
+        read_v.template read_bound_to<n / RegV::kCols, n % RegV::kCols, 4096>(rV(n / RegV::kCols, n % RegV::kCols));
+    });
+    wait_shared_reads<0>();
+
+    using First = compute::ScheduledGemm<RegA, RegB, RegS, compute::RegFile::kVgpr, compute::RegFile::kVgpr>;
+    static_for<RegB::kCols>([&](auto j_c) {
+        static_for<RegA::kCols>([&](auto k_c) { First::template at<0, decltype(j_c)::value, decltype(k_c)::value>(rA, rB, rS); });
+    });
+    asm volatile("s_nop 15\n\ts_nop 3");
+    compute::pin_tiles<compute::RegFile::kVgpr>(rS);
+    // accumulator tiles 2 j and 2 j + 1  ->  A operand tile j: elements 0..3 and 4..7
+    RegP rP;
+    static_for<RegP::kCols>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; e += 2)
+                compute::convert_pair_here(rS(0, 2 * j + h)(0, e), rS(0, 2 * j + h)(0, e + 1), rP(0, j).mutable_data() + 4 * h + e);
+    });
+    RegD rD;
+    compute::clear_pinned(rD);
+    using Second = compute::ScheduledGemm<RegP, RegV, RegD>;
+    static_for<RegV::kRows>([&](auto k_c) {
+        static_for<RegV::kCols>([&](auto j_c) { Second::template at<0, decltype(j_c)::value, decltype(k_c)::value>(rP, rV, rD); });
+    });
+    compute::settle_accumulators(rD);
+    GlobalD gD(dD);
+    RegToGlobalStorer<GlobalD, RegD, WarpLayout> r2g;
+    r2g(rD, gD);
+}
+
 // D = f16(A · B) · V on wavefronts that own 32 rows each: the 32 x 32 accumulator tiles of the first product, converted
 // to f16 in place, ARE the A operand of the second one, because V (row-major [kN, kP], transposing-read swizzle) is
 // fetched in the accumulator's own contraction order (SharedToRegTrPieces<..., kAccumulatorOrder = true>); every
@@ -770,6 +859,18 @@ void reg_gemm_pieces() {
                           kWR * kWC * 64,
                           (kM + kN) * kK * 2,
                           &launch_gemm<k_tile_gemm_pieces<kM, kN, kK, W>>});
+}
+
+template <int kM, int kN, int kK, int kP, int kWR>
+void reg_b2b_acc_order_k32() {
+    using W = tl::RowMajor<kWR, 1>;
+    registry().push_back({"tile_b2b",
+                          "accumulator_order_16x16x32_" + std::to_string(kM) + "x" + std::to_string(kN) + "x" + std::to_string(kK) +
+                              "x" + std::to_string(kP) + "_w" + std::to_string(kWR) + "x1",
+                          {kM, kN, kK, kP, 0, 0, 0, 0},
+                          kWR * 64,
+                          (kM * kK + kN * kK + kN * kP) * 2 + 4096,
+                          &launch_gemm<k_tile_b2b_accumulator_order_k32<kM, kN, kK, kP, W>>});
 }
 
 template <int kM, int kN, int kK, int kP, int kWR>
@@ -1159,6 +1260,9 @@ void build_registry() {
     reg_b2b_acc_order<32, 64, 64, 64, 1>();
     reg_b2b_acc_order<64, 128, 32, 64, 2>();
     reg_b2b_acc_order<128, 64, 128, 64, 4>();
+    reg_b2b_acc_order_k32<16, 32, 32, 128, 1>();
+    reg_b2b_acc_order_k32<32, 64, 128, 128, 2>();
+    reg_b2b_acc_order_k32<64, 128, 64, 128, 4>();
 }
 
 thread_local std::string g_err;
