@@ -348,7 +348,7 @@ def main():
                         "frac_mfma_peak": flops_long / (ms_long * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, "max_abs_err": err_long})
         del dql, dkl, dvl, dol
         configs.append({"name": "flash_attention_fwd_op_convention_b64_s2048_d128_v_col_major",
-                        "kernel": "flash_attention_fwd_w64<128, column-major V>", "ms": ms_op,
+                        "kernel": "flash_attention_w64_k32<128, column-major V>", "ms": ms_op,
                         "tflops": flops / (ms_op * 1e-3) / 1e12,
                         "frac_mfma_peak": flops / (ms_op * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, "max_abs_err": err_op})
 

@@ -102,6 +102,8 @@ DEVICE void issue(const DirectLoad& load) {
 /// tile's origin `src` (wave-uniform) and the stage `dst`. For kernels that spread the loads of the next tile over the
 /// matrix instructions of the current one instead of issuing them in a burst (the address unit of a CU takes one
 /// vector-memory instruction per ~14 cycles, and a wavefront that waits there issues nothing else).
+/// kGlobalPitch_ == 0: the pitch is a run-time value, given to the constructor (a tile cut out of an operand whose
+/// leading dimension is a run-time size, e.g. a column-major V of an attention layer: pitch = number of keys).
 template <typename Shared_, typename WarpLayout_, const int kGlobalPitch_>
 struct GlobalToSharedDirectPieces {
     using Shared = Shared_;
@@ -112,7 +114,10 @@ struct GlobalToSharedDirectPieces {
     static_assert((long)Shared::kLines * kGlobalPitch * (long)sizeof(DType) < (1l << 32),
                   "a tile's lines are addressed with 32-bit byte offsets from its origin");
 
-    DEVICE GlobalToSharedDirectPieces() {
+    DEVICE GlobalToSharedDirectPieces() : GlobalToSharedDirectPieces(kGlobalPitch_) {
+        static_assert(kGlobalPitch_ > 0, "a run-time pitch goes to the other constructor");
+    }
+    DEVICE explicit GlobalToSharedDirectPieces(int global_pitch) {
         const int lane = lane_id();
         wave_ = __builtin_amdgcn_readfirstlane(wave_id());
         const int line_in_load = lane / Loader::kPiecesPerLine;
@@ -122,7 +127,8 @@ struct GlobalToSharedDirectPieces {
             const int line = (wave_ * kPieces + j) * Loader::kLinesPerLoad + line_in_load;
             const int elem = Shared::kSwizzled ? Shared::Swizzle::apply(line, piece * Loader::kPieceElems)
                                                : piece * Loader::kPieceElems;
-            offset_[j] = (static_cast<unsigned int>(line) * kGlobalPitch + elem) * static_cast<unsigned int>(sizeof(DType));
+            offset_[j] = (static_cast<unsigned int>(line) * static_cast<unsigned int>(global_pitch) + elem) *
+                         static_cast<unsigned int>(sizeof(DType));
         }
     }
 

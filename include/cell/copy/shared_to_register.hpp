@@ -264,7 +264,13 @@ DEVICE unsigned int shared_view_address(const Shared& tile) {
 /// (sub-)tile it is pointed at: one vector addition per read.
 /// Shared_ is the tile type the offsets are computed for (a whole stage of a ring, or the sub-tile a wavefront's
 /// operand comes from); read() takes any view of that type whose origin is a multiple of the swizzle's line period.
-template <typename Reg_, typename Shared_, typename WarpLayout_, const WarpReuse kMode_,
+/// kDealtLines: the lines (rows of A, columns of B) of a PAIR of neighbouring operand tiles are dealt to the two tiles
+/// four at a time - tile 2 p + h holds lines 32 p + 8 q + 4 h + r (q, r = 0..3) as its lines 4 q + r - instead of 16
+/// consecutive ones each. The two 16 x 16 accumulators of a product with such a pair then hold, per lane, 8 CONSECUTIVE
+/// lines (accumulator 2 p: 8 g .. 8 g + 3, accumulator 2 p + 1: 8 g + 4 .. 8 g + 7 for lane group g): converted, they are
+/// an A operand in the standard contraction order, and the other operand of the next product can be read with plain
+/// 16-byte reads along its lines (a V stored column-major).
+template <typename Reg_, typename Shared_, typename WarpLayout_, const WarpReuse kMode_, const bool kDealtLines = false,
           typename Base = warp::CopyBase<WarpLayout_, kMode_>>
 struct SharedToRegPieces : public Base {
     using Reg = Reg_;
@@ -280,9 +286,16 @@ struct SharedToRegPieces : public Base {
                       Base::template col_exec_count<BaseShape, Shared::kCols>() == Reg::kCols,
                   "the register tile must hold exactly this wavefront's share of the shared tile");
 
+    static_assert(!kDealtLines || (G::kLaneMajor == 16 && (G::kRowMajor ? Reg::kRows : Reg::kCols) % 2 == 0),
+                  "lines are dealt to pairs of 16-line operand tiles");
+
     DEVICE SharedToRegPieces() {
         const int lane = lane_id();
         const int major = lane % G::kLaneMajor, minor = (lane / G::kLaneMajor) * G::kRunLen;
+        // line of operand tile t (along the major index) that this lane holds
+        auto line_of = [&](int t) {
+            return kDealtLines ? (t / 2) * 32 + 8 * (major / 4) + 4 * (t % 2) + major % 4 : t * G::kLaneMajor + major;
+        };
         const int row0 = Base::template warp_row0<Shared::kRows>();
         const int col0 = Base::template warp_col0<Shared::kCols>();
         const Shared whole(nullptr);
@@ -290,8 +303,8 @@ struct SharedToRegPieces : public Base {
         for (int i = 0; i < Reg::kRows; ++i)
 #pragma unroll
             for (int j = 0; j < Reg::kCols; ++j) {
-                const int row = row0 + i * BaseShape::kRows + (G::kRowMajor ? major : minor);
-                const int col = col0 + j * BaseShape::kCols + (G::kRowMajor ? minor : major);
+                const int row = row0 + (G::kRowMajor ? line_of(i) : i * BaseShape::kRows + minor);
+                const int col = col0 + (G::kRowMajor ? j * BaseShape::kCols + minor : line_of(j));
                 offset_[i][j] = static_cast<unsigned int>(whole.offset(row, col)) * static_cast<unsigned int>(sizeof(DType));
                 asm volatile("" : "+v"(offset_[i][j]));  // computed once, not again at every use
             }

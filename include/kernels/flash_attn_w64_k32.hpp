@@ -23,8 +23,9 @@
 // maximum that moves only when a partial sum could leave f16 range, f32 sums and output); the sums inside a matrix
 // instruction cover 32 instead of 16 indices and the final division is a reciprocal and a product, so results differ
 // from that kernel in the last bits.
-// Requirements: head size 128, row-major V, M % 256 == 0, N % 64 == 0, N >= 320 (Q passes through two ring stages
-// before the fifth block needs them). M, N and the batch count are run-time values.
+// Requirements: head size 128, M % 256 == 0, N % 64 == 0, N >= 320 (Q passes through two ring stages before the fifth
+// block needs them); V row-major [N, D] or column-major (the reference op's convention; see the traits). M, N and the
+// batch count are run-time values.
 #pragma once
 
 #include <type_traits>
@@ -40,9 +41,15 @@ using namespace tiledcuda::cell;
 using namespace tiledcuda::cell::copy;
 namespace tl = tiledcuda::cell::tile_layout;
 
-template <typename InType, const int kD_>
+/// kVColMajor_: V is stored column-major [N, D], i.e. as the array Vᵀ [D, N] (the convention of the reference's op,
+/// src/kernels/flash_attn.cu:314-327). Then a V block lies in LDS as two halves of 32 keys, column-major like K (lines
+/// of 64 bytes along the keys), its fragments are plain 16-byte reads in the standard contraction order, and the keys
+/// of a half are dealt to the two K operand tiles four at a time (copy::SharedToRegPieces<..., kDealtLines>), so that
+/// the two score accumulators of a lane hold 8 consecutive keys.
+template <typename InType, const int kD_, const bool kVColMajor_ = false>
 struct FlashW64K32Traits {
     static constexpr int kD = kD_;
+    static constexpr bool kVColMajor = kVColMajor_;
     using WarpLayout = tl::RowMajor<4, 1>;
     static constexpr int kWaves = 4, kThreads = kWaves * kWaveSize;
     static constexpr int kTM = 64 * kWaves, kTN = 64, kHalf = 32, kStages = 5;
@@ -59,8 +66,12 @@ struct FlashW64K32Traits {
     using GlobalO = GlobalTile<InType, tl::RowMajor<kTM, kD>>;
 
     // LDS: a ring stage is a K block followed by a V block; Q passes once through stages 3 and 4
-    using SharedK = SharedTile<InType, tl::ColMajor<kD, kTN>, true>;  // Kᵀ [d, keys], stored [keys, d]
-    using SharedV = SharedTile<InType, tl::RowMajor<kTN, kD>, true, tl::LdsSwizzleTr<kD, sizeof(InType), 8>>;
+    // Kᵀ [d, keys], stored [keys, d]
+    using SharedK = std::conditional_t<kVColMajor, SharedTile<InType, tl::ColMajor<kD, kTN>, true, tl::LdsSwizzleDealt<kD, sizeof(InType)>>,
+                                       SharedTile<InType, tl::ColMajor<kD, kTN>, true>>;
+    // a V block [keys, d] row-major, or one of its two halves [32 keys, d] column-major (the other one 8 KiB further on)
+    using SharedV = std::conditional_t<kVColMajor, SharedTile<InType, tl::ColMajor<kHalf, kD>, true>,
+                                       SharedTile<InType, tl::RowMajor<kTN, kD>, true, tl::LdsSwizzleTr<kD, sizeof(InType), 8>>>;
     static constexpr int kBlockNumel = kTN * kD;
     using RingK = SharedRing<SharedK, kStages, 2 * kBlockNumel>;
     using RingV = SharedRing<SharedV, kStages, 2 * kBlockNumel>;
@@ -71,9 +82,18 @@ struct FlashW64K32Traits {
 
     // the 32-key halves a step works on
     using KHalves = STileIterator<SharedK, TileShape<kD, kHalf>>;
-    using VHalves = STileIterator<SharedV, TileShape<kHalf, kD>>;
     using SharedKHalf = decltype(std::declval<KHalves>()(0));
-    using SharedVHalf = decltype(std::declval<VHalves>()(0));
+    struct RowMajorVHalf {  // half t of a row-major block: a view of 32 of its 64 lines
+        using Halves = STileIterator<SharedV, TileShape<kHalf, kD>>;
+        using type = decltype(std::declval<Halves>()(0));
+        DEVICE static type at(InType* block, int t) { return Halves(block)(t); }
+    };
+    struct ColMajorVHalf {  // half t of a column-major block: a tile of its own
+        using type = SharedV;
+        DEVICE static type at(InType* block, int t) { return SharedV(block + t * kHalf * kD); }
+    };
+    using VHalf = std::conditional_t<kVColMajor, ColMajorVHalf, RowMajorVHalf>;
+    using SharedVHalf = typename VHalf::type;
 
     // register tiles of one wavefront (64 queries)
     using RegQ = RegTile<typename Shape::TileA, tl::RowMajor<kQTiles, kDSteps>>;     // A of S = Q Kᵀ, in AGPRs
@@ -91,15 +111,17 @@ struct FlashW64K32Traits {
     using PiecesQ = GlobalToSharedDirectPieces<SharedQ, WarpLayout, kD>;  // the same copy a load at a time (the next item's Q)
     using QFragments = SharedToRegLoader<RegQ, WarpLayout, WarpReuse::kRowReuseCont>;
     using PiecesK = GlobalToSharedDirectPieces<SharedK, WarpLayout, kD>;
-    using PiecesV = GlobalToSharedDirectPieces<SharedV, WarpLayout, kD>;
-    using KFragmentsNow = SharedToRegLoader<RegKAll, WarpLayout, WarpReuse::kColReuseCont>;
-    using KFragments = SharedToRegPieces<RegKAll, SharedKHalf, WarpLayout, WarpReuse::kColReuseCont>;
-    using VFragments = SharedToRegTrPieces<RegVAll, SharedVHalf, WarpLayout, WarpReuse::kColReuseCont, true>;
+    // (a column-major V: the lines of a tile are N elements apart in memory, a run-time size)
+    using PiecesV = GlobalToSharedDirectPieces<SharedV, WarpLayout, kVColMajor ? 0 : kD>;
+    using KFragments = SharedToRegPieces<RegKAll, SharedKHalf, WarpLayout, WarpReuse::kColReuseCont, kVColMajor>;
+    using VFragments = std::conditional_t<kVColMajor, SharedToRegPieces<RegVAll, SharedVHalf, WarpLayout, WarpReuse::kColReuseCont>,
+                                          SharedToRegTrPieces<RegVAll, SharedVHalf, WarpLayout, WarpReuse::kColReuseCont, true>>;
+    static constexpr int kReadsV = kVColMajor ? 1 : 2;  // LDS read instructions per V fragment
     using Scores = compute::ScheduledGemm<RegQ, RegK, RegS, compute::RegFile::kVgpr, compute::RegFile::kAgpr>;
     using Output = compute::ScheduledGemm<RegP, RegV, RegO, compute::RegFile::kAgpr, compute::RegFile::kVgpr>;
     using OutToShared = RegToSharedStorer<RegOut, WarpLayout>;
     using OutToGlobal = SharedToGlobalStorer<SharedO, WarpLayout>;
-    static_assert(PiecesK::kPieces == 4 && PiecesV::kPieces == 4, "a wavefront issues 8 loads per block, one per group");
+    static_assert(PiecesK::kPieces == 4 && PiecesV::kPieces == (kVColMajor ? 2 : 4), "a wavefront issues 8 loads per block, one per group");
     static_assert(PiecesQ::kPieces == 16, "a wavefront fetches its 64 query rows with 16 loads: two steps' worth");
     static_assert(kDSteps * kKeyTiles == 8 && kDTiles == 8, "a step has 8 groups: a K fragment and a V fragment each");
 };
@@ -181,17 +203,27 @@ __global__ void __launch_bounds__(Traits::kThreads)
     typename Traits::SharedQ sQ(rows_over_two_stages(st(3), st(4)));
 
     typename Traits::PiecesK pieces_k;
-    typename Traits::PiecesV pieces_v;
+    typename Traits::PiecesV pieces_v = [&] {
+        if constexpr (Traits::kVColMajor) return typename Traits::PiecesV(kN);
+        else return typename Traits::PiecesV();
+    }();
     typename Traits::KFragments k_frag;
     typename Traits::VFragments v_frag;
 
-    // load s of this wavefront for key block `block` into ring stage `stage`: 4 pieces of K, then 4 of V
-    auto block_load = [&](int stage, int block, int s) -> DirectLoad {
-        return s < 4 ? pieces_k.piece(s, Kh + size_t(block) * kTN * kD, ringK[stage])
-                     : pieces_v.piece(s - 4, Vh + size_t(block) * kTN * kD, ringV[stage]);
+    // load s of this wavefront for key block `block` of the operands `Kb`, `Vb` into ring stage `stage`: 4 pieces of K,
+    // then 4 of V
+    auto v_half = [&](int stage, int t) { return Traits::VHalf::at(ringV.stage_data(stage), t); };
+    auto load_of = [&](const InType* Kb, const InType* Vb, int stage, int block, int s) -> DirectLoad {
+        if (s < 4) return pieces_k.piece(s, Kb + size_t(block) * kTN * kD, ringK[stage]);
+        if constexpr (Traits::kVColMajor) {  // element (key, d) of V at Vb[d * kN + key]: two loads per half
+            const int t = (s - 4) >> 1;
+            return pieces_v.piece((s - 4) & 1, Vb + size_t(block) * kTN + t * Traits::kHalf, v_half(stage, t));
+        } else {
+            return pieces_v.piece(s - 4, Vb + size_t(block) * kTN * kD, ringV[stage]);
+        }
     };
+    auto block_load = [&](int stage, int block, int s) -> DirectLoad { return load_of(Kh, Vh, stage, block, s); };
     auto k_half = [&](int stage, int t) { return typename Traits::KHalves(ringK.stage_data(stage))(t); };
-    auto v_half = [&](int stage, int t) { return typename Traits::VHalves(ringV.stage_data(stage))(t); };
 
     // ---- prologue: Q and block 0 are requested together (the cold latencies overlap); blocks 1 and 2 under the
     // first two score computations, blocks 3 and 4 (into the stages Q passed through) in the first block-iteration
@@ -244,13 +276,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
     // wavefront's loads of block `load_block` behind the groups
     auto scores_only = [&](int stage, int t, auto buf_c, int load_block) {
         constexpr int kBuf = decltype(buf_c)::value;
-        typename Traits::KFragmentsNow read_k;
         const auto sk = k_half(stage, t);
         typename Traits::RegKAll kf;
-        read_k.load_one(sk, kf, 0, 0);
+        k_frag.template read<0, 0>(sk, kf);
         static_for<8>([&](auto g_c) {
             constexpr int g = decltype(g_c)::value, ds = g % 4, kt = g / 4;
-            if constexpr (g + 1 < 8) read_k.load_one(sk, kf, (g + 1) % 4, (g + 1) / 4);
+            if constexpr (g + 1 < 8) {
+                k_frag.template read<(g + 1) % 4, (g + 1) / 4>(sk, kf);
+                wait_shared_reads<1>();
+            } else {
+                wait_shared_reads<0>();
+            }
             RegK one;
             one(ds, 0) = kf(ds, kt);
             static_for<kQT>([&](auto c_c) {
@@ -304,7 +340,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         int a, b, c, load;
     };
     constexpr int kAhead = 3;
-    constexpr int kReadsV = 2, kReadsQk = 3;  // LDS read instructions per group
+    constexpr int kReadsV = Traits::kReadsV, kReadsQk = kReadsV + 1;  // LDS read instructions per group
     constexpr int kHalfBytes = Traits::kHalf * kD * int(sizeof(InType));  // between the halves of a K or V block
     constexpr int kStageBytes = 2 * Traits::kBlockNumel * int(sizeof(InType));
 
@@ -323,7 +359,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
         static_for<decltype(last_c)::value - decltype(first_c)::value>([&](auto i_c) {
             constexpr int f = decltype(first_c)::value + decltype(i_c)::value;
             k_frag.template shift<f % 4, f / 4>(dK);
-            v_frag.template shift<f>(dV);
+            if constexpr (Traits::kVColMajor) v_frag.template shift<0, f>(dV);
+            else v_frag.template shift<f>(dV);
         });
     };
 
@@ -399,7 +436,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
             } else if constexpr (kLoads == 3) {
                 Output::template at<0, g % 4, 0>(
                     rP[kNxt], rV, rO[g / 4],
-                    g < 4 ? pieces_k.piece(g, Knext, ringK[next_s0]) : pieces_v.piece(g - 4, Vnext, ringV[next_s0]));
+                    load_of(Knext, Vnext, next_s0, 0, g));
             } else {
                 Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
             }

@@ -145,5 +145,21 @@ struct LdsSwizzleTr {
     }
 };
 
+/// XOR permutation for tiles of 2-byte elements with 256-byte lines whose lines are read 16 at a time in DEALT order
+/// (copy::SharedToRegPieces<..., kDealtLines = true>): one pass of a 16-byte-per-lane read touches lines
+/// 8 q + 4 h + r (q, r = 0..3; h fixed), which the standard permutation (unit ^= line % 16) would send to only 8 different
+/// places. Here the 16-byte unit is XORed with 4 q + r: bits 3, 4 and 0, 1 of the line.
+template <const int kPitch, const int kElemBytes>
+struct LdsSwizzleDealt {
+    static_assert(kElemBytes == 2 && kPitch == 128, "written for lines of 256 bytes of 2-byte elements");
+    static constexpr int kUnit = 8;  // elements per 16-byte unit
+    static constexpr int kLinePeriod = 32;
+
+    HOST_DEVICE static constexpr int apply(int line, int elem) {
+        const int s = (((line >> 3) & 3) << 2) | (line & 3);
+        return (((elem / kUnit) ^ s) * kUnit) | (elem % kUnit);
+    }
+};
+
 }  // namespace tile_layout
 }  // namespace tiledcuda::cell

@@ -863,7 +863,8 @@ def test_flash_attention_tile_wave64_is_wave64(tcu, oracle, device, batch, M, N)
 
 @pytest.mark.parametrize("batch,M,N", [(3, 256, 320), (8, 256, 640), (2, 512, 1024), (5, 768, 448), (64, 2048, 2048),
                                        (203, 1024, 448), (96, 2048, 384), (330, 256, 640)])
-def test_flash_attention_wave64_k32(tcu, oracle, device, batch, M, N):
+@pytest.mark.parametrize("v_col_major", [False, True])
+def test_flash_attention_wave64_k32(tcu, oracle, device, batch, M, N, v_col_major):
     """The one-wavefront-per-SIMD design on the 16x16x32 matrix instruction (wave64_k32): against the oracle on whole
     heads at small sizes and on a sample of rows at the benchmark size, and against the 32x32x16 kernel everywhere (same
     arithmetic up to the order of the sums inside a matrix instruction); at 5 key blocks (the minimum), an odd number of
@@ -873,7 +874,7 @@ def test_flash_attention_wave64_k32(tcu, oracle, device, batch, M, N):
     import torch
 
     D = 128
-    print(f"attention wave64_k32 b{batch} {M}x{N}", flush=True)
+    print(f"attention wave64_k32 b{batch} {M}x{N} v_col_major={v_col_major}", flush=True)
     q = oracle.fill_normal(batch * M * D, 91).reshape(batch, M, D).astype(np.float32)
     k = oracle.fill_normal(batch * N * D, 92).reshape(batch, N, D).astype(np.float32)
     v = oracle.fill_normal(batch * N * D, 93).reshape(batch, N, D)
@@ -885,7 +886,13 @@ def test_flash_attention_wave64_k32(tcu, oracle, device, batch, M, N):
     dq, dk, dv = dev(q, device), dev(k, device), dev(v, device)
     ref_kernel = tcu.flash_attention(dq, dk, dv, algo="wave64")
     out = torch.full_like(ref_kernel, float("nan"))
-    tcu.flash_attention(dq, dk, dv, out=out, algo="wave64_k32")
+    if v_col_major:
+        # V as the reference op takes it: the array V^T [D, N] per batch item
+        dvt = dv.transpose(1, 2).contiguous()
+        tcu.flash_attention_fwd(dq.view(-1), dk.view(-1), dvt.view(-1), out.view(-1), M, N, D, D, scale=1.0 / math.sqrt(D),
+                                batch=batch, algo="wave64_k32")
+    else:
+        tcu.flash_attention(dq, dk, dv, out=out, algo="wave64_k32")
     torch.cuda.synchronize()
     tol = 2e-2 if N == 640 else ABS_TOL
     assert torch.isfinite(out).all()

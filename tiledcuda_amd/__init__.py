@@ -211,19 +211,20 @@ def b2b_gemm(a: torch.Tensor, b_t: torch.Tensor, c_t: torch.Tensor, out: torch.T
 
 # ------------------------------------------------------------------------------ attention
 def flash_attention_fwd(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, O: torch.Tensor, m: int, n: int, k: int,
-                        p: int, scale: float = 1.0, batch: int = 1) -> None:
+                        p: int, scale: float = 1.0, batch: int = 1, algo: str = "auto") -> None:
     """Same call shape as the reference's ``pytiledcuda.flash_attention_fwd`` (flattened fp16
     device tensors; K as [n, k], V as [p, n]; O written in place; ``scale`` defaults to the
-    reference's 1).  Unsupported shapes raise ``RuntimeError`` like the reference op."""
+    reference's 1; ``algo`` picks a kernel, as in ``flash_attention``).  Unsupported shapes raise
+    ``RuntimeError`` like the reference op."""
     if min(m, n, k, p, batch) <= 0:
         raise ValueError("m, n, k, p and batch must be positive")
     for name, t, want in (("Q", Q, batch * m * k), ("K", K, batch * n * k), ("V", V, batch * p * n),
                           ("O", O, batch * m * p)):
         if t.numel() != want:
             raise ValueError(f"{name} must hold batch*rows*cols = {want} elements, got {t.numel()}")
-    _check(lib().tcu_flash_attn_fwd_f16(_dev_ptr(Q, torch.float16, "Q"), _dev_ptr(K, torch.float16, "K"),
-                                        _dev_ptr(V, torch.float16, "V"), _dev_ptr(O, torch.float16, "O"), batch, m, n,
-                                        k, p, float(scale), TCU_V_COL_MAJOR, _stream()))
+    _check(lib().tcu_flash_attn_fwd_f16_algo(_dev_ptr(Q, torch.float16, "Q"), _dev_ptr(K, torch.float16, "K"),
+                                             _dev_ptr(V, torch.float16, "V"), _dev_ptr(O, torch.float16, "O"), batch, m,
+                                             n, k, p, float(scale), TCU_V_COL_MAJOR, ATTN_ALGOS[algo], _stream()))
 
 
 def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float | None = None,

@@ -583,16 +583,12 @@ int fa_tile_w64_dispatch(const __half* Q, const __half* K, const __half* V, __ha
                                            "(M, N) in {(2048, 2048), (512, 1024), (256, 640), (256, 320)}");
 }
 
-/// The one-wavefront-per-SIMD kernel on the 16x16x32 instruction (tile-library functors, run-time M and N).
-int fa_w64_k32_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, int Kd,
-                        float scale, int v_layout, hipStream_t stream) {
-    using Traits = FlashW64K32Traits<__half, 128>;
-    if (Kd != 128 || v_layout != TCU_V_ROW_MAJOR)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel takes head size 128 and a row-major V");
-    if (M % Traits::kTM != 0 || N < Traits::kStages * Traits::kTN)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel needs M % 256 == 0 and N >= 320");
-    if ((long)N * 256 >= (1l << 32))
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel addresses a V block with 32-bit offsets");
+/// The one-wavefront-per-SIMD kernel on the 16x16x32 instruction (tile-library functors, run-time M and N, either V
+/// layout).
+template <bool kVColMajor>
+int launch_fa_w64_k32(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
+                      hipStream_t stream) {
+    using Traits = FlashW64K32Traits<__half, 128, kVColMajor>;
     // one workgroup per CU; a workgroup with more than one item fetches the next one's first operands under the last
     // steps of the current one. Items keep their XCD (item number modulo 8) only if the grid is a multiple of 8.
     int device = 0, cus = 0;
@@ -603,6 +599,19 @@ int fa_w64_k32_dispatch(const __half* Q, const __half* K, const __half* V, __hal
     const long grid = std::min<long>(items, cus - cus % 8);
     return launch(&flash_attention_w64_k32<__half, Traits>, dim3(unsigned(grid)), dim3(Traits::kThreads),
                   Traits::kShmBytes, stream, Q, K, V, O, batch, M, N, scale);
+}
+
+int fa_w64_k32_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, int Kd,
+                        float scale, int v_layout, hipStream_t stream) {
+    using Traits = FlashW64K32Traits<__half, 128>;
+    if (Kd != 128)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel is instantiated for head size 128");
+    if (M % Traits::kTM != 0 || N < Traits::kStages * Traits::kTN)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel needs M % 256 == 0 and N >= 320");
+    if ((long)N * 256 >= (1l << 32))
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel addresses a V block with 32-bit offsets");
+    return v_layout == TCU_V_ROW_MAJOR ? launch_fa_w64_k32<false>(Q, K, V, O, batch, M, N, scale, stream)
+                                       : launch_fa_w64_k32<true>(Q, K, V, O, batch, M, N, scale, stream);
 }
 
 template <int kD, bool kFused>
@@ -653,7 +662,12 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     }
     // column-major V (the reference op's convention), any N % 64 == 0
     if (Kd != 128) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for head size 128");
-    if (algo == TCU_ATTN_AUTO) return launch_fa_w64<true>(Q, K, V, O, batch, M, N, scale, stream);
+    if (algo == TCU_ATTN_AUTO) {
+        // long sequences with enough query blocks to fill the chip: the 16x16x32 kernel, as for a row-major V
+        if (M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 128)
+            return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
+        return launch_fa_w64<true>(Q, K, V, O, batch, M, N, scale, stream);
+    }
     // the kernel composed from tile primitives has the leading dimension of V (= N) as a compile-time constant, like
     // the reference op: one instantiation per N
     switch (N) {
