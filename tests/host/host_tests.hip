@@ -240,6 +240,38 @@ static void test_swizzle_tr8() {
     }
 }
 
+// The permutation for tiles whose lines are read 16 at a time in dealt order (lines 8 q + 4 h + r of a group of 32, h
+// fixed per read): a bijection per line that keeps 16-byte units whole and repeats every 32 lines, and every pass of a
+// 16-byte-per-lane read (16 lanes, one 16-byte unit column) touches 64 distinct banks.
+static void test_swizzle_dealt() {
+    constexpr int kPitch = 128;
+    using Swz = tl::LdsSwizzleDealt<kPitch, 2>;
+    CHECK(Swz::kLinePeriod == 32);
+    for (int line = 0; line < 64; ++line) {
+        std::set<int> seen;
+        for (int e = 0; e < kPitch; ++e) {
+            const int p = Swz::apply(line, e);
+            CHECK(p >= 0 && p < kPitch);
+            seen.insert(p);
+            if (e % 8 == 0)
+                for (int t = 1; t < 8; ++t) CHECK(Swz::apply(line, e + t) == p + t);
+            CHECK(Swz::apply(line + 32, e) == p);
+        }
+        CHECK(int(seen.size()) == kPitch);
+    }
+    for (int pair = 0; pair < 2; ++pair)
+        for (int h = 0; h < 2; ++h)
+            for (int unit = 0; unit < 16; ++unit) {
+                std::set<int> banks;
+                for (int lane = 0; lane < 16; ++lane) {
+                    const int line = 32 * pair + 8 * (lane / 4) + 4 * h + lane % 4;
+                    const int byte = (line * kPitch + Swz::apply(line, unit * 8)) * 2;
+                    for (int b = 0; b < 16; b += 4) banks.insert(((byte + b) / 4) % 64);
+                }
+                CHECK(int(banks.size()) == 64);
+            }
+}
+
 // A ring whose stages are further apart than a tile (two rings interleaved in one allocation).
 static void test_strided_ring() {
     using Shared = SharedTile<__half, tl::RowMajor<64, 128>, true>;
@@ -352,6 +384,7 @@ int main() {
     test_swizzle_tr<128>();
     test_swizzle_tr<64>();
     test_swizzle_tr8();
+    test_swizzle_dealt();
     test_strided_ring();
     test_swizzle<16, 4>(true);
     test_swizzle<32, 4>(true);
