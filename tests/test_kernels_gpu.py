@@ -862,7 +862,7 @@ def test_flash_attention_tile_wave64_is_wave64(tcu, oracle, device, batch, M, N)
 
 
 @pytest.mark.parametrize("batch,M,N", [(3, 256, 320), (8, 256, 640), (2, 512, 1024), (5, 768, 448), (64, 2048, 2048),
-                                       (203, 1024, 448), (96, 2048, 384), (330, 256, 640)])
+                                       (203, 1024, 448), (96, 2048, 384), (330, 256, 640), (1300, 256, 320)])
 @pytest.mark.parametrize("v_col_major", [False, True])
 def test_flash_attention_wave64_k32(tcu, oracle, device, batch, M, N, v_col_major):
     """The one-wavefront-per-SIMD design on the 16x16x32 matrix instruction (wave64_k32): against the oracle on whole
