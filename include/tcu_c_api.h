@@ -85,7 +85,8 @@ typedef enum {
 } tcu_v_layout;
 
 /* Which attention kernel to run (tcu_flash_attn_fwd_f16_algo). For a row-major V, AUTO picks WAVE64_K32 for long sequences
- * (head size 128, M % 256 == 0, N >= 1024, at least 128 blocks of 256 queries) and MFMA32_FUSED otherwise; for a
+ * (head size 128, M % 256 == 0, N >= 1024) with at least 256 blocks of 256 queries, WAVE64 with 128 to 255 such blocks,
+ * and MFMA32_FUSED otherwise; for a
  * column-major V (head size 128) AUTO picks WAVE64_K32 under the same conditions and WAVE64 otherwise (it takes every
  * M % 64 == 0 and N % 64 == 0). */
 typedef enum {

@@ -643,8 +643,11 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     if (v_layout == TCU_V_ROW_MAJOR && algo != TCU_ATTN_TILE_LIBRARY) {
         if (Kd != 128 && Kd != 64) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
         // long sequences with enough query blocks to fill the chip: the kernel with 64 queries per wavefront
+        // (with at least one block of 256 queries per CU the chip runs at its power limit, where the 16x16x32 instruction
+        // wins; a half-empty chip runs at full clock, where the 32x32x16 kernel's fewer issue cycles do)
         if (algo == TCU_ATTN_AUTO && Kd == 128 && M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 128)
-            return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
+            return (long)batch * (M / 256) >= 256 ? fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream)
+                                                  : launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream);
         if (algo == TCU_ATTN_MFMA32)
             return Kd == 128 ? fa_fwd_by_rows<128, false>(Q, K, V, O, batch, M, N, scale, stream)
                              : fa_fwd_by_rows<64, false>(Q, K, V, O, batch, M, N, scale, stream);
@@ -664,7 +667,7 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     if (Kd != 128) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for head size 128");
     if (algo == TCU_ATTN_AUTO) {
         // long sequences with enough query blocks to fill the chip: the 16x16x32 kernel, as for a row-major V
-        if (M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 128)
+        if (M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 256)
             return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
         return launch_fa_w64<true>(Q, K, V, O, batch, M, N, scale, stream);
     }
