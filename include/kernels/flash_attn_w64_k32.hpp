@@ -10,8 +10,8 @@
 //   (ds_read_b128, K) and SharedToRegTrPieces (ds_read_b64_tr_b16, V, in the order in which two 16 x 16 score
 //   accumulators hold their keys, so that the converted scores ARE the A operand of the second product) with addresses
 //   bound to the ring stage (bind / read_bound_to / shift: no addition in front of a read), awaited with
-//   wait_shared_reads<N>(); the softmax of 32 keys is sliced over the 64 matrix instructions of the neighbouring 32 -
-//   a v_exp_f32 behind every second one, the sums and conversions behind the others (compute::Exp2Raw,
+//   wait_shared_reads<N>(); the softmax of 32 keys is sliced over the 64 matrix instructions of the neighbouring 32 (at
+//   head size 128) - a v_exp_f32 behind every second one, the sums and conversions behind the others (compute::Exp2Raw,
 //   convert_pair_here); stages are handed over with wait_group_and_barrier_keep_reads<N>(); the last three steps fetch
 //   what the next workgroup on the XCD will ask for first; the output leaves through RegToSharedStorer /
 //   SharedToGlobalStorer.
@@ -23,9 +23,10 @@
 // maximum that moves only when a partial sum could leave f16 range, f32 sums and output); the sums inside a matrix
 // instruction cover 32 instead of 16 indices and the final division is a reciprocal and a product, so results differ
 // from that kernel in the last bits.
-// Requirements: head size 128, M % 256 == 0, N % 64 == 0, N >= 320 (Q passes through two ring stages before the fifth
-// block needs them); V row-major [N, D] or column-major (the reference op's convention; see the traits). M, N and the
-// batch count are run-time values.
+// Requirements: head size 128 (V row-major [N, D] or column-major, the reference op's convention; see the traits) or 64
+// (row-major V; a step then has 32 matrix instructions for the same softmax work and every one carries an exponential),
+// M % 256 == 0, N % 64 == 0, N >= 320 (Q passes through two ring stages before the fifth block needs them). M, N and
+// the batch count are run-time values.
 #pragma once
 
 #include <type_traits>
@@ -53,13 +54,15 @@ struct FlashW64K32Traits {
     using WarpLayout = tl::RowMajor<4, 1>;
     static constexpr int kWaves = 4, kThreads = kWaves * kWaveSize;
     static constexpr int kTM = 64 * kWaves, kTN = 64, kHalf = 32, kStages = 5;
-    static_assert(kD == 128, "the step schedule is written for head size 128");
+    static_assert(kD == 128 || (kD == 64 && !kVColMajor), "the step schedule is written for head sizes 128 and 64 (row-major V)");
 
     using Shape = traits::MfmaTileShape<InType, traits::MfmaShape::k16x16x32>;
     static constexpr int kQTiles = 64 / 16;     // 16-row query tiles of a wavefront
     static constexpr int kKeyTiles = kHalf / 16;  // 16-key tiles of a half
     static constexpr int kDSteps = kD / 32;     // contraction steps of S = Q Kᵀ
     static constexpr int kDTiles = kD / 16;     // 16-column tiles of O
+    static constexpr int kGroups = kDSteps * kKeyTiles;  // groups of a step: a K fragment and a V fragment each (8 or 4)
+    static constexpr int kKtPerReg = 4 / kDSteps;         // key tiles that the ring of 4 K fragments spans (1 or 2)
 
     // global views of one query block / key block
     using GlobalQ = GlobalTile<InType, tl::RowMajor<kTM, kD>>;
@@ -77,7 +80,7 @@ struct FlashW64K32Traits {
     using RingV = SharedRing<SharedV, kStages, 2 * kBlockNumel>;
     using SharedQ = SharedTile<InType, tl::RowMajor<kTM, kD>, true>;
     using SharedO = SharedTile<InType, tl::RowMajor<kTM, kD>, true>;
-    static constexpr int kShmBytes = kStages * 2 * kBlockNumel * int(sizeof(InType));  // 160 KiB
+    static constexpr int kShmBytes = kStages * 2 * kBlockNumel * int(sizeof(InType));  // 160 KiB (80 at head size 64)
     static_assert(kShmBytes <= kMaxLdsBytes && 2 * 2 * kBlockNumel == kTM * kD, "Q fills exactly two stages");
 
     // the 32-key halves a step works on
@@ -97,14 +100,14 @@ struct FlashW64K32Traits {
 
     // register tiles of one wavefront (64 queries)
     using RegQ = RegTile<typename Shape::TileA, tl::RowMajor<kQTiles, kDSteps>>;     // A of S = Q Kᵀ, in AGPRs
-    using RegK = RegTile<typename Shape::TileB, tl::ColMajor<kDSteps, 1>>;           // B of S: a ring of 4 fragments
+    using RegK = RegTile<typename Shape::TileB, tl::ColMajor<kDSteps, kKtPerReg>>;   // B of S: a ring of 4 fragments
     using RegKAll = RegTile<typename Shape::TileB, tl::ColMajor<kDSteps, kKeyTiles>>; // what the fragment loader addresses
-    using RegS = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, 1>>;         // scores of 16 keys
+    using RegS = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, kKtPerReg>>; // scores of 16 (or 32) keys
     using RegM = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, 1>>;         // where the score sums start
     using RegP = RegTile<typename Shape::TileA, tl::RowMajor<kQTiles, 1>>;           // probabilities: A of O += P V
     using RegV = RegTile<typename Shape::TileB, tl::ColMajor<1, 4>>;                 // B of O += P V: a ring of 4 fragments
     using RegVAll = RegTile<typename Shape::TileB, tl::ColMajor<1, kDTiles>>;
-    using RegO = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, 4>>;         // half of the head size; in AGPRs
+    using RegO = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kQTiles, 4>>;         // 4 of the head size's 16-column tiles; in AGPRs
     using RegOut = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kQTiles, kDTiles>>;
 
     using QLoader = GlobalToSharedDirectLoader<SharedQ, WarpLayout>;
@@ -121,9 +124,11 @@ struct FlashW64K32Traits {
     using Output = compute::ScheduledGemm<RegP, RegV, RegO, compute::RegFile::kAgpr, compute::RegFile::kVgpr>;
     using OutToShared = RegToSharedStorer<RegOut, WarpLayout>;
     using OutToGlobal = SharedToGlobalStorer<SharedO, WarpLayout>;
-    static_assert(PiecesK::kPieces == 4 && PiecesV::kPieces == (kVColMajor ? 2 : 4), "a wavefront issues 8 loads per block, one per group");
-    static_assert(PiecesQ::kPieces == 16, "a wavefront fetches its 64 query rows with 16 loads: two steps' worth");
-    static_assert(kDSteps * kKeyTiles == 8 && kDTiles == 8, "a step has 8 groups: a K fragment and a V fragment each");
+    static constexpr int kLoadsK = PiecesK::kPieces;  // of a wavefront, per block: then as many of V
+    static_assert(2 * kLoadsK == kGroups && PiecesV::kPieces == (kVColMajor ? kLoadsK / 2 : kLoadsK),
+                  "a wavefront issues one load per group of the step that loads a block");
+    static_assert(PiecesQ::kPieces == 2 * kGroups, "a wavefront fetches its 64 query rows with two steps' worth of loads");
+    static_assert(kDTiles == kGroups && (kGroups == 8 || kGroups == 4), "a step has 8 or 4 groups: a K fragment and a V fragment each");
 };
 
 /// grid = min((M / 256) * batch, number of CUs) workgroups (1-D), block = 256, dynamic LDS = Traits::kShmBytes. A workgroup
@@ -135,6 +140,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
                             float scale) {
     constexpr int kD = Traits::kD, kTN = Traits::kTN;
     constexpr int kQT = Traits::kQTiles, kDT = Traits::kDTiles, kStages = Traits::kStages;
+    constexpr int kDS = Traits::kDSteps, kG = Traits::kGroups, kKtPerReg = Traits::kKtPerReg;
+    constexpr int kSRegs = 2 / kKtPerReg, kORegs = kDT / 4;  // register tiles that hold a half's scores / the output
     using RegQ = typename Traits::RegQ;
     using RegK = typename Traits::RegK;
     using RegS = typename Traits::RegS;
@@ -210,16 +217,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
     typename Traits::KFragments k_frag;
     typename Traits::VFragments v_frag;
 
-    // load s of this wavefront for key block `block` of the operands `Kb`, `Vb` into ring stage `stage`: 4 pieces of K,
-    // then 4 of V
+    // load s of this wavefront for key block `block` of the operands `Kb`, `Vb` into ring stage `stage`: the pieces of K,
+    // then as many of V
     auto v_half = [&](int stage, int t) { return Traits::VHalf::at(ringV.stage_data(stage), t); };
     auto load_of = [&](const InType* Kb, const InType* Vb, int stage, int block, int s) -> DirectLoad {
-        if (s < 4) return pieces_k.piece(s, Kb + size_t(block) * kTN * kD, ringK[stage]);
+        constexpr int kLK = Traits::kLoadsK;
+        if (s < kLK) return pieces_k.piece(s, Kb + size_t(block) * kTN * kD, ringK[stage]);
         if constexpr (Traits::kVColMajor) {  // element (key, d) of V at Vb[d * kN + key]: two loads per half
-            const int t = (s - 4) >> 1;
-            return pieces_v.piece((s - 4) & 1, Vb + size_t(block) * kTN + t * Traits::kHalf, v_half(stage, t));
+            const int t = (s - kLK) >> 1;
+            return pieces_v.piece((s - kLK) & 1, Vb + size_t(block) * kTN + t * Traits::kHalf, v_half(stage, t));
         } else {
-            return pieces_v.piece(s - 4, Vb + size_t(block) * kTN * kD, ringV[stage]);
+            return pieces_v.piece(s - kLK, Vb + size_t(block) * kTN * kD, ringV[stage]);
         }
     };
     auto block_load = [&](int stage, int block, int s) -> DirectLoad { return load_of(Kh, Vh, stage, block, s); };
@@ -232,7 +240,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         typename Traits::GlobalQ gQ(Qb);
         load_q(gQ, sQ);
 #pragma unroll
-        for (int s = 0; s < 8; ++s) issue(block_load(st(0), 0, s));
+        for (int s = 0; s < kG; ++s) issue(block_load(st(0), 0, s));
         wait_group_and_barrier<0>();
     }
 
@@ -253,15 +261,15 @@ __global__ void __launch_bounds__(Traits::kThreads)
         compute::pin_tiles<compute::RegFile::kAgpr>(rQ);
     }
 
-    RegO rO[2];     // d tiles 0..3 and 4..7
-    compute::clear_pinned(rO[0]);
-    compute::clear_pinned(rO[1]);
+    RegO rO[kORegs];  // d tiles 0..3 (and 4..7)
+#pragma unroll
+    for (int h = 0; h < kORegs; ++h) compute::clear_pinned(rO[h]);
 
-    RegS rS[2][2];  // [half buffer][key tile]: score tiles of two consecutive halves, relative to the reference maximum
+    RegS rS[2][kSRegs];  // [half buffer][key tile / kKtPerReg]: score tiles of two consecutive halves, relative to the reference maximum
     RegP rP[2];     // their probabilities
     RegM neg_max;   // minus the reference maximum of this lane's query of each tile, in all 4 slots
     float m_run[kQT], l_run[kQT];
-    RegK rK;        // ring of the fragments in flight / in use: fragment g lives in tile g % 4
+    RegK rK;        // ring of the fragments in flight / in use: fragment g lives in tile g % 4 (column-major order)
     RegV rV;
 
     compute::Exp2Raw<float> exp2;
@@ -279,20 +287,20 @@ __global__ void __launch_bounds__(Traits::kThreads)
         const auto sk = k_half(stage, t);
         typename Traits::RegKAll kf;
         k_frag.template read<0, 0>(sk, kf);
-        static_for<8>([&](auto g_c) {
-            constexpr int g = decltype(g_c)::value, ds = g % 4, kt = g / 4;
-            if constexpr (g + 1 < 8) {
-                k_frag.template read<(g + 1) % 4, (g + 1) / 4>(sk, kf);
+        static_for<kG>([&](auto g_c) {
+            constexpr int g = decltype(g_c)::value, ds = g % kDS, kt = g / kDS;
+            if constexpr (g + 1 < kG) {
+                k_frag.template read<(g + 1) % kDS, (g + 1) / kDS>(sk, kf);
                 wait_shared_reads<1>();
             } else {
                 wait_shared_reads<0>();
             }
             RegK one;
-            one(ds, 0) = kf(ds, kt);
+            one(ds, kt % kKtPerReg) = kf(ds, kt);
             static_for<kQT>([&](auto c_c) {
                 constexpr int c = decltype(c_c)::value;
-                if constexpr (ds == 0) Scores::template at_from<c, 0, 0>(rQ, one, rS[kBuf][kt], neg_max(c, 0));
-                else Scores::template at<c, 0, ds>(rQ, one, rS[kBuf][kt]);
+                if constexpr (ds == 0) Scores::template at_from<c, kt % kKtPerReg, 0>(rQ, one, rS[kBuf][kt / kKtPerReg], neg_max(c, 0));
+                else Scores::template at<c, kt % kKtPerReg, ds>(rQ, one, rS[kBuf][kt / kKtPerReg]);
             });
             issue(block_load(st(load_block), load_block, g));
         });
@@ -309,6 +317,9 @@ __global__ void __launch_bounds__(Traits::kThreads)
         return (p0 + p1) + (p2 + p3);
     };
 
+    // score tile (query tile c, key tile kt) of a half
+    auto s_tile = [&](RegS(&rs)[kSRegs], int c, int kt) -> BaseTileRowMajor<float>& { return rs[kt / kKtPerReg](c, kt % kKtPerReg); };
+
     // ---- half 0: exact maxima
 #pragma unroll
     for (int c = 0; c < kQT; ++c)
@@ -317,19 +328,19 @@ __global__ void __launch_bounds__(Traits::kThreads)
     compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
     scores_only(st(0), 0, std::integral_constant<int, 0>{}, 1);
     asm volatile("s_nop 15\n\ts_nop 3");
-    compute::pin_tiles<compute::RegFile::kVgpr>(rS[0][0]);
-    compute::pin_tiles<compute::RegFile::kVgpr>(rS[0][1]);
+#pragma unroll
+    for (int h = 0; h < kSRegs; ++h) compute::pin_tiles<compute::RegFile::kVgpr>(rS[0][h]);
 #pragma unroll
     for (int c = 0; c < kQT; ++c) {
-        float mx = rS[0][0](c, 0)(0, 0);
+        float mx = s_tile(rS[0], c, 0)(0, 0);
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, rS[0][kt](c, 0)(0, e));
+            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, s_tile(rS[0], c, kt)(0, e));
         mx = row_max(mx);
         m_run[c] = mx;
         _Float16* p = reinterpret_cast<_Float16*>(rP[0](c, 0).mutable_data());
-        l_run[c] = tile_softmax_now(rS[0][0](c, 0), mx, p) + tile_softmax_now(rS[0][1](c, 0), mx, p + 4);
+        l_run[c] = tile_softmax_now(s_tile(rS[0], c, 0), mx, p) + tile_softmax_now(s_tile(rS[0], c, 1), mx, p + 4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) neg_max(c, 0)(0, e) = -mx;
     }
@@ -358,7 +369,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         const int dK = (ring.c - ring.b) * kStageBytes, dV = (ring.b - ring.a) * kStageBytes;
         static_for<decltype(last_c)::value - decltype(first_c)::value>([&](auto i_c) {
             constexpr int f = decltype(first_c)::value + decltype(i_c)::value;
-            k_frag.template shift<f % 4, f / 4>(dK);
+            k_frag.template shift<f % kDS, f / kDS>(dK);
             if constexpr (Traits::kVColMajor) v_frag.template shift<0, f>(dV);
             else v_frag.template shift<f>(dV);
         });
@@ -367,99 +378,169 @@ __global__ void __launch_bounds__(Traits::kThreads)
     // ---- one pipelined step on half i: softmax of half i (rS[kCur] -> rP[kCur]), scores of half i + 1 into rS[kNxt]
     // (if kQk), O += P V with half i - 1 (rP[kNxt]). ring: stages of blocks J, J + 1, J + 2 and of the block being
     // loaded. kLoads: 0 none, 1 block `load_block`, 2 / 4 / 3 the next item's Q (first, second half) / first block.
-    // A step is 8 groups of 8 matrix instructions: group g multiplies K fragment g (d-step g % 4 of key tile g / 4) with
-    // the 4 query tiles, then V fragment g (d tile g) with the 4 probability tiles, and takes score tile (g / 2, g % 2)
-    // of half i through the softmax. The fragments of group g + kAhead are requested inside group g (K behind the
-    // fourth, V behind the eighth matrix instruction), through addresses bound to the ring stage (no addition per
-    // read). What goes between two matrix instructions is measured, not guessed: every matrix instruction is followed
+    // A step is kG = 8 (head size 128) or 4 (64) groups of 8 matrix instructions: group g multiplies K fragment g (d-step
+    // g % kDS of key tile g / kDS) with the 4 query tiles, then V fragment g (d tile g) with the 4 probability tiles, and
+    // takes 32 / kG score values of half i through the softmax: score tile (query tile g / 2, key tile g % 2) with 8
+    // groups, both key tiles of query tile g with 4. The fragments of group g + kAhead are requested inside group g (K
+    // behind the fourth, V behind the eighth matrix instruction), through addresses bound to the ring stage (no
+    // addition per read). What goes between two matrix instructions is measured, not guessed: every matrix instruction is followed
     // by its dose in this order (the barriers keep the compiler from pairing the matrix instructions up), and the doses
     // come in pairs of issue slots - a v_exp_f32 counts as two, everything else as one; a pair costs 4 cycles on top of
-    // the matrix instruction's 16, a single slot costs as much, three or four cost 8.
+    // the matrix instruction's 16, a single slot costs as much, three or four cost 8. With 4 groups every matrix
+    // instruction has an exponential to carry, and its dose is four slots (the exponential, the addition of the one before
+    // to the sum, and a conversion or a fragment read).
     auto step = [&](const Stages& ring, auto cur_c, auto qk_c, auto loads_c, auto next_qk_c, int load_block) {
         constexpr int kCur = decltype(cur_c)::value, kNxt = kCur ^ 1;
         constexpr bool kQk = decltype(qk_c)::value, kNextQk = decltype(next_qk_c)::value;
         constexpr int kLoads = decltype(loads_c)::value;
         float lh[kQT] = {0.f, 0.f, 0.f, 0.f};
-        float x0 = 0.f, x1 = 0.f, x2 = 0.f, x3 = 0.f;
-        static_for<8>([&](auto g_c) {
+        float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I3 = std::integral_constant<int, 3>;
+        static_for<kG>([&](auto g_c) {
             constexpr int g = decltype(g_c)::value;
-            constexpr int gp = g + kAhead, f = gp % 8;
+            constexpr int gp = g + kAhead, f = gp % kG;
             // the fragments of group g + kAhead: halves 0 of the blocks in the first step of a block-iteration
             // (kCur == 1) until the step's end, halves 1 afterwards
-            constexpr int kImm = ((gp < 8) == (kCur == 1)) ? 0 : kHalfBytes;
-            constexpr bool kReadK = gp < 8 ? kQk : kNextQk;
+            constexpr int kImm = ((gp < kG) == (kCur == 1)) ? 0 : kHalfBytes;
+            constexpr bool kReadK = gp < kG ? kQk : kNextQk;
             // reads in flight that are younger than the fragments of this group and the next, at the top of the group
             // (the requests of this group are not yet issued): one wait per two groups
             constexpr int kPerGroup = kQk ? kReadsQk : kReadsV, kPerGroupNext = kNextQk ? kReadsQk : kReadsV;
-            constexpr int kYounger = gp < 8 ? (kAhead - 1) * kPerGroup : (7 - g) * kPerGroup + (gp - 8) * kPerGroupNext;
+            constexpr int kYounger = gp < kG ? (kAhead - 1) * kPerGroup : (kG - 1 - g) * kPerGroup + (gp - kG) * kPerGroupNext;
             if constexpr (g % 2 == 0) wait_shared_reads<kYounger - kPerGroup>();
-            constexpr int ds = g % 4, kt = g / 4;   // the K fragment of this group
-            constexpr int sc = g / 2, st = g % 2;   // the score tile of half i this group takes through the softmax
-            const auto& sv4 = rS[kCur][st](sc, 0);
-            _Float16* pdst = reinterpret_cast<_Float16*>(rP[kCur](sc, 0).mutable_data()) + 4 * st;
-            _Float16* pprev = reinterpret_cast<_Float16*>(rP[kCur]((g + 7) % 8 / 2, 0).mutable_data()) + 4 * ((g + 7) % 2);
+            constexpr int ds = g % kDS, kt = g / kDS;  // the K fragment of this group
             auto score = [&](auto c_c) {
                 constexpr int c = decltype(c_c)::value;
                 if constexpr (kQk) {
-                    if constexpr (ds == 0) Scores::template at_from<c, 0, 0>(rQ, rK, rS[kNxt][kt], neg_max(c, 0));
-                    else Scores::template at<c, 0, ds>(rQ, rK, rS[kNxt][kt]);
+                    if constexpr (ds == 0) Scores::template at_from<c, kt % kKtPerReg, 0>(rQ, rK, rS[kNxt][kt / kKtPerReg], neg_max(c, 0));
+                    else Scores::template at<c, kt % kKtPerReg, ds>(rQ, rK, rS[kNxt][kt / kKtPerReg]);
                 }
             };
-            using I0 = std::integral_constant<int, 0>;
-            using I1 = std::integral_constant<int, 1>;
-            using I2 = std::integral_constant<int, 2>;
-            using I3 = std::integral_constant<int, 3>;
-            score(I0{});
-            __builtin_amdgcn_sched_barrier(0);
-            x0 = exp2(sv4(0, 0));
-            __builtin_amdgcn_sched_barrier(0);
-            score(I1{});
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (g > 0) {  // the second pair of the group before
-                compute::convert_pair_here(x2, x3, reinterpret_cast<__half*>(pprev) + 2);
-                lh[(g - 1) / 2] += x3;
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            score(I2{});
-            __builtin_amdgcn_sched_barrier(0);
-            x1 = exp2(sv4(0, 1));
-            __builtin_amdgcn_sched_barrier(0);
-            score(I3{});
-            __builtin_amdgcn_sched_barrier(0);
-            lh[sc] += x0;
-            if constexpr (kReadK) k_frag.template read_bound_to<f % 4, f / 4, kImm>(rK(f % 4, 0));
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (kLoads == 1) {
-                Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4], block_load(ring.load, load_block, g));
-            } else if constexpr (kLoads == 2 || kLoads == 4) {
-                Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4], pieces_q.piece(kLoads == 2 ? g : 8 + g, Qnext, sQnext));
-            } else if constexpr (kLoads == 3) {
-                Output::template at<0, g % 4, 0>(
-                    rP[kNxt], rV, rO[g / 4],
-                    load_of(Knext, Vnext, next_s0, 0, g));
+            auto read_k = [&]() {
+                if constexpr (kReadK) k_frag.template read_bound_to<f % kDS, f / kDS, kImm>(rK(f % kDS, (f / kDS) % kKtPerReg));
+            };
+            // the first matrix instruction of O += P V carries this group's load
+            auto output0 = [&]() {
+                if constexpr (kLoads == 1) {
+                    Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4], block_load(ring.load, load_block, g));
+                } else if constexpr (kLoads == 2 || kLoads == 4) {
+                    Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4], pieces_q.piece(kLoads == 2 ? g : kG + g, Qnext, sQnext));
+                } else if constexpr (kLoads == 3) {
+                    Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4], load_of(Knext, Vnext, next_s0, 0, g));
+                } else {
+                    Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
+                }
+            };
+            if constexpr (kG == 8) {
+                constexpr int sc = g / 2, st = g % 2;  // the score tile of half i this group takes through the softmax
+                const auto& sv4 = rS[kCur][st](sc, 0);
+                _Float16* pdst = reinterpret_cast<_Float16*>(rP[kCur](sc, 0).mutable_data()) + 4 * st;
+                _Float16* pprev = reinterpret_cast<_Float16*>(rP[kCur]((g + 7) % 8 / 2, 0).mutable_data()) + 4 * ((g + 7) % 2);
+                score(I0{});
+                __builtin_amdgcn_sched_barrier(0);
+                x[0] = exp2(sv4(0, 0));
+                __builtin_amdgcn_sched_barrier(0);
+                score(I1{});
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (g > 0) {  // the second pair of the group before
+                    compute::convert_pair_here(x[2], x[3], reinterpret_cast<__half*>(pprev) + 2);
+                    lh[(g - 1) / 2] += x[3];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                score(I2{});
+                __builtin_amdgcn_sched_barrier(0);
+                x[1] = exp2(sv4(0, 1));
+                __builtin_amdgcn_sched_barrier(0);
+                score(I3{});
+                __builtin_amdgcn_sched_barrier(0);
+                lh[sc] += x[0];
+                read_k();
+                __builtin_amdgcn_sched_barrier(0);
+                output0();
+                __builtin_amdgcn_sched_barrier(0);
+                x[2] = exp2(sv4(0, 2));
+                __builtin_amdgcn_sched_barrier(0);
+                Output::template at<1, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
+                __builtin_amdgcn_sched_barrier(0);
+                compute::convert_pair_here(x[0], x[1], reinterpret_cast<__half*>(pdst));
+                lh[sc] += x[1];
+                __builtin_amdgcn_sched_barrier(0);
+                Output::template at<2, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
+                __builtin_amdgcn_sched_barrier(0);
+                x[3] = exp2(sv4(0, 3));
+                __builtin_amdgcn_sched_barrier(0);
+                Output::template at<3, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
+                __builtin_amdgcn_sched_barrier(0);
+                lh[sc] += x[2];
+                v_frag.template read_bound_to<0, f, kImm>(rV(0, f % 4));
+                __builtin_amdgcn_sched_barrier(0);
             } else {
-                Output::template at<0, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
+                // query tile g of half i: x[0..3] its key tile 0, x[4..7] its key tile 1; the last pair and the last two
+                // additions of a group wait for the first two gaps of the next one
+                const auto& sv0 = rS[kCur][0](g, 0);
+                const auto& sv1 = rS[kCur][0](g, 1);
+                __half* pdst = reinterpret_cast<__half*>(rP[kCur](g, 0).mutable_data());
+                __half* pprev = reinterpret_cast<__half*>(rP[kCur]((g + 3) % 4, 0).mutable_data());
+                score(I0{});
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (g > 0) {
+                    compute::convert_pair_here(x[6], x[7], pprev + 6);
+                    lh[g - 1] += x[7];
+                }
+                x[0] = exp2(sv0(0, 0));
+                __builtin_amdgcn_sched_barrier(0);
+                score(I1{});
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (g > 0) lh[g - 1] += x[6];
+                x[1] = exp2(sv0(0, 1));
+                lh[g] += x[0];
+                __builtin_amdgcn_sched_barrier(0);
+                score(I2{});
+                __builtin_amdgcn_sched_barrier(0);
+                x[2] = exp2(sv0(0, 2));
+                lh[g] += x[1];
+                compute::convert_pair_here(x[0], x[1], pdst);
+                __builtin_amdgcn_sched_barrier(0);
+                score(I3{});
+                __builtin_amdgcn_sched_barrier(0);
+                x[3] = exp2(sv0(0, 3));
+                lh[g] += x[2];
+                read_k();
+                __builtin_amdgcn_sched_barrier(0);
+                output0();
+                __builtin_amdgcn_sched_barrier(0);
+                x[4] = exp2(sv1(0, 0));
+                lh[g] += x[3];
+                compute::convert_pair_here(x[2], x[3], pdst + 2);
+                __builtin_amdgcn_sched_barrier(0);
+                Output::template at<1, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
+                __builtin_amdgcn_sched_barrier(0);
+                x[5] = exp2(sv1(0, 1));
+                lh[g] += x[4];
+                __builtin_amdgcn_sched_barrier(0);
+                Output::template at<2, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
+                __builtin_amdgcn_sched_barrier(0);
+                x[6] = exp2(sv1(0, 2));
+                lh[g] += x[5];
+                compute::convert_pair_here(x[4], x[5], pdst + 4);
+                __builtin_amdgcn_sched_barrier(0);
+                Output::template at<3, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
+                __builtin_amdgcn_sched_barrier(0);
+                x[7] = exp2(sv1(0, 3));
+                v_frag.template read_bound_to<0, f, kImm>(rV(0, f % 4));
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            x2 = exp2(sv4(0, 2));
-            __builtin_amdgcn_sched_barrier(0);
-            Output::template at<1, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
-            __builtin_amdgcn_sched_barrier(0);
-            compute::convert_pair_here(x0, x1, reinterpret_cast<__half*>(pdst));
-            lh[sc] += x1;
-            __builtin_amdgcn_sched_barrier(0);
-            Output::template at<2, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
-            __builtin_amdgcn_sched_barrier(0);
-            x3 = exp2(sv4(0, 3));
-            __builtin_amdgcn_sched_barrier(0);
-            Output::template at<3, g % 4, 0>(rP[kNxt], rV, rO[g / 4]);
-            __builtin_amdgcn_sched_barrier(0);
-            lh[sc] += x2;
-            v_frag.template read_bound_to<0, f, kImm>(rV(0, f % 4));
-            __builtin_amdgcn_sched_barrier(0);
         });
-        lh[kQT - 1] += x3;
-        compute::convert_pair_here(x2, x3, reinterpret_cast<__half*>(rP[kCur](kQT - 1, 0).mutable_data()) + 6);
+        if constexpr (kG == 8) {
+            lh[kQT - 1] += x[3];
+            compute::convert_pair_here(x[2], x[3], reinterpret_cast<__half*>(rP[kCur](kQT - 1, 0).mutable_data()) + 6);
+        } else {
+            lh[kQT - 1] += x[6] + x[7];
+            compute::convert_pair_here(x[6], x[7], reinterpret_cast<__half*>(rP[kCur](kQT - 1, 0).mutable_data()) + 6);
+        }
         // No probability of this half can have left f16 range while its sum stays below 2^14. The comparison first, then
         // work that does not depend on it, then the branch: the scalar unit sees the result of a vector comparison only
         // some 20 cycles after it was issued.
@@ -473,30 +554,30 @@ __global__ void __launch_bounds__(Traits::kThreads)
             l_run[c] += lh[c];
         }
         if constexpr (kCur == 1) shift_fragments(ring, std::integral_constant<int, 0>{}, std::integral_constant<int, 3>{});
-        else shift_fragments(ring, std::integral_constant<int, 3>{}, std::integral_constant<int, 8>{});
+        else shift_fragments(ring, std::integral_constant<int, 3>{}, std::integral_constant<int, kG>{});
         __builtin_amdgcn_sched_barrier(0);
         if (__builtin_expect(over != 0, 0)) {
             // rare path: move the reference maxima, rescale, re-bias the scores already computed, recompute
             asm volatile("s_nop 15\n\ts_nop 3");
             if constexpr (kQk) {
-                compute::pin_tiles<compute::RegFile::kVgpr>(rS[kNxt][0]);
-                compute::pin_tiles<compute::RegFile::kVgpr>(rS[kNxt][1]);
+#pragma unroll
+                for (int h = 0; h < kSRegs; ++h) compute::pin_tiles<compute::RegFile::kVgpr>(rS[kNxt][h]);
             }
-            compute::pin_tiles<compute::RegFile::kAgpr>(rO[0]);
-            compute::pin_tiles<compute::RegFile::kAgpr>(rO[1]);
+#pragma unroll
+            for (int h = 0; h < kORegs; ++h) compute::pin_tiles<compute::RegFile::kAgpr>(rO[h]);
 #pragma unroll
             for (int c = 0; c < kQT; ++c) {
-                float mx = rS[kCur][0](c, 0)(0, 0);
+                float mx = s_tile(rS[kCur], c, 0)(0, 0);
 #pragma unroll
                 for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) mx = fmaxf(mx, rS[kCur][kt2](c, 0)(0, e));
+                    for (int e = 0; e < 4; ++e) mx = fmaxf(mx, s_tile(rS[kCur], c, kt2)(0, e));
                 mx = row_max(mx);
                 const float shift = mx > 8.0f ? mx : 0.f;
                 const float alpha = exp2(-shift);
                 m_run[c] += shift;
 #pragma unroll
-                for (int h = 0; h < 2; ++h)
+                for (int h = 0; h < kORegs; ++h)
 #pragma unroll
                     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -505,17 +586,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
 #pragma unroll
                     for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) rS[kNxt][kt2](c, 0)(0, e) -= shift;
+                        for (int e = 0; e < 4; ++e) s_tile(rS[kNxt], c, kt2)(0, e) -= shift;
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) neg_max(c, 0)(0, e) = -m_run[c];
                 _Float16* p = reinterpret_cast<_Float16*>(rP[kCur](c, 0).mutable_data());
-                const float lsum = tile_softmax_now(rS[kCur][0](c, 0), shift, p) + tile_softmax_now(rS[kCur][1](c, 0), shift, p + 4);
+                const float lsum = tile_softmax_now(s_tile(rS[kCur], c, 0), shift, p) + tile_softmax_now(s_tile(rS[kCur], c, 1), shift, p + 4);
                 l_run[c] = l_before[c] * alpha + lsum;
             }
             compute::pin_tiles<compute::RegFile::kVgpr>(neg_max);
-            compute::pin_tiles<compute::RegFile::kAgpr>(rO[0]);
-            compute::pin_tiles<compute::RegFile::kAgpr>(rO[1]);
+#pragma unroll
+            for (int h = 0; h < kORegs; ++h) compute::pin_tiles<compute::RegFile::kAgpr>(rO[h]);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -543,7 +624,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         v_frag.bind(v_half(st(0), 0));
         static_for<kAhead>([&](auto a_c) {
             constexpr int a = decltype(a_c)::value;
-            k_frag.template read_bound_to<a % 4, a / 4>(rK(a % 4, 0));
+            k_frag.template read_bound_to<a % kDS, a / kDS>(rK(a % kDS, (a / kDS) % kKtPerReg));
             v_frag.template read_bound_to<0, a>(rV(0, a % 4));
         });
         Stages first = ring;
@@ -555,7 +636,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     // (left alone, the compiler unrolls these loops and the longer live ranges cost registers the kernel does not have)
 #pragma unroll 1
     for (; J + 4 < nb; advance()) {
-        wait_group_and_barrier_keep_reads<8>();
+        wait_group_and_barrier_keep_reads<kG>();
         step(ring, I1{}, Yes{}, I1{}, Yes{}, J + 4);
         step(ring, I0{}, Yes{}, I0{}, Yes{}, 0);
     }
@@ -587,14 +668,14 @@ __global__ void __launch_bounds__(Traits::kThreads)
     step(ring, I1{}, No{}, FetchKV{}, No{}, 0);
     {
         // O += P V with the last half (its first fragments were requested by the step before)
-        static_for<8>([&](auto g_c) {
+        static_for<kG>([&](auto g_c) {
             constexpr int g = decltype(g_c)::value;
             constexpr int gp = g + kAhead;
-            if constexpr (gp < 8) {
+            if constexpr (gp < kG) {
                 v_frag.template read_bound_to<0, gp, kHalfBytes>(rV(0, gp % 4));
                 wait_shared_reads<kAhead * kReadsV>();
             } else {
-                wait_shared_reads<(7 - g) * kReadsV>();
+                wait_shared_reads<(kG - 1 - g) * kReadsV>();
             }
             static_for<kQT>([&](auto c_c) { Output::template at<decltype(c_c)::value, g % 4, 0>(rP[1], rV, rO[g / 4]); });
         });
@@ -602,8 +683,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
 
     // ---- epilogue: O = O / l, to f16, through LDS for row-contiguous 16-byte stores (8-byte stores straight from the
     // accumulator layout were measured: three times slower)
-    compute::settle_accumulators(rO[0]);
-    compute::settle_accumulators(rO[1]);
+#pragma unroll
+    for (int h = 0; h < kORegs; ++h) compute::settle_accumulators(rO[h]);
     typename Traits::RegOut out;
 #pragma unroll
     for (int c = 0; c < kQT; ++c) {

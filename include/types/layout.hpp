@@ -129,18 +129,20 @@ struct LdsSwizzle {
 /// 256 bytes all start on bank 0, so the 4 lines are spread with unit ^= 2 * (line % 4); lines of 128 bytes alternate
 /// between the two halves of the banks, so only lines 2 apart collide: unit ^= line & 2. kLines = 8 (lines of 256
 /// bytes): the two groups sit on the same 32-byte unit of 8 consecutive lines (operand tiles 16 wide, each lane group
-/// 4 lines further down): unit ^= line % 8. 32-byte units (and with them the 16-byte pieces of direct-to-LDS loads)
-/// stay contiguous.
+/// 4 lines further down): unit ^= line % 8; with lines of 128 bytes, whose 4 units alternate between the halves of the
+/// banks by themselves, unit ^= (line / 2) % 4. 32-byte units (and with them the 16-byte pieces of direct-to-LDS
+/// loads) stay contiguous.
 template <const int kPitch, const int kElemBytes, const int kLines = 4>
 struct LdsSwizzleTr {
     static_assert(kElemBytes == 2 && (kPitch == 128 || kPitch == 64),
                   "written for lines of 128 or 256 bytes of 2-byte elements");
-    static_assert(kLines == 4 || (kLines == 8 && kPitch == 128), "4 lines per pass, or 8 lines of 256 bytes");
+    static_assert(kLines == 4 || kLines == 8, "4 or 8 lines per pass");
     static constexpr int kUnit = 16;  // elements per 32-byte unit
     static constexpr int kLinePeriod = kLines;
 
     HOST_DEVICE static constexpr int apply(int line, int elem) {
-        const int s = kLines == 8 ? (line & 7) : kPitch == 128 ? ((line & 3) << 1) : (line & 2);
+        const int s = kLines == 8 ? (kPitch == 128 ? (line & 7) : ((line >> 1) & 3))
+                                  : kPitch == 128 ? ((line & 3) << 1) : (line & 2);
         return (((elem / kUnit) ^ s) * kUnit) | (elem % kUnit);
     }
 };

@@ -210,8 +210,8 @@ static void test_swizzle_tr() {
 // The 8-line form (operand tiles 16 wide: the two 16-lane groups of a pass sit on the same 32-byte unit of 8 consecutive
 // lines, lane group g four lines below group g - 1): a bijection per line that keeps 32-byte units whole, repeats every 8
 // lines, and makes every pass of the read touch 64 distinct banks.
+template <int kPitch>
 static void test_swizzle_tr8() {
-    constexpr int kPitch = 128;
     using Swz = tl::LdsSwizzleTr<kPitch, 2, 8>;
     CHECK(Swz::kLinePeriod == 8);
     for (int line = 0; line < 64; ++line) {
@@ -383,7 +383,8 @@ int main() {
     test_swizzle<80, 2>(false);
     test_swizzle_tr<128>();
     test_swizzle_tr<64>();
-    test_swizzle_tr8();
+    test_swizzle_tr8<128>();
+    test_swizzle_tr8<64>();
     test_swizzle_dealt();
     test_strided_ring();
     test_swizzle<16, 4>(true);

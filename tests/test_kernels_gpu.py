@@ -907,6 +907,45 @@ def test_flash_attention_wave64_k32(tcu, oracle, device, batch, M, N, v_col_majo
     assert oracle.max_abs_err(host(out)[heads, M - 64:], ref_tail) <= tol
 
 
+@pytest.mark.parametrize("batch,M,N", [(3, 256, 320), (8, 256, 640), (5, 768, 448), (64, 2048, 2048), (203, 1024, 448),
+                                       (330, 256, 640), (1300, 256, 320)])
+def test_flash_attention_wave64_k32_head_size_64(tcu, oracle, device, batch, M, N):
+    """Head size 64 on the 16x16x32 one-wavefront-per-SIMD kernel (a step of 4 groups instead of 8: every matrix
+    instruction carries an exponential): against the oracle and against the 8-wavefront kernel, at the minimum of 5 key
+    blocks, an odd number of blocks, keys that force the rare re-basing path, and one to six items per workgroup.
+    The keys that force re-basing give logits up to 400; the kernels multiply Q by scale * log2(e) and round it to f16
+    once, which moves such a logit by up to ~400 * 2^-11 / sqrt(D) * a few: 0.026 on the output at D = 64 for these
+    inputs (0.015 at D = 128), computed on the host from that rounding alone. Hence 3e-2 there."""
+    import torch
+
+    D = 64
+    print(f"attention wave64_k32 d64 b{batch} {M}x{N}", flush=True)
+    q = oracle.fill_normal(batch * M * D, 94).reshape(batch, M, D).astype(np.float32)
+    k = oracle.fill_normal(batch * N * D, 95).reshape(batch, N, D).astype(np.float32)
+    v = oracle.fill_normal(batch * N * D, 96).reshape(batch, N, D)
+    if N == 640:
+        qdir = q / np.linalg.norm(q, axis=-1, keepdims=True)
+        for pos, gain in ((0, 30.0), (200, 60.0), (225, 120.0), (300, 200.0), (639, 400.0)):
+            k[:, pos] = qdir[:, pos % M] * gain
+    q, k = q.astype(np.float16), k.astype(np.float16)
+    dq, dk, dv = dev(q, device), dev(k, device), dev(v, device)
+    ref_kernel = tcu.flash_attention(dq, dk, dv, algo="mfma32_fused")
+    out = torch.full_like(ref_kernel, float("nan"))
+    tcu.flash_attention(dq, dk, dv, out=out, algo="wave64_k32")
+    torch.cuda.synchronize()
+    tol = 3e-2 if N == 640 else ABS_TOL
+    assert torch.isfinite(out).all()
+    assert (out.float() - ref_kernel.float()).abs().max().item() <= tol
+    heads = [0, batch - 1]
+    rows = M if batch * M * N <= (1 << 21) else 64
+    ref = oracle.attention(np.ascontiguousarray(q[heads, :rows]), np.ascontiguousarray(k[heads]), np.ascontiguousarray(v[heads]),
+                           1.0 / math.sqrt(D))
+    assert oracle.max_abs_err(host(out)[heads, :rows], ref) <= tol
+    ref_tail = oracle.attention(np.ascontiguousarray(q[heads, M - 64:]), np.ascontiguousarray(k[heads]),
+                                np.ascontiguousarray(v[heads]), 1.0 / math.sqrt(D))
+    assert oracle.max_abs_err(host(out)[heads, M - 64:], ref_tail) <= tol
+
+
 @pytest.mark.parametrize("algo", ["wave64", "tile_wave64", "wave64_k32"])
 def test_flash_attention_wave64_with_cold_caches(tcu, oracle, device, algo):
     """The one-wavefront-per-SIMD kernels request their first operand fragments of key block 1 only behind the barrier

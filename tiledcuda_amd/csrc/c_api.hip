@@ -585,10 +585,10 @@ int fa_tile_w64_dispatch(const __half* Q, const __half* K, const __half* V, __ha
 
 /// The one-wavefront-per-SIMD kernel on the 16x16x32 instruction (tile-library functors, run-time M and N, either V
 /// layout).
-template <bool kVColMajor>
+template <int kD, bool kVColMajor>
 int launch_fa_w64_k32(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, float scale,
                       hipStream_t stream) {
-    using Traits = FlashW64K32Traits<__half, 128, kVColMajor>;
+    using Traits = FlashW64K32Traits<__half, kD, kVColMajor>;
     // one workgroup per CU; a workgroup with more than one item fetches the next one's first operands under the last
     // steps of the current one. Items keep their XCD (item number modulo 8) only if the grid is a multiple of 8.
     int device = 0, cus = 0;
@@ -604,14 +604,16 @@ int launch_fa_w64_k32(const __half* Q, const __half* K, const __half* V, __half*
 int fa_w64_k32_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, int batch, int M, int N, int Kd,
                         float scale, int v_layout, hipStream_t stream) {
     using Traits = FlashW64K32Traits<__half, 128>;
-    if (Kd != 128)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel is instantiated for head size 128");
+    if (Kd != 128 && !(Kd == 64 && v_layout == TCU_V_ROW_MAJOR))
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel is instantiated for head size "
+                                               "128, and for head size 64 with a row-major V");
     if (M % Traits::kTM != 0 || N < Traits::kStages * Traits::kTN)
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel needs M % 256 == 0 and N >= 320");
     if ((long)N * 256 >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel addresses a V block with 32-bit offsets");
-    return v_layout == TCU_V_ROW_MAJOR ? launch_fa_w64_k32<false>(Q, K, V, O, batch, M, N, scale, stream)
-                                       : launch_fa_w64_k32<true>(Q, K, V, O, batch, M, N, scale, stream);
+    if (Kd == 64) return launch_fa_w64_k32<64, false>(Q, K, V, O, batch, M, N, scale, stream);
+    return v_layout == TCU_V_ROW_MAJOR ? launch_fa_w64_k32<128, false>(Q, K, V, O, batch, M, N, scale, stream)
+                                       : launch_fa_w64_k32<128, true>(Q, K, V, O, batch, M, N, scale, stream);
 }
 
 template <int kD, bool kFused>
@@ -648,6 +650,8 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
         if (algo == TCU_ATTN_AUTO && Kd == 128 && M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 128)
             return (long)batch * (M / 256) >= 256 ? fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream)
                                                   : launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream);
+        if (algo == TCU_ATTN_AUTO && Kd == 64 && M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 256)
+            return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
         if (algo == TCU_ATTN_MFMA32)
             return Kd == 128 ? fa_fwd_by_rows<128, false>(Q, K, V, O, batch, M, N, scale, stream)
                              : fa_fwd_by_rows<64, false>(Q, K, V, O, batch, M, N, scale, stream);
