@@ -484,6 +484,17 @@ def main():
                                 lambda: tcu.flash_attention(dq, dk, dv, out=do, algo="wave64_k32"), 40, 100)
             configs.append({"name": "flash_attn_fwd_b4_h16_s2048_d128_by_matrix_instruction", "kernel": "flash_attention_w64_k32 / flash_attention_fwd_w64",
                             "ms_16x16x32": ms_16, "ms_32x32x16": ms_32, "speed_16x16x32_vs_32x32x16": ms_32 / ms_16})
+            # head size 64 (8 x 16 heads of 2048): the 8-wavefront kernel against the 16x16x32 one-wavefront kernel
+            q64, k64, v64 = (torch.randn(128, 2048, 64, device=dev).half() for _ in range(3))
+            o64 = torch.empty_like(q64)
+            ms_8w, ms_1w = pair(lambda: tcu.flash_attention(q64, k64, v64, out=o64, algo="mfma32_fused"),
+                                lambda: tcu.flash_attention(q64, k64, v64, out=o64, algo="wave64_k32"), 40, 100)
+            flops64 = 4.0 * 128 * 2048 * 2048 * 64
+            configs.append({"name": "flash_attn_fwd_b8_h16_s2048_d64", "kernel": "flash_attention_w64_k32<64> (what AUTO runs)",
+                            "ms": ms_1w, "tflops": flops64 / (ms_1w * 1e-3) / 1e12,
+                            "frac_of_mfma_peak": flops64 / (ms_1w * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                            "ms_8_wavefront_kernel": ms_8w, "speed_vs_8_wavefront_kernel": ms_8w / ms_1w})
+            del q64, k64, v64, o64
         dCt = torch.empty_like(dC)
         ms_r, ms_t = pair(lambda: tcu.gemm(dA, dB, out=dCt, algo="wave128"), lambda: tcu.gemm(dA, dB, out=dCt, algo="tile_wave128"), 40, 100)
         configs.append({"name": "gemm_4096_tile_api_composition", "kernel": "gemm_tile_w128", "ms": ms_t,

@@ -1,5 +1,5 @@
 // The time loop of the fused LSTM layer as ONE launch, weight-stationary, for gfx950: after the input half of the
-// gates of all T steps has been computed by one large GEMM (pre[T, B, 4H] = x · W[:, :I]ᵀ, f32), this kernel runs the
+// gates of all T steps has been computed by one large GEMM (pre[T, B, 4H] = x · W[:, :I]ᵀ, f32 or f16), this kernel runs the
 // recurrence gates_t = pre_t + h_{t-1} · W[:, I:]ᵀ + bias, c_t = σ(f) c_{t-1} + σ(i) tanh(g), h_t = σ(o) tanh(c_t)
 // for t = 0 .. T-1 without returning to the host. Same contract and gate order (i, f, g, o) as kernels/lstm_fwd.hpp.
 // The reference has no LSTM kernel (its Makefile:3 only names a test).
@@ -28,8 +28,9 @@
 //     raises the error word and exits, and so does, in turn, every workgroup that waits for it. The outputs are then
 //     invalid; the host reads the word.
 // sync: 128-byte aligned device words, all zero at launch: [g] the XCDs group g runs on (one bit each), [8] error,
-// [32 (g + 1)] the step counter of group g (128 bytes apart). Requirements: H == 1024 (the register budget), B % 32 == 0,
-// B <= 256 (8 XCDs), grid == 256 workgroups of 256 threads.
+// [32 (g + 1)] the step counter of group g (128 bytes apart). Requirements: H in {256, 512, 768, 1024} (a CU always owns
+// 32 hidden units, so a group is H / 32 CUs of its XCD and a wavefront's weights are H / 4 registers: 1024 is the
+// register budget), B % 32 == 0, B <= 256 (8 XCDs), grid == 8 * H / 32 workgroups of 256 threads.
 #pragma once
 
 #include <type_traits>
@@ -45,21 +46,27 @@ template <const int kH_>
 struct LstmRecurrentTraits {
     static constexpr int kH = kH_;
     static constexpr int kRows = 32;          // batch rows per XCD
-    static constexpr int kCusPerXcd = 32;     // workgroups that share the rows of an XCD
+    static constexpr int kUnitsPerCu = 32;    // hidden units a workgroup owns
+    static constexpr int kCusPerXcd = kH / kUnitsPerCu;  // workgroups that share the rows of an XCD: 32 for H = 1024
     static constexpr int kXcds = 8;
-    static constexpr int kUnitsPerCu = kH / kCusPerXcd;  // 32
     static constexpr int kWaves = 4, kThreads = kWaves * kWaveSize;
     static constexpr int kUnitsPerWave = kUnitsPerCu / kWaves;  // 8 (x 4 gates = the 32 rows of an MFMA operand)
-    static constexpr int kKSteps = kH / 16;                      // 64 MFMAs per step and wavefront
+    static constexpr int kKSteps = kH / 16;                      // MFMAs per step and wavefront (64 for H = 1024)
     static constexpr int kRowBytes = kH * 2;
-    static constexpr int kLdsBytes = kRows * kRowBytes;  // h_{t-1} of the XCD's rows: 64 KiB
-    static constexpr int kPieces = 4;                    // h arrives in 4 pieces of 16 k-steps
-    static constexpr int kLoadsPerWave = kLdsBytes / 1024 / kWaves;  // 16 one-KiB load instructions
+    static constexpr int kHBytes = kRows * kRowBytes;    // h_{t-1} of the XCD's rows: 64 KiB for H = 1024
+    static constexpr int kStagingBytes = kWaves * 2 * 32 * 256;  // what the weights pass through on their way in
+    static constexpr int kLdsBytes = kHBytes > kStagingBytes ? kHBytes : kStagingBytes;
+    static constexpr int kPieces = 4;                    // h arrives in 4 pieces of kKSteps / 4 k-steps
+    static constexpr int kStepsPerPiece = kKSteps / kPieces;
+    static constexpr int kLoadsPerWave = kHBytes / 1024 / kWaves;  // one-KiB load instructions (16 for H = 1024)
+    static constexpr int kLoadsPerPiece = kLoadsPerWave / kPieces;
     static constexpr int kGrid = kXcds * kCusPerXcd;
     static constexpr int kSyncWords = 32 * (kXcds + 1);
     static constexpr int kErrorWord = 8;
-    static_assert(kUnitsPerWave == 8 && kKSteps * 4 == 256, "one wavefront's weights are exactly 256 registers per lane");
-    static_assert(kLoadsPerWave == 4 * kPieces);
+    static_assert(kH % 256 == 0 && kH >= 256 && kH <= 1024,
+                  "a wavefront's weights are H / 4 registers per lane (at most the 256 AGPRs), a piece of h is a whole "
+                  "number of load instructions and an even number of k-steps");
+    static_assert(kUnitsPerWave == 8 && kLoadsPerWave == kLoadsPerPiece * kPieces && kStepsPerPiece == 4 * kLoadsPerPiece);
 };
 
 namespace detail {
@@ -182,8 +189,8 @@ __global__ void __launch_bounds__(Traits::kThreads)
         pre_v[g] = widen_pre(load_pre(size_t(b), g));
     }
 
-    // ---- global -> LDS: load instruction j (0..15) of wavefront w brings rows 8 w .. 8 w + 7, logical 16-byte chunks
-    // 8 j .. 8 j + 7 (k-steps 4 j .. 4 j + 3): 128 contiguous bytes per row. LDS rows are 2 KiB; physical chunk p of
+    // ---- global -> LDS: load instruction j (0 .. kLoadsPerWave - 1) of wavefront w brings rows 8 w .. 8 w + 7, logical
+    // 16-byte chunks 8 j .. 8 j + 7 (k-steps 4 j .. 4 j + 3): 128 contiguous bytes per row.
     // The landing place of an instruction is 1 KiB of LDS, so h is stored piecewise: block (j, w) = [8 rows][8 chunks
     // of 16 B]; inside a block, physical chunk p of row r holds logical chunk p ^ key(r), key(r) = (r % 8) ^ (r / 8 % 2):
     // the ds_read_b128 of 16 consecutive rows at one k-offset then touches every bank once (rows of equal parity share
@@ -209,21 +216,22 @@ __global__ void __launch_bounds__(Traits::kThreads)
     };
 
     f32x16 acc0, acc1;
-    auto read_piece = [&](f16x8(&f)[16], int p) {
+    constexpr int kSPP = Traits::kStepsPerPiece, kLPP = Traits::kLoadsPerPiece;
+    auto read_piece = [&](f16x8(&f)[kSPP], int p) {
 #pragma unroll
-        for (int s = 0; s < 16; ++s) f[s] = read_frag(16 * p + s);
+        for (int s = 0; s < kSPP; ++s) f[s] = read_frag(kSPP * p + s);
     };
     // The MFMAs of piece p, and between them the fragment reads of piece p + 1 (one read per MFMA: issued in a block
     // they would hold up the matrix pipe for as long as eight MFMAs take). Weights first: accumulator rows = batch,
     // register quad = gate; two accumulators, so that consecutive MFMAs do not depend on each other; the first two
     // of a step start from zero.
-    auto mfma_piece = [&](const f16x8(&f)[16], f16x8(&next)[16], int p) {
+    auto mfma_piece = [&](const f16x8(&f)[kSPP], f16x8(&next)[kSPP], int p) {
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
+        for (int s = 0; s < kSPP; ++s) {
             f32x16& acc = (s & 1) ? acc1 : acc0;
             if (p == 0 && s < 2) detail::mfma32_weights_in_agprs_zero(acc, wf[s], f[s]);
-            else detail::mfma32_weights_in_agprs(acc, wf[16 * p + s], f[s]);
-            if (p + 1 < Traits::kPieces) next[s] = read_frag(16 * (p + 1) + s);
+            else detail::mfma32_weights_in_agprs(acc, wf[kSPP * p + s], f[s]);
+            if (p + 1 < Traits::kPieces) next[s] = read_frag(kSPP * (p + 1) + s);
         }
     };
 
@@ -266,18 +274,19 @@ __global__ void __launch_bounds__(Traits::kThreads)
             for (int g = 0; g < 4; ++g) pre_next[g] = load_pre(size_t(t + 1) * B + b, g);
         }
         if (h_prev) {
-            // Piece p (this wavefront's loads 4 p .. 4 p + 3) has landed when at most the loads issued after it are
-            // outstanding (`later`: the 4 loads of pre_next); then, behind the barrier, everyone's. The fragments of
-            // piece p + 1 are read between the MFMAs of piece p, so the barrier of piece p + 1 comes first.
-            f16x8 fa[16], fb[16];
-            if (t + 1 < T) detail::lds_barrier<12 + 4>();
-            else detail::lds_barrier<12>();
+            // Piece p (this wavefront's loads kLPP p .. kLPP (p + 1) - 1) has landed when at most the loads issued after
+            // it are outstanding (the later pieces and the 4 loads of pre_next); then, behind the barrier, everyone's.
+            // The fragments of piece p + 1 are read between the MFMAs of piece p, so the barrier of piece p + 1 comes
+            // first.
+            f16x8 fa[kSPP], fb[kSPP];
+            if (t + 1 < T) detail::lds_barrier<3 * kLPP + 4>();
+            else detail::lds_barrier<3 * kLPP>();
             read_piece(fa, 0);
-            if (t + 1 < T) detail::lds_barrier<8 + 4>();
-            else detail::lds_barrier<8>();
+            if (t + 1 < T) detail::lds_barrier<2 * kLPP + 4>();
+            else detail::lds_barrier<2 * kLPP>();
             mfma_piece(fa, fb, 0);
-            if (t + 1 < T) detail::lds_barrier<4 + 4>();
-            else detail::lds_barrier<4>();
+            if (t + 1 < T) detail::lds_barrier<kLPP + 4>();
+            else detail::lds_barrier<kLPP>();
             mfma_piece(fb, fa, 1);
             if (t + 1 < T) detail::lds_barrier<0 + 4>();
             else detail::lds_barrier<0>();

@@ -226,7 +226,7 @@ int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* 
 
 /*
  * The LSTM layer with the whole time loop in ONE launch, for the large-hidden-size case where a step is bound by
- * streaming the recurrent weights and by the cost of a dependent launch (H == 1024, I % 64 == 0, B % 32 == 0, B <= 256,
+ * streaming the recurrent weights and by the cost of a dependent launch (H in {256, 512, 768, 1024}, I % 64 == 0, B % 32 == 0, B <= 256,
  * T * B % 256 == 0; a device of 256 CUs in 8 XCDs). As in tcu_lstm_f16_ws the input half of the gates of all steps is
  * one GEMM into the workspace - here with its f32 sums rounded once to f16 (half the bytes to write and read back; the
  * gates' pre-activations then carry a relative error of 2^-11 on that half, far inside the layer's 1e-2 tolerance) -;

@@ -1182,17 +1182,18 @@ def test_lstm_config5(tcu, oracle, device):
             assert oracle.max_abs_err(cc[rows[0]:rows[1]], c_ref[rows[0]:rows[1]]) <= ABS_TOL, algo
 
 
-@pytest.mark.parametrize("T,B,I", [(4, 64, 64), (8, 32, 192), (2, 128, 1024), (1, 256, 64)])
+@pytest.mark.parametrize("T,B,I,H", [(4, 64, 64, 1024), (8, 32, 192, 1024), (2, 128, 1024, 1024), (1, 256, 64, 1024),
+                                     (8, 32, 64, 256), (4, 256, 256, 256), (8, 64, 128, 512), (2, 128, 512, 512),
+                                     (8, 96, 64, 768), (16, 256, 768, 768)])
 @pytest.mark.parametrize("with_state", [False, True])
-def test_lstm_persistent_single_launch(tcu, oracle, device, T, B, I, with_state):
-    """tcu_lstm_f16_persistent (H = 1024): the time loop in one weight-stationary launch, h exchanged inside each XCD.
-    One to eight XCDs in use, one to eight steps, with and without an initial state; against the oracle and against
-    the hoisted per-step path (same projection GEMM, other summation order); twice on one workspace, whose bytes past
-    the stated size stay untouched."""
+def test_lstm_persistent_single_launch(tcu, oracle, device, T, B, I, H, with_state):
+    """tcu_lstm_f16_persistent (H = 256, 512, 768, 1024: 8, 16, 24, 32 workgroups per XCD): the time loop in one
+    weight-stationary launch, h exchanged inside each XCD. One to eight XCDs in use, one to sixteen steps, with and
+    without an initial state; against the oracle and against the hoisted per-step path (same projection GEMM, other
+    summation order); twice on one workspace, whose bytes past the stated size stay untouched."""
     import torch
 
-    H = 1024
-    print(f"lstm persistent T{T} B{B} I{I} state={with_state}", flush=True)
+    print(f"lstm persistent T{T} B{B} I{I} H{H} state={with_state}", flush=True)
     x = oracle.fill_normal(T * B * I, 61, 0, 0.5).reshape(T, B, I)
     W = oracle.fill_normal(4 * H * (I + H), 62, 0, 0.03).reshape(4 * H, I + H)
     b = oracle.fill_normal(4 * H, 63, 0, 0.1)
@@ -1269,7 +1270,8 @@ def test_lstm_persistent_workspace_at_allocator_granularity(tcu, device):
 def test_lstm_persistent_rejects_what_it_cannot_do(tcu, device):
     import torch
 
-    assert tcu.lstm_persistent_workspace_bytes(4, 64, 64, 512) == 0    # H != 1024
+    assert tcu.lstm_persistent_workspace_bytes(4, 64, 64, 128) == 0    # H not in {256, 512, 768, 1024}
+    assert tcu.lstm_persistent_workspace_bytes(4, 64, 64, 2048) == 0
     assert tcu.lstm_persistent_workspace_bytes(4, 48, 64, 1024) == 0   # B not a multiple of 32
     assert tcu.lstm_persistent_workspace_bytes(1, 512, 64, 1024) == 0  # more rows than 8 XCDs x 32
     assert tcu.lstm_persistent_workspace_bytes(3, 64, 64, 1024) == 0   # T * B not a multiple of 256

@@ -292,7 +292,7 @@ def lstm(x: torch.Tensor, W: torch.Tensor, bias: torch.Tensor, h0: torch.Tensor 
     ``workspace=False`` (use that, or a workspace of your own, under HIP graph capture), else one fused kernel per step. ``out`` = (h_all, c_T) tensors to write into instead of allocating them.
 
     ``algo="persistent"`` runs the whole time loop in one weight-stationary launch after the same GEMM
-    (``tcu_lstm_f16_persistent``: H = 1024, B <= 256 in multiples of 32; ``lstm_persistent_workspace_bytes``). Its
+    (``tcu_lstm_f16_persistent``: H in {256, 512, 768, 1024}, B <= 256 in multiples of 32; ``lstm_persistent_workspace_bytes``). Its
     workgroups wait for each other with a time limit; with ``check=True`` (the default) the stream is synchronised and
     a RuntimeError raised if a wait expired, ``check=False`` leaves that to a later ``lstm_persistent_status(workspace)``."""
     if x.dim() != 3 or W.dim() != 2:

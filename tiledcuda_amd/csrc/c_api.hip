@@ -766,6 +766,18 @@ int launch_lstm_fwd(const __half* x, const __half* W, const __half* bias, const 
     return TCU_OK;
 }
 
+/// The weight-stationary recurrence for hidden size kH: 8 * kH / 32 workgroups, kH / 32 per XCD.
+template <int kH>
+int launch_lstm_recurrent_xcd(const __half* pre, const __half* W, const void* bias, const void* h0, const void* c0, void* h_all,
+                              void* c_out, int T, int B, int I, unsigned int* sync, unsigned long long spin_us,
+                              long peers_override, hipStream_t s) {
+    using Traits = LstmRecurrentTraits<kH>;
+    const unsigned int peers = peers_override >= 0 ? unsigned(peers_override) : unsigned(Traits::kCusPerXcd);
+    return launch(&lstm_recurrent_xcd<Traits, __half>, dim3(Traits::kGrid), dim3(Traits::kThreads), Traits::kLdsBytes, s, pre,
+                  W, I + kH, I, static_cast<const __half*>(bias), static_cast<const __half*>(h0),
+                  static_cast<const float*>(c0), static_cast<__half*>(h_all), static_cast<float*>(c_out), T, B, sync,
+                  spin_us * 100ull, peers);
+}
 }  // namespace
 
 extern "C" {
@@ -934,7 +946,7 @@ int tcu_lstm_f16_ws(const void* x, const void* W, const void* bias, const void* 
 
 unsigned long long tcu_lstm_persistent_workspace_bytes(int T, int B, int I, int H) {
     using Traits = LstmRecurrentTraits<1024>;
-    if (T <= 0 || B <= 0 || I <= 0 || H != Traits::kH) return 0;
+    if (T <= 0 || B <= 0 || I <= 0 || (H != 256 && H != 512 && H != 768 && H != 1024)) return 0;
     if (B % Traits::kRows != 0 || B > Traits::kRows * Traits::kXcds || I % 64 != 0) return 0;
     if ((long)T * B % 256 != 0 || (long)T * B > INT_MAX) return 0;
     // the pre-activations of all steps in f16: [T, B, 4H]
@@ -952,11 +964,12 @@ int tcu_lstm_f16_persistent(const void* x, const void* W, const void* bias, cons
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: operands must be 16-byte aligned, the workspace 128-byte aligned");
     const unsigned long long need = tcu_lstm_persistent_workspace_bytes(T, B, I, H);
     if (need == 0)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_persistent: needs H == 1024, I % 64 == 0, B % 32 == 0, B <= 256 "
-                                               "and T * B % 256 == 0");
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_persistent: needs H in {256, 512, 768, 1024}, I % 64 == 0, B % 32 == 0, "
+                                               "B <= 256 and T * B % 256 == 0");
     if (workspace_bytes < need)
         return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_lstm_f16_persistent: workspace smaller than tcu_lstm_persistent_workspace_bytes()");
-    // one workgroup per CU, all resident at once, 32 per XCD: the grid is the chip
+    // one workgroup per CU, all resident at once, H / 32 per XCD (dealt to the 8 XCDs in turn): at H = 1024 the grid is
+    // the chip
     int device = 0, cus = 0;
     if (hipGetDevice(&device) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
@@ -965,9 +978,9 @@ int tcu_lstm_f16_persistent(const void* x, const void* W, const void* bias, cons
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "tcu_lstm_f16_persistent: written for a device of 256 CUs in 8 XCDs; this one has " +
                                                    std::to_string(cus) + " CUs");
     unsigned long long spin_us = 2000000;  // a wait is microseconds when every workgroup is resident
-    unsigned int peers = Traits::kCusPerXcd;
+    long peers = -1;                       // (the number of workgroups per XCD)
     if (const char* e = std::getenv("TCU_LSTM_PERSISTENT_SPIN_US")) spin_us = std::strtoull(e, nullptr, 10);
-    if (const char* e = std::getenv("TCU_LSTM_PERSISTENT_PEERS")) peers = unsigned(std::strtoul(e, nullptr, 10));
+    if (const char* e = std::getenv("TCU_LSTM_PERSISTENT_PEERS")) peers = long(std::strtoul(e, nullptr, 10));
     auto s = static_cast<hipStream_t>(stream);
     auto sync = static_cast<unsigned int*>(workspace);
     auto pre = reinterpret_cast<__half*>(static_cast<unsigned char*>(workspace) + kPersistentSyncBytes);
@@ -977,10 +990,12 @@ int tcu_lstm_f16_persistent(const void* x, const void* W, const void* bias, cons
     // synchronisation words on the side (its first workgroup): no launch of its own.
     int rc = gemm_w128_dispatch<__half>(xp, wp, pre, T * B, 4 * H, I, s, I, I + H, 0, sync, Traits::kSyncWords);
     if (rc != TCU_OK) return rc;
-    return launch(&lstm_recurrent_xcd<Traits, __half>, dim3(Traits::kGrid), dim3(Traits::kThreads), Traits::kLdsBytes, s,
-                  static_cast<const __half*>(pre), wp, I + H, I, static_cast<const __half*>(bias),
-                  static_cast<const __half*>(h0), static_cast<const float*>(c0), static_cast<__half*>(h_all),
-                  static_cast<float*>(c_out), T, B, sync, spin_us * 100ull, peers);
+    switch (H) {
+        case 256: return launch_lstm_recurrent_xcd<256>(pre, wp, bias, h0, c0, h_all, c_out, T, B, I, sync, spin_us, peers, s);
+        case 512: return launch_lstm_recurrent_xcd<512>(pre, wp, bias, h0, c0, h_all, c_out, T, B, I, sync, spin_us, peers, s);
+        case 768: return launch_lstm_recurrent_xcd<768>(pre, wp, bias, h0, c0, h_all, c_out, T, B, I, sync, spin_us, peers, s);
+        default: return launch_lstm_recurrent_xcd<1024>(pre, wp, bias, h0, c0, h_all, c_out, T, B, I, sync, spin_us, peers, s);
+    }
 }
 
 int tcu_lstm_persistent_status(const void* workspace, void* stream) {
