@@ -19,7 +19,9 @@
 //     stores its 32 x 8 piece of h_t;
 //   * h is exchanged only between the 32 CUs of an XCD, through that XCD's L2: plain stores (the vector L1 writes
 //     through), loads that bypass the L1 (sc1), and one counter per XCD: a CU adds 1 when its stores of h_t have been
-//     acknowledged, and polls for 32 (t + 1) before it loads h_t. No traffic crosses XCDs, no cache is flushed;
+//     acknowledged, and polls for 32 (t + 1) before it loads h_t. No traffic crosses XCDs, no cache is flushed. (A
+//     counter per quarter of the hidden units, polled right before that quarter is requested, was measured: the
+//     three extra polls and barriers cost 0.7 us per step, far more than the skew between the CUs they could hide);
 //   * workgroups whose ids are equal modulo 8 form a group (the dispatcher deals workgroups to the XCDs in turn, so
 //     they share an XCD); that they really do is checked from the hardware's XCC_ID before the first exchange. The
 //     launch needs every workgroup resident at once (grid = number of CUs, one workgroup per CU by register use),
@@ -84,6 +86,14 @@ DEVICE void mfma32_weights_in_agprs(f32x16& acc, const f16x8& w, const f16x8& h)
 DEVICE void mfma32_weights_in_agprs_zero(f32x16& acc, const f16x8& w, const f16x8& h) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "a"(w), "v"(h));
 }
+/// sigmoid(a) * tanh(b) as one quotient: (1 - E_b) / ((1 + E_a) (1 + E_b)) with E_a = e^-a, E_b = e^-2b - two v_exp_f32
+/// and ONE v_rcp_f32 where the factors taken separately need two of each (the cell update sits on the critical path of
+/// every step, and these instructions run at a quarter of the rate). b is clamped to +-20, where tanh is 1 to f32
+/// precision and E_b stays finite; E_a may overflow (a < -88): the quotient is then 0, the limit.
+DEVICE float sigmoid_times_tanh(float a, float b) {
+    const float ea = __expf(-a), eb = __expf(-2.0f * __builtin_amdgcn_fmed3f(b, -20.0f, 20.0f));
+    return (1.0f - eb) * __builtin_amdgcn_rcpf((1.0f + ea) * (1.0f + eb));
+}
 }  // namespace detail
 
 /// pre: [T, B, 4H] f32 or f16 (PreType; gate-major columns, as W's rows); W: [4H, ldw] f16, the recurrent block starts at column
@@ -121,7 +131,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int frow = lane & 31, fhalf = lane >> 5;
     const int unit0 = slot * Traits::kUnitsPerCu + wave * Traits::kUnitsPerWave;
     f16x8 wf[Traits::kKSteps];
-    {
+    auto load_weights = [&]() {
         // A lane's share of a fragment is 16 bytes of one weight row, so loading fragments straight from memory asks
         // for 32-byte pieces of 32 rows per instruction; instead the wavefront's 32 rows x 2 KiB pass through its
         // quarter of the LDS (not yet in use) in 8 chunks of 32 rows x 256 B (8 k-steps), loaded directly to LDS in
@@ -162,7 +172,9 @@ __global__ void __launch_bounds__(Traits::kThreads)
         // into the AGPR half, where the MFMAs below take them from
 #pragma unroll
         for (int ks = 0; ks < Traits::kKSteps; ++ks) asm volatile("" : "+a"(wf[ks]));
-    }
+    };
+    // Without an initial hidden state step 0 multiplies nothing: the weights are fetched behind it (64 MiB through the
+    // fabric for the chip, ~10 us), and the XCD's first exchange of h runs under that fetch.
 
     // ---- the lane's share of the cell update: accumulator register 4 g + e is gate g of batch row row0 + lane % 32,
     // hidden unit unit0 + 4 (lane / 32) + e
@@ -186,7 +198,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         const f16x4 bv = *reinterpret_cast<const f16x4*>(bias + g * kH + hid);
 #pragma unroll
         for (int e = 0; e < 4; ++e) bias_v[g][e] = static_cast<float>(bv[e]);
-        pre_v[g] = widen_pre(load_pre(size_t(b), g));
+        pre_v[g] = widen_pre(load_pre(size_t(b), g)) + bias_v[g];
     }
 
     // ---- global -> LDS: load instruction j (0 .. kLoadsPerWave - 1) of wavefront w brings rows 8 w .. 8 w + 7, logical
@@ -198,9 +210,11 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
     const int lrow = 8 * wave + (lane >> 3), lchk = lane & 7;
     auto key = [](int r) { return (r & 7) ^ ((r >> 3) & 1); };
-    auto issue_h = [&](const __half* src_rows) {
+    // (piece p: this wavefront's loads kLoadsPerPiece p .. kLoadsPerPiece (p + 1) - 1, a quarter of the hidden units)
+    auto issue_h_piece = [&](const __half* src_rows, int p) {
 #pragma unroll
-        for (int j = 0; j < Traits::kLoadsPerWave; ++j) {
+        for (int jj = 0; jj < Traits::kLoadsPerPiece; ++jj) {
+            const int j = p * Traits::kLoadsPerPiece + jj;
             const int chunk = 8 * j + (lchk ^ key(lrow));
             detail::load_lds_16B_untracked_sc1(src_rows + size_t(lrow) * kH + chunk * 8,
                                                __builtin_amdgcn_readfirstlane(lds_base + (j * Traits::kWaves + wave) * 1024));
@@ -236,13 +250,15 @@ __global__ void __launch_bounds__(Traits::kThreads)
     };
 
     constexpr unsigned long long kNoLimit = ~0ull;
-    for (int t = 0; t < T; ++t) {
+    // one time step; kHasH = false: step 0 without an initial hidden state (nothing to multiply)
+    auto time_step = [&](int t, auto has_h_c) {
+        constexpr bool kHasH = decltype(has_h_c)::value;
         const __half* h_prev = t == 0 ? h0 : h_all + size_t(t - 1) * B * kH;
-        if (!h_prev) {
+        if constexpr (!kHasH) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc0[e] = acc1[e] = 0.f;
         }
-        if (h_prev) {
+        if constexpr (kHasH) {
             // ---- everybody's piece of h_{t-1} is in the L2 when the XCD's counter has reached peers * t
             if (t > 0 && threadIdx.x == 0) {
                 const unsigned int target = peers * unsigned(t);
@@ -264,8 +280,10 @@ __global__ void __launch_bounds__(Traits::kThreads)
             }
             // the poll is over; everyone has finished reading the previous h from LDS (they stored h_{t-1} after it)
             detail::lds_barrier<0>();
-            if (__builtin_amdgcn_readfirstlane(*const_cast<volatile int*>(&s_abort))) return;
-            issue_h(h_prev + size_t(row0) * kH);
+            if (__builtin_amdgcn_readfirstlane(*const_cast<volatile int*>(&s_abort))) return false;
+            const __half* src_rows = h_prev + size_t(row0) * kH;
+#pragma unroll
+            for (int p = 0; p < Traits::kPieces; ++p) issue_h_piece(src_rows, p);
         }
         // pre-activations of the next step, a step ahead (independent of h)
         PreRaw pre_next[4];
@@ -273,7 +291,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
 #pragma unroll
             for (int g = 0; g < 4; ++g) pre_next[g] = load_pre(size_t(t + 1) * B + b, g);
         }
-        if (h_prev) {
+        if constexpr (kHasH) {
             // Piece p (this wavefront's loads kLPP p .. kLPP (p + 1) - 1) has landed when at most the loads issued after
             // it are outstanding (the later pieces and the 4 loads of pre_next); then, behind the barrier, everyone's.
             // The fragments of piece p + 1 are read between the MFMAs of piece p, so the barrier of piece p + 1 comes
@@ -301,23 +319,32 @@ __global__ void __launch_bounds__(Traits::kThreads)
         f16x4 h_new;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float gi = acc0[0 + e] + acc1[0 + e] + pre_v[0][e] + bias_v[0][e];
-            const float gf = acc0[4 + e] + acc1[4 + e] + pre_v[1][e] + bias_v[1][e];
-            const float gg = acc0[8 + e] + acc1[8 + e] + pre_v[2][e] + bias_v[2][e];
-            const float go = acc0[12 + e] + acc1[12 + e] + pre_v[3][e] + bias_v[3][e];
-            const float cn = detail::sigmoid_fast(gf) * c_state[e] + detail::sigmoid_fast(gi) * detail::tanh_fast(gg);
+            // (pre_v already holds the bias)
+            const float gi = acc0[0 + e] + acc1[0 + e] + pre_v[0][e];
+            const float gf = acc0[4 + e] + acc1[4 + e] + pre_v[1][e];
+            const float gg = acc0[8 + e] + acc1[8 + e] + pre_v[2][e];
+            const float go = acc0[12 + e] + acc1[12 + e] + pre_v[3][e];
+            const float cn = detail::sigmoid_fast(gf) * c_state[e] + detail::sigmoid_times_tanh(gi, gg);
             c_state[e] = cn;
-            h_new[e] = static_cast<_Float16>(detail::sigmoid_fast(go) * detail::tanh_fast(cn));
+            h_new[e] = static_cast<_Float16>(detail::sigmoid_times_tanh(go, cn));
         }
         *reinterpret_cast<f16x4*>(h_all + (size_t(t) * B + b) * kH + hid) = h_new;
         if (t + 1 < T) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) pre_v[g] = widen_pre(pre_next[g]);
+            for (int g = 0; g < 4; ++g) pre_v[g] = widen_pre(pre_next[g]) + bias_v[g];  // (while the stores are under way)
             // arrival: every wavefront's stores of h_t have been acknowledged by the L2, then one lane counts
             detail::lds_barrier<0>();
             if (threadIdx.x == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-    }
+        return true;
+    };
+    // Without an initial hidden state step 0 multiplies nothing: it runs first, and the weights are fetched behind it
+    // (64 MiB through the fabric for the chip, ~10 us) while the XCD's first exchange of h is under way.
+    const int t0 = h0 ? 0 : 1;
+    if (!h0) time_step(0, std::false_type{});
+    if (t0 < T) load_weights();
+    for (int t = t0; t < T; ++t)
+        if (!time_step(t, std::true_type{})) return;
     *reinterpret_cast<f32x4*>(c_out + size_t(b) * kH + hid) = c_state;
 }
 
