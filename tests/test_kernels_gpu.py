@@ -944,6 +944,10 @@ def test_flash_attention_wave64_k32_head_size_64(tcu, oracle, device, batch, M, 
     ref_tail = oracle.attention(np.ascontiguousarray(q[heads, M - 64:]), np.ascontiguousarray(k[heads]),
                                 np.ascontiguousarray(v[heads]), 1.0 / math.sqrt(D))
     assert oracle.max_abs_err(host(out)[heads, M - 64:], ref_tail) <= tol
+    if N >= 1024 and batch * (M // 256) >= 256:
+        # long sequences with a block of 256 queries per CU: what AUTO runs
+        auto = tcu.flash_attention(dq, dk, dv)
+        assert torch.equal(auto, out)
 
 
 @pytest.mark.parametrize("algo", ["wave64", "tile_wave64", "wave64_k32"])
