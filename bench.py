@@ -458,6 +458,42 @@ def main():
         nbytes = 2.0 * (2 * Mr * 128 + 2 * 256 * 128)
         configs.append({"name": "b2b_65536x256x128x128_auto", "kernel": "b2b_gemm_rows<__half>", "ms": ms,
                         "gbs": nbytes / (ms * 1e-3) / 1e9, "tflops": 4.0 * Mr * 256 * 128 / (ms * 1e-3) / 1e12})
+        # the shapes the fast paths were widened to: a mid-size GEMM with edge tiles, b2b at K = P = 64 (the reference
+        # driver's inner sizes, fused_gemm.cu:212-259), the one-launch LSTM layer at a smaller hidden size
+        a_, b_ = rand16(1552, 4096), rand16(1552, 4096)
+        c_ = torch.empty(1552, 1552, dtype=torch.float16, device=dev)
+        ms = time_kernel(lambda: tcu.gemm(a_, b_, out=c_), 40, 20)
+        ms_v = time_kernel(lambda: torch.matmul(a_, b_.t(), out=c_), 40, 20)
+        configs.append({"name": "gemm_1552x1552x4096_auto", "kernel": "gemm_w128k<__half, edge tiles>", "ms": ms,
+                        "tflops": 2.0 * 1552 * 1552 * 4096 / (ms * 1e-3) / 1e12, "hipblaslt_ms": ms_v,
+                        "speed_vs_hipblaslt": ms_v / ms})
+        a_ = (torch.randn(8192, 64, device=dev) * 0.1).half()
+        b_ = (torch.randn(128, 64, device=dev) * 0.1).half()
+        c_ = (torch.randn(64, 128, device=dev) * 0.1).half()
+        d_ = torch.empty(8192, 64, dtype=torch.float16, device=dev)
+        ms_g = time_graph(lambda: tcu.b2b_gemm(a_, b_, c_, out=d_), 10 * args.steps, args.warmup)
+        ms_k = time_graph(lambda: tcu.b2b_gemm(a_, b_, c_, out=d_, algo="tile_library"), 10 * args.steps, args.warmup)
+        configs.append({"name": "b2b_8192x128x64x64_auto", "kernel": "b2b_gemm_tile_resident<N, 64, 64>",
+                        "us_in_hip_graph": None if ms_g is None else ms_g * 1e3,
+                        "tile_library_kernel_us_in_hip_graph": None if ms_k is None else ms_k * 1e3})
+        if want("lstm"):
+            Th, Bh, Hh2 = 16, 256, 512
+            xh = (torch.randn(Th, Bh, Hh2, device=dev) * 0.5).half()
+            Wh = (torch.randn(4 * Hh2, 2 * Hh2, device=dev) * 0.05).half()
+            bh = (torch.randn(4 * Hh2, device=dev) * 0.1).half()
+            wsh = torch.empty(tcu.lstm_persistent_workspace_bytes(Th, Bh, Hh2, Hh2), dtype=torch.uint8, device=dev)
+            outh = (torch.empty(Th, Bh, Hh2, dtype=torch.float16, device=dev), torch.empty(Bh, Hh2, dtype=torch.float32, device=dev))
+            ms_p = time_kernel(lambda: tcu.lstm(xh, Wh, bh, algo="persistent", workspace=wsh, out=outh, check=False), 20, 10)
+            ms_a = time_kernel(lambda: tcu.lstm(xh, Wh, bh, out=outh), 20, 10)
+            failure = None
+            try:
+                tcu.lstm_persistent_status(wsh)
+            except RuntimeError as exc:
+                failure = str(exc)
+            configs.append({"name": "lstm_b256_i512_h512_t16_persistent_single_launch", "kernel": "gemm_w128<__half> + lstm_recurrent_xcd<512>",
+                            "ms": ms_p, "us_per_step": ms_p * 1e3 / Th, "gave_up_waiting": failure,
+                            "launch_per_step_ms": ms_a})
+            del xh, Wh, bh, wsh, outh
         # the tile-API compositions beside their hand-indexed counterparts: interleaved (hand-indexed, composition, twice),
         # the better pass of each, so that both are timed in the same power state
         def pair(fn_hand, fn_tile, steps, warmup):
