@@ -17,8 +17,9 @@
 //     is still ahead of the LDS-bound tiling: 2048^3 24.4 us against 26.8 us (the vendor library: 24.6-25.8 us).
 //   * Accumulators in AGPRs through inline assembly, scalar-base addressing, XCD-aware tile order: as in gemm_w128.
 // The sum over K is taken in four interleaved parts, so results differ from the other kernels by f32 rounding.
-// K % 128 == 0; M % 128 == 0 and N % 128 == 0, or with kEdges any M, N in multiples of 16: the grid then covers
-// ceil(M / 128) x ceil(N / 128) tiles, rows beyond the edge are loaded from the last valid row (their products are
+// The tile is 128 x 128 or 128 x 96 (GemmW128kTraitsN: the numbers above are those of the wider one).
+// K % 128 == 0; M % 128 == 0 and N a multiple of the tile width, or with kEdges any M, N in multiples of 16: the grid
+// then covers ceil(M / 128) x ceil(N / width) tiles, rows beyond the edge are loaded from the last valid row (their products are
 // computed and dropped) and the stores are guarded per 16 x 16 block (checked by the launcher).
 #pragma once
 
@@ -30,25 +31,33 @@
 
 namespace tiledcuda::kernels {
 
-struct GemmW128kTraits {
-    static constexpr int kBM = 128, kBN = 128, kBK = 128;
+/// kNT_: 16-column tiles of a workgroup's tile: 8 (128 x 128) or 6 (128 x 96, for products that would fill two thirds of
+/// the chip with 128 x 128 tiles: a quarter more workgroups, each with a quarter less to multiply and an eighth less to
+/// load).
+template <const int kNT_ = 8>
+struct GemmW128kTraitsN {
+    static constexpr int kNT = kNT_;
+    static constexpr int kBM = 128, kBN = 16 * kNT, kBK = 128;
     static constexpr int kWaves = 4, kThreads = kWaves * kWaveSize;
     static constexpr int kRowBytes = kBK * 2;                      // 256
     static constexpr int kABytes = kBM * kRowBytes, kBBytes = kBN * kRowBytes;
-    static constexpr int kStageBytes = kABytes + kBBytes;          // 64 KiB
-    static constexpr int kLoads = kBM * kRowBytes / 1024 / kWaves;  // 1 KiB load instructions per operand per wavefront
-    static constexpr int kLdsBytes = 2 * kStageBytes;              // 128 KiB; the reduction reuses it
-    static_assert(kLoads == 8, "the phase schedule below is written for 8 + 8 loads per wavefront");
-    static_assert(kLdsBytes <= kMaxLdsBytes);
+    static constexpr int kStageBytes = kABytes + kBBytes;          // 64 KiB (56)
+    static constexpr int kLoads = kBM * kRowBytes / 1024 / kWaves;   // 1 KiB load instructions of A per wavefront
+    static constexpr int kLoadsB = kBN * kRowBytes / 1024 / kWaves;  // ... of B: 8 (6)
+    static constexpr int kFrags = 8 + kNT;                         // operand fragments of a phase
+    static constexpr int kLdsBytes = 2 * (kABytes + 128 * kRowBytes);  // 128 KiB; the reduction reuses it
+    static_assert(kLoads == 8 && (kNT == 8 || kNT == 6), "the phase schedule below is written for 8 + 8 or 8 + 6 loads per wavefront");
+    static_assert(kLdsBytes <= kMaxLdsBytes && 2 * kStageBytes <= kLdsBytes);
 };
+using GemmW128kTraits = GemmW128kTraitsN<8>;
 
-/// grid = (M / 128) * (N / 128), block = 256, dynamic LDS = GemmW128kTraits::kLdsBytes. lda / ldb / ldc: elements
-/// between consecutive rows of A, of the stored [N, K] array and of C. kEdges: grid = ceil(M / 128) * ceil(N / 128).
-template <typename OutType, bool kEdges = false>
-__global__ void __launch_bounds__(GemmW128kTraits::kThreads)
+/// grid = (M / 128) * (N / kBN), block = 256, dynamic LDS = T::kLdsBytes. lda / ldb / ldc: elements between consecutive
+/// rows of A, of the stored [N, K] array and of C. kEdges: grid = ceil(M / 128) * ceil(N / kBN).
+template <typename OutType, bool kEdges = false, typename T = GemmW128kTraits>
+__global__ void __launch_bounds__(T::kThreads)
     gemm_w128k(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
                int lda, int ldb, int ldc) {
-    using T = GemmW128kTraits;
+    constexpr int kNT = T::kNT, kNumLoads = 8 + T::kLoadsB;
     extern __shared__ __align__(1024) unsigned char lds[];
 
     const int lane = lane_id();
@@ -61,10 +70,10 @@ __global__ void __launch_bounds__(GemmW128kTraits::kThreads)
     // writes physical 16-byte chunk i % 16 of row i / 16, which must hold logical chunk (i % 16) ^ (row % 16).
     // kEdges: a row beyond the matrix is fetched from the last valid row instead (its LDS place and swizzle are its own)
     const int lrow = lane >> 4, lchk = lane & 15;
-    unsigned int voff[16];
+    unsigned int voff[kNumLoads];
 #pragma unroll
-    for (int q = 0; q < 16; ++q) {
-        const int row = (wave * T::kLoads + (q & 7)) * 4 + lrow;
+    for (int q = 0; q < kNumLoads; ++q) {
+        const int row = (q < 8 ? wave * T::kLoads + q : wave * T::kLoadsB + (q - 8)) * 4 + lrow;
         int src_row = row;
         if constexpr (kEdges) {
             const int last = (q < 8 ? M - m0 : N - n0) - 1;
@@ -77,7 +86,7 @@ __global__ void __launch_bounds__(GemmW128kTraits::kThreads)
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
     auto load_dst = [&](int stage, int q) -> unsigned int {
         return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +
-                                              (wave * T::kLoads + (q & 7)) * 1024);
+                                              (q < 8 ? wave * T::kLoads + q : wave * T::kLoadsB + (q - 8)) * 1024);
     };
     auto load_src = [&](int kt, int q) -> const __half* { return (q < 8 ? a_base : b_base) + kt * T::kBK; };
 
@@ -92,34 +101,40 @@ __global__ void __launch_bounds__(GemmW128kTraits::kThreads)
                                                chunk * 16);
     };
 
-    f16x8 fx[16], fy[16];  // fragments of the tile being multiplied / of the next one: [0..7] A, [8..15] B
+    f16x8 fx[T::kFrags], fy[T::kFrags];  // fragments of the tile being multiplied / of the next one: [0..7] A, [8..] B
     const int ktiles = K / T::kBK;
 #pragma unroll
-    for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
+    for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
 #pragma unroll
-    for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(ktiles > 1 ? 1 : 0, q), load_dst(1, q));
-    f32x4 acc[8][8];
+    for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(ktiles > 1 ? 1 : 0, q), load_dst(1, q));
+    // the accumulators are pinned to the AGPR half row group by row group
+    auto pin_row = [](f32x4 (&row)[kNT]) {
+        if constexpr (kNT == 8)
+            asm volatile("" : "+a"(row[0]), "+a"(row[1]), "+a"(row[2]), "+a"(row[3]), "+a"(row[4]), "+a"(row[5]), "+a"(row[6]), "+a"(row[7]));
+        else
+            asm volatile("" : "+a"(row[0]), "+a"(row[1]), "+a"(row[2]), "+a"(row[3]), "+a"(row[4]), "+a"(row[5]));
+    };
+    f32x4 acc[8][kNT];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        asm volatile(""
-                     : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),
-                       "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]));
+        for (int j = 0; j < kNT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        pin_row(acc[i]);
     }
-    detail::lds_barrier<16>();  // tile 0 has landed, for everyone
+    detail::lds_barrier<kNumLoads>();  // tile 0 has landed, for everyone
 #pragma unroll
-    for (int r = 0; r < 16; ++r) fx[r] = read_frag(0, r);
+    for (int r = 0; r < T::kFrags; ++r) fx[r] = read_frag(0, r);
 
-    constexpr int kOrder[16] = {0, 8, 9, 10, 11, 12, 13, 14, 15, 1, 2, 3, 4, 5, 6, 7};
-    auto snake = [](int i, int n) { return (i & 1) ? 7 - n : n; };
+    // the order in which the fragments of the next tile are read: its first row group needs A fragment 0 and all of B
+    auto order = [](int r) { return r == 0 ? 0 : r <= kNT ? 7 + r : r - kNT; };
+    auto snake = [](int i, int n) { return (i & 1) ? kNT - 1 - n : n; };
 
     // One tile of K out of `cur`, reading the next tile's fragments into `nxt` and loading the tile after that into
     // the stage `cur`'s tile came from. Every phase is the same straight-line code: behind the last tile of K the
     // fragment reads fetch stale data that nobody uses and the loads fetch the last tile once more (clamped index) -
     // cheaper than peeled copies of the phase, whose control-flow merges made the compiler shuffle and spill
     // accumulators between the assembly statements, where it knows of no wait states.
-    auto tile = [&](int kt, f16x8 (&cur)[16], f16x8 (&nxt)[16]) {
+    auto tile = [&](int kt, f16x8 (&cur)[T::kFrags], f16x8 (&nxt)[T::kFrags]) {
         const int stage = kt & 1;
         const int kload = kt + 2 < ktiles ? kt + 2 : ktiles - 1;
         // tile kt + 1 has landed and this wavefront's reads of `stage` (issued during the previous phase) have
@@ -128,12 +143,12 @@ __global__ void __launch_bounds__(GemmW128kTraits::kThreads)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
-            for (int n = 0; n < 8; ++n) {
+            for (int n = 0; n < kNT; ++n) {
                 const int j = snake(i, n);
-                const int r = 4 * i + (n >> 1);
-                if ((n & 1) == 0 && r < 16) nxt[kOrder[r]] = read_frag(stage ^ 1, kOrder[r]);
-                if ((n & 3) == 1) {
-                    const int q = 2 * i + (n >> 2);
+                const int r = (kNT / 2) * i + (n >> 1);
+                if ((n & 1) == 0 && r < T::kFrags) nxt[order(r)] = read_frag(stage ^ 1, order(r));
+                const int q = 2 * i + (n >> 2);
+                if ((n & 3) == 1 && q < kNumLoads) {
                     detail::mfma_16x16x32_agpr_then_load(acc[i][j], cur[8 + j], cur[i], voff[q], load_src(kload, q),
                                                          load_dst(stage, q));
                 } else {
@@ -153,35 +168,33 @@ __global__ void __launch_bounds__(GemmW128kTraits::kThreads)
 
     detail::mfma_results_wait();
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-        asm volatile(""
-                     : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),
-                       "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]));
+    for (int i = 0; i < 8; ++i) pin_row(acc[i]);
 
-    // ---- the four partial tiles are added through LDS, two row groups (32 rows, 16 MFMA tiles) per round. Every
-    // wavefront writes its 16 partial tiles of the round - tile t = 8 (row group % 2) + column tile, 1 KiB each, a
+    // ---- the four partial tiles are added through LDS, two row groups (32 rows, 2 kNT MFMA tiles) per round. Every
+    // wavefront writes its partial tiles of the round - tile t = kNT (row group % 2) + column tile, 1 KiB each, a
     // lane's f32x4 at 16 * lane: conflict-free and the same for writer and reader - and then sums the four partials
-    // of tiles 4 w .. 4 w + 3 into registers of its own. Which tiles a wavefront sums is a matter of LDS addresses
-    // only: register indices are the same in all four wavefronts (an index that depended on the wavefront would put
-    // the accumulators into scratch memory). Two buffers of 64 KiB alternate, so one barrier per round is enough: a
+    // of tiles (kNT / 2) w .. + kNT / 2 - 1 into registers of its own. Which tiles a wavefront sums is a matter of LDS
+    // addresses only: register indices are the same in all four wavefronts (an index that depended on the wavefront would
+    // put the accumulators into scratch memory). Two buffers of 64 KiB alternate, so one barrier per round is enough: a
     // buffer is written again two rounds later, after the barrier of the round in between.
-    // Wavefront w ends up with rows 32 r + 16 (w / 2) .. + 15 (r = 0 .. 3), columns 64 (w % 2) .. + 63.
+    // Wavefront w ends up with rows 32 r + 16 (w / 2) .. + 15 (r = 0 .. 3), column tiles (kNT / 2) (w % 2) .. + kNT / 2 - 1.
     detail::lds_barrier<0>();  // nothing is on its way into LDS any more, every wavefront is done with the operand stages
     using lds_f32x4_ptr = __attribute__((address_space(3))) f32x4*;
-    f32x4 res[4][4];
+    constexpr int kPerRound = 2 * kNT, kMine = kNT / 2;
+    f32x4 res[4][kMine];
 #pragma unroll
     for (int round = 0; round < 4; ++round) {
         const unsigned int buf = lds_base + (round & 1) * (64 * 1024) + lane * 16;
 #pragma unroll
-        for (int t = 0; t < 16; ++t)
-            *reinterpret_cast<lds_f32x4_ptr>(buf + (wave * 16 + t) * 1024) = acc[2 * round + t / 8][t % 8];
+        for (int t = 0; t < kPerRound; ++t)
+            *reinterpret_cast<lds_f32x4_ptr>(buf + (wave * kPerRound + t) * 1024) = acc[2 * round + t / kNT][t % kNT];
         __syncthreads();
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-            f32x4 sum = *reinterpret_cast<lds_f32x4_ptr>(buf + (4 * wave + jj) * 1024);
+        for (int jj = 0; jj < kMine; ++jj) {
+            f32x4 sum = *reinterpret_cast<lds_f32x4_ptr>(buf + (kMine * wave + jj) * 1024);
 #pragma unroll
             for (int w = 1; w < 4; ++w) {
-                const f32x4 v = *reinterpret_cast<lds_f32x4_ptr>(buf + (w * 16 + 4 * wave + jj) * 1024);
+                const f32x4 v = *reinterpret_cast<lds_f32x4_ptr>(buf + (w * kPerRound + kMine * wave + jj) * 1024);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sum[e] += v[e];
             }
@@ -189,16 +202,16 @@ __global__ void __launch_bounds__(GemmW128kTraits::kThreads)
         }
     }
 
-    // ---- store: res[r][jj][e] = C[32 r + 16 (w / 2) + lane % 16][64 (w % 2) + 16 jj + 4 (lane / 16) + e] of the tile
-    OutType* cbase = C + size_t(m0 + 16 * (wave >> 1) + frow) * ldc + n0 + 64 * (wave & 1) + 4 * fquad;
+    // ---- store: res[r][jj][e] = C[32 r + 16 (w / 2) + lane % 16][16 (kMine (w % 2) + jj) + 4 (lane / 16) + e] of the tile
+    OutType* cbase = C + size_t(m0 + 16 * (wave >> 1) + frow) * ldc + n0 + 16 * kMine * (wave & 1) + 4 * fquad;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
+        for (int jj = 0; jj < kMine; ++jj) {
             OutType* p = cbase + size_t(32 * r) * ldc + 16 * jj;
             if constexpr (kEdges) {
                 // M and N are multiples of 16: a 16 x 16 block lies inside the matrix or outside it as a whole
-                if (m0 + 32 * r + 16 * (wave >> 1) >= M || n0 + 64 * (wave & 1) + 16 * jj >= N) continue;
+                if (m0 + 32 * r + 16 * (wave >> 1) >= M || n0 + 16 * kMine * (wave & 1) + 16 * jj >= N) continue;
             }
             if constexpr (sizeof(OutType) == 4) {
                 *reinterpret_cast<f32x4*>(p) = res[r][jj];

@@ -121,13 +121,15 @@ def test_gemm_ragged_shapes(tcu, oracle, device, M, N, K, out_dtype):
 
 
 @pytest.mark.parametrize("M,N,K,splits", [(256, 256, 8192, 16), (512, 512, 16384, 32), (1024, 1024, 16384, 16),
-                                          (2048, 2048, 8192, 4), (1024, 1024, 8192, 1), (256, 512, 512, 1), (2048, 2048, 2048, 1)])
+                                          (2048, 2048, 16384, 4), (2048, 2048, 8192, 1), (1536, 1536, 4096, 1),
+                                          (1024, 1024, 8192, 1), (256, 512, 512, 1), (2048, 2048, 2048, 1)])
 @pytest.mark.parametrize("out_dtype", ["f32", "f16"])
 def test_gemm_split_k_with_workspace(tcu, oracle, device, M, N, K, splits, out_dtype):
     """tcu_gemm_f16_ws: few output tiles and a long K are split over K (f32 partial products in the caller's workspace,
     then a reduction) where that is expected to beat the unsplit launch; against the oracle and against the unsplit
-    kernel; the workspace size is splits * M * N * 4, bytes past it stay untouched; shapes that are not split (last three
-    cases) take the ordinary path and need no workspace."""
+    kernel; the workspace size is splits * M * N * 4, bytes past it stay untouched; shapes that are not split (last five
+    cases: among them 2048 x 2048 x 8192 and 1536 x 1536 x 4096, where the kernel whose wavefronts split K inside the
+    workgroup is the faster plan) take the ordinary path and need no workspace."""
     import torch
 
     print(f"gemm split-K {M}x{N}x{K} {out_dtype}", flush=True)
@@ -333,13 +335,16 @@ def test_gemm_wave128_ksplit(tcu, oracle, device, M, N, K, out_dtype):
         assert np.max(np.abs(got - want)) <= (5.0 if out_dtype == "f16" else 0.1)
 
 
-@pytest.mark.parametrize("M,N,K", [(16, 16, 128), (144, 112, 256), (272, 400, 384), (1552, 1552, 4096), (1536, 1616, 2048)])
+@pytest.mark.parametrize("M,N,K", [(16, 16, 128), (144, 112, 256), (272, 400, 384), (1552, 1552, 4096), (1536, 1616, 2048),
+                                   (1808, 1936, 256), (1536, 1536, 512)])
 @pytest.mark.parametrize("out_dtype", ["f16", "f32"])
 def test_gemm_wave128_ksplit_edge_tiles(tcu, oracle, device, M, N, K, out_dtype):
-    """The K-splitting kernel on shapes that are not whole 128 x 128 tiles (M, N in multiples of 16): rows beyond the
-    edge are fetched from the last valid row and their results dropped, the stores are guarded - nothing outside C is
-    written (guard rows and guard columns around it) and every element of C matches the oracle. 1552 x 1552 x 4096
-    (169 tiles) is a shape AUTO sends to it."""
+    """The K-splitting kernel on shapes that are not whole tiles (M, N in multiples of 16): rows beyond the edge are
+    fetched from the last valid row and their results dropped, the stores are guarded - nothing outside C is written
+    (guard rows and guard columns around it) and every element of C matches the oracle. Both tile widths: 128 x 96
+    where 128 x 128 tiles would leave a quarter of the CUs idle (1552 x 1552 x 4096: 221 instead of 169 workgroups, a
+    shape AUTO sends to this kernel; 1536 x 1536: whole 128 x 96 tiles), 128 x 128 otherwise (1808 x 1936: 240 tiles
+    with edges)."""
     import torch
 
     print(f"gemm wave128_ksplit edges {M}x{N}x{K} {out_dtype}", flush=True)

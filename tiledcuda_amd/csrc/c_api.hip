@@ -239,6 +239,18 @@ int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int 
                   C, M, N, K, lda, ldb, ldc, zero_words, zero_count);
 }
 
+template <typename OutType, typename T>
+int launch_gemm_w128k(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    const long grid = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
+    if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many tiles for one launch");
+    if (M % T::kBM == 0 && N % T::kBN == 0)
+        return launch(&gemm_w128k<OutType, false, T>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C,
+                      M, N, K, K, K, N);
+    // edge tiles: rows beyond M or N loaded from the last valid row, stores guarded per 16 x 16 block
+    return launch(&gemm_w128k<OutType, true, T>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M,
+                  N, K, K, K, N);
+}
+
 template <typename OutType>
 int gemm_w128k_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
     using T = GemmW128kTraits;
@@ -247,14 +259,17 @@ int gemm_w128k_dispatch(const __half* A, const __half* B, OutType* C, int M, int
                                                "and K in multiples of 128");
     if ((long)K * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the K-splitting GEMM addresses a 128-row panel with 32-bit offsets");
-    const long grid = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
-    if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many tiles for one launch");
-    if (M % T::kBM == 0 && N % T::kBN == 0)
-        return launch(&gemm_w128k<OutType, false>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M,
-                      N, K, K, K, N);
-    // edge tiles: rows beyond M or N loaded from the last valid row, stores guarded per 16 x 16 block
-    return launch(&gemm_w128k<OutType, true>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M, N,
-                  K, K, K, N);
+    // All workgroups run at once (one per CU), so the launch takes as long as one tile: when 128 x 128 tiles would
+    // leave a quarter of the CUs idle and 128 x 96 tiles still fit one round, the smaller tile is the shorter launch
+    const long rows = (M + 127) / 128;
+    const long tiles128 = rows * ((N + 127) / 128), tiles96 = rows * ((N + 95) / 96);
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
+        cus = 0;
+    if (cus > 0 && tiles128 <= (3l * cus) / 4 && tiles96 <= cus)
+        return launch_gemm_w128k<OutType, GemmW128kTraitsN<6>>(A, B, C, M, N, K, stream);
+    return launch_gemm_w128k<OutType, T>(A, B, C, M, N, K, stream);
 }
 
 template <typename OutType, int kM, int kN, int kK, int kTM, int kTN, typename WarpLayout>
@@ -327,12 +342,29 @@ int gemm_main_and_strips(const __half* A, const __half* B, OutType* C, int M, in
 /// expected to beat the unsplit launch by 5 %. Expected cost of s ranges (measured, one workgroup per CU at most):
 /// 10 us for the two launches and the epilogues + 1.4 us per k-tile of a range + the partial products written and
 /// read once (2 x s x M x N x 4 bytes at 5.3 TB/s); of the unsplit launch: pipelined_plan().
+/// Whether AUTO sends an unsplit product to the kernel whose wavefronts split K: about one 128 x 128 tile per CU and a
+/// long enough K (2048^3: 24.4 against 26.8 us for the LDS-bound 64 x 64-per-wavefront tilings, 1536 x 1536 x 4096: 32.5
+/// against 38.5 us); with a short K its reduction through LDS costs more than it saves (1792 x 1792 x 1024: 16.0 against
+/// 13.1 us).
+bool gemm_w128k_is_the_choice(int M, int N, int K) {
+    if (M % 16 != 0 || N % 16 != 0 || K % 128 != 0 || K < 2048 || (long)K * 256 >= (1l << 32)) return false;
+    const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    return tiles >= 128 && tiles <= 256;
+}
+
 int gemm_split_count(int M, int N, int K) {
     using T = GemmW128Traits;
     if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0) return 1;
     const long tiles = (long)(M / T::kBM) * (N / T::kBN);
     if (tiles > 128) return 1;
-    const double unsplit_us = pipelined_plan(M, N, K).us;
+    double unsplit_us = pipelined_plan(M, N, K).us;
+    // the K-splitting kernel, where AUTO would run it: one round of workgroups, 5 us + 1.2 us per 128 of K with 128 x 128
+    // tiles, 0.85 us with 128 x 96 tiles (measured)
+    if (gemm_w128k_is_the_choice(M, N, K)) {
+        const long tiles128 = (long)(M / 128) * (N / 128), tiles96 = (long)(M / 128) * ((N + 95) / 96);
+        const double per_tile = tiles128 <= 192 && tiles96 <= 256 ? 0.85 : 1.05;
+        unsplit_us = std::min(unsplit_us, 5.0 + per_tile * (K / 128));
+    }
     int best = 1;
     double best_us = 0.95 * unsplit_us;
     for (int s = 2; s * tiles <= 256 && K % (s * T::kBK) == 0 && K / s >= 512; s *= 2) {
@@ -388,13 +420,8 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
                 (long)K * 512 < (1l << 32))
                 return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
             // too few 256 x 256 tiles for the chip, but about one 128 x 128 tile per CU and a long enough K: the
-            // kernel whose wavefronts split K (each owns the whole 128 x 128 tile) beats the LDS-bound 64 x 64-per-
-            // wavefront tilings (2048^3: 24.4 against 26.8 us, 1536 x 1536 x 4096: 35.7 against 39.8 us); with a
-            // short K its reduction through LDS costs more than it saves (1792 x 1792 x 1024: 16.0 against 13.1 us)
-            if (M % 16 == 0 && N % 16 == 0 && K % 128 == 0 && K >= 2048 && (long)K * 256 < (1l << 32)) {
-                const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-                if (tiles >= 128 && tiles <= 256) return gemm_w128k_dispatch<OutType>(A, B, C, M, N, K, stream);
-            }
+            // kernel whose wavefronts split K (each owns the whole tile)
+            if (gemm_w128k_is_the_choice(M, N, K)) return gemm_w128k_dispatch<OutType>(A, B, C, M, N, K, stream);
             if (M % 16 == 0 && N % 16 == 0) {
                 const int rc = gemm_main_and_strips<OutType>(A, B, C, M, N, K, stream);
                 if (rc != kPlanNotTaken) return rc;
