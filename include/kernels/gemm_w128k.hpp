@@ -8,13 +8,16 @@
 //     (16 reads per 64 instructions, half the LDS traffic, the gemm_w128 ratio) over a quarter of K: a tile of K is
 //     128 wide, wavefront w multiplies columns 32 w .. 32 w + 31 of it. The four partial tiles are added through LDS
 //     at the end, after which wavefront w holds rows 32 w .. 32 w + 31 of the result and stores them.
-//   * A stage is 128 + 128 rows of 256 bytes = 64 KiB; two stages. One phase per tile of K: 64 MFMAs, with the 16
-//     fragment reads of the next tile (one per two MFMAs) and this wavefront's 16 direct-to-LDS loads of the tile after
-//     that (one per four MFMAs, each in one statement with its MFMA), then one LDS-only barrier. The loads of a tile
-//     have one phase to land (a third stage does not fit), and a workgroup pulls 64 KiB per 1024 cycles of matrix
-//     work through its CU's load path: the loop runs at the pace of those loads (a phase measures about 1.2 us at
-//     2048^3, the same whether the loads are issued one per four, three or two MFMAs), not of the matrix pipe. That
-//     is still ahead of the LDS-bound tiling: 2048^3 24.4 us against 26.8 us (the vendor library: 24.6-25.8 us).
+//   * The A part and the B part of a tile of K (128 rows of 256 bytes = 32 KiB each) pass through a ring of five 32 KiB
+//     slots in the order A0 B0 A1 B1 A2 ... One phase per tile of K: 64 MFMAs, with the 16 fragment reads of the next
+//     tile (one per two MFMAs) and this wavefront's 16 direct-to-LDS loads (one per four MFMAs, each in one statement
+//     with its MFMA): first B of the tile after the next, then A of the one after that, into the two slots the current
+//     tile came from; then one LDS-only barrier, which waits for that B part but not for the A part requested behind it.
+//     B has most of a phase to land and A a phase more. (With two stages of 64 KiB the last load of a tile was
+//     requested at the very end of the phase whose closing barrier waited for it, so a phase took as long as a load:
+//     1.2 us at 2048^3 for 0.5 us of matrix work, whether the loads were issued one per four, three or two MFMAs. The
+//     ring: 1536 x 1536 x 4096 32.4 -> 26.6 us, 2048^3 22.8 -> 21.9 us; a full third stage does not fit 160 KiB.)
+//     Against the LDS-bound tiling: 2048^3 21.9 us against 26.8 us (the vendor library: 21-23.4 us).
 //   * Accumulators in AGPRs through inline assembly, scalar-base addressing, XCD-aware tile order: as in gemm_w128.
 // The sum over K is taken in four interleaved parts, so results differ from the other kernels by f32 rounding.
 // The tile is 128 x 128 or 128 x 96 (GemmW128kTraitsN: the numbers above are those of the wider one).
@@ -41,13 +44,14 @@ struct GemmW128kTraitsN {
     static constexpr int kWaves = 4, kThreads = kWaves * kWaveSize;
     static constexpr int kRowBytes = kBK * 2;                      // 256
     static constexpr int kABytes = kBM * kRowBytes, kBBytes = kBN * kRowBytes;
-    static constexpr int kStageBytes = kABytes + kBBytes;          // 64 KiB (56)
+    static constexpr int kSlotBytes = kABytes;                     // a ring slot holds the A or the B part of a tile of K
+    static constexpr int kSlots = 5;
     static constexpr int kLoads = kBM * kRowBytes / 1024 / kWaves;   // 1 KiB load instructions of A per wavefront
     static constexpr int kLoadsB = kBN * kRowBytes / 1024 / kWaves;  // ... of B: 8 (6)
     static constexpr int kFrags = 8 + kNT;                         // operand fragments of a phase
-    static constexpr int kLdsBytes = 2 * (kABytes + 128 * kRowBytes);  // 128 KiB; the reduction reuses it
+    static constexpr int kLdsBytes = kSlots * kSlotBytes;          // 160 KiB; the reduction reuses 128 of it
     static_assert(kLoads == 8 && (kNT == 8 || kNT == 6), "the phase schedule below is written for 8 + 8 or 8 + 6 loads per wavefront");
-    static_assert(kLdsBytes <= kMaxLdsBytes && 2 * kStageBytes <= kLdsBytes);
+    static_assert(kLdsBytes <= kMaxLdsBytes && kBBytes <= kSlotBytes);
 };
 using GemmW128kTraits = GemmW128kTraitsN<8>;
 
@@ -84,8 +88,11 @@ __global__ void __launch_bounds__(T::kThreads)
     const __half* a_base = A + size_t(m0) * lda;
     const __half* b_base = Bt + size_t(n0) * ldb;
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
-    auto load_dst = [&](int stage, int q) -> unsigned int {
-        return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +
+    // The A and B parts of the tiles of K pass through a ring of five 32 KiB slots in the order A0 B0 A1 B1 A2 ...:
+    // part u lives in slot u % 5 (A of tile t: u = 2 t, B: u = 2 t + 1).
+    auto slot_bytes = [](int unit) -> unsigned int { return static_cast<unsigned int>(unit % T::kSlots) * T::kSlotBytes; };
+    auto load_dst = [&](unsigned int slot, int q) -> unsigned int {
+        return __builtin_amdgcn_readfirstlane(lds_base + slot +
                                               (q < 8 ? wave * T::kLoads + q : wave * T::kLoadsB + (q - 8)) * 1024);
     };
     auto load_src = [&](int kt, int q) -> const __half* { return (q < 8 ? a_base : b_base) + kt * T::kBK; };
@@ -94,19 +101,22 @@ __global__ void __launch_bounds__(T::kThreads)
     // k = 32 wave + 8 (l / 16) .. + 7 of the tile = logical chunk 4 wave + l / 16 of its row. The 16 rows a 16-lane
     // group reads have 16 different values of row % 16: 16 different chunks, no bank conflict.
     const int frow = lane & 15, fquad = lane >> 4;
-    auto read_frag = [&](int stage, int r) -> f16x8 {
+    auto read_frag = [&](unsigned int slot_a, unsigned int slot_b, int r) -> f16x8 {
         const int row = (r & 7) * 16 + frow;
         const int chunk = (4 * wave + fquad) ^ (row & 15);
-        return *reinterpret_cast<const f16x8*>(lds + stage * T::kStageBytes + (r < 8 ? 0 : T::kABytes) + row * T::kRowBytes +
-                                               chunk * 16);
+        return *reinterpret_cast<const f16x8*>(lds + (r < 8 ? slot_a : slot_b) + row * T::kRowBytes + chunk * 16);
     };
 
     f16x8 fx[T::kFrags], fy[T::kFrags];  // fragments of the tile being multiplied / of the next one: [0..7] A, [8..] B
     const int ktiles = K / T::kBK;
+    auto clamped = [&](int kt) { return kt < ktiles ? kt : ktiles - 1; };
+    // prologue: A0 B0 A1 B1 A2 fill the ring
 #pragma unroll
-    for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
+    for (int u = 0; u < T::kSlots; ++u) {
 #pragma unroll
-    for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(ktiles > 1 ? 1 : 0, q), load_dst(1, q));
+        for (int q = (u & 1) ? 8 : 0; q < ((u & 1) ? kNumLoads : 8); ++q)
+            detail::load_lds_16B_sbase(voff[q], load_src(clamped(u >> 1), q), load_dst(u * T::kSlotBytes, q));
+    }
     // the accumulators are pinned to the AGPR half row group by row group
     auto pin_row = [](f32x4 (&row)[kNT]) {
         if constexpr (kNT == 8)
@@ -121,36 +131,42 @@ __global__ void __launch_bounds__(T::kThreads)
         for (int j = 0; j < kNT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
         pin_row(acc[i]);
     }
-    detail::lds_barrier<kNumLoads>();  // tile 0 has landed, for everyone
+    detail::lds_barrier<16 + T::kLoadsB>();  // tile 0 has landed (behind it: A1 B1 A2), for everyone
 #pragma unroll
-    for (int r = 0; r < T::kFrags; ++r) fx[r] = read_frag(0, r);
+    for (int r = 0; r < T::kFrags; ++r) fx[r] = read_frag(0, T::kSlotBytes, r);
 
     // the order in which the fragments of the next tile are read: its first row group needs A fragment 0 and all of B
     auto order = [](int r) { return r == 0 ? 0 : r <= kNT ? 7 + r : r - kNT; };
     auto snake = [](int i, int n) { return (i & 1) ? kNT - 1 - n : n; };
 
-    // One tile of K out of `cur`, reading the next tile's fragments into `nxt` and loading the tile after that into
-    // the stage `cur`'s tile came from. Every phase is the same straight-line code: behind the last tile of K the
-    // fragment reads fetch stale data that nobody uses and the loads fetch the last tile once more (clamped index) -
-    // cheaper than peeled copies of the phase, whose control-flow merges made the compiler shuffle and spill
-    // accumulators between the assembly statements, where it knows of no wait states.
+    // One tile of K out of `cur`, reading the next tile's fragments into `nxt`, and loading B of tile kt + 2 and then A of
+    // tile kt + 3 into the slots `cur`'s tile came from. B of a tile is requested first in its phase and has the rest
+    // of it to land (the barrier at the top of the next phase waits for it, not for the A part requested behind it); A
+    // has a phase more. With two 64 KiB stages the last load of a tile was requested at the very end of the phase
+    // whose closing barrier waited for it: the phase took as long as a load.
+    // Every phase is the same straight-line code: behind the last tile of K the fragment reads fetch stale data that
+    // nobody uses and the loads fetch the last tile once more (clamped index) - cheaper than peeled copies of the
+    // phase, whose control-flow merges made the compiler shuffle and spill accumulators between the assembly
+    // statements, where it knows of no wait states.
     auto tile = [&](int kt, f16x8 (&cur)[T::kFrags], f16x8 (&nxt)[T::kFrags]) {
-        const int stage = kt & 1;
-        const int kload = kt + 2 < ktiles ? kt + 2 : ktiles - 1;
-        // tile kt + 1 has landed and this wavefront's reads of `stage` (issued during the previous phase) have
-        // returned; then everyone's
-        detail::lds_barrier<0>();
+        const unsigned int read_a = slot_bytes(2 * kt + 2), read_b = slot_bytes(2 * kt + 3);  // tile kt + 1
+        const unsigned int load_b = slot_bytes(2 * kt + 5), load_a = slot_bytes(2 * kt + 6);  // = the slots of tile kt
+        const int kt_b = clamped(kt + 2), kt_a = clamped(kt + 3);
+        // tile kt + 1 has landed (behind its B part: the A part of tile kt + 2) and this wavefront's reads of tile kt's
+        // slots (issued during the previous phase) have returned; then everyone's
+        detail::lds_barrier<8>();
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
             for (int n = 0; n < kNT; ++n) {
                 const int j = snake(i, n);
                 const int r = (kNT / 2) * i + (n >> 1);
-                if ((n & 1) == 0 && r < T::kFrags) nxt[order(r)] = read_frag(stage ^ 1, order(r));
-                const int q = 2 * i + (n >> 2);
-                if ((n & 3) == 1 && q < kNumLoads) {
-                    detail::mfma_16x16x32_agpr_then_load(acc[i][j], cur[8 + j], cur[i], voff[q], load_src(kload, q),
-                                                         load_dst(stage, q));
+                if ((n & 1) == 0 && r < T::kFrags) nxt[order(r)] = read_frag(read_a, read_b, order(r));
+                const int s = 2 * i + (n >> 2);  // load slot of the phase: B of tile kt + 2 first, then A of tile kt + 3
+                if ((n & 3) == 1 && s < kNumLoads) {
+                    const int q = s < T::kLoadsB ? 8 + s : s - T::kLoadsB;
+                    detail::mfma_16x16x32_agpr_then_load(acc[i][j], cur[8 + j], cur[i], voff[q],
+                                                         load_src(q < 8 ? kt_a : kt_b, q), load_dst(q < 8 ? load_a : load_b, q));
                 } else {
                     detail::mfma_16x16x32_agpr(acc[i][j], cur[8 + j], cur[i]);
                 }

@@ -359,10 +359,10 @@ int gemm_split_count(int M, int N, int K) {
     if (tiles > 128) return 1;
     double unsplit_us = pipelined_plan(M, N, K).us;
     // the K-splitting kernel, where AUTO would run it: one round of workgroups, 5 us + 1.2 us per 128 of K with 128 x 128
-    // tiles, 0.85 us with 128 x 96 tiles (measured)
+    // tiles, 0.75 us with 128 x 96 tiles (measured)
     if (gemm_w128k_is_the_choice(M, N, K)) {
         const long tiles128 = (long)(M / 128) * (N / 128), tiles96 = (long)(M / 128) * ((N + 95) / 96);
-        const double per_tile = tiles128 <= 192 && tiles96 <= 256 ? 0.85 : 1.05;
+        const double per_tile = tiles128 <= 192 && tiles96 <= 256 ? 0.75 : 1.05;
         unsplit_us = std::min(unsplit_us, 5.0 + per_tile * (K / 128));
     }
     int best = 1;
