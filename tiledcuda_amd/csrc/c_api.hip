@@ -343,11 +343,11 @@ int gemm_main_and_strips(const __half* A, const __half* B, OutType* C, int M, in
 /// 10 us for the two launches and the epilogues + 1.4 us per k-tile of a range + the partial products written and
 /// read once (2 x s x M x N x 4 bytes at 5.3 TB/s); of the unsplit launch: pipelined_plan().
 /// Whether AUTO sends an unsplit product to the kernel whose wavefronts split K: about one 128 x 128 tile per CU and a
-/// long enough K (2048^3: 24.4 against 26.8 us for the LDS-bound 64 x 64-per-wavefront tilings, 1536 x 1536 x 4096: 32.5
-/// against 38.5 us); with a short K its reduction through LDS costs more than it saves (1792 x 1792 x 1024: 16.0 against
-/// 13.1 us).
+/// long enough K (2048^3: 21.9 against 26.8 us for the LDS-bound 64 x 64-per-wavefront tilings, 1536 x 1536 x 4096: 26.6
+/// against 38.5 us, 2048 x 2048 x 1536: 19.8 against 22.6 us); with a short K its reduction through LDS costs more than
+/// it saves (1792 x 1792 x 1024: 15.6 against 14.1 us).
 bool gemm_w128k_is_the_choice(int M, int N, int K) {
-    if (M % 16 != 0 || N % 16 != 0 || K % 128 != 0 || K < 2048 || (long)K * 256 >= (1l << 32)) return false;
+    if (M % 16 != 0 || N % 16 != 0 || K % 128 != 0 || K < 1536 || (long)K * 256 >= (1l << 32)) return false;
     const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
     return tiles >= 128 && tiles <= 256;
 }
