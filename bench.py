@@ -447,7 +447,7 @@ def main():
         c_ = torch.empty(1024, 1024, dtype=torch.float16, device=dev)
         ws_ = torch.empty(max(16, tcu.gemm_workspace_bytes(1024, 1024, 16384)), dtype=torch.uint8, device=dev)
         ms = time_kernel(lambda: tcu.gemm(a_, b_, out=c_, workspace=ws_), 40, 20)
-        configs.append({"name": "gemm_1024x1024x16384_split_k", "kernel": "gemm_w128<float> over K-ranges + splitk_reduce<__half>",
+        configs.append({"name": "gemm_1024x1024x16384_split_k", "kernel": "gemm_w128k<float> over 4 K-ranges + splitk_reduce<__half>",
                         "ms": ms, "workspace_bytes": int(ws_.numel()), "tflops": 2.0 * 1024 * 1024 * 16384 / (ms * 1e-3) / 1e12})
         Mr = 65536
         a_ = (torch.randn(Mr, 128, device=dev) * 0.1).half()

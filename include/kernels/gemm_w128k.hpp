@@ -55,8 +55,10 @@ struct GemmW128kTraitsN {
 };
 using GemmW128kTraits = GemmW128kTraitsN<8>;
 
-/// grid = (M / 128) * (N / kBN), block = 256, dynamic LDS = T::kLdsBytes. lda / ldb / ldc: elements between consecutive
-/// rows of A, of the stored [N, K] array and of C. kEdges: grid = ceil(M / 128) * ceil(N / kBN).
+/// grid = ((M / 128) * (N / kBN), splits), block = 256, dynamic LDS = T::kLdsBytes. lda / ldb / ldc: elements between
+/// consecutive rows of A, of the stored [N, K] array and of C. kEdges: grid.x = ceil(M / 128) * ceil(N / kBN). With
+/// splits > 1 workgroup row z multiplies the K-range [z K, (z + 1) K) of wider operands (lda, ldb >= splits * K) and
+/// writes plane z of C ([splits, M, N]: partial sums for splitk_reduce).
 template <typename OutType, bool kEdges = false, typename T = GemmW128kTraits>
 __global__ void __launch_bounds__(T::kThreads)
     gemm_w128k(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
@@ -85,8 +87,10 @@ __global__ void __launch_bounds__(T::kThreads)
         }
         voff[q] = static_cast<unsigned int>(src_row) * static_cast<unsigned int>(q < 8 ? lda : ldb) * 2u + (lchk ^ (row & 15)) * 16;
     }
-    const __half* a_base = A + size_t(m0) * lda;
-    const __half* b_base = Bt + size_t(n0) * ldb;
+    const size_t z = blockIdx.y;
+    const __half* a_base = A + size_t(m0) * lda + z * K;
+    const __half* b_base = Bt + size_t(n0) * ldb + z * K;
+    C += z * size_t(M) * ldc;
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
     // The A and B parts of the tiles of K pass through a ring of five 32 KiB slots in the order A0 B0 A1 B1 A2 ...:
     // part u lives in slot u % 5 (A of tile t: u = 2 t, B: u = 2 t + 1).

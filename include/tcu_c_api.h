@@ -146,9 +146,10 @@ int tcu_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K, int
 
 /*
  * tcu_gemm_f16 (TCU_GEMM_AUTO) for products with few output tiles and a long K, where one workgroup per output
- * tile leaves most of the chip idle or short of work (e.g. 1024 x 1024 x 16384, 2048 x 2048 x 8192): K is split into
- * ranges multiplied by different workgroups (the WAVE128 kernel, f32 partial products into `workspace`,
- * [splits, M, N]) and a second kernel adds the partial products. tcu_gemm_workspace_bytes(M, N, K) is the workspace
+ * tile leaves most of the chip idle or short of work (e.g. 1024 x 1024 x 16384, 2048 x 2048 x 32768): K is split into
+ * ranges multiplied by different workgroups (the WAVE128_KSPLIT kernel with 128 x 128 tiles, or the WAVE128 kernel where
+ * those tiles fill the chip by themselves; f32 partial products into `workspace`, [splits, M, N]) and a second kernel
+ * adds the partial products. tcu_gemm_workspace_bytes(M, N, K) is the workspace
  * this takes, or 0 when the product is not split (more than 128 tiles of 256 x 256, M or N not multiples of 256,
  * less than 512 of K per range, or the unsplit kernel expected to be as fast): then, and when `workspace` is NULL,
  * the call is tcu_gemm_f16 with TCU_GEMM_AUTO. The workspace (16-byte aligned device

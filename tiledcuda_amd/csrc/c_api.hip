@@ -337,11 +337,6 @@ int gemm_main_and_strips(const __half* A, const __half* B, OutType* C, int M, in
     return rc;
 }
 
-/// Number of K-ranges a product is split into when the caller brings a workspace: 1 unless 256 x 256 tiles would leave
-/// at least half of the chip idle (at most 128 tiles), K gives every workgroup at least 512 of it, and the split is
-/// expected to beat the unsplit launch by 5 %. Expected cost of s ranges (measured, one workgroup per CU at most):
-/// 10 us for the two launches and the epilogues + 1.4 us per k-tile of a range + the partial products written and
-/// read once (2 x s x M x N x 4 bytes at 5.3 TB/s); of the unsplit launch: pipelined_plan().
 /// Whether AUTO sends an unsplit product to the kernel whose wavefronts split K: about one 128 x 128 tile per CU and a
 /// long enough K (2048^3: 21.9 against 26.8 us for the LDS-bound 64 x 64-per-wavefront tilings, 1536 x 1536 x 4096: 26.6
 /// against 38.5 us, 2048 x 2048 x 1536: 19.8 against 22.6 us); with a short K its reduction through LDS costs more than
@@ -352,44 +347,82 @@ bool gemm_w128k_is_the_choice(int M, int N, int K) {
     return tiles >= 128 && tiles <= 256;
 }
 
-int gemm_split_count(int M, int N, int K) {
+/// How tcu_gemm_f16_ws runs a product: unsplit (splits == 1), or split over K into `splits` ranges whose f32 partial
+/// products come from gemm_w128 (256 x 256 tiles) or from gemm_w128k (128 x 128 tiles: four times the workgroups per
+/// range, so a quarter of the ranges - and of the partial products to write and add - fills the chip).
+/// Split only if 256 x 256 tiles would leave at least half of the chip idle (at most 128 tiles), K gives every workgroup
+/// at least 512 of it (1024 with 128 x 128 tiles), and the split is expected to beat the unsplit launch by 5 %. Expected
+/// cost of s ranges (measured, one workgroup per CU at most): 10 us for the two launches and the epilogues + 1.4 us per
+/// k-tile of a range + the partial products written and read once (2 x s x M x N x 4 bytes at 5.3 TB/s); of the unsplit
+/// launch: pipelined_plan(), or the K-splitting kernel's time where AUTO would run it.
+struct GemmSplitPlan {
+    int splits;
+    bool tiles128;
+};
+
+GemmSplitPlan gemm_split_plan(int M, int N, int K) {
     using T = GemmW128Traits;
-    if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0) return 1;
+    GemmSplitPlan plan{1, false};
+    if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0) return plan;
     const long tiles = (long)(M / T::kBM) * (N / T::kBN);
-    if (tiles > 128) return 1;
+    if (tiles > 128) return plan;
     double unsplit_us = pipelined_plan(M, N, K).us;
-    // the K-splitting kernel, where AUTO would run it: one round of workgroups, 5 us + 1.2 us per 128 of K with 128 x 128
+    // the K-splitting kernel, where AUTO would run it: one round of workgroups, 5 us + 0.95 us per 128 of K with 128 x 128
     // tiles, 0.75 us with 128 x 96 tiles (measured)
     if (gemm_w128k_is_the_choice(M, N, K)) {
         const long tiles128 = (long)(M / 128) * (N / 128), tiles96 = (long)(M / 128) * ((N + 95) / 96);
-        const double per_tile = tiles128 <= 192 && tiles96 <= 256 ? 0.75 : 1.05;
+        const double per_tile = tiles128 <= 192 && tiles96 <= 256 ? 0.75 : 0.95;
         unsplit_us = std::min(unsplit_us, 5.0 + per_tile * (K / 128));
     }
-    int best = 1;
     double best_us = 0.95 * unsplit_us;
+    const double plane_us = 2.0 * double(M) * N * 4 / 5.3e6;  // a plane of partial products written and read once
     for (int s = 2; s * tiles <= 256 && K % (s * T::kBK) == 0 && K / s >= 512; s *= 2) {
-        const double us = 10.0 + 1.4 * (K / s / T::kBK) + 2.0 * s * double(M) * N * 4 / 5.3e6;
+        const double us = 10.0 + 1.4 * (K / s / T::kBK) + s * plane_us;
         if (us < best_us) {
-            best = s;
+            plan = {s, false};
             best_us = us;
         }
     }
-    return best;
+    // partial products from the kernel whose wavefronts split K inside the workgroup: 11.5 us for the two launches, the
+    // reduction through LDS and the epilogues + per 128 of a range 0.62 us with up to 128 workgroups, rising to 0.95 us
+    // with 256 (their loads share the L2s) - measured on 256^2 x 8192 ... 1024 x 2048 x 16384 with 2 to 16 ranges
+    if ((long)K * 256 < (1l << 32)) {
+        for (int s = 2; s * tiles * 4 <= 256 && K % (s * 128) == 0 && K / s >= 512; s *= 2) {
+            const long groups = s * tiles * 4;
+            const double per_tile = 0.62 + 0.33 * (groups > 128 ? double(groups - 128) / 128.0 : 0.0);
+            const double us = 11.5 + per_tile * (K / s / 128) + s * plane_us;
+            if (us < best_us) {
+                plan = {s, true};
+                best_us = us;
+            }
+        }
+    }
+    return plan;
 }
 
+int gemm_split_count(int M, int N, int K) { return gemm_split_plan(M, N, K).splits; }
+
 template <typename OutType>
-int gemm_splitk(const __half* A, const __half* B, OutType* C, int M, int N, int K, int splits, float* partial,
+int gemm_splitk(const __half* A, const __half* B, OutType* C, int M, int N, int K, GemmSplitPlan plan, float* partial,
                 hipStream_t stream) {
     using T = GemmW128Traits;
     if ((long)K * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
-    const int tiles = (M / T::kBM) * (N / T::kBN);
-    int rc = launch(&gemm_w128<float>, dim3(tiles, splits), dim3(T::kThreads), T::kLdsBytes, stream, A, B, partial, M, N,
-                    K / splits, K, K, N, static_cast<unsigned int*>(nullptr), 0);
+    int rc;
+    if (plan.tiles128) {
+        using Tk = GemmW128kTraits;
+        const int tiles = (M / Tk::kBM) * (N / Tk::kBN);
+        rc = launch(&gemm_w128k<float, false, Tk>, dim3(tiles, plan.splits), dim3(Tk::kThreads), Tk::kLdsBytes, stream, A, B,
+                    partial, M, N, K / plan.splits, K, K, N);
+    } else {
+        const int tiles = (M / T::kBM) * (N / T::kBN);
+        rc = launch(&gemm_w128<float>, dim3(tiles, plan.splits), dim3(T::kThreads), T::kLdsBytes, stream, A, B, partial, M, N,
+                    K / plan.splits, K, K, N, static_cast<unsigned int*>(nullptr), 0);
+    }
     if (rc != TCU_OK) return rc;
     const size_t n = size_t(M) * N;
     return launch(&splitk_reduce<OutType>, dim3(unsigned((n / 4 + 255) / 256)), dim3(256), 0, stream,
-                  static_cast<const float*>(partial), C, n, splits);
+                  static_cast<const float*>(partial), C, n, plan.splits);
 }
 
 template <typename OutType>
@@ -852,9 +885,9 @@ int tcu_gemm_f16_ws(const void* A, const void* B, void* C, int M, int N, int K, 
     auto a = static_cast<const __half*>(A), b = static_cast<const __half*>(B);
     auto s = static_cast<hipStream_t>(stream);
     auto ws = static_cast<float*>(workspace);
-    const int splits = gemm_split_count(M, N, K);
-    if (out_dtype == TCU_DTYPE_F32) return gemm_splitk<float>(a, b, static_cast<float*>(C), M, N, K, splits, ws, s);
-    if (out_dtype == TCU_DTYPE_F16) return gemm_splitk<__half>(a, b, static_cast<__half*>(C), M, N, K, splits, ws, s);
+    const GemmSplitPlan plan = gemm_split_plan(M, N, K);
+    if (out_dtype == TCU_DTYPE_F32) return gemm_splitk<float>(a, b, static_cast<float*>(C), M, N, K, plan, ws, s);
+    if (out_dtype == TCU_DTYPE_F16) return gemm_splitk<__half>(a, b, static_cast<__half*>(C), M, N, K, plan, ws, s);
     return fail(TCU_ERR_INVALID_ARGUMENT, "tcu_gemm_f16_ws: out_dtype must be TCU_DTYPE_F32 or TCU_DTYPE_F16");
 }
 
