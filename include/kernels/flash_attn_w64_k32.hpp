@@ -25,8 +25,8 @@
 // from that kernel in the last bits.
 // Requirements: head size 128 (V row-major [N, D] or column-major, the reference op's convention; see the traits) or 64
 // (row-major V; a step then has 32 matrix instructions for the same softmax work and every one carries an exponential),
-// M % 256 == 0, N % 64 == 0, N >= 320 (Q passes through two ring stages before the fifth block needs them). M, N and
-// the batch count are run-time values.
+// M % 64 == 0 (wavefronts of a head's last block of 256 whose queries lie beyond M idle), N % 64 == 0, N >= 320 (Q passes
+// through two ring stages before the fifth block needs them). M, N and the batch count are run-time values.
 #pragma once
 
 #include <type_traits>
@@ -131,7 +131,7 @@ struct FlashW64K32Traits {
     static_assert(kDTiles == kGroups && (kGroups == 8 || kGroups == 4), "a step has 8 or 4 groups: a K fragment and a V fragment each");
 };
 
-/// grid = min((M / 256) * batch, number of CUs) workgroups (1-D), block = 256, dynamic LDS = Traits::kShmBytes. A workgroup
+/// grid = min(ceil(M / 256) * batch, number of CUs) workgroups (1-D), block = 256, dynamic LDS = Traits::kShmBytes. A workgroup
 /// takes the items (blocks of 256 queries of one batch item) blockIdx.x, blockIdx.x + gridDim.x, ... one after the
 /// other: gridDim.x must be a multiple of 8 (or hold every item), so that a workgroup's items stay on its XCD's mapping.
 template <typename InType, typename Traits>
@@ -155,7 +155,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     const int nb = kN / kTN;
 
     // query blocks of one (batch, head) item get item numbers congruent modulo 8: one XCD, K and V fetched once
-    const int q_blocks = kM / Traits::kTM;
+    const int q_blocks = (kM + Traits::kTM - 1) / Traits::kTM;
     const int items = q_blocks * batch;
     auto locate = [&](int w, size_t& head, int& q_block) {
         if (batch % 8 == 0) {
@@ -177,7 +177,13 @@ __global__ void __launch_bounds__(Traits::kThreads)
     size_t head;
     int q_block;
     locate(w, head, q_block);
-    const InType* Qb = dQ + (head * kM + size_t(q_block) * Traits::kTM) * kD;
+    // kM need only be a multiple of 64: a wavefront of a head's last block whose 64 queries lie beyond kM takes part in
+    // the loads of K and V and in the barriers, reads the block's first 64 rows of Q in place of its own and writes
+    // nothing
+    auto rows_of = [&](int qb) { return wave_u * 64 < kM - qb * Traits::kTM ? wave_u * 64 : 0; };
+    const bool active = wave_u * 64 < kM - q_block * Traits::kTM;
+    // (the loaders address a wavefront's rows from the tile's origin: the origin is moved instead)
+    const InType* Qb = dQ + (long(head) * kM + long(q_block) * Traits::kTM + rows_of(q_block) - wave_u * 64) * kD;
     const InType* Kh = dK + head * size_t(kN) * kD;
     const InType* Vh = dV + head * size_t(kN) * kD;
     InType* Ob = dO + (head * kM + size_t(q_block) * Traits::kTM) * kD;
@@ -187,7 +193,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         size_t nhead;
         int nqb;
         locate(w + int(gridDim.x) < items ? w + int(gridDim.x) : w, nhead, nqb);
-        Qnext = dQ + (nhead * kM + size_t(nqb) * Traits::kTM) * kD;
+        Qnext = dQ + (long(nhead) * kM + long(nqb) * Traits::kTM + rows_of(nqb) - wave_u * 64) * kD;
         Knext = dK + nhead * size_t(kN) * kD;
         Vnext = dV + nhead * size_t(kN) * kD;
     }
@@ -709,7 +715,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
     typename Traits::OutToGlobal to_global;
     typename Traits::GlobalO gO(Ob);
     to_shared(out, sO);
-    to_global(sO, gO);
+    if (active) to_global(sO, gO);
     // the next item loads its blocks 1 and 2 into these two stages: not before everyone has read its rows back
     __builtin_amdgcn_s_barrier();
     s0 = next_s0;

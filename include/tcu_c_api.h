@@ -86,7 +86,7 @@ typedef enum {
 } tcu_v_layout;
 
 /* Which attention kernel to run (tcu_flash_attn_fwd_f16_algo). For a row-major V, AUTO picks WAVE64_K32 for long sequences
- * (M % 256 == 0, N >= 1024) with at least 256 blocks of 256 queries, at head size 128 also WAVE64 with 128 to 255 such
+ * (N >= 1024) with at least 256 whole blocks of 256 queries, at head size 128 also WAVE64 with 128 to 255 such
  * blocks, and MFMA32_FUSED otherwise; for a column-major V (head size 128) AUTO picks WAVE64_K32 under the same
  * conditions and WAVE64 otherwise (it takes every M % 64 == 0 and N % 64 == 0). */
 typedef enum {
@@ -109,8 +109,9 @@ typedef enum {
                                   instructions, each contracting 32 indices: the chip sustains a higher clock on them),
                                   launched as one workgroup per CU that takes its blocks of 256 queries one after the
                                   other and fetches the next one's first operands under the last steps of the current;
-                                  head size 128 with either V layout or head size 64 with a row-major V, M % 256 == 0,
-                                  N % 64 == 0, N >= 320; results equal to WAVE64 (MFMA32_FUSED at head size 64) up to the
+                                  head size 128 with either V layout or head size 64 with a row-major V, M % 64 == 0
+                                  (wavefronts of a head's last block whose 64 queries lie beyond M idle), N % 64 == 0,
+                                  N >= 320; results equal to WAVE64 (MFMA32_FUSED at head size 64) up to the
                                   summation order inside a matrix instruction */
 } tcu_attn_algo;
 

@@ -139,7 +139,6 @@ def test_unsupported_shapes_are_reported_not_launched(tcu):
     assert l.tcu_flash_attn_fwd_f16_algo(p, p, p, p, 1, 512, 512, 128, 128, 1.0, 1, 5, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # tile-API wave64: fixed (M, N)
     assert l.tcu_flash_attn_fwd_f16_algo(p, p, p, p, 1, 2048, 2048, 128, 128, 1.0, 0, 5, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # ... and a row-major V
     assert l.tcu_flash_attn_fwd_f16_algo(p, p, p, p, 1, 256, 256, 128, 128, 1.0, 1, 6, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # 16x16x32 wave64: N >= 320
-    assert l.tcu_flash_attn_fwd_f16_algo(p, p, p, p, 1, 320, 640, 128, 128, 1.0, 1, 6, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # ... M % 256
     assert l.tcu_flash_attn_fwd_f16_algo(p, p, p, p, 1, 256, 640, 64, 64, 1.0, 0, 6, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # ... head size 64 only with a row-major V
     assert l.tcu_flash_attn_fwd_f16_algo(p, p, p, p, 1, 256, 256, 128, 128, 1.0, 1, 7, 0) == tcu.TCU_ERR_INVALID_ARGUMENT  # no such algo
     assert l.tcu_b2b_gemm_f16_algo(p, p, p, p, 64, 512, 128, 128, 1, 1, 4, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # tile-API resident: fixed N

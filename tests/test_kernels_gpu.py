@@ -958,6 +958,42 @@ def test_flash_attention_wave64_k32_head_size_64(tcu, oracle, device, batch, M, 
         assert torch.equal(auto, out)
 
 
+@pytest.mark.parametrize("batch,M,N,D", [(2, 64, 320, 128), (1, 192, 384, 128), (3, 320, 640, 128), (2, 448, 704, 128),
+                                         (130, 576, 1024, 128), (3, 320, 448, 64), (2, 192, 320, 64)])
+@pytest.mark.parametrize("v_col_major", [False, True])
+def test_flash_attention_wave64_k32_partial_workgroups(tcu, oracle, device, batch, M, N, D, v_col_major):
+    """Query counts that are multiples of 64 but not of 256 on the 16x16x32 kernel: the wavefronts of a head's last block
+    whose queries lie beyond M take part in the loads and barriers, read the block's first rows in place of their own
+    and write nothing (the output is followed by a guard region that must stay untouched) - also as the second and
+    third item of a workgroup, whose Q is fetched under the steps of the item before (130 x 3 blocks on 256 CUs)."""
+    import torch
+
+    if v_col_major and D != 128:
+        pytest.skip("a column-major V is instantiated for head size 128")
+    print(f"attention wave64_k32 partial b{batch} {M}x{N}x{D} v_col_major={v_col_major}", flush=True)
+    q = oracle.fill_normal(batch * M * D, 97).reshape(batch, M, D)
+    k = oracle.fill_normal(batch * N * D, 98).reshape(batch, N, D)
+    v = oracle.fill_normal(batch * N * D, 99).reshape(batch, N, D)
+    dq, dk, dv = dev(q, device), dev(k, device), dev(v, device)
+    buf = torch.full((batch * M * D + 256 * D,), 7.0, dtype=torch.float16, device=device)
+    out = buf[:batch * M * D].view(batch, M, D)
+    if v_col_major:
+        dvt = dv.transpose(1, 2).contiguous()
+        tcu.flash_attention_fwd(dq.view(-1), dk.view(-1), dvt.view(-1), out.view(-1), M, N, D, D, scale=1.0 / math.sqrt(D),
+                                batch=batch, algo="wave64_k32")
+    else:
+        tcu.flash_attention(dq, dk, dv, out=out, algo="wave64_k32")
+    torch.cuda.synchronize()
+    assert bool((buf[batch * M * D:] == 7.0).all())
+    heads = list(range(batch)) if batch <= 3 else [0, 57, batch - 1]
+    ref = oracle.attention(np.ascontiguousarray(q[heads]), np.ascontiguousarray(k[heads]), np.ascontiguousarray(v[heads]),
+                           1.0 / math.sqrt(D))
+    assert oracle.max_abs_err(host(out)[heads], ref) <= ABS_TOL
+    if batch > 3:  # every head, against the 8-wavefront kernel
+        other = tcu.flash_attention(dq, dk, dv, algo="mfma32_fused")
+        assert (out.float() - other.float()).abs().max().item() <= ABS_TOL
+
+
 @pytest.mark.parametrize("algo", ["wave64", "tile_wave64", "wave64_k32"])
 def test_flash_attention_wave64_with_cold_caches(tcu, oracle, device, algo):
     """The one-wavefront-per-SIMD kernels request their first operand fragments of key block 1 only behind the barrier

@@ -655,7 +655,7 @@ int launch_fa_w64_k32(const __half* Q, const __half* K, const __half* V, __half*
     if (hipGetDevice(&device) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus < 8)
         return fail(TCU_ERR_HIP, "attention: cannot read the number of compute units");
-    const long items = (long)(M / Traits::kTM) * batch;
+    const long items = (long)((M + Traits::kTM - 1) / Traits::kTM) * batch;
     const long grid = std::min<long>(items, cus - cus % 8);
     return launch(&flash_attention_w64_k32<__half, Traits>, dim3(unsigned(grid)), dim3(Traits::kThreads),
                   Traits::kShmBytes, stream, Q, K, V, O, batch, M, N, scale);
@@ -667,8 +667,8 @@ int fa_w64_k32_dispatch(const __half* Q, const __half* K, const __half* V, __hal
     if (Kd != 128 && !(Kd == 64 && v_layout == TCU_V_ROW_MAJOR))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel is instantiated for head size "
                                                "128, and for head size 64 with a row-major V");
-    if (M % Traits::kTM != 0 || N < Traits::kStages * Traits::kTN)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel needs M % 256 == 0 and N >= 320");
+    if (N < Traits::kStages * Traits::kTN)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the 16x16x32 one-wavefront-per-SIMD attention kernel needs N >= 320");
     if ((long)N * 256 >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD attention kernel addresses a V block with 32-bit offsets");
     if (Kd == 64) return launch_fa_w64_k32<64, false>(Q, K, V, O, batch, M, N, scale, stream);
@@ -707,10 +707,12 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
         // long sequences with enough query blocks to fill the chip: the kernel with 64 queries per wavefront
         // (with at least one block of 256 queries per CU the chip runs at its power limit, where the 16x16x32 instruction
         // wins; a half-empty chip runs at full clock, where the 32x32x16 kernel's fewer issue cycles do)
-        if (algo == TCU_ATTN_AUTO && Kd == 128 && M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 128)
-            return (long)batch * (M / 256) >= 256 ? fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream)
-                                                  : launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream);
-        if (algo == TCU_ATTN_AUTO && Kd == 64 && M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 256)
+        // (M any multiple of 64: wavefronts of a head's last block beyond M idle; blocks counts the whole blocks)
+        const long blocks = (long)batch * (M / 256);
+        if (algo == TCU_ATTN_AUTO && Kd == 128 && N >= 1024 && blocks >= 128)
+            return blocks >= 256 ? fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream)
+                                 : launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream);
+        if (algo == TCU_ATTN_AUTO && Kd == 64 && N >= 1024 && blocks >= 256)
             return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
         if (algo == TCU_ATTN_MFMA32)
             return Kd == 128 ? fa_fwd_by_rows<128, false>(Q, K, V, O, batch, M, N, scale, stream)
@@ -731,7 +733,7 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     if (Kd != 128) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for head size 128");
     if (algo == TCU_ATTN_AUTO) {
         // long sequences with enough query blocks to fill the chip: the 16x16x32 kernel, as for a row-major V
-        if (M % 256 == 0 && N >= 1024 && (long)batch * (M / 256) >= 256)
+        if (N >= 1024 && (long)batch * (M / 256) >= 256)
             return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
         return launch_fa_w64<true>(Q, K, V, O, batch, M, N, scale, stream);
     }
