@@ -704,16 +704,16 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     }
     if (v_layout == TCU_V_ROW_MAJOR && algo != TCU_ATTN_TILE_LIBRARY) {
         if (Kd != 128 && Kd != 64) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "attention is instantiated for head sizes 64 and 128");
-        // long sequences with enough query blocks to fill the chip: the kernel with 64 queries per wavefront
-        // (with at least one block of 256 queries per CU the chip runs at its power limit, where the 16x16x32 instruction
-        // wins; a half-empty chip runs at full clock, where the 32x32x16 kernel's fewer issue cycles do)
-        // (M any multiple of 64: wavefronts of a head's last block beyond M idle; blocks counts the whole blocks)
+        // Enough query blocks to fill the chip: the kernels with 64 queries per wavefront. From one block of 256 queries
+        // per CU on (counting a sequence's whole blocks; M is any multiple of 64) the chip runs at its power limit, where
+        // the 16x16x32 instruction wins, at every sequence length that kernel takes (256 x 512 x 512 x 128: 45.6 against
+        // 57.9 us for the 8-wavefront kernel, 1024 x 320 x 320: 117.7 against 203); a half-empty chip runs at full clock,
+        // where the 32x32x16 kernel's fewer issue cycles do (long sequences, head size 128).
         const long blocks = (long)batch * (M / 256);
-        if (algo == TCU_ATTN_AUTO && Kd == 128 && N >= 1024 && blocks >= 128)
-            return blocks >= 256 ? fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream)
-                                 : launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream);
-        if (algo == TCU_ATTN_AUTO && Kd == 64 && N >= 1024 && blocks >= 256)
+        if (algo == TCU_ATTN_AUTO && N >= 320 && blocks >= 256)
             return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
+        if (algo == TCU_ATTN_AUTO && Kd == 128 && N >= 1024 && blocks >= 128)
+            return launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream);
         if (algo == TCU_ATTN_MFMA32)
             return Kd == 128 ? fa_fwd_by_rows<128, false>(Q, K, V, O, batch, M, N, scale, stream)
                              : fa_fwd_by_rows<64, false>(Q, K, V, O, batch, M, N, scale, stream);
@@ -732,8 +732,8 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     // column-major V (the reference op's convention), any N % 64 == 0
     if (Kd != 128) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for head size 128");
     if (algo == TCU_ATTN_AUTO) {
-        // long sequences with enough query blocks to fill the chip: the 16x16x32 kernel, as for a row-major V
-        if (N >= 1024 && (long)batch * (M / 256) >= 256)
+        // enough query blocks to fill the chip: the 16x16x32 kernel, as for a row-major V
+        if (N >= 320 && (long)batch * (M / 256) >= 256)
             return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
         return launch_fa_w64<true>(Q, K, V, O, batch, M, N, scale, stream);
     }
