@@ -708,9 +708,10 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
         // per CU on (counting a sequence's whole blocks; M is any multiple of 64) the chip runs at its power limit, where
         // the 16x16x32 instruction wins, at every sequence length that kernel takes (256 x 512 x 512 x 128: 45.6 against
         // 57.9 us for the 8-wavefront kernel, 1024 x 320 x 320: 117.7 against 203); a half-empty chip runs at full clock,
-        // where the 32x32x16 kernel's fewer issue cycles do (long sequences, head size 128).
+        // where the 32x32x16 kernel's fewer issue cycles do (long sequences, head size 128: 16 x 2048^2 45.7 against 48.8
+        // us; with 192 blocks the 16x16x32 kernel is ahead again, 52.6 against 55.5).
         const long blocks = (long)batch * (M / 256);
-        if (algo == TCU_ATTN_AUTO && N >= 320 && blocks >= 256)
+        if (algo == TCU_ATTN_AUTO && N >= 320 && (blocks >= 256 || (blocks >= 192 && N >= 1024)))
             return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
         if (algo == TCU_ATTN_AUTO && Kd == 128 && N >= 1024 && blocks >= 128)
             return launch_fa_w64<false>(Q, K, V, O, batch, M, N, scale, stream);
