@@ -86,9 +86,8 @@ typedef enum {
 } tcu_v_layout;
 
 /* Which attention kernel to run (tcu_flash_attn_fwd_f16_algo). For a row-major V, AUTO picks WAVE64_K32 with at least 256
- * whole blocks of 256 queries and N >= 320 (192 with N >= 1024), at head size 128 also WAVE64 with 128 to 191 such blocks and
- * N >= 1024, and
- * MFMA32_FUSED otherwise; for a column-major V (head size 128) AUTO picks WAVE64_K32 under the same conditions and
+ * whole blocks of 256 queries and N >= 320 (192 with N >= 1024), at head size 128 also WAVE64 with 128 to 191 such blocks
+ * and N >= 1024, and MFMA32_FUSED otherwise; for a column-major V (head size 128) AUTO picks WAVE64_K32 under the same conditions and
  * WAVE64 otherwise (it takes every M % 64 == 0 and N % 64 == 0). */
 typedef enum {
     TCU_ATTN_AUTO = 0,

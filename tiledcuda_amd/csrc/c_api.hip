@@ -734,7 +734,8 @@ int fa_dispatch(const __half* Q, const __half* K, const __half* V, __half* O, in
     if (Kd != 128) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "column-major V is instantiated for head size 128");
     if (algo == TCU_ATTN_AUTO) {
         // enough query blocks to fill the chip: the 16x16x32 kernel, as for a row-major V
-        if (N >= 320 && (long)batch * (M / 256) >= 256)
+        const long blocks = (long)batch * (M / 256);
+        if (N >= 320 && (blocks >= 256 || (blocks >= 192 && N >= 1024)))
             return fa_w64_k32_dispatch(Q, K, V, O, batch, M, N, Kd, scale, v_layout, stream);
         return launch_fa_w64<true>(Q, K, V, O, batch, M, N, scale, stream);
     }
