@@ -37,21 +37,28 @@
 
 namespace tiledcuda::kernels {
 
-struct GemmW128Traits {
-    static constexpr int kBM = 256, kBN = 256, kBK = 64;
+/// kNT_: 16-column tiles of a wavefront's block of C: 8 (workgroup tile 256 x 256) or 4 (256 x 128, for products with too
+/// few 256 x 256 tiles to fill the chip and too many 128 x 128 tiles for one round of the K-splitting kernel).
+template <const int kNT_ = 8>
+struct GemmW128TraitsN {
+    static constexpr int kNT = kNT_;
+    static constexpr int kBM = 256, kBN = 2 * 16 * kNT, kBK = 64;
     static constexpr int kWaves = 4, kThreads = kWaves * kWaveSize;
-    static constexpr int kWaveM = 128, kWaveN = 128;
-    static constexpr int kMT = kWaveM / 16, kNT = kWaveN / 16;  // 8 x 8 MFMA tiles of 16 x 16 per wavefront
+    static constexpr int kWaveM = 128, kWaveN = 16 * kNT;
+    static constexpr int kMT = kWaveM / 16;                     // 8 x kNT MFMA tiles of 16 x 16 per wavefront
     static constexpr int kRowBytes = kBK * 2;                   // 128
     static constexpr int kABytes = kBM * kRowBytes, kBBytes = kBN * kRowBytes;
-    static constexpr int kStageBytes = kABytes + kBBytes;  // 64 KiB
-    static constexpr int kLoads = kBM / 8 / kWaves;        // 1 KiB load instructions per operand per wavefront per stage
+    static constexpr int kStageBytes = kABytes + kBBytes;  // 64 KiB (48)
+    static constexpr int kLoads = kBM / 8 / kWaves;        // 1 KiB load instructions of A per wavefront per stage
+    static constexpr int kLoadsB = kBN / 8 / kWaves;       // ... of B: 8 (4)
+    static constexpr int kFrags = 8 + kNT;                 // operand fragments of a substep
     static constexpr int kLdsBytesMain = 2 * kStageBytes;  // 128 KiB of operand stages
     static constexpr int kEpilogueBytesPerWave = 2 * 16 * kWaveN * 2;  // f16 epilogue: two buffers of 16 rows
     static constexpr int kLdsBytes = kLdsBytesMain + kWaves * kEpilogueBytesPerWave;  // 160 KiB
-    static_assert(kLoads == 8 && kMT == 8 && kNT == 8, "the phase schedule below is written for these counts");
+    static_assert(kLoads == 8 && kMT == 8 && (kNT == 8 || kNT == 4), "the phase schedule below is written for these counts");
     static_assert(kLdsBytes <= kMaxLdsBytes);
 };
+using GemmW128Traits = GemmW128TraitsN<8>;
 
 namespace detail {
 
@@ -97,18 +104,18 @@ __global__ void __launch_bounds__(256) splitk_reduce(const float* __restrict__ p
     }
 }
 
-/// grid = ((M / 256) * (N / 256), splits), block = 256, dynamic LDS = GemmW128Traits::kLdsBytes.
+/// grid = ((M / 256) * (N / kBN), splits), block = 256, dynamic LDS = T::kLdsBytes.
 /// lda / ldb: elements between consecutive rows of A / of the stored [N, K] array (K for dense operands; larger when
 /// the operand is a column block of a wider matrix); ldc: elements between consecutive rows of C (N for a dense C;
 /// larger when C is the leading block of a wider matrix). With splits > 1 workgroup row z multiplies the
 /// K-range [z K, (z + 1) K) and writes plane z of C ([splits, M, N]; partial sums for splitk_reduce).
 /// zero_words / zero_count: device words that the first workgroup sets to zero on the side (null / 0: none) - the
 /// synchronisation words of a kernel that follows this one on the stream, cleared without a launch of their own.
-template <typename OutType>
-__global__ void __launch_bounds__(GemmW128Traits::kThreads)
+template <typename OutType, typename T = GemmW128Traits>
+__global__ void __launch_bounds__(T::kThreads)
     gemm_w128(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
               int lda, int ldb, int ldc, unsigned int* __restrict__ zero_words, int zero_count) {
-    using T = GemmW128Traits;
+    constexpr int kNT = T::kNT, kNumLoads = 8 + T::kLoadsB, kFrags = T::kFrags;
     extern __shared__ __align__(1024) unsigned char lds[];
 
     const int lane = lane_id();
@@ -124,10 +131,10 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
     // ---- global -> LDS: load instruction q of this wavefront (q < 8: A, else B) fills 8 rows of 128 bytes; lane i
     // writes physical 16-byte chunk i % 8 of row i / 8, which must hold logical chunk (i % 8) ^ ((row / 2) % 8)
     const int lrow = lane >> 3, lchk = lane & 7;
-    unsigned int voff[16];
+    unsigned int voff[kNumLoads];
 #pragma unroll
-    for (int q = 0; q < 16; ++q) {
-        const int row = (wave * T::kLoads + (q & 7)) * 8 + lrow;
+    for (int q = 0; q < kNumLoads; ++q) {
+        const int row = (q < 8 ? wave * T::kLoads + q : wave * T::kLoadsB + (q - 8)) * 8 + lrow;
         voff[q] = static_cast<unsigned int>(row) * static_cast<unsigned int>(q < 8 ? lda : ldb) * 2u +
                   (lchk ^ ((row >> 1) & 7)) * 16;
     }
@@ -140,7 +147,7 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
     auto load_dst = [&](int stage, int q) -> unsigned int {
         return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +
-                                              (wave * T::kLoads + (q & 7)) * 1024);
+                                              (q < 8 ? wave * T::kLoads + q : wave * T::kLoadsB + (q - 8)) * 1024);
     };
     // Rows a multiple of 32 KiB apart put the same k-tile of every row of every panel into the same few memory
     // channels, and all workgroups walk K in step. Each XCD then starts at a different eighth of K and wraps around
@@ -165,35 +172,40 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
                                                row * T::kRowBytes + chunk * 16);
     };
 
-    f16x8 fx[16], fy[16];  // fragments of substep 0 / substep 1: [0..7] A, [8..15] B
+    f16x8 fx[kFrags], fy[kFrags];  // fragments of substep 0 / substep 1: [0..7] A, [8..] B
 
 #pragma unroll
-    for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
+    for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
     if (ktiles > 1) {
 #pragma unroll
-        for (int q = 0; q < 16; ++q) detail::load_lds_16B_sbase(voff[q], load_src(1, q), load_dst(1, q));
+        for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(1, q), load_dst(1, q));
     }
     // the 256 accumulators are cleared while the first tiles are on their way (the empty asm statements keep the
     // compiler from sinking the clears below the barrier, where nothing would hide them)
-    f32x4 acc[8][8];
+    // the accumulators are pinned to the AGPR half row group by row group
+    auto pin_row = [](f32x4 (&row)[kNT]) {
+        if constexpr (kNT == 8)
+            asm volatile("" : "+a"(row[0]), "+a"(row[1]), "+a"(row[2]), "+a"(row[3]), "+a"(row[4]), "+a"(row[5]), "+a"(row[6]), "+a"(row[7]));
+        else
+            asm volatile("" : "+a"(row[0]), "+a"(row[1]), "+a"(row[2]), "+a"(row[3]));
+    };
+    f32x4 acc[8][kNT];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        asm volatile(""
-                     : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),
-                       "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]));
+        for (int j = 0; j < kNT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        pin_row(acc[i]);
     }
-    if (ktiles > 1) detail::lds_barrier<16>();  // this wavefront's part of tile 0 has landed; then everyone's
+    if (ktiles > 1) detail::lds_barrier<kNumLoads>();  // this wavefront's part of tile 0 has landed; then everyone's
     else detail::lds_barrier<0>();
 #pragma unroll
-    for (int r = 0; r < 16; ++r) fx[r] = read_frag(0, 0, r);
+    for (int r = 0; r < kFrags; ++r) fx[r] = read_frag(0, 0, r);
 
-    // Order of the 16 fragment reads of a phase: row group 0 of the next phase needs A fragment 0 and all B fragments.
-    constexpr int kOrder[16] = {0, 8, 9, 10, 11, 12, 13, 14, 15, 1, 2, 3, 4, 5, 6, 7};
+    // Order of the fragment reads of a phase: row group 0 of the next phase needs A fragment 0 and all B fragments.
+    auto order = [](int r) { return r == 0 ? 0 : r <= kNT ? 7 + r : r - kNT; };
     // MFMA n of row group i works on tile (i, j): odd row groups walk their tiles backwards, so that one operand of
     // every MFMA, also the first of a row group, is the operand of the MFMA before it
-    auto snake = [](int i, int n) { return (i & 1) ? 7 - n : n; };
+    auto snake = [](int i, int n) { return (i & 1) ? kNT - 1 - n : n; };
 
     // One tile of K. kMore: there is a tile kt+1 (read its substep 0 during phase 2); kMore2: there is a tile kt+2
     // (load it during phase 2). Row group i = MFMA tiles (i, 0..7): the MFMA order is fixed by the asm statements, the
@@ -204,10 +216,10 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
-            for (int n = 0; n < 8; ++n) {
+            for (int n = 0; n < kNT; ++n) {
                 const int j = snake(i, n);
-                const int r = 4 * i + (n >> 1);
-                if ((n & 1) == 0 && r < 16) fy[kOrder[r]] = read_frag(stage, 1, kOrder[r]);
+                const int r = (kNT / 2) * i + (n >> 1);
+                if ((n & 1) == 0 && r < kFrags) fy[order(r)] = read_frag(stage, 1, order(r));
                 detail::mfma_16x16x32_agpr(acc[i][j], fx[8 + j], fx[i]);
             }
         }
@@ -216,12 +228,15 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
-            for (int n = 0; n < 8; ++n) {
+            for (int n = 0; n < kNT; ++n) {
                 const int j = snake(i, n);
-                const int r = 4 * i + (n >> 1);
-                if (kMore && (n & 1) == 0 && r < 16) fx[kOrder[r]] = read_frag(stage ^ 1, 0, kOrder[r]);
-                if (kMore2 && (n & 3) == 1) {
-                    const int q = 2 * i + (n >> 2);
+                const int r = (kNT / 2) * i + (n >> 1);
+                if (kMore && (n & 1) == 0 && r < kFrags) fx[order(r)] = read_frag(stage ^ 1, 0, order(r));
+                // one load per four MFMAs (256 x 256) or per two and a half (256 x 128: 12 loads over 32 MFMAs)
+                const int m = kNT * i + n;  // (256 x 128: 12 loads over 32 MFMAs, behind MFMAs 0, 3, 6 of every 8)
+                const int q = kNT == 8 ? 2 * i + (n >> 2) : (3 * m) / 8;
+                const bool load_here = kNT == 8 ? (n & 3) == 1 : (3 * m) % 8 < 3;
+                if (kMore2 && load_here && q < kNumLoads) {
                     detail::mfma_16x16x32_agpr_then_load(acc[i][j], fy[8 + j], fy[i], voff[q], load_src(kt + 2, q),
                                                          load_dst(stage, q));
                 } else {
@@ -244,34 +259,33 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
     // accumulator through a statement that comes after the wait
     detail::mfma_results_wait();
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-        asm volatile(""
-                     : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),
-                       "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]));
+    for (int i = 0; i < 8; ++i) pin_row(acc[i]);
 
     // ---- epilogue: acc[i][j][e] = C[16 i + lane % 16][16 j + 4 (lane / 16) + e] of the wavefront's block
     if constexpr (sizeof(OutType) == 2) {
         // f16: 16 rows at a time through a private LDS buffer (beyond the operand stages, so no workgroup barrier),
         // so that global stores are 16 bytes per lane and row-contiguous; two buffers per wavefront, so the
         // conversion and staging of rows 16 (i + 1).. overlap the stores of rows 16 i..
-        constexpr int kPitch = T::kWaveN * 2;              // 256 bytes per staged row
+        constexpr int kPitch = T::kWaveN * 2;              // 256 (128) bytes per staged row
         constexpr int kSlotMask = (kPitch / 8 - 1) & ~1;   // 8-byte slots of a row are XOR-ed with 2 * row
+        constexpr int kLanesPerRow = kPitch / 16, kRowsPerRead = kWaveSize / kLanesPerRow, kReads = 16 / kRowsPerRead;
         unsigned char* stg = lds + T::kLdsBytesMain + wave * T::kEpilogueBytesPerWave;
-        const int rr = lane >> 4, cc = lane & 15;  // read-back: 16 lanes x 16 B per row, 4 rows per instruction
+        // read-back: 16 (8) lanes x 16 B per row, 4 (8) rows per instruction
+        const int rr = lane / kLanesPerRow, cc = lane % kLanesPerRow;
         OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * ldc + n0 + wave_n * T::kWaveN;
         // LDS addresses of this lane's 8 staging writes and 4 read-backs of a row group (the same for every group but
         // for the buffer), computed once: with one wavefront per SIMD the epilogue is bound by instruction issue
-        unsigned int waddr[8], raddr[4];
+        unsigned int waddr[kNT], raddr[kReads];
         const unsigned int stg_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(stg));
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < kNT; ++j) {
             const int slot = (j * 16 + 4 * fquad) >> 2;
             waddr[j] = stg_base + frow * kPitch + (slot ^ ((frow << 1) & kSlotMask)) * 8;
             asm volatile("" : "+v"(waddr[j]));
         }
 #pragma unroll
-        for (int it = 0; it < 4; ++it) {
-            const int row = it * 4 + rr;
+        for (int it = 0; it < kReads; ++it) {
+            const int row = it * kRowsPerRead + rr;
             raddr[it] = stg_base + row * kPitch + ((2 * cc) ^ ((row << 1) & kSlotMask)) * 8;
             asm volatile("" : "+v"(raddr[it]));
         }
@@ -282,7 +296,7 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
         for (int i = 0; i < 8; ++i) {
             const unsigned int buf = (i & 1) * (16 * kPitch);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < kNT; ++j) {
                 f16x4 v;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc[i][j][e]);
@@ -290,9 +304,9 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
             }
             // LDS operations of one wavefront execute in order: the reads below see the writes above
 #pragma unroll
-            for (int it = 0; it < 4; ++it) {
+            for (int it = 0; it < kReads; ++it) {
                 const u32x4 v = *reinterpret_cast<lds_u32x4_ptr>(raddr[it] + buf);
-                *reinterpret_cast<u32x4*>(crow + size_t(i * 16 + it * 4) * ldc * sizeof(OutType)) = v;
+                *reinterpret_cast<u32x4*>(crow + size_t(i * 16 + it * kRowsPerRead) * ldc * sizeof(OutType)) = v;
             }
         }
     } else {
@@ -300,7 +314,7 @@ __global__ void __launch_bounds__(GemmW128Traits::kThreads)
 #pragma unroll
         for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+            for (int j = 0; j < kNT; ++j)
                 *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * ldc + j * 16 + 4 * fquad) = acc[i][j];
     }
 }

@@ -54,12 +54,16 @@ typedef enum {
                                 a piece at a time, single-fragment LDS reads, gemm_scheduled() with accumulators pinned
                                 in AGPRs); compile-time shapes: 4096^3, 1024^3, 512x768x192, 256x256x64; results
                                 identical to WAVE128 and PIPELINED bit for bit */
-    TCU_GEMM_WAVE128_KSPLIT = 8 /* 128 x 128 tile (128 x 96 where that fills the GPU better) on 4 wavefronts (one per SIMD)
+    TCU_GEMM_WAVE128_KSPLIT = 8, /* 128 x 128 tile (128 x 96 where that fills the GPU better) on 4 wavefronts (one per SIMD)
                                 that each own the whole tile over a quarter of every 128-wide step of K, partial tiles
                                 added through LDS: for products with too few 256 x 256 tiles to fill the GPU (2048^3,
                                 1552 x 1552 x 4096); K a multiple of 128,
                                 M and N multiples of 16 (edge tiles: rows clamped, stores guarded); the sum over K is
                                 taken in four interleaved parts (differs from the other kernels by f32 rounding) */
+    TCU_GEMM_WAVE128_NARROW = 9 /* the WAVE128 kernel with 256 x 128 workgroup tiles (a wavefront owns 128 x 64): for
+                                products between the two above - too few 256 x 256 tiles to fill the GPU, too many
+                                128 x 128 tiles for one round of WAVE128_KSPLIT (2048 x 2560 x 4096); M % 256 == 0,
+                                N % 128 == 0, K % 64 == 0; results identical to WAVE128 and PIPELINED bit for bit */
 } tcu_gemm_algo;
 
 /* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks ROWS for many rows, else RESIDENT, where

@@ -337,6 +337,33 @@ def test_gemm_wave128_ksplit(tcu, oracle, device, M, N, K, out_dtype):
         assert np.max(np.abs(got - want)) <= (5.0 if out_dtype == "f16" else 0.1)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 128, 64), (256, 384, 128), (512, 640, 320), (1024, 1152, 1984), (2048, 2560, 4096)])
+@pytest.mark.parametrize("out_dtype", ["f16", "f32"])
+def test_gemm_wave128_narrow(tcu, oracle, device, M, N, K, out_dtype):
+    """The one-wavefront-per-SIMD kernel with 256 x 128 workgroup tiles (a wavefront owns 128 x 64): 1 to 64 tiles of K,
+    odd and even counts, against the oracle and bit for bit against the pipelined kernel (same order of the sum), guard
+    rows around C; 2048 x 2560 x 4096 (160 tiles: more than half a round of 256 x 256 tiles would idle, 128 x 128 tiles
+    need two rounds) is a shape AUTO sends to it."""
+    import torch
+
+    print(f"gemm wave128_narrow {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float16 if out_dtype == "f16" else torch.float32
+    A = oracle.fill_uniform(M * K, 7300 + K).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 8300 + K).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    guard = torch.full((M + 2, N), -7.0, dtype=dt, device=device)
+    out = guard[1:M + 1]
+    tcu.gemm(dA, dB, out=out, algo="wave128_narrow")
+    torch.cuda.synchronize()
+    assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
+    rows = (0, M) if M <= 1024 else (M - 192, M)
+    ref = oracle.gemm(A, Bt, rows=rows)
+    assert oracle.max_rel_err(host(out)[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
+    assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))
+    if M == 2048:
+        assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, workspace=False))  # AUTO takes this kernel here
+
+
 @pytest.mark.parametrize("M,N,K", [(16, 16, 128), (144, 112, 256), (272, 400, 384), (1552, 1552, 4096), (1536, 1616, 2048),
                                    (1808, 1936, 256), (1536, 1536, 512)])
 @pytest.mark.parametrize("out_dtype", ["f16", "f32"])

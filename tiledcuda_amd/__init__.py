@@ -35,7 +35,7 @@ TCU_ERR_NO_DEVICE = -4
 TCU_DTYPE_F32 = 0
 TCU_DTYPE_F16 = 1
 
-GEMM_ALGOS = {"auto": 0, "global_reg": 1, "all_mem": 2, "pipelined": 3, "wave128": 4, "tile_pipelined": 5, "ragged": 6, "tile_wave128": 7, "wave128_ksplit": 8}
+GEMM_ALGOS = {"auto": 0, "global_reg": 1, "all_mem": 2, "pipelined": 3, "wave128": 4, "tile_pipelined": 5, "ragged": 6, "tile_wave128": 7, "wave128_ksplit": 8, "wave128_narrow": 9}
 
 TCU_V_COL_MAJOR = 0
 TCU_V_ROW_MAJOR = 1

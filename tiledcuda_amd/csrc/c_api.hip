@@ -239,6 +239,20 @@ int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int 
                   C, M, N, K, lda, ldb, ldc, zero_words, zero_count);
 }
 
+/// gemm_w128 with 256 x 128 workgroup tiles: for products with too few 256 x 256 tiles to fill the chip and too many
+/// 128 x 128 tiles for one round of the K-splitting kernel.
+template <typename OutType>
+int gemm_w128_narrow_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    using T = GemmW128TraitsN<4>;
+    if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM with 256 x 128 tiles needs M % 256 == 0, "
+                                               "N % 128 == 0, K % 64 == 0");
+    if ((long)K * 2 * T::kBM >= (1l << 32))
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
+    return launch(&gemm_w128<OutType, T>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
+                  C, M, N, K, K, K, N, static_cast<unsigned int*>(nullptr), 0);
+}
+
 template <typename OutType, typename T>
 int launch_gemm_w128k(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
     const long grid = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
@@ -447,6 +461,8 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             return gemm_tile_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_WAVE128_KSPLIT:
             return gemm_w128k_dispatch<OutType>(A, B, C, M, N, K, stream);
+        case TCU_GEMM_WAVE128_NARROW:
+            return gemm_w128_narrow_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_AUTO:
             // where the 256 x 256 tile is the choice anyway, the one-wavefront-per-SIMD kernel is the faster one
             if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) >= 128 &&
@@ -455,6 +471,13 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             // too few 256 x 256 tiles for the chip, but about one 128 x 128 tile per CU and a long enough K: the
             // kernel whose wavefronts split K (each owns the whole tile)
             if (gemm_w128k_is_the_choice(M, N, K)) return gemm_w128k_dispatch<OutType>(A, B, C, M, N, K, stream);
+            // between the two: more than half a round of 256 x 256 tiles would idle and 128 x 128 tiles need two rounds of
+            // the K-splitting kernel, but 256 x 128 tiles fill one round (2048 x 2560 x 4096: 52.3 against 60.2 us for the
+            // pipelined kernel, 3072 x 2560 x 4096: 57.3 against 64); a short K is left to the pipelined kernel's ring
+            if (M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && K >= 1024 && (long)K * 512 < (1l << 32)) {
+                const long narrow = (long)(M / 256) * (N / 128);
+                if (narrow > 128 && narrow <= 256) return gemm_w128_narrow_dispatch<OutType>(A, B, C, M, N, K, stream);
+            }
             if (M % 16 == 0 && N % 16 == 0) {
                 const int rc = gemm_main_and_strips<OutType>(A, B, C, M, N, K, stream);
                 if (rc != kPlanNotTaken) return rc;
