@@ -467,6 +467,13 @@ def main():
         configs.append({"name": "gemm_1552x1552x4096_auto", "kernel": "gemm_w128k<__half, edge tiles>", "ms": ms,
                         "tflops": 2.0 * 1552 * 1552 * 4096 / (ms * 1e-3) / 1e12, "hipblaslt_ms": ms_v,
                         "speed_vs_hipblaslt": ms_v / ms})
+        a_, b_ = rand16(2048, 4096), rand16(2560, 4096)
+        c_ = torch.empty(2048, 2560, dtype=torch.float16, device=dev)
+        ms = time_kernel(lambda: tcu.gemm(a_, b_, out=c_), 40, 40)
+        ms_v = time_kernel(lambda: torch.matmul(a_, b_.t(), out=c_), 40, 40)
+        configs.append({"name": "gemm_2048x2560x4096_auto", "kernel": "gemm_w128<__half, 256 x 128 tiles, three stages>", "ms": ms,
+                        "tflops": 2.0 * 2048 * 2560 * 4096 / (ms * 1e-3) / 1e12, "hipblaslt_ms": ms_v,
+                        "speed_vs_hipblaslt": ms_v / ms})
         a_ = (torch.randn(8192, 64, device=dev) * 0.1).half()
         b_ = (torch.randn(128, 64, device=dev) * 0.1).half()
         c_ = (torch.randn(64, 128, device=dev) * 0.1).half()

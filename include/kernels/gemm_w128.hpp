@@ -24,6 +24,13 @@
 //   * LDS layout, XOR swizzle and XCD-aware tile order are those of gemm_pipelined.hpp; the f16 epilogue stages 16
 //     rows at a time through 8 KiB of LDS per wavefront beyond the operand stages (no workgroup barrier, staging
 //     overlapped with the 16-byte row-contiguous stores).
+//   * a second tile width, 256 x 128 (GemmW128TraitsN<4>: a wavefront owns 128 x 64, 32 MFMAs per phase with 12 fragment
+//     reads and 12 loads per tile), for products with too few 256 x 256 tiles to fill the chip. Its stages are 48 KiB, so
+//     a third one fits, and it runs with three: the barrier in the middle of tile kt waits for tile kt + 1 with the loads
+//     of tile kt + 2 still on their way, and phase 2 requests tile kt + 3 - three phases to land instead of one to two
+//     (2048 x 2560 x 4096: 52.8 us with two stages, 45.9 us with three). Per multiply-add it moves half as much again
+//     through LDS and the load path as the 256 x 256 tile, which is why it loses where that one fills the chip
+//     (4096^3: 115 against 99 us).
 // Because the compiler does not know these asm statements are MFMAs it inserts none of the wait states MFMA results
 // need before other instructions read them; the only such reads are in the epilogue, and every accumulator passes
 // through a waiting statement first (see below). M % 256 == 0, N % 256 == 0, K % 64 == 0 (checked by the launcher).
@@ -37,8 +44,9 @@
 
 namespace tiledcuda::kernels {
 
-/// kNT_: 16-column tiles of a wavefront's block of C: 8 (workgroup tile 256 x 256) or 4 (256 x 128, for products with too
-/// few 256 x 256 tiles to fill the chip and too many 128 x 128 tiles for one round of the K-splitting kernel).
+/// kNT_: 16-column tiles of a wavefront's block of C: 8 (workgroup tile 256 x 256, two stages) or 4 (256 x 128, three
+/// stages: for products with too few 256 x 256 tiles to fill the chip and too many 128 x 128 tiles for one round of the
+/// K-splitting kernel).
 template <const int kNT_ = 8>
 struct GemmW128TraitsN {
     static constexpr int kNT = kNT_;
@@ -52,7 +60,8 @@ struct GemmW128TraitsN {
     static constexpr int kLoads = kBM / 8 / kWaves;        // 1 KiB load instructions of A per wavefront per stage
     static constexpr int kLoadsB = kBN / 8 / kWaves;       // ... of B: 8 (4)
     static constexpr int kFrags = 8 + kNT;                 // operand fragments of a substep
-    static constexpr int kLdsBytesMain = 2 * kStageBytes;  // 128 KiB of operand stages
+    static constexpr int kStages = kNT == 8 ? 2 : 3;       // the narrower tile's stages are 48 KiB: a third one fits
+    static constexpr int kLdsBytesMain = kStages * kStageBytes;  // 128 KiB (144) of operand stages
     static constexpr int kEpilogueBytesPerWave = 2 * 16 * kWaveN * 2;  // f16 epilogue: two buffers of 16 rows
     static constexpr int kLdsBytes = kLdsBytesMain + kWaves * kEpilogueBytesPerWave;  // 160 KiB
     static_assert(kLoads == 8 && kMT == 8 && (kNT == 8 || kNT == 4), "the phase schedule below is written for these counts");
@@ -174,11 +183,20 @@ __global__ void __launch_bounds__(T::kThreads)
 
     f16x8 fx[kFrags], fy[kFrags];  // fragments of substep 0 / substep 1: [0..7] A, [8..] B
 
+    auto clamped = [&](int kt) { return kt < ktiles ? kt : ktiles - 1; };
+    if constexpr (T::kStages == 3) {
+        // three stages: tiles 0, 1, 2 (behind the end of K: the last tile again, so that every phase is the same code)
 #pragma unroll
-    for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
-    if (ktiles > 1) {
+        for (int st = 0; st < 3; ++st)
 #pragma unroll
-        for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(1, q), load_dst(1, q));
+            for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(clamped(st), q), load_dst(st, q));
+    } else {
+#pragma unroll
+        for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
+        if (ktiles > 1) {
+#pragma unroll
+            for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(1, q), load_dst(1, q));
+        }
     }
     // the 256 accumulators are cleared while the first tiles are on their way (the empty asm statements keep the
     // compiler from sinking the clears below the barrier, where nothing would hide them)
@@ -196,7 +214,9 @@ __global__ void __launch_bounds__(T::kThreads)
         for (int j = 0; j < kNT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
         pin_row(acc[i]);
     }
-    if (ktiles > 1) detail::lds_barrier<kNumLoads>();  // this wavefront's part of tile 0 has landed; then everyone's
+    // this wavefront's part of tile 0 has landed; then everyone's
+    if constexpr (T::kStages == 3) detail::lds_barrier<2 * kNumLoads>();
+    else if (ktiles > 1) detail::lds_barrier<kNumLoads>();
     else detail::lds_barrier<0>();
 #pragma unroll
     for (int r = 0; r < kFrags; ++r) fx[r] = read_frag(0, 0, r);
@@ -245,7 +265,49 @@ __global__ void __launch_bounds__(T::kThreads)
             }
         }
     };
-    {
+    // The same with three stages: tile kt + 1 landed a whole tile ago, the barrier in the middle waits for it with the
+    // loads of tile kt + 2 still on their way, and phase 2 requests tile kt + 3 into the stage just vacated: a load has
+    // three phases to land instead of one to two. Straight-line code: behind the end of K the loads fetch the last tile
+    // again and the fragment reads fetch data nobody uses.
+    auto tile3 = [&](int kt, int stage, int next) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int n = 0; n < kNT; ++n) {
+                const int j = snake(i, n);
+                const int r = (kNT / 2) * i + (n >> 1);
+                if ((n & 1) == 0 && r < kFrags) fy[order(r)] = read_frag(stage, 1, order(r));
+                detail::mfma_16x16x32_agpr(acc[i][j], fx[8 + j], fx[i]);
+            }
+        }
+        detail::lds_barrier<kNumLoads>();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int n = 0; n < kNT; ++n) {
+                const int j = snake(i, n);
+                const int r = (kNT / 2) * i + (n >> 1);
+                if ((n & 1) == 0 && r < kFrags) fx[order(r)] = read_frag(next, 0, order(r));
+                const int m = kNT * i + n;  // 12 loads over 32 MFMAs: behind MFMAs 0, 3, 6 of every 8
+                const int q = (3 * m) / 8;
+                if ((3 * m) % 8 < 3 && q < kNumLoads) {
+                    detail::mfma_16x16x32_agpr_then_load(acc[i][j], fy[8 + j], fy[i], voff[q], load_src(clamped(kt + 3), q),
+                                                         load_dst(stage, q));
+                } else {
+                    detail::mfma_16x16x32_agpr(acc[i][j], fy[8 + j], fy[i]);
+                }
+            }
+        }
+    };
+    if constexpr (T::kStages == 3) {
+        int stage = 0;
+        for (int kt = 0; kt < ktiles; ++kt) {
+            const int next = stage == 2 ? 0 : stage + 1;
+            tile3(kt, stage, next);
+            stage = next;
+        }
+        detail::wait_vmcnt<0>();  // (the last loads, of data nobody uses, have landed before the workgroup ends)
+    } else {
         int kt = 0;
         for (; kt + 2 < ktiles; ++kt) tile(kt, std::true_type{}, std::true_type{});
         if (kt + 1 < ktiles) {

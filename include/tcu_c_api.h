@@ -60,7 +60,7 @@ typedef enum {
                                 1552 x 1552 x 4096); K a multiple of 128,
                                 M and N multiples of 16 (edge tiles: rows clamped, stores guarded); the sum over K is
                                 taken in four interleaved parts (differs from the other kernels by f32 rounding) */
-    TCU_GEMM_WAVE128_NARROW = 9 /* the WAVE128 kernel with 256 x 128 workgroup tiles (a wavefront owns 128 x 64): for
+    TCU_GEMM_WAVE128_NARROW = 9 /* the WAVE128 kernel with 256 x 128 workgroup tiles (a wavefront owns 128 x 64; three stages): for
                                 products between the two above - too few 256 x 256 tiles to fill the GPU, too many
                                 128 x 128 tiles for one round of WAVE128_KSPLIT (2048 x 2560 x 4096); M % 256 == 0,
                                 N % 128 == 0, K % 64 == 0; results identical to WAVE128 and PIPELINED bit for bit */

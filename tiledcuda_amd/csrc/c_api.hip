@@ -472,8 +472,8 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             // kernel whose wavefronts split K (each owns the whole tile)
             if (gemm_w128k_is_the_choice(M, N, K)) return gemm_w128k_dispatch<OutType>(A, B, C, M, N, K, stream);
             // between the two: more than half a round of 256 x 256 tiles would idle and 128 x 128 tiles need two rounds of
-            // the K-splitting kernel, but 256 x 128 tiles fill one round (2048 x 2560 x 4096: 52.3 against 60.2 us for the
-            // pipelined kernel, 3072 x 2560 x 4096: 57.3 against 64); a short K is left to the pipelined kernel's ring
+            // the K-splitting kernel, but 256 x 128 tiles fill one round (2048 x 2560 x 4096: 45.9 against 59.1 us for the
+            // pipelined kernel, 3072 x 2560 x 4096: 57.0 against 67.3); a short K is left to the pipelined kernel's ring
             if (M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && K >= 1024 && (long)K * 512 < (1l << 32)) {
                 const long narrow = (long)(M / 256) * (N / 128);
                 if (narrow > 128 && narrow <= 256) return gemm_w128_narrow_dispatch<OutType>(A, B, C, M, N, K, stream);
