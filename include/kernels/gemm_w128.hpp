@@ -14,8 +14,8 @@
 //     per two MFMAs; then one LDS-only barrier per tile: tile kt+1 has landed, everyone has left tile kt's stage;
 //     phase 2 (substep 1) also issues the reads of tile kt+1 / substep 0 and this wavefront's 16 direct-to-LDS loads
 //     of tile kt+2 into the stage just vacated, one per four MFMAs (the CU's address unit takes one vector-memory
-//     instruction per ~14 cycles, and a wavefront that has to wait for it issues no MFMAs). A load has a full tile
-//     of MFMA time to land;
+//     instruction per ~14 cycles, and a wavefront that has to wait for it issues no MFMAs). A load has one to two
+//     phases to land;
 //   * the loads address memory as scalar base + 32-bit lane offset (the k offset advances in scalar registers: no
 //     vector ALU work per load), and each load is one asm statement with the MFMA that precedes it, which is the
 //     wait state the load needs after the write of m0;
@@ -33,7 +33,8 @@
 //     (4096^3: 115 against 99 us).
 // Because the compiler does not know these asm statements are MFMAs it inserts none of the wait states MFMA results
 // need before other instructions read them; the only such reads are in the epilogue, and every accumulator passes
-// through a waiting statement first (see below). M % 256 == 0, N % 256 == 0, K % 64 == 0 (checked by the launcher).
+// through a waiting statement first (see below). M % 256 == 0, N a multiple of the tile width, K % 64 == 0 (checked by the
+// launcher).
 #pragma once
 
 #include <type_traits>
