@@ -462,15 +462,16 @@ def main():
         # driver's inner sizes, fused_gemm.cu:212-259), the one-launch LSTM layer at a smaller hidden size
         a_, b_ = rand16(1552, 4096), rand16(1552, 4096)
         c_ = torch.empty(1552, 1552, dtype=torch.float16, device=dev)
-        ms = time_kernel(lambda: tcu.gemm(a_, b_, out=c_), 40, 20)
-        ms_v = time_kernel(lambda: torch.matmul(a_, b_.t(), out=c_), 40, 20)
+        # both libraries as in the comparison table further down: 60 untimed + 40 timed launches, the better of two passes
+        ms = min(time_kernel(lambda: tcu.gemm(a_, b_, out=c_), 40, 60) for _ in range(2))
+        ms_v = min(time_kernel(lambda: torch.matmul(a_, b_.t(), out=c_), 40, 60) for _ in range(2))
         configs.append({"name": "gemm_1552x1552x4096_auto", "kernel": "gemm_w128k<__half, edge tiles>", "ms": ms,
                         "tflops": 2.0 * 1552 * 1552 * 4096 / (ms * 1e-3) / 1e12, "hipblaslt_ms": ms_v,
                         "speed_vs_hipblaslt": ms_v / ms})
         a_, b_ = rand16(2048, 4096), rand16(2560, 4096)
         c_ = torch.empty(2048, 2560, dtype=torch.float16, device=dev)
-        ms = time_kernel(lambda: tcu.gemm(a_, b_, out=c_), 40, 40)
-        ms_v = time_kernel(lambda: torch.matmul(a_, b_.t(), out=c_), 40, 40)
+        ms = min(time_kernel(lambda: tcu.gemm(a_, b_, out=c_), 40, 60) for _ in range(2))
+        ms_v = min(time_kernel(lambda: torch.matmul(a_, b_.t(), out=c_), 40, 60) for _ in range(2))
         configs.append({"name": "gemm_2048x2560x4096_auto", "kernel": "gemm_w128<__half, 256 x 128 tiles, three stages>", "ms": ms,
                         "tflops": 2.0 * 2048 * 2560 * 4096 / (ms * 1e-3) / 1e12, "hipblaslt_ms": ms_v,
                         "speed_vs_hipblaslt": ms_v / ms})
