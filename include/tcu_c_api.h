@@ -28,7 +28,7 @@ typedef enum {
 
 typedef enum { TCU_DTYPE_F32 = 0, TCU_DTYPE_F16 = 1 } tcu_dtype;
 
-/* Which GEMM kernel to run. AUTO picks WAVE128 when M and N are multiples of 256 with at least 128 tiles of 256 x 256;
+/* Which GEMM kernel to run. AUTO picks WAVE128 when M and N are multiples of 256 with more than 128 tiles of 256 x 256;
  * WAVE128 on the leading block of whole tiles plus PIPELINED on the remaining columns and rows (three launches on
  * disjoint parts of C, bit for bit the result of one launch) when M or N lie a little above such multiples and that
  * saves a round of workgroups; else PIPELINED; RAGGED for problems below 64 x 64. Every shape made of whole 16 x 16
@@ -62,7 +62,7 @@ typedef enum {
                                 taken in four interleaved parts (differs from the other kernels by f32 rounding) */
     TCU_GEMM_WAVE128_NARROW = 9 /* the WAVE128 kernel with 256 x 128 workgroup tiles (a wavefront owns 128 x 64; three stages): for
                                 products between the two above - too few 256 x 256 tiles to fill the GPU, too many
-                                128 x 128 tiles for one round of WAVE128_KSPLIT (2048 x 2560 x 4096); M % 256 == 0,
+                                128 x 128 tiles for one round of WAVE128_KSPLIT (2048 x 2560 x 4096, 4096 x 2048 x 8192); M % 256 == 0,
                                 N % 128 == 0, K % 64 == 0; results identical to WAVE128 and PIPELINED bit for bit */
 } tcu_gemm_algo;
 

@@ -122,6 +122,7 @@ def test_gemm_ragged_shapes(tcu, oracle, device, M, N, K, out_dtype):
 
 @pytest.mark.parametrize("M,N,K,splits", [(256, 256, 8192, 16), (512, 512, 16384, 8), (1024, 1024, 16384, 4),
                                           (1024, 2048, 16384, 2), (2048, 2048, 32768, 4), (2048, 2048, 8192, 1),
+                                          (2048, 4096, 2048, 1),
                                           (1536, 1536, 4096, 1), (1024, 1024, 8192, 1), (256, 512, 512, 1),
                                           (2048, 2048, 2048, 1)])
 @pytest.mark.parametrize("out_dtype", ["f32", "f16"])
@@ -129,7 +130,7 @@ def test_gemm_split_k_with_workspace(tcu, oracle, device, M, N, K, splits, out_d
     """tcu_gemm_f16_ws: few output tiles and a long K are split over K (f32 partial products in the caller's workspace,
     then a reduction) where that is expected to beat the unsplit launch - the partial products from the kernel with
     128 x 128 tiles whose wavefronts split K once more (first four cases) or, where those tiles alone fill the chip, from
-    the one with 256 x 256 tiles (2048 x 2048 x 32768); against the oracle and against the unsplit kernel; the workspace size is splits * M * N * 4, bytes past it stay untouched; shapes that are not split (last five
+    the one with 256 x 256 tiles (2048 x 2048 x 32768); against the oracle and against the unsplit kernel; the workspace size is splits * M * N * 4, bytes past it stay untouched; shapes that are not split (last six
     cases: among them 2048 x 2048 x 8192 and 1536 x 1536 x 4096, where the kernel whose wavefronts split K inside the
     workgroup is the faster plan) take the ordinary path and need no workspace."""
     import torch
@@ -337,13 +338,14 @@ def test_gemm_wave128_ksplit(tcu, oracle, device, M, N, K, out_dtype):
         assert np.max(np.abs(got - want)) <= (5.0 if out_dtype == "f16" else 0.1)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 128, 64), (256, 384, 128), (512, 640, 320), (1024, 1152, 1984), (2048, 2560, 4096)])
+@pytest.mark.parametrize("M,N,K", [(256, 128, 64), (256, 384, 128), (512, 640, 320), (1024, 1152, 1984), (2048, 2560, 4096),
+                                   (2048, 4096, 1024)])
 @pytest.mark.parametrize("out_dtype", ["f16", "f32"])
 def test_gemm_wave128_narrow(tcu, oracle, device, M, N, K, out_dtype):
     """The one-wavefront-per-SIMD kernel with 256 x 128 workgroup tiles (a wavefront owns 128 x 64): 1 to 64 tiles of K,
     odd and even counts, against the oracle and bit for bit against the pipelined kernel (same order of the sum), guard
     rows around C; 2048 x 2560 x 4096 (160 tiles: more than half a round of 256 x 256 tiles would idle, 128 x 128 tiles
-    need two rounds) is a shape AUTO sends to it."""
+    need two rounds) and 2048 x 4096 x 1024 (exactly 128 tiles of 256 x 256, half of the chip) are shapes AUTO sends to it."""
     import torch
 
     print(f"gemm wave128_narrow {M}x{N}x{K} {out_dtype}", flush=True)

@@ -361,6 +361,18 @@ bool gemm_w128k_is_the_choice(int M, int N, int K) {
     return tiles >= 128 && tiles <= 256;
 }
 
+/// Whether AUTO sends an unsplit product to the 256 x 128 tile: at most 128 tiles of 256 x 256 (half of the chip or
+/// more would idle), 128 x 128 tiles need two rounds of the K-splitting kernel, but 256 x 128 tiles fill one round
+/// (2048 x 2560 x 4096: 45.9 against 59.1 us for the pipelined kernel, 3072 x 2560 x 4096: 57.0 against 67.3,
+/// 4096 x 2048 x 8192: 106.5 against 134.7 us for 128 tiles of 256 x 256); a short K is left to the pipelined kernel's
+/// ring.
+bool gemm_narrow_is_the_choice(int M, int N, int K) {
+    if (M % 256 != 0 || N % 128 != 0 || K % 64 != 0 || K < 1024 || (long)K * 512 >= (1l << 32)) return false;
+    if (gemm_w128k_is_the_choice(M, N, K)) return false;
+    const long narrow = (long)(M / 256) * (N / 128);
+    return narrow > 128 && narrow <= 256;
+}
+
 /// How tcu_gemm_f16_ws runs a product: unsplit (splits == 1), or split over K into `splits` ranges whose f32 partial
 /// products come from gemm_w128 (256 x 256 tiles) or from gemm_w128k (128 x 128 tiles: four times the workgroups per
 /// range, so a quarter of the ranges - and of the partial products to write and add - fills the chip).
@@ -387,6 +399,13 @@ GemmSplitPlan gemm_split_plan(int M, int N, int K) {
         const long tiles128 = (long)(M / 128) * (N / 128), tiles96 = (long)(M / 128) * ((N + 95) / 96);
         const double per_tile = tiles128 <= 192 && tiles96 <= 256 ? 0.75 : 0.95;
         unsplit_us = std::min(unsplit_us, 5.0 + per_tile * (K / 128));
+    }
+    // the 256 x 128 tile, where AUTO would run it: 6 us + per 64 of K 0.70 us with up to 160 tiles, rising to 0.83 us with
+    // 256 (measured)
+    if (gemm_narrow_is_the_choice(M, N, K)) {
+        const long narrow = (long)(M / 256) * (N / 128);
+        const double per_tile = 0.70 + 0.13 * (narrow > 160 ? double(narrow - 160) / 96.0 : 0.0);
+        unsplit_us = std::min(unsplit_us, 6.0 + per_tile * (K / 64));
     }
     double best_us = 0.95 * unsplit_us;
     const double plane_us = 2.0 * double(M) * N * 4 / 5.3e6;  // a plane of partial products written and read once
@@ -465,19 +484,14 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             return gemm_w128_narrow_dispatch<OutType>(A, B, C, M, N, K, stream);
         case TCU_GEMM_AUTO:
             // where the 256 x 256 tile is the choice anyway, the one-wavefront-per-SIMD kernel is the faster one
-            if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) >= 128 &&
+            if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) > 128 &&
                 (long)K * 512 < (1l << 32))
                 return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
             // too few 256 x 256 tiles for the chip, but about one 128 x 128 tile per CU and a long enough K: the
             // kernel whose wavefronts split K (each owns the whole tile)
             if (gemm_w128k_is_the_choice(M, N, K)) return gemm_w128k_dispatch<OutType>(A, B, C, M, N, K, stream);
-            // between the two: more than half a round of 256 x 256 tiles would idle and 128 x 128 tiles need two rounds of
-            // the K-splitting kernel, but 256 x 128 tiles fill one round (2048 x 2560 x 4096: 45.9 against 59.1 us for the
-            // pipelined kernel, 3072 x 2560 x 4096: 57.0 against 67.3); a short K is left to the pipelined kernel's ring
-            if (M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && K >= 1024 && (long)K * 512 < (1l << 32)) {
-                const long narrow = (long)(M / 256) * (N / 128);
-                if (narrow > 128 && narrow <= 256) return gemm_w128_narrow_dispatch<OutType>(A, B, C, M, N, K, stream);
-            }
+            // between the two: 256 x 128 tiles fill one round
+            if (gemm_narrow_is_the_choice(M, N, K)) return gemm_w128_narrow_dispatch<OutType>(A, B, C, M, N, K, stream);
             if (M % 16 == 0 && N % 16 == 0) {
                 const int rc = gemm_main_and_strips<OutType>(A, B, C, M, N, K, stream);
                 if (rc != kPlanNotTaken) return rc;
