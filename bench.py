@@ -475,6 +475,16 @@ def main():
         configs.append({"name": "gemm_2048x2560x4096_auto", "kernel": "gemm_w128<__half, 256 x 128 tiles, three stages>", "ms": ms,
                         "tflops": 2.0 * 2048 * 2560 * 4096 / (ms * 1e-3) / 1e12, "hipblaslt_ms": ms_v,
                         "speed_vs_hipblaslt": ms_v / ms})
+        # 320 tiles of 256 x 256: the first 256 by gemm_w128, the rest of C by the kernel whose wavefronts split K
+        a_, b_ = rand16(2560, 4096), rand16(8192, 4096)
+        c_ = torch.empty(2560, 8192, dtype=torch.float16, device=dev)
+        ms = min(time_kernel(lambda: tcu.gemm(a_, b_, out=c_, workspace=False), 40, 60) for _ in range(2))
+        ms_1 = min(time_kernel(lambda: tcu.gemm(a_, b_, out=c_, algo="wave128"), 40, 60) for _ in range(2))
+        ms_v = min(time_kernel(lambda: torch.matmul(a_, b_.t(), out=c_), 40, 60) for _ in range(2))
+        configs.append({"name": "gemm_2560x8192x4096_auto", "kernel": "gemm_w128<__half> on 2048 rows + gemm_w128k<__half> on 512",
+                        "ms": ms, "tflops": 2.0 * 2560 * 8192 * 4096 / (ms * 1e-3) / 1e12, "ms_single_launch": ms_1,
+                        "hipblaslt_ms": ms_v, "speed_vs_hipblaslt": ms_v / ms})
+        del a_, b_, c_
         a_ = (torch.randn(8192, 64, device=dev) * 0.1).half()
         b_ = (torch.randn(128, 64, device=dev) * 0.1).half()
         c_ = (torch.randn(64, 128, device=dev) * 0.1).half()

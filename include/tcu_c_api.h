@@ -31,7 +31,9 @@ typedef enum { TCU_DTYPE_F32 = 0, TCU_DTYPE_F16 = 1 } tcu_dtype;
 /* Which GEMM kernel to run. AUTO picks WAVE128 when M and N are multiples of 256 with more than 128 tiles of 256 x 256;
  * WAVE128 on the leading block of whole tiles plus PIPELINED on the remaining columns and rows (three launches on
  * disjoint parts of C, bit for bit the result of one launch) when M or N lie a little above such multiples and that
- * saves a round of workgroups; else PIPELINED; RAGGED for problems below 64 x 64. Every shape made of whole 16 x 16
+ * saves a round of workgroups; WAVE128 on the leading rows or columns that fill whole rounds of 256 workgroups plus a
+ * kernel with smaller tiles (WAVE128_KSPLIT, WAVE128_NARROW or PIPELINED) on the rest of C when the last round would be
+ * far from full (2560 x 8192: 320 tiles); WAVE128_KSPLIT and WAVE128_NARROW as described below; else PIPELINED; RAGGED for problems below 64 x 64. Every shape made of whole 16 x 16
  * BaseTiles (M, N, K multiples of 16), the granularity of the reference's tile types, is accepted. */
 typedef enum {
     TCU_GEMM_AUTO = 0,

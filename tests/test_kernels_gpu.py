@@ -366,6 +366,44 @@ def test_gemm_wave128_narrow(tcu, oracle, device, M, N, K, out_dtype):
         assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, workspace=False))  # AUTO takes this kernel here
 
 
+@pytest.mark.parametrize("M,N,K,main,rest_algo", [(2560, 8192, 2048, (2048, 8192), "wave128_ksplit"),
+                                                  (8192, 2560, 2048, (8192, 2048), "wave128_ksplit"),
+                                                  (4608, 4608, 4096, None, "wave128_narrow")])
+@pytest.mark.parametrize("out_dtype", ["f16", "f32"])
+def test_gemm_full_rounds_and_rest(tcu, oracle, device, M, N, K, main, rest_algo, out_dtype):
+    """More than 256 tiles of 256 x 256 with a last round that is far from full (320 = 256 + 64, 324 = 252 + 72): AUTO
+    gives the leading rows (first and third case) or columns (second case) to the one-wavefront-per-SIMD kernel and the
+    rest of C to a kernel with smaller tiles, as a second launch. Against the oracle on rows of both parts; the main
+    part bit for bit what the one-wavefront-per-SIMD kernel writes there in one launch, the rest bit for bit what the
+    named kernel gives on that sub-problem (the kernel with 256 x 128 tiles sums in the same order as the one with
+    256 x 256, so there all of C is compared with the single launch); guard rows around C."""
+    import torch
+
+    print(f"gemm rounds and rest {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float16 if out_dtype == "f16" else torch.float32
+    A = oracle.fill_uniform(M * K, 9100 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 9200 + N).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    guard = torch.full((M + 2, N), -7.0, dtype=dt, device=device)
+    out = guard[1:M + 1]
+    tcu.gemm(dA, dB, out=out, workspace=False)
+    torch.cuda.synchronize()
+    assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
+    for rows in ((0, 32), (M - 32, M)):
+        ref = oracle.gemm(A, Bt, rows=rows)
+        assert oracle.max_rel_err(host(out)[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
+    whole = tcu.gemm(dA, dB, out_dtype=dt, algo="wave128")
+    if main is None:
+        assert torch.equal(out, whole)
+        return
+    Mm, Nm = main
+    assert torch.equal(out[:Mm, :Nm], whole[:Mm, :Nm])
+    if Mm < M:
+        assert torch.equal(out[Mm:], tcu.gemm(dA[Mm:], dB, out_dtype=dt, algo=rest_algo))
+    else:
+        assert torch.equal(out[:, Nm:], tcu.gemm(dA, dB[Nm:], out_dtype=dt, algo=rest_algo))
+
+
 @pytest.mark.parametrize("M,N,K", [(16, 16, 128), (144, 112, 256), (272, 400, 384), (1552, 1552, 4096), (1536, 1616, 2048),
                                    (1808, 1936, 256), (1536, 1536, 512)])
 @pytest.mark.parametrize("out_dtype", ["f16", "f32"])

@@ -242,32 +242,36 @@ int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int 
 /// gemm_w128 with 256 x 128 workgroup tiles: for products with too few 256 x 256 tiles to fill the chip and too many
 /// 128 x 128 tiles for one round of the K-splitting kernel.
 template <typename OutType>
-int gemm_w128_narrow_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+int gemm_w128_narrow_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream,
+                              int ldc = 0) {
     using T = GemmW128TraitsN<4>;
+    if (ldc == 0) ldc = N;
     if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0)
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM with 256 x 128 tiles needs M % 256 == 0, "
                                                "N % 128 == 0, K % 64 == 0");
     if ((long)K * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
     return launch(&gemm_w128<OutType, T>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
-                  C, M, N, K, K, K, N, static_cast<unsigned int*>(nullptr), 0);
+                  C, M, N, K, K, K, ldc, static_cast<unsigned int*>(nullptr), 0);
 }
 
 template <typename OutType, typename T>
-int launch_gemm_w128k(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+int launch_gemm_w128k(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream, int ldc) {
     const long grid = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
     if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many tiles for one launch");
     if (M % T::kBM == 0 && N % T::kBN == 0)
         return launch(&gemm_w128k<OutType, false, T>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C,
-                      M, N, K, K, K, N);
+                      M, N, K, K, K, ldc);
     // edge tiles: rows beyond M or N loaded from the last valid row, stores guarded per 16 x 16 block
     return launch(&gemm_w128k<OutType, true, T>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M,
-                  N, K, K, K, N);
+                  N, K, K, K, ldc);
 }
 
 template <typename OutType>
-int gemm_w128k_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+int gemm_w128k_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream,
+                        int ldc = 0) {
     using T = GemmW128kTraits;
+    if (ldc == 0) ldc = N;
     if (M % 16 != 0 || N % 16 != 0 || K % T::kBK != 0)
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the K-splitting one-wavefront-per-SIMD GEMM needs M and N in multiples of 16 "
                                                "and K in multiples of 128");
@@ -282,8 +286,8 @@ int gemm_w128k_dispatch(const __half* A, const __half* B, OutType* C, int M, int
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
         cus = 0;
     if (cus > 0 && tiles128 <= (3l * cus) / 4 && tiles96 <= cus)
-        return launch_gemm_w128k<OutType, GemmW128kTraitsN<6>>(A, B, C, M, N, K, stream);
-    return launch_gemm_w128k<OutType, T>(A, B, C, M, N, K, stream);
+        return launch_gemm_w128k<OutType, GemmW128kTraitsN<6>>(A, B, C, M, N, K, stream, ldc);
+    return launch_gemm_w128k<OutType, T>(A, B, C, M, N, K, stream, ldc);
 }
 
 template <typename OutType, int kM, int kN, int kK, int kTM, int kTN, typename WarpLayout>
@@ -373,6 +377,70 @@ bool gemm_narrow_is_the_choice(int M, int N, int K) {
     return narrow > 128 && narrow <= 256;
 }
 
+/// Expected time of one launch, in us, of the kernels above where AUTO runs them (measured on whole-chip launches): the
+/// K-splitting kernel 5 us + 0.95 us per 128 of K with 128 x 128 tiles, 0.75 us with 128 x 96 tiles; the 256 x 128 tile
+/// 6 us + per 64 of K 0.70 us with up to 160 tiles, rising to 0.83 us with 256; 256 x 256 tiles 3 us + per 1024 of K
+/// 23.5 us for every full round of 256 workgroups and, for a last round of t, 10.6 + 12.9 t / 256 us (the chip is
+/// power-limited: fewer busy CUs run at a higher clock) but not below 17 us (what one workgroup needs by itself).
+double gemm_w128k_us(int M, int N, int K) {
+    const long rows = (M + 127) / 128;
+    const long tiles128 = rows * ((N + 127) / 128), tiles96 = rows * ((N + 95) / 96);
+    return 5.0 + (tiles128 <= 192 && tiles96 <= 256 ? 0.75 : 0.95) * (K / 128);
+}
+
+double gemm_narrow_us(int M, int N, int K) {
+    const long narrow = (long)(M / 256) * (N / 128);
+    return 6.0 + (0.70 + 0.13 * (narrow > 160 ? double(narrow - 160) / 96.0 : 0.0)) * (K / 64);
+}
+
+double gemm_w128_us(long tiles, int K) {
+    const long full = (tiles - 1) / 256, last = tiles - 256 * full;
+    // a later round starts unevenly - the XCDs differ by about 4 % - which hides some of a last round that is far from full
+    const double fill = last / 256.0;
+    const double last_us = std::max(17.0, 10.6 + 12.9 * fill) - 0.04 * 23.5 * full * (1.0 - fill);
+    return 3.0 + (K / 1024.0) * (23.5 * full + std::max(9.0, last_us));
+}
+
+/// More than one round of 256 x 256 tiles, the last of them far from full (2560 x 8192: 320 tiles, the last 64 of which
+/// cost as much again as the first 256): the leading rows (or columns) whose tiles fill whole rounds go to gemm_w128, the
+/// rest of C to the kernel that fills the chip with smaller tiles - the K-splitting kernel (32 to 64 tiles of 256 x 256
+/// left), the 256 x 128 tile (65 to 128 left), else the pipelined kernel. Two launches on disjoint parts of C; taken
+/// when the cost model expects 7 % over the single launch (2560 x 8192 x 4096: 134.6 against 166.3 us, 4352^2 x 4096:
+/// 127.8 against 164.1, 3072 x 6144 x 4096: 125.6 against 160.9). Returns kPlanNotTaken otherwise.
+template <typename OutType>
+int gemm_rounds_and_rest(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+    if (M % 256 != 0 || N % 256 != 0 || K % 64 != 0 || (long)K * 512 >= (1l << 32)) return kPlanNotTaken;
+    const int tm = M / 256, tn = N / 256;
+    const long tiles = (long)tm * tn;
+    if (tiles <= 256 || tiles % 256 == 0) return kPlanNotTaken;
+    auto rest_us = [&](int Mr, int Nr) {
+        if (gemm_w128k_is_the_choice(Mr, Nr, K)) return gemm_w128k_us(Mr, Nr, K);
+        if (gemm_narrow_is_the_choice(Mr, Nr, K)) return gemm_narrow_us(Mr, Nr, K);
+        return pipelined_plan(Mr, Nr, K).us;
+    };
+    double best_us = 0.93 * gemm_w128_us(tiles, K);
+    int main_rows = 0, main_cols = 0;  // in tiles; one of them set when a split wins
+    for (int t = 1; t < tm; ++t) {
+        const double us = gemm_w128_us((long)t * tn, K) + 2.0 + rest_us(M - 256 * t, N);
+        if (us < best_us) best_us = us, main_rows = t, main_cols = 0;
+    }
+    for (int t = 1; t < tn; ++t) {
+        const double us = gemm_w128_us((long)t * tm, K) + 2.0 + rest_us(M, N - 256 * t);
+        if (us < best_us) best_us = us, main_rows = 0, main_cols = t;
+    }
+    if (main_rows == 0 && main_cols == 0) return kPlanNotTaken;
+    const int Mm = main_rows ? 256 * main_rows : M, Nm = main_cols ? 256 * main_cols : N;
+    int rc = gemm_w128_dispatch<OutType>(A, B, C, Mm, Nm, K, stream, K, K, N);
+    if (rc != TCU_OK) return rc;
+    const __half* Ar = main_rows ? A + size_t(Mm) * K : A;
+    const __half* Br = main_cols ? B + size_t(Nm) * K : B;
+    OutType* Cr = main_rows ? C + size_t(Mm) * N : C + Nm;
+    const int Mr = main_rows ? M - Mm : M, Nr = main_cols ? N - Nm : N;
+    if (gemm_w128k_is_the_choice(Mr, Nr, K)) return gemm_w128k_dispatch<OutType>(Ar, Br, Cr, Mr, Nr, K, stream, N);
+    if (gemm_narrow_is_the_choice(Mr, Nr, K)) return gemm_w128_narrow_dispatch<OutType>(Ar, Br, Cr, Mr, Nr, K, stream, N);
+    return gemm_pipelined_dispatch<OutType>(Ar, Br, Cr, Mr, Nr, K, stream, N);
+}
+
 /// How tcu_gemm_f16_ws runs a product: unsplit (splits == 1), or split over K into `splits` ranges whose f32 partial
 /// products come from gemm_w128 (256 x 256 tiles) or from gemm_w128k (128 x 128 tiles: four times the workgroups per
 /// range, so a quarter of the ranges - and of the partial products to write and add - fills the chip).
@@ -393,20 +461,9 @@ GemmSplitPlan gemm_split_plan(int M, int N, int K) {
     const long tiles = (long)(M / T::kBM) * (N / T::kBN);
     if (tiles > 128) return plan;
     double unsplit_us = pipelined_plan(M, N, K).us;
-    // the K-splitting kernel, where AUTO would run it: one round of workgroups, 5 us + 0.95 us per 128 of K with 128 x 128
-    // tiles, 0.75 us with 128 x 96 tiles (measured)
-    if (gemm_w128k_is_the_choice(M, N, K)) {
-        const long tiles128 = (long)(M / 128) * (N / 128), tiles96 = (long)(M / 128) * ((N + 95) / 96);
-        const double per_tile = tiles128 <= 192 && tiles96 <= 256 ? 0.75 : 0.95;
-        unsplit_us = std::min(unsplit_us, 5.0 + per_tile * (K / 128));
-    }
-    // the 256 x 128 tile, where AUTO would run it: 6 us + per 64 of K 0.70 us with up to 160 tiles, rising to 0.83 us with
-    // 256 (measured)
-    if (gemm_narrow_is_the_choice(M, N, K)) {
-        const long narrow = (long)(M / 256) * (N / 128);
-        const double per_tile = 0.70 + 0.13 * (narrow > 160 ? double(narrow - 160) / 96.0 : 0.0);
-        unsplit_us = std::min(unsplit_us, 6.0 + per_tile * (K / 64));
-    }
+    // the kernels AUTO would run instead of the pipelined one
+    if (gemm_w128k_is_the_choice(M, N, K)) unsplit_us = std::min(unsplit_us, gemm_w128k_us(M, N, K));
+    if (gemm_narrow_is_the_choice(M, N, K)) unsplit_us = std::min(unsplit_us, gemm_narrow_us(M, N, K));
     double best_us = 0.95 * unsplit_us;
     const double plane_us = 2.0 * double(M) * N * 4 / 5.3e6;  // a plane of partial products written and read once
     for (int s = 2; s * tiles <= 256 && K % (s * T::kBK) == 0 && K / s >= 512; s *= 2) {
@@ -485,8 +542,10 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
         case TCU_GEMM_AUTO:
             // where the 256 x 256 tile is the choice anyway, the one-wavefront-per-SIMD kernel is the faster one
             if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) > 128 &&
-                (long)K * 512 < (1l << 32))
-                return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
+                (long)K * 512 < (1l << 32)) {
+                const int rc = gemm_rounds_and_rest<OutType>(A, B, C, M, N, K, stream);
+                return rc != kPlanNotTaken ? rc : gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
+            }
             // too few 256 x 256 tiles for the chip, but about one 128 x 128 tile per CU and a long enough K: the
             // kernel whose wavefronts split K (each owns the whole tile)
             if (gemm_w128k_is_the_choice(M, N, K)) return gemm_w128k_dispatch<OutType>(A, B, C, M, N, K, stream);
