@@ -33,8 +33,8 @@
 //     (4096^3: 115 against 99 us).
 // Because the compiler does not know these asm statements are MFMAs it inserts none of the wait states MFMA results
 // need before other instructions read them; the only such reads are in the epilogue, and every accumulator passes
-// through a waiting statement first (see below). M % 256 == 0, N a multiple of the tile width, K % 64 == 0 (checked by the
-// launcher).
+// through a waiting statement first (see below). M % 256 == 0, N a multiple of the tile width - or, with edge tiles
+// (kEdges: rows clamped on the way in, stores guarded), any multiples of 16 - and K % 64 == 0 (checked by the launcher).
 #pragma once
 
 #include <type_traits>
@@ -121,7 +121,10 @@ __global__ void __launch_bounds__(256) splitk_reduce(const float* __restrict__ p
 /// K-range [z K, (z + 1) K) and writes plane z of C ([splits, M, N]; partial sums for splitk_reduce).
 /// zero_words / zero_count: device words that the first workgroup sets to zero on the side (null / 0: none) - the
 /// synchronisation words of a kernel that follows this one on the stream, cleared without a launch of their own.
-template <typename OutType, typename T = GemmW128Traits>
+/// kEdges: M and N need not be multiples of the tile (multiples of 16 suffice): the grid covers ceil(M / 256) x
+/// ceil(N / kBN) tiles, rows beyond the edge are loaded from the last valid row (their products are computed and
+/// dropped) and the stores are guarded. Nothing changes inside the loop over K.
+template <typename OutType, typename T = GemmW128Traits, bool kEdges = false>
 __global__ void __launch_bounds__(T::kThreads)
     gemm_w128(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
               int lda, int ldb, int ldc, unsigned int* __restrict__ zero_words, int zero_count) {
@@ -135,7 +138,8 @@ __global__ void __launch_bounds__(T::kThreads)
         for (int i = threadIdx.x; i < zero_count; i += T::kThreads) zero_words[i] = 0u;
     }
     int tile_m, tile_n;
-    detail::xcd_tile_coords(blockIdx.x, M / T::kBM, N / T::kBN, tile_m, tile_n);
+    detail::xcd_tile_coords(blockIdx.x, kEdges ? (M + T::kBM - 1) / T::kBM : M / T::kBM,
+                            kEdges ? (N + T::kBN - 1) / T::kBN : N / T::kBN, tile_m, tile_n);
     const int m0 = tile_m * T::kBM, n0 = tile_n * T::kBN;
 
     // ---- global -> LDS: load instruction q of this wavefront (q < 8: A, else B) fills 8 rows of 128 bytes; lane i
@@ -145,7 +149,8 @@ __global__ void __launch_bounds__(T::kThreads)
 #pragma unroll
     for (int q = 0; q < kNumLoads; ++q) {
         const int row = (q < 8 ? wave * T::kLoads + q : wave * T::kLoadsB + (q - 8)) * 8 + lrow;
-        voff[q] = static_cast<unsigned int>(row) * static_cast<unsigned int>(q < 8 ? lda : ldb) * 2u +
+        const int last = q < 8 ? M - 1 - m0 : N - 1 - n0;  // the tile's last row that exists
+        voff[q] = static_cast<unsigned int>(kEdges && row > last ? last : row) * static_cast<unsigned int>(q < 8 ? lda : ldb) * 2u +
                   (lchk ^ ((row >> 1) & 7)) * 16;
     }
     // blockIdx.y = z selects the z-th K-range of length K of wider operands (split-K: lda, ldb >= gridDim.y * K) and
@@ -369,7 +374,9 @@ __global__ void __launch_bounds__(T::kThreads)
 #pragma unroll
             for (int it = 0; it < kReads; ++it) {
                 const u32x4 v = *reinterpret_cast<lds_u32x4_ptr>(raddr[it] + buf);
-                *reinterpret_cast<u32x4*>(crow + size_t(i * 16 + it * kRowsPerRead) * ldc * sizeof(OutType)) = v;
+                if (!kEdges || (m0 + wave_m * T::kWaveM + i * 16 + it * kRowsPerRead + rr < M &&
+                                n0 + wave_n * T::kWaveN + cc * 8 < N))
+                    *reinterpret_cast<u32x4*>(crow + size_t(i * 16 + it * kRowsPerRead) * ldc * sizeof(OutType)) = v;
             }
         }
     } else {
@@ -378,7 +385,8 @@ __global__ void __launch_bounds__(T::kThreads)
         for (int i = 0; i < 8; ++i)
 #pragma unroll
             for (int j = 0; j < kNT; ++j)
-                *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * ldc + j * 16 + 4 * fquad) = acc[i][j];
+                if (!kEdges || (m0 + wave_m * T::kWaveM + i * 16 + frow < M && n0 + wave_n * T::kWaveN + j * 16 + 4 * fquad < N))
+                    *reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * ldc + j * 16 + 4 * fquad) = acc[i][j];
     }
 }
 

@@ -44,7 +44,8 @@ typedef enum {
                                 workgroups a launch takes; edge tiles (rows clamped, stores guarded, k tail zeroed in
                                 LDS) where the shape is not whole tiles */
     TCU_GEMM_WAVE128 = 4,    /* same pipeline, 256 x 256 tile on 4 wavefronts (one per SIMD, 128 x 128 each),
-                                accumulators in AGPRs; results identical to PIPELINED bit for bit, except where K is a
+                                accumulators in AGPRs; M and N multiples of 16 (edge tiles: rows clamped, stores
+                                guarded), K % 64 == 0; results identical to PIPELINED bit for bit, except where K is a
                                 multiple of 16384 (rows a multiple of 32 KiB apart): there each XCD sums over K in
                                 rotated order, which differs by f32 rounding */
     TCU_GEMM_TILE_PIPELINED = 5, /* the PIPELINED kernel composed from tile-library functors only (direct-to-LDS loader,
@@ -64,8 +65,9 @@ typedef enum {
                                 taken in four interleaved parts (differs from the other kernels by f32 rounding) */
     TCU_GEMM_WAVE128_NARROW = 9 /* the WAVE128 kernel with 256 x 128 workgroup tiles (a wavefront owns 128 x 64; three stages): for
                                 products between the two above - too few 256 x 256 tiles to fill the GPU, too many
-                                128 x 128 tiles for one round of WAVE128_KSPLIT (2048 x 2560 x 4096, 4096 x 2048 x 8192); M % 256 == 0,
-                                N % 128 == 0, K % 64 == 0; results identical to WAVE128 and PIPELINED bit for bit */
+                                128 x 128 tiles for one round of WAVE128_KSPLIT (2048 x 2560 x 4096, 4096 x 2048 x 8192,
+                                1552 x 3088 x 4096); M and N multiples of 16 (edge tiles: rows clamped, stores guarded),
+                                K % 64 == 0; results identical to WAVE128 and PIPELINED bit for bit */
 } tcu_gemm_algo;
 
 /* Which back-to-back GEMM kernel to run (tcu_b2b_gemm_f16_algo). AUTO picks ROWS for many rows, else RESIDENT, where

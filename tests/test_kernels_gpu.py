@@ -258,9 +258,38 @@ def test_gemm_main_block_and_strips(tcu, oracle, device, M, N, K, out_dtype):
 def test_gemm_wave128_rejects_other_shapes(tcu, device):
     import torch
 
-    A = torch.zeros(128, 64, dtype=torch.float16, device=device)
+    A = torch.zeros(128, 96, dtype=torch.float16, device=device)  # K must be a multiple of 64
     with pytest.raises(RuntimeError):
         tcu.gemm(A, A, algo="wave128")
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 16, 64), (272, 400, 128), (1040, 528, 192), (4112, 272, 64), (240, 4112, 320),
+                                   (3088, 3088, 256)])
+@pytest.mark.parametrize("out_dtype", ["f16", "f32"])
+def test_gemm_wave128_edge_tiles(tcu, oracle, device, M, N, K, out_dtype):
+    """The one-wavefront-per-SIMD kernel on shapes that are not whole 256 x 256 tiles (M, N in multiples of 16): rows
+    beyond the edge are fetched from the last valid row and their results dropped, the stores are guarded - a single
+    partial tile, edges in M, in N and in both, a tile row and a tile column that are 16 wide; against the oracle, bit
+    for bit against the pipelined kernel, with guard rows around C. 3088 x 3088 is a shape AUTO sends to it (169 tiles in one round)."""
+    import torch
+
+    print(f"gemm wave128 edge tiles {M}x{N}x{K} {out_dtype}", flush=True)
+    dt = torch.float16 if out_dtype == "f16" else torch.float32
+    A = oracle.fill_uniform(M * K, 6100 + M).reshape(M, K)
+    Bt = oracle.fill_uniform(N * K, 6200 + N).reshape(N, K)
+    dA, dB = dev(A, device), dev(Bt, device)
+    guard = torch.full((M + 2, N), -7.0, dtype=dt, device=device)
+    out = guard[1:M + 1]
+    tcu.gemm(dA, dB, out=out, algo="wave128")
+    torch.cuda.synchronize()
+    assert torch.all(guard[0] == -7.0) and torch.all(guard[M + 1] == -7.0)
+    rows = (0, M) if M * N * K <= 2 ** 28 else (M - 64, M)
+    ref = oracle.gemm(A, Bt, rows=rows)
+    assert oracle.max_rel_err(host(out)[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
+    assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))
+    if M == 3088:
+        auto = tcu.gemm(dA, dB, out_dtype=dt, workspace=False)
+        assert torch.equal(out, auto)
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 768, 192), (1024, 1024, 1024), (4096, 4096, 4096)])
@@ -339,13 +368,15 @@ def test_gemm_wave128_ksplit(tcu, oracle, device, M, N, K, out_dtype):
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 128, 64), (256, 384, 128), (512, 640, 320), (1024, 1152, 1984), (2048, 2560, 4096),
-                                   (2048, 4096, 1024)])
+                                   (2048, 4096, 1024), (16, 16, 64), (272, 400, 128), (1040, 528, 192), (1552, 3088, 1024)])
 @pytest.mark.parametrize("out_dtype", ["f16", "f32"])
 def test_gemm_wave128_narrow(tcu, oracle, device, M, N, K, out_dtype):
     """The one-wavefront-per-SIMD kernel with 256 x 128 workgroup tiles (a wavefront owns 128 x 64): 1 to 64 tiles of K,
     odd and even counts, against the oracle and bit for bit against the pipelined kernel (same order of the sum), guard
     rows around C; 2048 x 2560 x 4096 (160 tiles: more than half a round of 256 x 256 tiles would idle, 128 x 128 tiles
-    need two rounds) and 2048 x 4096 x 1024 (exactly 128 tiles of 256 x 256, half of the chip) are shapes AUTO sends to it."""
+    need two rounds) and 2048 x 4096 x 1024 (exactly 128 tiles of 256 x 256, half of the chip) are shapes AUTO sends to it,
+    and so is 1552 x 3088 x 1024 (175 tiles, with edge tiles: the last four shapes are not whole tiles - rows beyond the edge
+    are fetched from the last valid row, the stores are guarded)."""
     import torch
 
     print(f"gemm wave128_narrow {M}x{N}x{K} {out_dtype}", flush=True)
@@ -362,7 +393,7 @@ def test_gemm_wave128_narrow(tcu, oracle, device, M, N, K, out_dtype):
     ref = oracle.gemm(A, Bt, rows=rows)
     assert oracle.max_rel_err(host(out)[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
     assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))
-    if M == 2048:
+    if M == 2048 or M == 1552:
         assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, workspace=False))  # AUTO takes this kernel here
 
 

@@ -231,12 +231,18 @@ int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int 
     if (lda == 0) lda = K;
     if (ldb == 0) ldb = K;
     if (ldc == 0) ldc = N;
-    if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM needs M % 256 == 0, N % 256 == 0, K % 64 == 0");
+    if (M % 16 != 0 || N % 16 != 0 || K % T::kBK != 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM needs M and N in multiples of 16 and K % 64 == 0");
     if ((long)std::max(lda, ldb) * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
-    return launch(&gemm_w128<OutType>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
-                  C, M, N, K, lda, ldb, ldc, zero_words, zero_count);
+    if (M % T::kBM == 0 && N % T::kBN == 0)
+        return launch(&gemm_w128<OutType>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
+                      C, M, N, K, lda, ldb, ldc, zero_words, zero_count);
+    // edge tiles: rows beyond M or N loaded from the last valid row, stores guarded
+    const long grid = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
+    if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many tiles for one launch");
+    return launch(&gemm_w128<OutType, T, true>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M, N,
+                  K, lda, ldb, ldc, zero_words, zero_count);
 }
 
 /// gemm_w128 with 256 x 128 workgroup tiles: for products with too few 256 x 256 tiles to fill the chip and too many
@@ -246,13 +252,19 @@ int gemm_w128_narrow_dispatch(const __half* A, const __half* B, OutType* C, int 
                               int ldc = 0) {
     using T = GemmW128TraitsN<4>;
     if (ldc == 0) ldc = N;
-    if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM with 256 x 128 tiles needs M % 256 == 0, "
-                                               "N % 128 == 0, K % 64 == 0");
+    if (M % 16 != 0 || N % 16 != 0 || K % T::kBK != 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM with 256 x 128 tiles needs M and N in "
+                                               "multiples of 16 and K % 64 == 0");
     if ((long)K * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
-    return launch(&gemm_w128<OutType, T>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
-                  C, M, N, K, K, K, ldc, static_cast<unsigned int*>(nullptr), 0);
+    if (M % T::kBM == 0 && N % T::kBN == 0)
+        return launch(&gemm_w128<OutType, T>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A,
+                      B, C, M, N, K, K, K, ldc, static_cast<unsigned int*>(nullptr), 0);
+    // edge tiles: rows beyond M or N loaded from the last valid row, stores guarded
+    const long grid = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
+    if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many tiles for one launch");
+    return launch(&gemm_w128<OutType, T, true>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M, N,
+                  K, K, K, ldc, static_cast<unsigned int*>(nullptr), 0);
 }
 
 template <typename OutType, typename T>
@@ -337,17 +349,19 @@ int gemm_tile_w128_dispatch(const __half* A, const __half* B, OutType* C, int M,
 /// everywhere, so the result is bit for bit that of one launch. Returns kPlanNotTaken when the plain launch is the
 /// better plan.
 constexpr int kPlanNotTaken = INT_MIN;
+double gemm_w128_us(long tiles, int K);
 template <typename OutType>
-int gemm_main_and_strips(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
+int gemm_main_and_strips(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream,
+                         double other_us) {
     using T = GemmW128Traits;
     const int Mm = M / T::kBM * T::kBM, Nm = N / T::kBN * T::kBN;
     if ((Mm == M && Nm == N) || K % T::kBK != 0 || (long)K * 512 >= (1l << 32)) return kPlanNotTaken;
     const long tiles = (long)(Mm / T::kBM) * (Nm / T::kBN);
     if (tiles < 128) return kPlanNotTaken;
-    const double main_us = 2.5 + double((tiles + 255) / 256) * 24.0 * K / 1024.0;
+    const double main_us = gemm_w128_us(tiles, K);
     const double right_us = N > Nm ? 2.0 + pipelined_plan(M, N - Nm, K).us : 0.0;
     const double bottom_us = M > Mm ? 2.0 + pipelined_plan(M - Mm, Nm, K).us : 0.0;
-    if (main_us + right_us + bottom_us >= pipelined_plan(M, N, K).us) return kPlanNotTaken;
+    if (main_us + right_us + bottom_us >= std::min(other_us, pipelined_plan(M, N, K).us)) return kPlanNotTaken;
     int rc = gemm_w128_dispatch<OutType>(A, B, C, Mm, Nm, K, stream, K, K, N);
     if (rc == TCU_OK && N > Nm) rc = gemm_pipelined_dispatch<OutType>(A, B + size_t(Nm) * K, C + Nm, M, N - Nm, K, stream, N);
     if (rc == TCU_OK && M > Mm)
@@ -371,9 +385,9 @@ bool gemm_w128k_is_the_choice(int M, int N, int K) {
 /// 4096 x 2048 x 8192: 106.5 against 134.7 us for 128 tiles of 256 x 256); a short K is left to the pipelined kernel's
 /// ring.
 bool gemm_narrow_is_the_choice(int M, int N, int K) {
-    if (M % 256 != 0 || N % 128 != 0 || K % 64 != 0 || K < 1024 || (long)K * 512 >= (1l << 32)) return false;
+    if (M % 16 != 0 || N % 16 != 0 || K % 64 != 0 || K < 1024 || (long)K * 512 >= (1l << 32)) return false;
     if (gemm_w128k_is_the_choice(M, N, K)) return false;
-    const long narrow = (long)(M / 256) * (N / 128);
+    const long narrow = (long)((M + 255) / 256) * ((N + 127) / 128);  // with edge tiles where M, N are not whole tiles
     return narrow > 128 && narrow <= 256;
 }
 
@@ -389,7 +403,7 @@ double gemm_w128k_us(int M, int N, int K) {
 }
 
 double gemm_narrow_us(int M, int N, int K) {
-    const long narrow = (long)(M / 256) * (N / 128);
+    const long narrow = (long)((M + 255) / 256) * ((N + 127) / 128);
     return 6.0 + (0.70 + 0.13 * (narrow > 160 ? double(narrow - 160) / 96.0 : 0.0)) * (K / 64);
 }
 
@@ -552,8 +566,15 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             // between the two: 256 x 128 tiles fill one round
             if (gemm_narrow_is_the_choice(M, N, K)) return gemm_w128_narrow_dispatch<OutType>(A, B, C, M, N, K, stream);
             if (M % 16 == 0 && N % 16 == 0) {
-                const int rc = gemm_main_and_strips<OutType>(A, B, C, M, N, K, stream);
+                // M or N not multiples of 256: the one-wavefront-per-SIMD kernel with edge tiles, that kernel on the
+                // leading block of whole tiles plus the pipelined kernel on the strips beyond it, or the pipelined kernel
+                // with the tile its cost model picks - whichever is expected to be the shortest
+                const long tiles_e = (long)((M + 255) / 256) * ((N + 255) / 256);
+                const double edge_us = K % 64 == 0 && tiles_e >= 128 && (long)K * 512 < (1l << 32)
+                                           ? gemm_w128_us(tiles_e, K) : 1e30;
+                const int rc = gemm_main_and_strips<OutType>(A, B, C, M, N, K, stream, edge_us);
                 if (rc != kPlanNotTaken) return rc;
+                if (edge_us < pipelined_plan(M, N, K).us) return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
             }
             // tiny problems: the kernel that takes its operand tiles straight from global memory has the shorter start
             if ((long)M * N < 64 * 64) return gemm_ragged_dispatch<OutType>(A, B, C, M, N, K, stream);
