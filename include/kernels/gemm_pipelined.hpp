@@ -147,23 +147,27 @@ DEVICE void lds_barrier() {
 }
 
 /// Tile coordinates for workgroup `bid` of a grid of tiles_m x tiles_n tiles: ids that are
-/// congruent modulo 8 (same XCD) are gathered into compact blocks of tiles.
+/// congruent modulo 8 (same XCD) are gathered into compact blocks of tiles. Any grid: with total = 8 q + r tiles the
+/// first r XCDs hold q + 1 ids and the others q, each XCD takes a run of that many consecutive positions of a walk
+/// through the grid in row panels 4 tiles tall (the last panel has the tiles_m % 4 rows that are left).
 HOST_DEVICE void xcd_tile_coords(int bid, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
     const int total = tiles_m * tiles_n;
     constexpr int kXcds = 8;
-    if (total % kXcds == 0 && tiles_m % 4 == 0) {
-        const int per_xcd = total / kXcds;
-        const int xcd = bid % kXcds;
-        const int local = bid / kXcds;
-        const int lin = xcd * per_xcd + local;  // consecutive `lin` = same XCD
-        // walk the grid in column panels 4 tiles tall so that an XCD's run of per_xcd tiles is compact
+    const int q = total / kXcds, r = total % kXcds;
+    const int xcd = bid % kXcds;
+    const int local = bid / kXcds;
+    const int lin = xcd * q + (xcd < r ? xcd : r) + local;  // consecutive `lin` = same XCD
+    const int whole = (tiles_m / 4) * 4 * tiles_n;          // positions inside panels of full height
+    if (lin < whole) {
         const int panel = lin / (4 * tiles_n);
         const int in_panel = lin % (4 * tiles_n);
         tile_m = panel * 4 + in_panel % 4;
         tile_n = in_panel / 4;
     } else {
-        tile_m = bid % tiles_m;
-        tile_n = bid / tiles_m;
+        const int height = tiles_m % 4;
+        const int in_panel = lin - whole;
+        tile_m = (tiles_m / 4) * 4 + in_panel % height;
+        tile_n = in_panel / height;
     }
 }
 

@@ -359,6 +359,23 @@ static void test_pipelined_gemm_maps() {
         }
         CHECK(int(seen.size()) == tiles * tiles);
     }
+    // ... also for grids that are neither a multiple of 8 tiles nor of 4 rows: a bijection, and the ids of one XCD
+    // stay inside a few row panels (a run of ceil(total / 8) positions spans at most that many / (4 tiles_n) + 2)
+    for (int tiles_m = 1; tiles_m <= 33; ++tiles_m)
+        for (int tiles_n : {1, 2, 3, 5, 9, 13, 16, 27, 32}) {
+            std::set<std::pair<int, int>> seen;
+            std::set<int> panels_of_xcd[8];
+            for (int bid = 0; bid < tiles_m * tiles_n; ++bid) {
+                int tm, tn;
+                kernels::detail::xcd_tile_coords(bid, tiles_m, tiles_n, tm, tn);
+                CHECK(tm >= 0 && tm < tiles_m && tn >= 0 && tn < tiles_n);
+                seen.insert({tm, tn});
+                panels_of_xcd[bid % 8].insert(tm / 4);
+            }
+            CHECK(int(seen.size()) == tiles_m * tiles_n);
+            const int run = (tiles_m * tiles_n + 7) / 8;
+            for (const auto& panels : panels_of_xcd) CHECK(int(panels.size()) <= run / (4 * tiles_n) + 2);
+        }
     std::set<int> rows, cols;
     for (int bid = 3; bid < 256; bid += 8) {
         int tm, tn;
