@@ -399,12 +399,14 @@ def test_gemm_wave128_narrow(tcu, oracle, device, M, N, K, out_dtype):
 
 @pytest.mark.parametrize("M,N,K,main,rest_algo", [(2560, 8192, 2048, (2048, 8192), "wave128_ksplit"),
                                                   (8192, 2560, 2048, (8192, 2048), "wave128_ksplit"),
-                                                  (4608, 4608, 4096, None, "wave128_narrow")])
+                                                  (4608, 4608, 4096, None, "wave128_narrow"),
+                                                  (2688, 6912, 2048, (2304, 6912), "wave128_ksplit")])
 @pytest.mark.parametrize("out_dtype", ["f16", "f32"])
 def test_gemm_full_rounds_and_rest(tcu, oracle, device, M, N, K, main, rest_algo, out_dtype):
     """More than 256 tiles of 256 x 256 with a last round that is far from full (320 = 256 + 64, 324 = 252 + 72): AUTO
     gives the leading rows (first and third case) or columns (second case) to the one-wavefront-per-SIMD kernel and the
-    rest of C to a kernel with smaller tiles, as a second launch. Against the oracle on rows of both parts; the main
+    rest of C to a kernel with smaller tiles, as a second launch; the last case is not whole tiles (10.5 x 27 tiles: both
+    launches have edge tiles). Against the oracle on rows of both parts; the main
     part bit for bit what the one-wavefront-per-SIMD kernel writes there in one launch, the rest bit for bit what the
     named kernel gives on that sub-problem (the kernel with 256 x 128 tiles sums in the same order as the one with
     256 x 256, so there all of C is compared with the single launch); guard rows around C."""

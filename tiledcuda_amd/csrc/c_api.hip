@@ -418,38 +418,47 @@ double gemm_w128_us(long tiles, int K) {
 /// More than one round of 256 x 256 tiles, the last of them far from full (2560 x 8192: 320 tiles, the last 64 of which
 /// cost as much again as the first 256): the leading rows (or columns) whose tiles fill whole rounds go to gemm_w128, the
 /// rest of C to the kernel that fills the chip with smaller tiles - the K-splitting kernel (32 to 64 tiles of 256 x 256
-/// left), the 256 x 128 tile (65 to 128 left), else the pipelined kernel. Two launches on disjoint parts of C; taken
-/// when the cost model expects 7 % over the single launch (2560 x 8192 x 4096: 134.6 against 166.3 us, 4352^2 x 4096:
-/// 127.8 against 164.1, 3072 x 6144 x 4096: 125.6 against 160.9). Returns kPlanNotTaken otherwise.
-template <typename OutType>
-int gemm_rounds_and_rest(const __half* A, const __half* B, OutType* C, int M, int N, int K, hipStream_t stream) {
-    if (M % 256 != 0 || N % 256 != 0 || K % 64 != 0 || (long)K * 512 >= (1l << 32)) return kPlanNotTaken;
-    const int tm = M / 256, tn = N / 256;
+/// left), the 256 x 128 tile (65 to 128 left), else the pipelined kernel. Two launches on disjoint parts of C
+/// (2560 x 8192 x 4096: 134.6 against 166.3 us, 4352^2 x 4096: 127.8 against 164.1, 3072 x 6144 x 4096: 125.6 against
+/// 160.9). M and N in multiples of 16: the split falls on a multiple of 256, every kernel involved has edge tiles.
+/// The plan: the best split and what it is expected to cost (1e30: none).
+struct GemmRoundsPlan {
+    double us;
+    int main_rows, main_cols;  // in tiles of 256; one of them is set
+};
+
+GemmRoundsPlan gemm_rounds_and_rest_plan(int M, int N, int K) {
+    GemmRoundsPlan plan{1e30, 0, 0};
+    if (M % 16 != 0 || N % 16 != 0 || K % 64 != 0 || (long)K * 512 >= (1l << 32)) return plan;
+    const int tm = (M + 255) / 256, tn = (N + 255) / 256;
     const long tiles = (long)tm * tn;
-    if (tiles <= 256 || tiles % 256 == 0) return kPlanNotTaken;
+    if (tiles <= 256 || tiles % 256 == 0) return plan;
     auto rest_us = [&](int Mr, int Nr) {
         if (gemm_w128k_is_the_choice(Mr, Nr, K)) return gemm_w128k_us(Mr, Nr, K);
         if (gemm_narrow_is_the_choice(Mr, Nr, K)) return gemm_narrow_us(Mr, Nr, K);
         return pipelined_plan(Mr, Nr, K).us;
     };
-    double best_us = 0.93 * gemm_w128_us(tiles, K);
-    int main_rows = 0, main_cols = 0;  // in tiles; one of them set when a split wins
     for (int t = 1; t < tm; ++t) {
         const double us = gemm_w128_us((long)t * tn, K) + 2.0 + rest_us(M - 256 * t, N);
-        if (us < best_us) best_us = us, main_rows = t, main_cols = 0;
+        if (us < plan.us) plan = {us, t, 0};
     }
     for (int t = 1; t < tn; ++t) {
         const double us = gemm_w128_us((long)t * tm, K) + 2.0 + rest_us(M, N - 256 * t);
-        if (us < best_us) best_us = us, main_rows = 0, main_cols = t;
+        if (us < plan.us) plan = {us, 0, t};
     }
-    if (main_rows == 0 && main_cols == 0) return kPlanNotTaken;
-    const int Mm = main_rows ? 256 * main_rows : M, Nm = main_cols ? 256 * main_cols : N;
+    return plan;
+}
+
+template <typename OutType>
+int gemm_rounds_and_rest(const __half* A, const __half* B, OutType* C, int M, int N, int K, GemmRoundsPlan plan,
+                         hipStream_t stream) {
+    const int Mm = plan.main_rows ? 256 * plan.main_rows : M, Nm = plan.main_cols ? 256 * plan.main_cols : N;
     int rc = gemm_w128_dispatch<OutType>(A, B, C, Mm, Nm, K, stream, K, K, N);
     if (rc != TCU_OK) return rc;
-    const __half* Ar = main_rows ? A + size_t(Mm) * K : A;
-    const __half* Br = main_cols ? B + size_t(Nm) * K : B;
-    OutType* Cr = main_rows ? C + size_t(Mm) * N : C + Nm;
-    const int Mr = main_rows ? M - Mm : M, Nr = main_cols ? N - Nm : N;
+    const __half* Ar = plan.main_rows ? A + size_t(Mm) * K : A;
+    const __half* Br = plan.main_cols ? B + size_t(Nm) * K : B;
+    OutType* Cr = plan.main_rows ? C + size_t(Mm) * N : C + Nm;
+    const int Mr = plan.main_rows ? M - Mm : M, Nr = plan.main_cols ? N - Nm : N;
     if (gemm_w128k_is_the_choice(Mr, Nr, K)) return gemm_w128k_dispatch<OutType>(Ar, Br, Cr, Mr, Nr, K, stream, N);
     if (gemm_narrow_is_the_choice(Mr, Nr, K)) return gemm_w128_narrow_dispatch<OutType>(Ar, Br, Cr, Mr, Nr, K, stream, N);
     return gemm_pipelined_dispatch<OutType>(Ar, Br, Cr, Mr, Nr, K, stream, N);
@@ -557,8 +566,12 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             // where the 256 x 256 tile is the choice anyway, the one-wavefront-per-SIMD kernel is the faster one
             if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (long)(M / 256) * (N / 256) > 128 &&
                 (long)K * 512 < (1l << 32)) {
-                const int rc = gemm_rounds_and_rest<OutType>(A, B, C, M, N, K, stream);
-                return rc != kPlanNotTaken ? rc : gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
+                // ... in one launch, or - where its last round would be far from full and the cost model expects 7 % -
+                // on the leading rows or columns, with a second launch of smaller tiles on the rest of C
+                const GemmRoundsPlan rounds = gemm_rounds_and_rest_plan(M, N, K);
+                if (rounds.us < 0.93 * gemm_w128_us((long)(M / 256) * (N / 256), K))
+                    return gemm_rounds_and_rest<OutType>(A, B, C, M, N, K, rounds, stream);
+                return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
             }
             // too few 256 x 256 tiles for the chip, but about one 128 x 128 tile per CU and a long enough K: the
             // kernel whose wavefronts split K (each owns the whole tile)
@@ -567,14 +580,20 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
             if (gemm_narrow_is_the_choice(M, N, K)) return gemm_w128_narrow_dispatch<OutType>(A, B, C, M, N, K, stream);
             if (M % 16 == 0 && N % 16 == 0) {
                 // M or N not multiples of 256: the one-wavefront-per-SIMD kernel with edge tiles, that kernel on the
-                // leading block of whole tiles plus the pipelined kernel on the strips beyond it, or the pipelined kernel
-                // with the tile its cost model picks - whichever is expected to be the shortest
+                // leading block of whole tiles plus the pipelined kernel on the strips beyond it, that kernel on the
+                // rows or columns that fill whole rounds plus smaller tiles on the rest, or the pipelined kernel with the
+                // tile its cost model picks - whichever is expected to be the shortest
                 const long tiles_e = (long)((M + 255) / 256) * ((N + 255) / 256);
                 const double edge_us = K % 64 == 0 && tiles_e >= 128 && (long)K * 512 < (1l << 32)
                                            ? gemm_w128_us(tiles_e, K) : 1e30;
-                const int rc = gemm_main_and_strips<OutType>(A, B, C, M, N, K, stream, edge_us);
+                const GemmRoundsPlan rounds = gemm_rounds_and_rest_plan(M, N, K);
+                const double rounds_us = rounds.us / 0.93;  // (two launches have to promise 7 % over the other plans)
+                const int rc = gemm_main_and_strips<OutType>(A, B, C, M, N, K, stream, std::min(edge_us, rounds_us));
                 if (rc != kPlanNotTaken) return rc;
-                if (edge_us < pipelined_plan(M, N, K).us) return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
+                const double pipelined_us = pipelined_plan(M, N, K).us;
+                if (rounds_us < edge_us && rounds_us < pipelined_us)
+                    return gemm_rounds_and_rest<OutType>(A, B, C, M, N, K, rounds, stream);
+                if (edge_us < pipelined_us) return gemm_w128_dispatch<OutType>(A, B, C, M, N, K, stream);
             }
             // tiny problems: the kernel that takes its operand tiles straight from global memory has the shorter start
             if ((long)M * N < 64 * 64) return gemm_ragged_dispatch<OutType>(A, B, C, M, N, K, stream);
