@@ -376,7 +376,7 @@ int gemm_main_and_strips(const __half* A, const __half* B, OutType* C, int M, in
 bool gemm_w128k_is_the_choice(int M, int N, int K) {
     if (M % 16 != 0 || N % 16 != 0 || K % 128 != 0 || K < 1536 || (long)K * 256 >= (1l << 32)) return false;
     const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-    return tiles >= 128 && tiles <= 256;
+    return tiles >= (K >= 2048 ? 96 : 128) && tiles <= 256;  // (1424 x 1280 x 4096, 120 tiles: 25.6 against 29.2 us)
 }
 
 /// Whether AUTO sends an unsplit product to the 256 x 128 tile: at most 128 tiles of 256 x 256 (half of the chip or
@@ -394,7 +394,7 @@ bool gemm_narrow_is_the_choice(int M, int N, int K) {
 /// Expected time of one launch, in us, of the kernels above where AUTO runs them (measured on whole-chip launches): the
 /// K-splitting kernel 5 us + 0.95 us per 128 of K with 128 x 128 tiles, 0.75 us with 128 x 96 tiles; the 256 x 128 tile
 /// 6 us + per 64 of K 0.70 us with up to 160 tiles, rising to 0.83 us with 256; 256 x 256 tiles 3 us + per 1024 of K
-/// 23.5 us for every full round of 256 workgroups and, for a last round of t, 10.6 + 12.9 t / 256 us (the chip is
+/// 23.5 us for every full round of 256 workgroups and, for a single round of t, 10.6 + 12.9 t / 256 us (the chip is
 /// power-limited: fewer busy CUs run at a higher clock) but not below 17 us (what one workgroup needs by itself).
 double gemm_w128k_us(int M, int N, int K) {
     const long rows = (M + 127) / 128;
@@ -409,10 +409,11 @@ double gemm_narrow_us(int M, int N, int K) {
 
 double gemm_w128_us(long tiles, int K) {
     const long full = (tiles - 1) / 256, last = tiles - 256 * full;
-    // a later round starts unevenly - the XCDs differ by about 4 % - which hides some of a last round that is far from full
+    // a last round behind full ones starts unevenly (the XCDs differ by about 4 %) and runs beside their stragglers:
+    // 13 to 23 us measured, rising with its fill (8192 x 8448, 7168^2, 6144^2, 2560 x 8192, 6976 x 8192)
     const double fill = last / 256.0;
-    const double last_us = std::max(17.0, 10.6 + 12.9 * fill) - 0.04 * 23.5 * full * (1.0 - fill);
-    return 3.0 + (K / 1024.0) * (23.5 * full + std::max(9.0, last_us));
+    const double last_us = full == 0 ? std::max(17.0, 10.6 + 12.9 * fill) : std::min(23.5, 12.0 + 20.0 * fill);
+    return 3.0 + (K / 1024.0) * (23.5 * full + last_us);
 }
 
 /// More than one round of 256 x 256 tiles, the last of them far from full (2560 x 8192: 320 tiles, the last 64 of which
