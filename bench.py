@@ -485,6 +485,32 @@ def main():
                         "ms": ms, "tflops": 2.0 * 2560 * 8192 * 4096 / (ms * 1e-3) / 1e12, "ms_single_launch": ms_1,
                         "hipblaslt_ms": ms_v, "speed_vs_hipblaslt": ms_v / ms})
         del a_, b_, c_
+        if not args.no_vendor:
+            # AUTO on shapes nobody tuned for: 48 seeded random shapes (M, N multiples of 16, 128 or 256 in 512..8192, K from
+            # six values), no workspace; both libraries 40 untimed + 30 timed launches, the better of two passes
+            import random
+            rng = random.Random(20)
+            ratios, worst, best = [], None, None
+            for _ in range(48):
+                pick = lambda: rng.choice([rng.randrange(512, 8193, 16), rng.randrange(512, 8193, 256),
+                                           rng.randrange(512, 4097, 128)])
+                m_, n_, k_ = pick(), pick(), rng.choice([1024, 1536, 2048, 3072, 4096, 8192])
+                a_, b_ = rand16(m_, k_), rand16(n_, k_)
+                c_ = torch.empty(m_, n_, dtype=torch.float16, device=dev)
+                ours = min(time_kernel(lambda: tcu.gemm(a_, b_, out=c_, workspace=False), 30, 40) for _ in range(2))
+                blas = min(time_kernel(lambda: torch.matmul(a_, b_.t(), out=c_), 30, 40) for _ in range(2))
+                ratios.append(blas / ours)
+                if worst is None or ratios[-1] < worst[1]:
+                    worst = ([m_, n_, k_], ratios[-1])
+                if best is None or ratios[-1] > best[1]:
+                    best = ([m_, n_, k_], ratios[-1])
+                del a_, b_, c_
+            configs.append({"name": "gemm_auto_48_random_shapes_vs_hipblaslt",
+                            "geomean_speed_vs_hipblaslt": float(np.exp(np.mean(np.log(ratios)))),
+                            "share_at_or_above_hipblaslt": sum(r >= 1.0 for r in ratios) / len(ratios),
+                            "share_below_0.9": sum(r < 0.9 for r in ratios) / len(ratios),
+                            "slowest_against_it": {"shape": worst[0], "speed_vs_hipblaslt": worst[1]},
+                            "fastest_against_it": {"shape": best[0], "speed_vs_hipblaslt": best[1]}})
         a_ = (torch.randn(8192, 64, device=dev) * 0.1).half()
         b_ = (torch.randn(128, 64, device=dev) * 0.1).half()
         c_ = (torch.randn(64, 128, device=dev) * 0.1).half()
