@@ -35,7 +35,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
 HBM_PEAK_GBS = 8000.0
 # The kernel the headline workload runs on (what tcu.gemm(..., algo="auto") dispatches to at 4096^3) and the committed
 # rocprofv3 summary that holds its measured HBM-side traffic.
-GEMM_4096_KERNEL = "gemm_w128<__half, tiledcuda::kernels::GemmW128TraitsN<8> >"
+GEMM_4096_KERNEL = "gemm_w128<__half, tiledcuda::kernels::GemmW128TraitsN<8>, false>"
 GEMM_4096_PROFILE = os.path.join(ROOT, "profiles", "gemm_w128_f16_4096x4096x4096.md")
 
 
