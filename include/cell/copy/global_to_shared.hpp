@@ -22,7 +22,8 @@ namespace detail {
 /// Per-wavefront line-by-line copy between a pitched global block and a shared tile view.
 /// The block is kLines lines of kLineLen contiguous elements, starting at line `line0`,
 /// element `elem0` of both tiles. kToShared selects the direction.
-template <typename Global, typename Shared, const int kLines, const int kLineLen, const bool kToShared>
+template <typename Global, typename Shared, const int kLines, const int kLineLen, const bool kToShared,
+          const bool kStream = false>
 struct LineCopy {
     using DType = typename Shared::DType;
     static constexpr int kVec = TraitsBase<DType>::kNumPerAccess;  // 8 x f16 or 4 x f32 = 16 B
@@ -52,7 +53,8 @@ struct LineCopy {
                 } else {
                     DType tmp[kVec];
                     vec_load<kVec>(s, tmp);
-                    vec_store<kVec>(tmp, const_cast<DType*>(g));
+                    if constexpr (kStream) vec_store_stream<kVec>(tmp, const_cast<DType*>(g));
+                    else vec_store<kVec>(tmp, const_cast<DType*>(g));
                 }
             }
         }
@@ -100,8 +102,10 @@ struct GlobalToSharedLoader : public Base {
     }
 };
 
-/// Copy a shared tile into a global tile of the same shape.
-template <typename Shared_, typename WarpLayout_, typename Base = warp::CopyBase<WarpLayout_, WarpReuse::kCont>>
+/// Copy a shared tile into a global tile of the same shape. kStream: with non-temporal stores (an output that the
+/// kernel does not read again: nothing stays dirty in the L2 for the write-back at the kernel's end).
+template <typename Shared_, typename WarpLayout_, typename Base = warp::CopyBase<WarpLayout_, WarpReuse::kCont>,
+          const bool kStream = false>
 struct SharedToGlobalStorer : public Base {
     using Shared = Shared_;
     using DType = typename Shared::DType;
@@ -120,13 +124,18 @@ struct SharedToGlobalStorer : public Base {
         const int col0 = Base::template warp_col0<Shared::kCols>();
 
         if constexpr (Shared::kIsRowMajor) {
-            detail::LineCopy<Global, Shared, kBlockRows, kBlockCols, false> copy;
+            detail::LineCopy<Global, Shared, kBlockRows, kBlockCols, false, kStream> copy;
             copy(dst.mutable_data(), src, row0, col0);
         } else {
-            detail::LineCopy<Global, Shared, kBlockCols, kBlockRows, false> copy;
+            detail::LineCopy<Global, Shared, kBlockCols, kBlockRows, false, kStream> copy;
             copy(dst.mutable_data(), src, col0, row0);
         }
     }
 };
+
+/// SharedToGlobalStorer with non-temporal stores.
+template <typename Shared_, typename WarpLayout_>
+using SharedToGlobalStreamStorer =
+    SharedToGlobalStorer<Shared_, WarpLayout_, warp::CopyBase<WarpLayout_, WarpReuse::kCont>, true>;
 
 }  // namespace tiledcuda::cell::copy

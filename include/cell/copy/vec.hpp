@@ -34,4 +34,14 @@ DEVICE void vec_store(const T* src, T* dst) {
     *reinterpret_cast<V*>(dst) = v;
 }
 
+/// The same with a non-temporal store: the data is streamed to memory instead of staying dirty in the XCD's L2 until
+/// the kernel's end (whole lines written by neighbouring lanes only: pieces of lines are better gathered by the L2).
+template <int kN, typename T>
+DEVICE void vec_store_stream(const T* src, T* dst) {
+    using V = typename VecOf<kN * sizeof(T)>::type;
+    V v;
+    __builtin_memcpy(&v, src, sizeof(V));
+    __builtin_nontemporal_store(v, reinterpret_cast<V*>(dst));
+}
+
 }  // namespace tiledcuda::cell::copy

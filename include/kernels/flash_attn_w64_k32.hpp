@@ -123,7 +123,7 @@ struct FlashW64K32Traits {
     using Scores = compute::ScheduledGemm<RegQ, RegK, RegS, compute::RegFile::kVgpr, compute::RegFile::kAgpr>;
     using Output = compute::ScheduledGemm<RegP, RegV, RegO, compute::RegFile::kAgpr, compute::RegFile::kVgpr>;
     using OutToShared = RegToSharedStorer<RegOut, WarpLayout>;
-    using OutToGlobal = SharedToGlobalStorer<SharedO, WarpLayout>;
+    using OutToGlobal = SharedToGlobalStreamStorer<SharedO, WarpLayout>;
     static constexpr int kLoadsK = PiecesK::kPieces;  // of a wavefront, per block: then as many of V
     static_assert(2 * kLoadsK == kGroups && PiecesV::kPieces == (kVColMajor ? kLoadsK / 2 : kLoadsK),
                   "a wavefront issues one load per group of the step that loads a block");

@@ -77,7 +77,10 @@ __global__ void __launch_bounds__(256)
             if constexpr (kVec == 1) {
                 *dst = *src;
             } else {
-                *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src);
+                // streamed both ways: nothing here is touched twice, and lines left dirty in the L2s would be written
+                // back after the last wavefront (65536 rows of 4 KiB: 103.5 -> 99.8 us, a plain device copy takes 99.2)
+                __builtin_nontemporal_store(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src)),
+                                            reinterpret_cast<u32x4*>(dst));
             }
         } else {
             static_assert(kMode == ScatterMode::kAssign || kVec == 1, "atomic add is per element");
