@@ -35,7 +35,7 @@ template <bool kRowMajor, int kRows, int kCols>
 using LayoutOf = std::conditional_t<kRowMajor, tl::RowMajor<kRows, kCols>, tl::ColMajor<kRows, kCols>>;
 
 // ------------------------------------------------------------------ global -> shared -> global
-template <typename Element, bool kRowMajor, int kRows, int kCols, typename WarpLayout, bool kSwizzled>
+template <typename Element, bool kRowMajor, int kRows, int kCols, typename WarpLayout, bool kSwizzled, bool kStream = false>
 __global__ void __launch_bounds__(512) k_g2s_roundtrip(const Element* src, Element* dst) {
     extern __shared__ __align__(16) unsigned char buf[];
     auto* smem = reinterpret_cast<Element*>(buf);
@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(512) k_g2s_roundtrip(const Element* src, Eleme
     Global g_dst(dst);
     Shared s(smem);
     GlobalToSharedLoader<Shared, WarpLayout> loader;
-    SharedToGlobalStorer<Shared, WarpLayout> storer;
+    std::conditional_t<kStream, SharedToGlobalStreamStorer<Shared, WarpLayout>, SharedToGlobalStorer<Shared, WarpLayout>> storer;
     loader(g_src, s);
     __copy_async();
     __syncthreads();
@@ -890,17 +890,17 @@ constexpr const char* ename() {
     return sizeof(E) == 2 ? "f16" : "f32";
 }
 
-template <typename E, bool kRowMajor, int kRows, int kCols, int kWR, int kWC, bool kSwz>
+template <typename E, bool kRowMajor, int kRows, int kCols, int kWR, int kWC, bool kSwz, bool kStream = false>
 void reg_g2s() {
     using W = tl::RowMajor<kWR, kWC>;
     registry().push_back({"g2s_roundtrip",
                           std::string(ename<E>()) + (kRowMajor ? "_row_" : "_col_") + std::to_string(kRows) + "x" +
                               std::to_string(kCols) + "_w" + std::to_string(kWR) + "x" + std::to_string(kWC) +
-                              (kSwz ? "_swz" : "_plain"),
+                              (kSwz ? "_swz" : "_plain") + (kStream ? "_stream_storer" : ""),
                           {kRows, kCols, 0, int(sizeof(E)), kRowMajor, 0, 0, 0},
                           kWR * kWC * 64,
                           int(kRows * kCols * sizeof(E)),
-                          &launch2<k_g2s_roundtrip<E, kRowMajor, kRows, kCols, W, kSwz>, E>});
+                          &launch2<k_g2s_roundtrip<E, kRowMajor, kRows, kCols, W, kSwz, kStream>, E>});
 }
 
 template <typename E, bool kRowMajor, int kRows, int kCols, int kChunk, int kWR, int kWC, bool kSwz>
@@ -1064,6 +1064,8 @@ void reg_g2s_family() {
     reg_g2s<E, true, 32, 32, 2, 2, kSwz>();
     reg_g2s<E, true, 64, 64, 2, 2, kSwz>();
     reg_g2s<E, true, 96, 128, 2, 4, kSwz>();
+    reg_g2s<E, true, 96, 128, 2, 4, kSwz, true>();  // ... leaving through SharedToGlobalStreamStorer
+    reg_g2s<E, false, 128, 96, 2, 2, kSwz, true>();
     reg_g2s<E, true, 192, 32, 2, 2, kSwz>();
     reg_g2s<E, false, 16, 16, 1, 1, kSwz>();
     reg_g2s<E, false, 64, 16, 4, 1, kSwz>();
