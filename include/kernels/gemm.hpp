@@ -402,7 +402,7 @@ struct ScheduledGemmTileTraits {
     using SharedC = SharedTile<OutType, tl::RowMajor<kTM, kTN>, true>;
     using GlobalC = GlobalTile<OutType, tl::RowMajor<kTM, kTN, kN>>;
     using R2SStorerC = RegToSharedStorer<RegC, WarpLayout>;
-    using S2GStorerC = SharedToGlobalStorer<SharedC, WarpLayout>;
+    using S2GStorerC = SharedToGlobalStreamStorer<SharedC, WarpLayout>;  // whole rows, never read again: streamed out
 
     static constexpr int kShmInput = RingA::kBytes + RingB::kBytes;
     static constexpr int kShmOutput = sizeof(OutType) == 2 ? kTM * kTN * int(sizeof(OutType)) : 0;
