@@ -329,15 +329,10 @@ __global__ void __launch_bounds__(T::kThreads)
 #pragma unroll
     for (int i = 0; i < 8; ++i) pin_row(acc[i]);
 
-    // f16 C leaves through non-temporal stores: the XCDs' L2s are not coherent with each other, so whatever a kernel
-    // leaves dirty in them is written back when it ends, after the last wavefront - whole lines streamed out while
-    // others still compute are not (4096^3: -1.5 %, 4096 x 4096 x 1024: -3.5 %). Not the f32 output: its stores are
-    // 16-byte pieces of 16 different rows per instruction, which the L2 has to gather into lines (+4 ... +19 % when
-    // streamed).
-    auto store_c = [](auto* p, const auto& v) {
-        if constexpr (sizeof(OutType) == 2) __builtin_nontemporal_store(v, p);
-        else *p = v;
-    };
+    // C leaves through non-temporal stores of whole rows: the XCDs' L2s are not coherent with each other, so whatever a
+    // kernel leaves dirty in them is written back when it ends, after the last wavefront - lines streamed out while
+    // others still compute are not (f16, 4096^3: -1.5 %, 4096 x 4096 x 1024: -3.5 %)
+    auto store_c = [](auto* p, const auto& v) { __builtin_nontemporal_store(v, p); };
     // ---- epilogue: acc[i][j][e] = C[16 i + lane % 16][16 j + 4 (lane / 16) + e] of the wavefront's block
     if constexpr (sizeof(OutType) == 2) {
         // f16: 16 rows at a time through a private LDS buffer (beyond the operand stages, so no workgroup barrier),
@@ -389,13 +384,47 @@ __global__ void __launch_bounds__(T::kThreads)
             }
         }
     } else {
+        // f32: the same through one buffer of 16 rows (512 or 256 bytes each: the 16-byte slots of a row XOR-ed with the
+        // row, so that the 16 rows a write instruction touches fall into different banks) - an accumulator register
+        // holds 4 columns of 16 different rows, and 16-byte pieces of 16 rows per store instruction are what the
+        // memory side handles worst
+        constexpr int kPitch = T::kWaveN * 4;
+        constexpr int kLanesPerRow = kPitch / 16, kRowsPerRead = kWaveSize / kLanesPerRow, kReads = 16 / kRowsPerRead;
+        static_assert(16 * kPitch <= T::kEpilogueBytesPerWave);
+        const unsigned int stg_base =
+            static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds + T::kLdsBytesMain + wave * T::kEpilogueBytesPerWave));
+        const int rr = lane / kLanesPerRow, cc = lane % kLanesPerRow;
+        unsigned int waddr[kNT], raddr[kReads];
+#pragma unroll
+        for (int j = 0; j < kNT; ++j) {
+            waddr[j] = stg_base + frow * kPitch + ((j * 4 + fquad) ^ frow) * 16;
+            asm volatile("" : "+v"(waddr[j]));
+        }
+#pragma unroll
+        for (int it = 0; it < kReads; ++it) {
+            const int row = it * kRowsPerRead + rr;
+            raddr[it] = stg_base + row * kPitch + (cc ^ row) * 16;
+            asm volatile("" : "+v"(raddr[it]));
+        }
+        using lds_f32x4_ptr = __attribute__((address_space(3))) f32x4*;
+        using lds_u32x4_ptr = __attribute__((address_space(3))) const u32x4*;
         OutType* cbase = C + size_t(m0 + wave_m * T::kWaveM) * ldc + n0 + wave_n * T::kWaveN;
+        unsigned char* crow = reinterpret_cast<unsigned char*>(cbase + size_t(rr) * ldc) + cc * 16;
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < 8; ++i) {
 #pragma unroll
-            for (int j = 0; j < kNT; ++j)
-                if (!kEdges || (m0 + wave_m * T::kWaveM + i * 16 + frow < M && n0 + wave_n * T::kWaveN + j * 16 + 4 * fquad < N))
-                    store_c(reinterpret_cast<f32x4*>(cbase + size_t(i * 16 + frow) * ldc + j * 16 + 4 * fquad), acc[i][j]);
+            for (int j = 0; j < kNT; ++j) *reinterpret_cast<lds_f32x4_ptr>(waddr[j]) = acc[i][j];
+            // LDS operations of one wavefront execute in order: the reads see the writes above, and the next group's
+            // writes come behind them
+#pragma unroll
+            for (int it = 0; it < kReads; ++it) {
+                const u32x4 v = *reinterpret_cast<lds_u32x4_ptr>(raddr[it]);
+                if (!kEdges || (m0 + wave_m * T::kWaveM + i * 16 + it * kRowsPerRead + rr < M &&
+                                n0 + wave_n * T::kWaveN + cc * 4 < N))
+                    __builtin_nontemporal_store(
+                        v, reinterpret_cast<u32x4*>(crow + size_t(i * 16 + it * kRowsPerRead) * ldc * sizeof(OutType)));
+            }
+        }
     }
 }
 
