@@ -222,24 +222,57 @@ __global__ void __launch_bounds__(T::kThreads)
         }
     }
 
-    // ---- store: res[r][jj][e] = C[32 r + 16 (w / 2) + lane % 16][16 (kMine (w % 2) + jj) + 4 (lane / 16) + e] of the tile
-    OutType* cbase = C + size_t(m0 + 16 * (wave >> 1) + frow) * ldc + n0 + 16 * kMine * (wave & 1) + 4 * fquad;
+    // ---- store: res[r][jj][e] = C[32 r + 16 (w / 2) + lane % 16][16 (kMine (w % 2) + jj) + 4 (lane / 16) + e] of the tile.
+    // f16: the 16 rows of a round pass through 2 KiB of LDS of this wavefront's own (beyond the two reduction buffers; the
+    // 8-byte slots of a row XOR-ed with twice the row) and leave as whole rows of 16 kMine elements through non-temporal
+    // stores, 16 bytes per lane: 8-byte pieces of lines would have to be gathered by the L2, and lines left dirty there
+    // are written back after the kernel's last wavefront.
+    if constexpr (sizeof(OutType) == 2) {
+        constexpr int kPitch = 16 * kMine * 2;                     // bytes per staged row: 128 (96)
+        constexpr int kSlots = kPitch / 8;                         // 8-byte slots per row: 16 (12)
+        constexpr int kChunks = kPitch / 16;                       // 16-byte pieces per row: 8 (6)
+        constexpr int kPieces = 16 * kChunks;                      // per round: 128 (96)
+        const unsigned int stg = lds_base + 128 * 1024 + wave * 2048;
+        using lds_f16x4_ptr = __attribute__((address_space(3))) f16x4*;
+        using lds_u32x4_ptr = __attribute__((address_space(3))) const u32x4*;
+        // slot s of row q lies at slot s ^ (2 q % 16) where that stays inside the row (kSlots = 16), else unpermuted
+        auto slot_of = [](int q, int s) { return kSlots == 16 ? s ^ ((2 * q) & 15) : s; };
+        OutType* cblock = C + size_t(m0 + 16 * (wave >> 1)) * ldc + n0 + 16 * kMine * (wave & 1);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+        for (int r = 0; r < 4; ++r) {
 #pragma unroll
-        for (int jj = 0; jj < kMine; ++jj) {
-            OutType* p = cbase + size_t(32 * r) * ldc + 16 * jj;
-            if constexpr (kEdges) {
-                // M and N are multiples of 16: a 16 x 16 block lies inside the matrix or outside it as a whole
-                if (m0 + 32 * r + 16 * (wave >> 1) >= M || n0 + 16 * kMine * (wave & 1) + 16 * jj >= N) continue;
-            }
-            if constexpr (sizeof(OutType) == 4) {
-                *reinterpret_cast<f32x4*>(p) = res[r][jj];
-            } else {
+            for (int jj = 0; jj < kMine; ++jj) {
                 f16x4 h;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(res[r][jj][e]);
-                *reinterpret_cast<f16x4*>(p) = h;
+                *reinterpret_cast<lds_f16x4_ptr>(stg + frow * kPitch + slot_of(frow, 4 * jj + fquad) * 8) = h;
+            }
+            // LDS operations of one wavefront execute in order: the reads see the writes above
+#pragma unroll
+            for (int it = 0; it < (kPieces + kWaveSize - 1) / kWaveSize; ++it) {
+                const int piece = it * kWaveSize + lane;
+                const int q = piece / kChunks, c = piece % kChunks;
+                if (kPieces % kWaveSize != 0 && piece >= kPieces) continue;
+                const u32x4 v = *reinterpret_cast<lds_u32x4_ptr>(stg + q * kPitch + slot_of(q, 2 * c) * 8);
+                if constexpr (kEdges) {
+                    // M and N are multiples of 16: a 16-byte piece lies inside the matrix or outside it as a whole
+                    if (m0 + 32 * r + 16 * (wave >> 1) + q >= M || n0 + 16 * kMine * (wave & 1) + 8 * c >= N) continue;
+                }
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(cblock + size_t(32 * r + q) * ldc + 8 * c));
+            }
+        }
+    } else {
+        OutType* cbase = C + size_t(m0 + 16 * (wave >> 1) + frow) * ldc + n0 + 16 * kMine * (wave & 1) + 4 * fquad;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+#pragma unroll
+            for (int jj = 0; jj < kMine; ++jj) {
+                OutType* p = cbase + size_t(32 * r) * ldc + 16 * jj;
+                if constexpr (kEdges) {
+                    // M and N are multiples of 16: a 16 x 16 block lies inside the matrix or outside it as a whole
+                    if (m0 + 32 * r + 16 * (wave >> 1) >= M || n0 + 16 * kMine * (wave & 1) + 16 * jj >= N) continue;
+                }
+                *reinterpret_cast<f32x4*>(p) = res[r][jj];
             }
         }
     }
