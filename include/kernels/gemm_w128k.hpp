@@ -262,17 +262,28 @@ __global__ void __launch_bounds__(T::kThreads)
             }
         }
     } else {
-        OutType* cbase = C + size_t(m0 + 16 * (wave >> 1) + frow) * ldc + n0 + 16 * kMine * (wave & 1) + 4 * fquad;
+        // f32 (also the partial products of a split-K launch): the same with 16-byte slots, 4 KiB per wavefront
+        constexpr int kPitch = 16 * kMine * 4;                     // bytes per staged row: 256 (192)
+        constexpr int kChunks = kPitch / 16;                       // 16-byte pieces per row: 16 (12)
+        constexpr int kPieces = 16 * kChunks;                      // per round: 256 (192)
+        const unsigned int stg = lds_base + 128 * 1024 + wave * 4096;
+        using lds_u32x4_ptr = __attribute__((address_space(3))) const u32x4*;
+        auto slot_of = [](int q, int s) { return kChunks == 16 ? s ^ q : s; };
+        OutType* cblock = C + size_t(m0 + 16 * (wave >> 1)) * ldc + n0 + 16 * kMine * (wave & 1);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
 #pragma unroll
-            for (int jj = 0; jj < kMine; ++jj) {
-                OutType* p = cbase + size_t(32 * r) * ldc + 16 * jj;
+            for (int jj = 0; jj < kMine; ++jj)
+                *reinterpret_cast<lds_f32x4_ptr>(stg + frow * kPitch + slot_of(frow, 4 * jj + fquad) * 16) = res[r][jj];
+#pragma unroll
+            for (int it = 0; it < kPieces / kWaveSize; ++it) {
+                const int piece = it * kWaveSize + lane;
+                const int q = piece / kChunks, c = piece % kChunks;
+                const u32x4 v = *reinterpret_cast<lds_u32x4_ptr>(stg + q * kPitch + slot_of(q, c) * 16);
                 if constexpr (kEdges) {
-                    // M and N are multiples of 16: a 16 x 16 block lies inside the matrix or outside it as a whole
-                    if (m0 + 32 * r + 16 * (wave >> 1) >= M || n0 + 16 * kMine * (wave & 1) + 16 * jj >= N) continue;
+                    if (m0 + 32 * r + 16 * (wave >> 1) + q >= M || n0 + 16 * kMine * (wave & 1) + 4 * c >= N) continue;
                 }
-                *reinterpret_cast<f32x4*>(p) = res[r][jj];
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(cblock + size_t(32 * r + q) * ldc + 4 * c));
             }
         }
     }
