@@ -174,7 +174,8 @@ using PipeSmallRing = PipelinedGemmTraits<64, 64, 64, 2, 2, 4>;  // 4-stage ring
 /// and a round costs K / 1024 x 25.5, 16 or 13 us for 256 x 256, 128 x 128 and 64 x 64 tiles (measured on full rounds at
 /// K = 1024 .. 4096); the larger tile wins a tie. With few 64 x 64 tiles per CU there is no neighbour workgroup to hide
 /// the latency of a tile's loads behind: then the same tile with a 4-stage ring (3 tiles in flight, 2 workgroups per
-/// CU) is the choice: 3.75 us per K / 1024 with at most one workgroup per CU, 5.8 with two, 7 per round beyond.
+/// CU) is the choice: 4.2 us per K / 1024 with at most one workgroup per CU (1024^2 x 8192: 36.7 us), 5.8 with two, 7 per
+/// round beyond.
 enum PipeConfig { kPipeLarge, kPipeMid, kPipeSmall, kPipeSmallRing };
 struct PipePlan {
     PipeConfig config;
@@ -184,7 +185,7 @@ PipePlan pipelined_plan(int M, int N, int K) {
     const auto tiles = [&](int tile) { return (long)((M + tile - 1) / tile) * ((N + tile - 1) / tile); };
     const auto rounds = [&](int tile, int per_cu) { return double((tiles(tile) + 256l * per_cu - 1) / (256l * per_cu)); };
     const double large = rounds(256, 1) * 25.5, mid = rounds(128, 2) * 16.0, small = rounds(64, 4) * 13.0;
-    const double ring = tiles(64) <= 256 ? 3.75 : tiles(64) <= 512 ? 5.8 : rounds(64, 2) * 7.0;
+    const double ring = tiles(64) <= 256 ? 4.2 : tiles(64) <= 512 ? 5.8 : rounds(64, 2) * 7.0;
     const double least_small = small < ring ? small : ring;
     PipePlan plan;
     if (large <= mid && large <= least_small) plan = {kPipeLarge, large};
@@ -497,14 +498,14 @@ GemmSplitPlan gemm_split_plan(int M, int N, int K) {
             best_us = us;
         }
     }
-    // partial products from the kernel whose wavefronts split K inside the workgroup: 11.5 us for the two launches, the
+    // partial products from the kernel whose wavefronts split K inside the workgroup: 8 us for the two launches, the
     // reduction through LDS and the epilogues + per 128 of a range 0.62 us with up to 128 workgroups, rising to 0.95 us
     // with 256 (their loads share the L2s) - measured on 256^2 x 8192 ... 1024 x 2048 x 16384 with 2 to 16 ranges
     if ((long)K * 256 < (1l << 32)) {
         for (int s = 2; s * tiles * 4 <= 256 && K % (s * 128) == 0 && K / s >= 512; s *= 2) {
             const long groups = s * tiles * 4;
             const double per_tile = 0.62 + 0.33 * (groups > 128 ? double(groups - 128) / 128.0 : 0.0);
-            const double us = 11.5 + per_tile * (K / s / 128) + s * plane_us;
+            const double us = 8.0 + per_tile * (K / s / 128) + s * plane_us;
             if (us < best_us) {
                 plan = {s, true};
                 best_us = us;
