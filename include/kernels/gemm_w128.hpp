@@ -123,7 +123,9 @@ __global__ void __launch_bounds__(256) splitk_reduce(const float* __restrict__ p
 /// synchronisation words of a kernel that follows this one on the stream, cleared without a launch of their own.
 /// kEdges: M and N need not be multiples of the tile (multiples of 16 suffice): the grid covers ceil(M / 256) x
 /// ceil(N / kBN) tiles, rows beyond the edge are loaded from the last valid row (their products are computed and
-/// dropped) and the stores are guarded. Nothing changes inside the loop over K.
+/// dropped) and the stores are guarded. With 256 x 256 tiles K may be any multiple of 16 as well: the loop runs over
+/// ceil(K / 64) tiles and the pieces of the last one beyond K are zeros in LDS. Nothing changes inside the loop over K
+/// but for its last three tiles.
 template <typename OutType, typename T = GemmW128Traits, bool kEdges = false>
 __global__ void __launch_bounds__(T::kThreads)
     gemm_w128(const __half* __restrict__ A, const __half* __restrict__ Bt, OutType* __restrict__ C, int M, int N, int K,
@@ -169,7 +171,23 @@ __global__ void __launch_bounds__(T::kThreads)
     // (its workgroups stay in step with each other, which is what makes its L2 work): 7-14 % at K = 16384, nothing at
     // smaller K. The sum over K is then taken in rotated order: the same value on every run, but not bit for bit the
     // in-order sum of the other kernels (f32 rounding).
-    const int ktiles = K / T::kBK;
+    // K a multiple of 16 (two-stage form with edge tiles only): the last tile of K is partial. Its 16-byte pieces that lie
+    // beyond K are fetched from the row's first piece of that tile instead (tail_back[p]: how far back that is for loads of
+    // parity p, 0 for pieces inside K) and overwritten with zeros in LDS once they have landed.
+    constexpr bool kTail = kEdges && T::kStages == 2;
+    const int ktiles = kTail ? (K + T::kBK - 1) / T::kBK : K / T::kBK;
+    const int tail_pieces = kTail ? (K % T::kBK) / 8 : 0;  // 0: K is whole tiles
+    unsigned int tail_back[2] = {0u, 0u};
+    if constexpr (kTail) {
+        if (tail_pieces != 0) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int piece = lchk ^ ((4 * p + (lrow >> 1)) & 7);  // logical piece this lane fetches in loads of parity p
+                tail_back[p] = piece >= tail_pieces ? piece * 16u : 0u;
+            }
+        }
+    }
+    auto tail_voff = [&](int q) { return voff[q] - tail_back[q & 1]; };
     const int k_start = __builtin_amdgcn_readfirstlane(
         ((lda | ldb) & 16383) == 0 && ktiles >= 64 ? int(blockIdx.x & 7) * (ktiles / 8) : 0);
     auto load_src = [&](int kt, int q) -> const __half* {
@@ -198,10 +216,12 @@ __global__ void __launch_bounds__(T::kThreads)
             for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(clamped(st), q), load_dst(st, q));
     } else {
 #pragma unroll
-        for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(0, q), load_dst(0, q));
+        for (int q = 0; q < kNumLoads; ++q)
+            detail::load_lds_16B_sbase(kTail && ktiles == 1 ? tail_voff(q) : voff[q], load_src(0, q), load_dst(0, q));
         if (ktiles > 1) {
 #pragma unroll
-            for (int q = 0; q < kNumLoads; ++q) detail::load_lds_16B_sbase(voff[q], load_src(1, q), load_dst(1, q));
+            for (int q = 0; q < kNumLoads; ++q)
+                detail::load_lds_16B_sbase(kTail && ktiles == 2 ? tail_voff(q) : voff[q], load_src(1, q), load_dst(1, q));
         }
     }
     // the 256 accumulators are cleared while the first tiles are on their way (the empty asm statements keep the
@@ -221,9 +241,24 @@ __global__ void __launch_bounds__(T::kThreads)
         pin_row(acc[i]);
     }
     // this wavefront's part of tile 0 has landed; then everyone's
-    if constexpr (T::kStages == 3) detail::lds_barrier<2 * kNumLoads>();
-    else if (ktiles > 1) detail::lds_barrier<kNumLoads>();
-    else detail::lds_barrier<0>();
+    // the pieces of a partial last tile that lie beyond K: zeros, once the loads into `stage` have landed
+    auto zero_tail = [&](int stage) {
+        using lds_u32x4_ptr = __attribute__((address_space(3))) u32x4*;
+#pragma unroll
+        for (int q = 0; q < kNumLoads; ++q)
+            if (tail_back[q & 1] != 0u) *reinterpret_cast<lds_u32x4_ptr>(load_dst(stage, q) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    };
+    if constexpr (T::kStages == 3) {
+        detail::lds_barrier<2 * kNumLoads>();
+    } else if (ktiles > 1) {
+        detail::lds_barrier<kNumLoads>();
+    } else {
+        if (kTail && tail_pieces != 0) {
+            detail::wait_vmcnt<0>();
+            zero_tail(0);
+        }
+        detail::lds_barrier<0>();
+    }
 #pragma unroll
     for (int r = 0; r < kFrags; ++r) fx[r] = read_frag(0, 0, r);
 
@@ -236,8 +271,10 @@ __global__ void __launch_bounds__(T::kThreads)
     // One tile of K. kMore: there is a tile kt+1 (read its substep 0 during phase 2); kMore2: there is a tile kt+2
     // (load it during phase 2). Row group i = MFMA tiles (i, 0..7): the MFMA order is fixed by the asm statements, the
     // fragment reads (plain loads) are written where they should issue and the compiler keeps them there.
-    auto tile = [&](int kt, auto more_c, auto more2_c) {
+    // kTailLoads: the tile loaded here is the last one and may be partial.
+    auto tile = [&](int kt, auto more_c, auto more2_c, auto tail_loads_c) {
         constexpr bool kMore = decltype(more_c)::value, kMore2 = decltype(more2_c)::value;
+        constexpr bool kTailLoads = decltype(tail_loads_c)::value;
         const int stage = kt & 1;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -250,6 +287,12 @@ __global__ void __launch_bounds__(T::kThreads)
             }
         }
         // this wavefront's part of tile kt+1 has landed and its reads of `stage` are done; then everyone's
+        if constexpr (kTail && kMore && !kMore2) {  // tile kt+1 is the last one
+            if (tail_pieces != 0) {
+                detail::wait_vmcnt<0>();
+                zero_tail(stage ^ 1);
+            }
+        }
         detail::lds_barrier<0>();
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -263,8 +306,8 @@ __global__ void __launch_bounds__(T::kThreads)
                 const int q = kNT == 8 ? 2 * i + (n >> 2) : (3 * m) / 8;
                 const bool load_here = kNT == 8 ? (n & 3) == 1 : (3 * m) % 8 < 3;
                 if (kMore2 && load_here && q < kNumLoads) {
-                    detail::mfma_16x16x32_agpr_then_load(acc[i][j], fy[8 + j], fy[i], voff[q], load_src(kt + 2, q),
-                                                         load_dst(stage, q));
+                    detail::mfma_16x16x32_agpr_then_load(acc[i][j], fy[8 + j], fy[i], kTailLoads ? tail_voff(q) : voff[q],
+                                                         load_src(kt + 2, q), load_dst(stage, q));
                 } else {
                     detail::mfma_16x16x32_agpr(acc[i][j], fy[8 + j], fy[i]);
                 }
@@ -315,12 +358,18 @@ __global__ void __launch_bounds__(T::kThreads)
         detail::wait_vmcnt<0>();  // (the last loads, of data nobody uses, have landed before the workgroup ends)
     } else {
         int kt = 0;
-        for (; kt + 2 < ktiles; ++kt) tile(kt, std::true_type{}, std::true_type{});
+        for (; kt + (kTail ? 3 : 2) < ktiles; ++kt) tile(kt, std::true_type{}, std::true_type{}, std::false_type{});
+        if constexpr (kTail) {  // the iteration that loads the last tile: with the offsets of a partial one
+            if (kt + 2 < ktiles) {
+                tile(kt, std::true_type{}, std::true_type{}, std::true_type{});
+                ++kt;
+            }
+        }
         if (kt + 1 < ktiles) {
-            tile(kt, std::true_type{}, std::false_type{});
+            tile(kt, std::true_type{}, std::false_type{}, std::false_type{});
             ++kt;
         }
-        tile(kt, std::false_type{}, std::false_type{});
+        tile(kt, std::false_type{}, std::false_type{}, std::false_type{});
     }
 
     // the compiler does not know the statements above are MFMAs: wait once for the last results, then pass every

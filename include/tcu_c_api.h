@@ -44,8 +44,8 @@ typedef enum {
                                 workgroups a launch takes; edge tiles (rows clamped, stores guarded, k tail zeroed in
                                 LDS) where the shape is not whole tiles */
     TCU_GEMM_WAVE128 = 4,    /* same pipeline, 256 x 256 tile on 4 wavefronts (one per SIMD, 128 x 128 each),
-                                accumulators in AGPRs; M and N multiples of 16 (edge tiles: rows clamped, stores
-                                guarded), K % 64 == 0; results identical to PIPELINED bit for bit, except where K is a
+                                accumulators in AGPRs; M, N and K multiples of 16 (edge tiles: rows clamped, stores
+                                guarded, a partial last tile of K zero-filled in LDS); results identical to PIPELINED bit for bit, except where K is a
                                 multiple of 16384 (rows a multiple of 32 KiB apart): there each XCD sums over K in
                                 rotated order, which differs by f32 rounding */
     TCU_GEMM_TILE_PIPELINED = 5, /* the PIPELINED kernel composed from tile-library functors only (direct-to-LDS loader,

@@ -125,8 +125,8 @@ def test_unsupported_shapes_are_reported_not_launched(tcu):
     assert l.tcu_gemm_f16(p, p, p, 64, 72, 64, 0, 6, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # whole 16 x 16 tiles only
     assert l.tcu_gemm_f16(p, p, p, 64, 64, 40, 0, 0, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_gemm_f16(p, p, p, 256, 256, 256, 0, 1, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
-    assert l.tcu_gemm_f16(p, p, p, 128, 256, 96, 0, 4, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # one wavefront per SIMD: K % 64
-    assert l.tcu_gemm_f16(p, p, p, 120, 256, 64, 0, 4, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # ... and M, N % 16 (edge tiles)
+    assert l.tcu_gemm_f16(p, p, p, 128, 256, 40, 0, 4, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # one wavefront per SIMD: M, N, K % 16
+    assert l.tcu_gemm_f16(p, p, p, 120, 256, 64, 0, 4, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE
     assert l.tcu_gemm_f16(p, p, p, 512, 512, 512, 0, 7, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # tile-API kernels: fixed shapes
     assert l.tcu_gemm_f16(p, p, p, 256, 256, 192, 0, 8, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # K-splitting kernel: K % 128
     assert l.tcu_gemm_f16(p, p, p, 200, 256, 256, 0, 8, 0) == tcu.TCU_ERR_UNSUPPORTED_SHAPE  # ... and M, N % 16 (edge tiles)

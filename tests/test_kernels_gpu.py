@@ -258,19 +258,23 @@ def test_gemm_main_block_and_strips(tcu, oracle, device, M, N, K, out_dtype):
 def test_gemm_wave128_rejects_other_shapes(tcu, device):
     import torch
 
-    A = torch.zeros(128, 96, dtype=torch.float16, device=device)  # K must be a multiple of 64
+    A = torch.zeros(128, 40, dtype=torch.float16, device=device)  # K must be a multiple of 16
     with pytest.raises(RuntimeError):
         tcu.gemm(A, A, algo="wave128")
 
 
 @pytest.mark.parametrize("M,N,K", [(16, 16, 64), (272, 400, 128), (1040, 528, 192), (4112, 272, 64), (240, 4112, 320),
-                                   (3088, 3088, 256)])
+                                   (3088, 3088, 256), (256, 256, 48), (256, 512, 80), (512, 768, 144), (1040, 528, 272),
+                                   (272, 400, 16), (2064, 2320, 1072), (3600, 3600, 1200)])
 @pytest.mark.parametrize("out_dtype", ["f16", "f32"])
 def test_gemm_wave128_edge_tiles(tcu, oracle, device, M, N, K, out_dtype):
     """The one-wavefront-per-SIMD kernel on shapes that are not whole 256 x 256 tiles (M, N in multiples of 16): rows
     beyond the edge are fetched from the last valid row and their results dropped, the stores are guarded - a single
     partial tile, edges in M, in N and in both, a tile row and a tile column that are 16 wide; against the oracle, bit
-    for bit against the pipelined kernel, with guard rows around C. 3088 x 3088 is a shape AUTO sends to it (169 tiles in one round)."""
+    for bit against the pipelined kernel, with guard rows around C. 3088 x 3088 is a shape AUTO sends to it (169 tiles in one
+    round). The last seven shapes have a K that is not whole tiles of 64 (tails of 16, 32 and 48 behind 0, 1, 2, 4, 16 and 18
+    whole tiles): the pieces of the last tile beyond K are fetched from inside the row and zeroed in LDS; 3600 x 3600 x 1200
+    is such a shape that AUTO sends here."""
     import torch
 
     print(f"gemm wave128 edge tiles {M}x{N}x{K} {out_dtype}", flush=True)
@@ -287,7 +291,7 @@ def test_gemm_wave128_edge_tiles(tcu, oracle, device, M, N, K, out_dtype):
     ref = oracle.gemm(A, Bt, rows=rows)
     assert oracle.max_rel_err(host(out)[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= REL_TOL
     assert torch.equal(out, tcu.gemm(dA, dB, out_dtype=dt, algo="pipelined"))
-    if M == 3088:
+    if M == 3088 or M == 3600:
         auto = tcu.gemm(dA, dB, out_dtype=dt, workspace=False)
         assert torch.equal(out, auto)
 

@@ -232,14 +232,14 @@ int gemm_w128_dispatch(const __half* A, const __half* B, OutType* C, int M, int 
     if (lda == 0) lda = K;
     if (ldb == 0) ldb = K;
     if (ldc == 0) ldc = N;
-    if (M % 16 != 0 || N % 16 != 0 || K % T::kBK != 0)
-        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM needs M and N in multiples of 16 and K % 64 == 0");
+    if (M % 16 != 0 || N % 16 != 0 || K % 16 != 0)
+        return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM needs M, N and K in multiples of 16");
     if ((long)std::max(lda, ldb) * 2 * T::kBM >= (1l << 32))
         return fail(TCU_ERR_UNSUPPORTED_SHAPE, "the one-wavefront-per-SIMD GEMM addresses a 256-row panel with 32-bit offsets");
-    if (M % T::kBM == 0 && N % T::kBN == 0)
+    if (M % T::kBM == 0 && N % T::kBN == 0 && K % T::kBK == 0)
         return launch(&gemm_w128<OutType>, dim3((M / T::kBM) * (N / T::kBN)), dim3(T::kThreads), T::kLdsBytes, stream, A, B,
                       C, M, N, K, lda, ldb, ldc, zero_words, zero_count);
-    // edge tiles: rows beyond M or N loaded from the last valid row, stores guarded
+    // edge tiles: rows beyond M or N loaded from the last valid row, stores guarded, a partial last tile of K zero-filled
     const long grid = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
     if (grid > INT_MAX) return fail(TCU_ERR_UNSUPPORTED_SHAPE, "GEMM: too many tiles for one launch");
     return launch(&gemm_w128<OutType, T, true>, dim3(unsigned(grid)), dim3(T::kThreads), T::kLdsBytes, stream, A, B, C, M, N,
@@ -586,8 +586,8 @@ int gemm_dispatch(const __half* A, const __half* B, OutType* C, int M, int N, in
                 // rows or columns that fill whole rounds plus smaller tiles on the rest, or the pipelined kernel with the
                 // tile its cost model picks - whichever is expected to be the shortest
                 const long tiles_e = (long)((M + 255) / 256) * ((N + 255) / 256);
-                const double edge_us = K % 64 == 0 && tiles_e >= 128 && (long)K * 512 < (1l << 32)
-                                           ? gemm_w128_us(tiles_e, K) : 1e30;
+                const double edge_us = K % 16 == 0 && tiles_e >= 128 && (long)K * 512 < (1l << 32)
+                                           ? gemm_w128_us(tiles_e, (K + 63) / 64 * 64) : 1e30;
                 const GemmRoundsPlan rounds = gemm_rounds_and_rest_plan(M, N, K);
                 const double rounds_us = rounds.us / 0.93;  // (two launches have to promise 7 % over the other plans)
                 const int rc = gemm_main_and_strips<OutType>(A, B, C, M, N, K, stream, std::min(edge_us, rounds_us));
