@@ -373,11 +373,13 @@ int gemm_main_and_strips(const __half* A, const __half* B, OutType* C, int M, in
 /// Whether AUTO sends an unsplit product to the kernel whose wavefronts split K: about one 128 x 128 tile per CU and a
 /// long enough K (2048^3: 21.9 against 26.8 us for the LDS-bound 64 x 64-per-wavefront tilings, 1536 x 1536 x 4096: 26.6
 /// against 38.5 us, 2048 x 2048 x 1536: 19.8 against 22.6 us); with a short K its reduction through LDS costs more than
-/// it saves (1792 x 1792 x 1024: 15.6 against 14.1 us).
+/// it saves.
 bool gemm_w128k_is_the_choice(int M, int N, int K) {
-    if (M % 16 != 0 || N % 16 != 0 || K % 128 != 0 || K < 1536 || (long)K * 256 >= (1l << 32)) return false;
+    if (M % 16 != 0 || N % 16 != 0 || K % 128 != 0 || K < 1024 || (long)K * 256 >= (1l << 32)) return false;
     const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-    return tiles >= (K >= 2048 ? 96 : 128) && tiles <= 256;  // (1424 x 1280 x 4096, 120 tiles: 25.6 against 29.2 us)
+    // the fewer tiles, the longer K has to be (1408 x 1280 x 4096, 110 tiles: 24.7 against 26.1 us; 1536 x 1280 x 2048, 120:
+    // 15.6 against 14.2; 1792^2 x 1024, 196: 11.8 against 13.2; 1536^2 x 1024, 144: 10.3 against 10.0)
+    return tiles >= (K >= 4096 ? 100 : K >= 1536 ? 128 : 150) && tiles <= 256;
 }
 
 /// Whether AUTO sends an unsplit product to the 256 x 128 tile: at most 128 tiles of 256 x 256 (half of the chip or
