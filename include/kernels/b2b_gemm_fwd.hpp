@@ -229,7 +229,9 @@ struct B2bRowsTraits {
     static constexpr int kRowBytesK = 2 * kK, kRowBytesN = 2 * kN;
     static constexpr int kBOff = 0;
     static constexpr int kCOff = kBOff + kN * kRowBytesK;
-    static constexpr int kLdsBytes = kCOff + kP * kRowBytesN;  // 128 KiB
+    static constexpr int kStageOff = kCOff + kP * kRowBytesN;   // 128 KiB of weights, then the f16 output staging:
+    static constexpr int kStageBytesPerWave = 16 * kP * 2;      // 16 rows of D per wavefront
+    static constexpr int kLdsBytes = kStageOff + kWaves * kStageBytesPerWave;  // 144 KiB
     static_assert(kLdsBytes <= kMaxLdsBytes);
 };
 
@@ -380,20 +382,41 @@ __global__ void __launch_bounds__(B2bRowsTraits::kThreads)
 #pragma unroll
             for (int pt = 0; pt < 8; ++pt)
                 asm volatile("" : "+a"(acc2[pt][0]), "+a"(acc2[pt][1]), "+a"(acc2[pt][2]), "+a"(acc2[pt][3]));
+            if constexpr (sizeof(OutType) == 4) {
 #pragma unroll
-            for (int pt = 0; pt < 8; ++pt)
+                for (int pt = 0; pt < 8; ++pt)
+#pragma unroll
+                    for (int mt = 0; mt < kMT; ++mt)
+                        *reinterpret_cast<f32x4*>(Db + size_t(row0 + 16 * mt + L) * kP + 16 * pt + 4 * g) = acc2[pt][mt];
+            } else {
+                // f16: 16 rows at a time through 4 KiB of LDS of this wavefront's own (the 8-byte slots of a row XOR-ed with
+                // twice the row), so that D leaves as whole 256-byte rows, 16 bytes per lane, through non-temporal stores:
+                // 8-byte pieces would have to be gathered into lines by the L2, and lines left dirty there are written
+                // back after the kernel's last wavefront
+                using lds_f16x4_ptr = __attribute__((address_space(3))) f16x4*;
+                using lds_u32x4_ptr = __attribute__((address_space(3))) const u32x4*;
+                const unsigned int stg = lds_base + T::kStageOff + wave * T::kStageBytesPerWave;
+                const int q4 = lane >> 4, c = lane & 15;  // read-back: row 4 it + q4, 16-byte piece c
 #pragma unroll
                 for (int mt = 0; mt < kMT; ++mt) {
-                    OutType* dst = Db + size_t(row0 + 16 * mt + L) * kP + 16 * pt + 4 * g;
-                    if constexpr (sizeof(OutType) == 4) {
-                        *reinterpret_cast<f32x4*>(dst) = acc2[pt][mt];
-                    } else {
+#pragma unroll
+                    for (int pt = 0; pt < 8; ++pt) {
                         f16x4 v;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc2[pt][mt][e]);
-                        *reinterpret_cast<f16x4*>(dst) = v;
+                        *reinterpret_cast<lds_f16x4_ptr>(stg + L * (kP * 2) + (((4 * pt + g) ^ (2 * L)) & 31) * 8) = v;
+                    }
+                    // LDS operations of one wavefront execute in order: the reads see the writes above, the next
+                    // row group's writes come behind them
+#pragma unroll
+                    for (int it = 0; it < 4; ++it) {
+                        const int q = 4 * it + q4;
+                        const u32x4 v = *reinterpret_cast<lds_u32x4_ptr>(stg + q * (kP * 2) + (((2 * c) ^ (2 * q)) & 31) * 8);
+                        __builtin_nontemporal_store(
+                            v, reinterpret_cast<u32x4*>(Db + size_t(row0 + 16 * mt + q) * kP + 8 * c));
                     }
                 }
+            }
         }
         if (next0 < M) {
 #pragma unroll
