@@ -38,7 +38,8 @@ struct B2bResidentTraits {
     static constexpr int kBOff = kAOff + kTM * kRowBytesK;
     static constexpr int kCOff = kBOff + kN * kRowBytesK;
     static constexpr int kSOff = kCOff + kP * kRowBytesN;
-    static constexpr int kLdsBytes = kSOff + kTM * kRowBytesN;
+    static constexpr int kDOff = kSOff + kTM * kRowBytesN;  // the f16 output tile on its way out: 32 rows of 256 bytes
+    static constexpr int kLdsBytes = kDOff + kTM * kP * 2;  // 160 KiB
     static_assert(kLdsBytes <= kMaxLdsBytes);
     /// Physical 16-byte chunk of logical chunk c in row `row` (rows of 16 or 32 chunks).
     HOST_DEVICE static constexpr int swz(int c, int row) { return (c & 16) | ((c & 15) ^ (row & 15)); }
@@ -162,17 +163,26 @@ __global__ void __launch_bounds__(B2bResidentTraits::kThreads)
         load_c(nb + 1);
     }
     }  // blocks of N
+    if constexpr (sizeof(OutType) == 4) {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-        OutType* dst = Db + size_t(16 * mt + L) * kP + 16 * wave + 4 * g;
-        if constexpr (sizeof(OutType) == 4) {
-            *reinterpret_cast<f32x4*>(dst) = acc2[mt];
-        } else {
+        for (int mt = 0; mt < 2; ++mt)
+            *reinterpret_cast<f32x4*>(Db + size_t(16 * mt + L) * kP + 16 * wave + 4 * g) = acc2[mt];
+    } else {
+        // f16: the tile is gathered in LDS (8-byte slots of a row XOR-ed with twice the row) and leaves as whole 256-byte
+        // rows, one 16-byte piece per lane, through non-temporal stores - a wavefront's own share is 32 bytes of every
+        // row, which the L2 would have to gather into lines and write back after the kernel's last wavefront
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
             f16x4 v;
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = static_cast<_Float16>(acc2[mt][e]);
-            *reinterpret_cast<f16x4*>(dst) = v;
+            const int row = 16 * mt + L;
+            *reinterpret_cast<f16x4*>(lds + T::kDOff + row * (kP * 2) + (((4 * wave + g) ^ (2 * row)) & 31) * 8) = v;
         }
+        __syncthreads();
+        const int row = threadIdx.x >> 4, c = threadIdx.x & 15;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(lds + T::kDOff + row * (kP * 2) + (((2 * c) ^ (2 * row)) & 31) * 8);
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(Db + size_t(row) * kP + 8 * c));
     }
 }
 
