@@ -199,8 +199,13 @@ struct ResidentFusedGemmTraits {
     using SharedB = SharedTile<InType, tl::ColMajor<kK, kTN>, true>;
     using SharedC = SharedTile<InType, tl::ColMajor<kTN, kP>, true>;
     using SharedS = SharedTile<InType, tl::RowMajor<kTM, kTN>, true>;  // the intermediate of one block
-    static constexpr int kShmBytes =
+    // a 2-byte output tile is gathered in LDS behind the operands and leaves as whole rows (SharedToGlobalStreamStorer);
+    // a 4-byte one would not fit beside them and goes from registers to memory
+    static constexpr bool kStageD = sizeof(OutType) == 2;
+    using SharedD = SharedTile<OutType, tl::RowMajor<kTM, kP>, true>;
+    static constexpr int kShmOperands =
         (SharedA::kNumel + SharedB::kNumel + SharedC::kNumel + SharedS::kNumel) * int(sizeof(InType));  // 152 KiB by default
+    static constexpr int kShmBytes = kShmOperands + (kStageD ? SharedD::kNumel * int(sizeof(OutType)) : 0);  // 160 KiB
     static_assert(kShmBytes <= kMaxLdsBytes);
 
     using LoadA = GlobalToSharedDirectLoader<SharedA, WarpLayout>;
@@ -226,6 +231,8 @@ struct ResidentFusedGemmTraits {
     using ReadC = SharedToRegLoader<RegC, WarpLayout, WarpReuse::kColReuseCont>;
     using ConvertD = compute::RegTileConvert<RegD, RegDCast>;
     using StoreD = RegToGlobalStorer<GlobalD, RegDCast, WarpLayout>;
+    using StageD = RegToSharedStorer<RegDCast, WarpLayout>;
+    using StreamD = SharedToGlobalStreamStorer<SharedD, WarpLayout>;
 };
 
 /// grid = (M / 32, batch), block = 512, dynamic LDS = Traits::kShmBytes.
@@ -299,8 +306,17 @@ __global__ void __launch_bounds__(Traits::kThreads)
     typename Traits::ConvertD cast_d;
     cast_d(rD, rD_out);
     typename Traits::GlobalD gD(D);
-    typename Traits::StoreD store_d;
-    store_d(rD_out, gD);
+    if constexpr (Traits::kStageD) {
+        typename Traits::SharedD sD(reinterpret_cast<OutType*>(shared_buf + Traits::kShmOperands));
+        typename Traits::StageD stage_d;
+        typename Traits::StreamD stream_d;
+        stage_d(rD_out, sD);
+        __syncthreads();
+        stream_d(sD, gD);
+    } else {
+        typename Traits::StoreD store_d;
+        store_d(rD_out, gD);
+    }
 }
 
 }  // namespace tiledcuda::kernels
