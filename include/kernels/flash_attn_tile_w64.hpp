@@ -84,7 +84,7 @@ struct FlashW64TileTraits {
     using Scores = compute::ScheduledGemm<RegQ, RegK, RegS, compute::RegFile::kVgpr, compute::RegFile::kAgpr>;
     using Output = compute::ScheduledGemm<RegP, RegV, RegO, compute::RegFile::kAgpr, compute::RegFile::kVgpr>;
     using OutToShared = RegToSharedStorer<RegOut, WarpLayout>;
-    using OutToGlobal = SharedToGlobalStorer<SharedO, WarpLayout>;
+    using OutToGlobal = SharedToGlobalStreamStorer<SharedO, WarpLayout>;
     static_assert(PiecesK::kPieces == 4 && PiecesV::kPieces == 4, "a wavefront issues 8 loads per block, one per d-step");
 };
 

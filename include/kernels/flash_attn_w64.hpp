@@ -753,7 +753,7 @@ __global__ void __launch_bounds__(Traits::kThreads)
         const int row = it * kRowsPerIter + rr;
         const int pslot = (2 * cc) ^ (((row & 15) << 1) & kSlotMask);
         const u32x4 v = *reinterpret_cast<const u32x4*>(stg + row * kRowBytes + pslot * 8);
-        if (active) *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(Oh + size_t(row) * kD) + cc * 16) = v;
+        if (active) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(Oh + size_t(row) * kD) + cc * 16));  // whole rows, streamed
     }
 }
 
