@@ -98,19 +98,20 @@ __global__ void __launch_bounds__(256) splitk_reduce(const float* __restrict__ p
                                                      size_t n, int splits) {
     const size_t i = (size_t(blockIdx.x) * 256 + threadIdx.x) * 4;
     if (i >= n) return;
-    f32x4 acc = *reinterpret_cast<const f32x4*>(partial + i);
+    // (read once, written once: streamed both ways)
+    f32x4 acc = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(partial + i));
     for (int z = 1; z < splits; ++z) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(partial + size_t(z) * n + i);
+        const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(partial + size_t(z) * n + i));
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[e] += v[e];
     }
     if constexpr (sizeof(OutType) == 4) {
-        *reinterpret_cast<f32x4*>(C + i) = acc;
+        __builtin_nontemporal_store(acc, reinterpret_cast<f32x4*>(C + i));
     } else {
         f16x4 h;
 #pragma unroll
         for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[e]);
-        *reinterpret_cast<f16x4*>(C + i) = h;
+        __builtin_nontemporal_store(h, reinterpret_cast<f16x4*>(C + i));
     }
 }
 
