@@ -199,11 +199,32 @@ __global__ void __launch_bounds__(T::kThreads)
     // ---- LDS -> registers: fragment r of a substep (r < 8: A rows 16 r.., else B rows 16 (r - 8)..); lane l holds
     // row l % 16, k = 8 (l / 16) .. +7 of the 32-wide substep = logical chunk 4 kk + l / 16 of its row
     const int frow = lane & 15, fquad = lane >> 4;
-    auto read_frag = [&](int stage, int kk, int r) -> f16x8 {
-        const int row = (r < 8 ? wave_m * T::kWaveM + r * 16 : wave_n * T::kWaveN + (r - 8) * 16) + frow;
-        const int chunk = (4 * kk + fquad) ^ ((row >> 1) & 7);
-        return *reinterpret_cast<const f16x8*>(lds + stage * T::kStageBytes + (r < 8 ? 0 : T::kABytes) +
-                                               row * T::kRowBytes + chunk * 16);
+    // Two stages: the lane's address of fragment 0 of A and of B, per stage and substep, in registers of their own (the
+    // XOR term depends on lane % 16 only, so fragment r lies r * 2 KiB further on: an immediate) - the second stage
+    // begins 64 KiB further on, which no immediate reaches.
+    unsigned int frag_a[2][2], frag_b[2][2];  // [stage][kk]
+    if constexpr (T::kStages == 2) {
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            const unsigned int lane_off = frow * T::kRowBytes + (((4 * kk + fquad) ^ ((frow >> 1) & 7)) * 16);
+            frag_a[0][kk] = lds_base + wave_m * T::kWaveM * T::kRowBytes + lane_off;
+            frag_b[0][kk] = lds_base + T::kABytes + wave_n * T::kWaveN * T::kRowBytes + lane_off;
+            frag_a[1][kk] = frag_a[0][kk] + T::kStageBytes;
+            frag_b[1][kk] = frag_b[0][kk] + T::kStageBytes;
+            asm volatile("" : "+v"(frag_a[0][kk]), "+v"(frag_b[0][kk]), "+v"(frag_a[1][kk]), "+v"(frag_b[1][kk]));
+        }
+    }
+    auto read_frag = [&](int stage, int kk, int r) __attribute__((always_inline)) -> f16x8 {
+        if constexpr (T::kStages == 2) {
+            using lds_f16x8_ptr = __attribute__((address_space(3))) const f16x8*;
+            const unsigned int base = r < 8 ? (stage ? frag_a[1][kk] : frag_a[0][kk]) : (stage ? frag_b[1][kk] : frag_b[0][kk]);
+            return *reinterpret_cast<lds_f16x8_ptr>(base + (r < 8 ? r : r - 8) * 16 * T::kRowBytes);
+        } else {
+            const int row = (r < 8 ? wave_m * T::kWaveM + r * 16 : wave_n * T::kWaveN + (r - 8) * 16) + frow;
+            const int chunk = (4 * kk + fquad) ^ ((row >> 1) & 7);
+            return *reinterpret_cast<const f16x8*>(lds + stage * T::kStageBytes + (r < 8 ? 0 : T::kABytes) +
+                                                   row * T::kRowBytes + chunk * 16);
+        }
     };
 
     f16x8 fx[kFrags], fy[kFrags];  // fragments of substep 0 / substep 1: [0..7] A, [8..] B
@@ -272,11 +293,13 @@ __global__ void __launch_bounds__(T::kThreads)
     // One tile of K. kMore: there is a tile kt+1 (read its substep 0 during phase 2); kMore2: there is a tile kt+2
     // (load it during phase 2). Row group i = MFMA tiles (i, 0..7): the MFMA order is fixed by the asm statements, the
     // fragment reads (plain loads) are written where they should issue and the compiler keeps them there.
-    // kTailLoads: the tile loaded here is the last one and may be partial.
-    auto tile = [&](int kt, auto more_c, auto more2_c, auto tail_loads_c) {
+    // kTailLoads: the tile loaded here is the last one and may be partial. In the loop over K, unrolled by two, the stage
+    // is a constant, so that every LDS address there is a register fixed for the kernel plus an immediate (with the stage a
+    // run-time value a tile pays 8 vector additions in front of fragment reads and 26 scalar ones).
+    auto tile = [&](int kt, auto more_c, auto more2_c, auto tail_loads_c, auto stage_v) __attribute__((always_inline)) {
         constexpr bool kMore = decltype(more_c)::value, kMore2 = decltype(more2_c)::value;
         constexpr bool kTailLoads = decltype(tail_loads_c)::value;
-        const int stage = kt & 1;
+        const int stage = stage_v;  // an integral_constant in the unrolled loop, kt % 2 in the tiles behind it
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
@@ -358,19 +381,27 @@ __global__ void __launch_bounds__(T::kThreads)
         }
         detail::wait_vmcnt<0>();  // (the last loads, of data nobody uses, have landed before the workgroup ends)
     } else {
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        constexpr int kTailTiles = kTail ? 1 : 0;  // (the tile that requests a partial last tile is not part of the loop)
         int kt = 0;
-        for (; kt + (kTail ? 3 : 2) < ktiles; ++kt) tile(kt, std::true_type{}, std::true_type{}, std::false_type{});
+        for (; kt + 3 + kTailTiles < ktiles; kt += 2) {
+            tile(kt, std::true_type{}, std::true_type{}, std::false_type{}, I0{});
+            tile(kt + 1, std::true_type{}, std::true_type{}, std::false_type{}, I1{});
+        }
+        // the tiles behind the unrolled loop: one more that loads a tile, then the last two peeled
+        for (; kt + 2 + kTailTiles < ktiles; ++kt) tile(kt, std::true_type{}, std::true_type{}, std::false_type{}, kt & 1);
         if constexpr (kTail) {  // the iteration that loads the last tile: with the offsets of a partial one
             if (kt + 2 < ktiles) {
-                tile(kt, std::true_type{}, std::true_type{}, std::true_type{});
+                tile(kt, std::true_type{}, std::true_type{}, std::true_type{}, kt & 1);
                 ++kt;
             }
         }
         if (kt + 1 < ktiles) {
-            tile(kt, std::true_type{}, std::false_type{}, std::false_type{});
+            tile(kt, std::true_type{}, std::false_type{}, std::false_type{}, kt & 1);
             ++kt;
         }
-        tile(kt, std::false_type{}, std::false_type{}, std::false_type{});
+        tile(kt, std::false_type{}, std::false_type{}, std::false_type{}, kt & 1);
     }
 
     // the compiler does not know the statements above are MFMAs: wait once for the last results, then pass every
