@@ -199,32 +199,30 @@ __global__ void __launch_bounds__(T::kThreads)
     // ---- LDS -> registers: fragment r of a substep (r < 8: A rows 16 r.., else B rows 16 (r - 8)..); lane l holds
     // row l % 16, k = 8 (l / 16) .. +7 of the 32-wide substep = logical chunk 4 kk + l / 16 of its row
     const int frow = lane & 15, fquad = lane >> 4;
-    // Two stages: the lane's address of fragment 0 of A and of B, per stage and substep, in registers of their own (the
-    // XOR term depends on lane % 16 only, so fragment r lies r * 2 KiB further on: an immediate) - the second stage
-    // begins 64 KiB further on, which no immediate reaches.
-    unsigned int frag_a[2][2], frag_b[2][2];  // [stage][kk]
-    if constexpr (T::kStages == 2) {
+    // The lane's address of fragment 0 of A and of B, per stage and substep, in registers of their own (the XOR term
+    // depends on lane % 16 only, so fragment r lies r * 2 KiB further on: an immediate) - the later stages begin 48 or
+    // 64 KiB further on, which no immediate reaches.
+    unsigned int frag_a[T::kStages][2], frag_b[T::kStages][2];  // [stage][kk]
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-            const unsigned int lane_off = frow * T::kRowBytes + (((4 * kk + fquad) ^ ((frow >> 1) & 7)) * 16);
-            frag_a[0][kk] = lds_base + wave_m * T::kWaveM * T::kRowBytes + lane_off;
-            frag_b[0][kk] = lds_base + T::kABytes + wave_n * T::kWaveN * T::kRowBytes + lane_off;
-            frag_a[1][kk] = frag_a[0][kk] + T::kStageBytes;
-            frag_b[1][kk] = frag_b[0][kk] + T::kStageBytes;
-            asm volatile("" : "+v"(frag_a[0][kk]), "+v"(frag_b[0][kk]), "+v"(frag_a[1][kk]), "+v"(frag_b[1][kk]));
+    for (int kk = 0; kk < 2; ++kk) {
+        const unsigned int lane_off = frow * T::kRowBytes + (((4 * kk + fquad) ^ ((frow >> 1) & 7)) * 16);
+#pragma unroll
+        for (int st = 0; st < T::kStages; ++st) {
+            frag_a[st][kk] = lds_base + st * T::kStageBytes + wave_m * T::kWaveM * T::kRowBytes + lane_off;
+            frag_b[st][kk] = lds_base + st * T::kStageBytes + T::kABytes + wave_n * T::kWaveN * T::kRowBytes + lane_off;
+            asm volatile("" : "+v"(frag_a[st][kk]), "+v"(frag_b[st][kk]));
         }
     }
-    auto read_frag = [&](int stage, int kk, int r) __attribute__((always_inline)) -> f16x8 {
-        if constexpr (T::kStages == 2) {
-            using lds_f16x8_ptr = __attribute__((address_space(3))) const f16x8*;
-            const unsigned int base = r < 8 ? (stage ? frag_a[1][kk] : frag_a[0][kk]) : (stage ? frag_b[1][kk] : frag_b[0][kk]);
-            return *reinterpret_cast<lds_f16x8_ptr>(base + (r < 8 ? r : r - 8) * 16 * T::kRowBytes);
+    // (stage: a constant, or with two stages a run-time 0 / 1 in the tiles behind the unrolled loop)
+    auto read_frag = [&](auto stage, int kk, int r) __attribute__((always_inline)) -> f16x8 {
+        using lds_f16x8_ptr = __attribute__((address_space(3))) const f16x8*;
+        unsigned int base;
+        if constexpr (std::is_same_v<decltype(stage), int>) {  // (two stages only: the three-stage form never gets here)
+            base = r < 8 ? (stage ? frag_a[1][kk] : frag_a[0][kk]) : (stage ? frag_b[1][kk] : frag_b[0][kk]);
         } else {
-            const int row = (r < 8 ? wave_m * T::kWaveM + r * 16 : wave_n * T::kWaveN + (r - 8) * 16) + frow;
-            const int chunk = (4 * kk + fquad) ^ ((row >> 1) & 7);
-            return *reinterpret_cast<const f16x8*>(lds + stage * T::kStageBytes + (r < 8 ? 0 : T::kABytes) +
-                                                   row * T::kRowBytes + chunk * 16);
+            base = r < 8 ? frag_a[decltype(stage)::value][kk] : frag_b[decltype(stage)::value][kk];
         }
+        return *reinterpret_cast<lds_f16x8_ptr>(base + (r < 8 ? r : r - 8) * 16 * T::kRowBytes);
     };
 
     f16x8 fx[kFrags], fy[kFrags];  // fragments of substep 0 / substep 1: [0..7] A, [8..] B
@@ -282,7 +280,7 @@ __global__ void __launch_bounds__(T::kThreads)
         detail::lds_barrier<0>();
     }
 #pragma unroll
-    for (int r = 0; r < kFrags; ++r) fx[r] = read_frag(0, 0, r);
+    for (int r = 0; r < kFrags; ++r) fx[r] = read_frag(std::integral_constant<int, 0>{}, 0, r);
 
     // Order of the fragment reads of a phase: row group 0 of the next phase needs A fragment 0 and all B fragments.
     auto order = [](int r) { return r == 0 ? 0 : r <= kNT ? 7 + r : r - kNT; };
@@ -342,14 +340,15 @@ __global__ void __launch_bounds__(T::kThreads)
     // loads of tile kt + 2 still on their way, and phase 2 requests tile kt + 3 into the stage just vacated: a load has
     // three phases to land instead of one to two. Straight-line code: behind the end of K the loads fetch the last tile
     // again and the fragment reads fetch data nobody uses.
-    auto tile3 = [&](int kt, int stage, int next) {
+    auto tile3 = [&](int kt, auto stage_c, auto next_c) __attribute__((always_inline)) {
+        constexpr int stage = decltype(stage_c)::value;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
             for (int n = 0; n < kNT; ++n) {
                 const int j = snake(i, n);
                 const int r = (kNT / 2) * i + (n >> 1);
-                if ((n & 1) == 0 && r < kFrags) fy[order(r)] = read_frag(stage, 1, order(r));
+                if ((n & 1) == 0 && r < kFrags) fy[order(r)] = read_frag(stage_c, 1, order(r));
                 detail::mfma_16x16x32_agpr(acc[i][j], fx[8 + j], fx[i]);
             }
         }
@@ -360,7 +359,7 @@ __global__ void __launch_bounds__(T::kThreads)
             for (int n = 0; n < kNT; ++n) {
                 const int j = snake(i, n);
                 const int r = (kNT / 2) * i + (n >> 1);
-                if ((n & 1) == 0 && r < kFrags) fx[order(r)] = read_frag(next, 0, order(r));
+                if ((n & 1) == 0 && r < kFrags) fx[order(r)] = read_frag(next_c, 0, order(r));
                 const int m = kNT * i + n;  // 12 loads over 32 MFMAs: behind MFMAs 0, 3, 6 of every 8
                 const int q = (3 * m) / 8;
                 if ((3 * m) % 8 < 3 && q < kNumLoads) {
@@ -373,12 +372,18 @@ __global__ void __launch_bounds__(T::kThreads)
         }
     };
     if constexpr (T::kStages == 3) {
-        int stage = 0;
-        for (int kt = 0; kt < ktiles; ++kt) {
-            const int next = stage == 2 ? 0 : stage + 1;
-            tile3(kt, stage, next);
-            stage = next;
+        // unrolled by three: the stage of every fragment read and load is a constant
+        using S0 = std::integral_constant<int, 0>;
+        using S1 = std::integral_constant<int, 1>;
+        using S2 = std::integral_constant<int, 2>;
+        int kt = 0;
+        for (; kt + 2 < ktiles; kt += 3) {
+            tile3(kt, S0{}, S1{});
+            tile3(kt + 1, S1{}, S2{});
+            tile3(kt + 2, S2{}, S0{});
         }
+        if (kt < ktiles) tile3(kt, S0{}, S1{});
+        if (kt + 1 < ktiles) tile3(kt + 1, S1{}, S2{});
         detail::wait_vmcnt<0>();  // (the last loads, of data nobody uses, have landed before the workgroup ends)
     } else {
         using I0 = std::integral_constant<int, 0>;
