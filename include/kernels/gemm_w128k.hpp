@@ -105,10 +105,14 @@ __global__ void __launch_bounds__(T::kThreads)
     // k = 32 wave + 8 (l / 16) .. + 7 of the tile = logical chunk 4 wave + l / 16 of its row. The 16 rows a 16-lane
     // group reads have 16 different values of row % 16: 16 different chunks, no bank conflict.
     const int frow = lane & 15, fquad = lane >> 4;
-    auto read_frag = [&](unsigned int slot_a, unsigned int slot_b, int r) -> f16x8 {
-        const int row = (r & 7) * 16 + frow;
-        const int chunk = (4 * wave + fquad) ^ (row & 15);
-        return *reinterpret_cast<const f16x8*>(lds + (r < 8 ? slot_a : slot_b) + row * T::kRowBytes + chunk * 16);
+    // The XOR term depends on lane % 16 only: the lane's address of fragment 0 of a slot is one register (frag_lane, fixed
+    // for the kernel) plus the slot's offset - one addition per part and tile - and fragment r lies (r % 8) * 2 KiB
+    // further on: an immediate.
+    unsigned int frag_lane = lds_base + frow * T::kRowBytes + (((4 * wave + fquad) ^ frow) * 16);
+    asm volatile("" : "+v"(frag_lane));
+    auto read_frag = [&](unsigned int base_a, unsigned int base_b, int r) __attribute__((always_inline)) -> f16x8 {
+        using lds_f16x8_ptr = __attribute__((address_space(3))) const f16x8*;
+        return *reinterpret_cast<lds_f16x8_ptr>((r < 8 ? base_a : base_b) + (r & 7) * 16 * T::kRowBytes);
     };
 
     f16x8 fx[T::kFrags], fy[T::kFrags];  // fragments of the tile being multiplied / of the next one: [0..7] A, [8..] B
@@ -137,7 +141,7 @@ __global__ void __launch_bounds__(T::kThreads)
     }
     detail::lds_barrier<16 + T::kLoadsB>();  // tile 0 has landed (behind it: A1 B1 A2), for everyone
 #pragma unroll
-    for (int r = 0; r < T::kFrags; ++r) fx[r] = read_frag(0, T::kSlotBytes, r);
+    for (int r = 0; r < T::kFrags; ++r) fx[r] = read_frag(frag_lane, frag_lane + T::kSlotBytes, r);
 
     // the order in which the fragments of the next tile are read: its first row group needs A fragment 0 and all of B
     auto order = [](int r) { return r == 0 ? 0 : r <= kNT ? 7 + r : r - kNT; };
@@ -153,7 +157,8 @@ __global__ void __launch_bounds__(T::kThreads)
     // phase, whose control-flow merges made the compiler shuffle and spill accumulators between the assembly
     // statements, where it knows of no wait states.
     auto tile = [&](int kt, f16x8 (&cur)[T::kFrags], f16x8 (&nxt)[T::kFrags]) {
-        const unsigned int read_a = slot_bytes(2 * kt + 2), read_b = slot_bytes(2 * kt + 3);  // tile kt + 1
+        unsigned int read_a = frag_lane + slot_bytes(2 * kt + 2), read_b = frag_lane + slot_bytes(2 * kt + 3);  // tile kt + 1
+        asm volatile("" : "+v"(read_a), "+v"(read_b));  // (these two sums, not one per fragment)
         const unsigned int load_b = slot_bytes(2 * kt + 5), load_a = slot_bytes(2 * kt + 6);  // = the slots of tile kt
         const int kt_b = clamped(kt + 2), kt_a = clamped(kt + 3);
         // tile kt + 1 has landed (behind its B part: the A part of tile kt + 2) and this wavefront's reads of tile kt's
