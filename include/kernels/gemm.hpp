@@ -467,9 +467,10 @@ __global__ void __launch_bounds__(Traits::kThreads) gemm_tile_w128(const InType*
     for (int r = 0; r < 16; ++r) read_fragment(0, 0, 0, r);
 
     // kMore: there is a tile k1 + 1; kMore2: there is a tile k1 + 2
-    auto tile = [&](int k1, auto more_c, auto more2_c) {
+    // (stage: k1 % 2 - a constant in the loop unrolled by two, so that the addresses there are immediates)
+    auto tile = [&](int k1, auto more_c, auto more2_c, auto stage_v) __attribute__((always_inline)) {
         constexpr bool kMore = decltype(more_c)::value, kMore2 = decltype(more2_c)::value;
-        const int stage = k1 & 1;
+        const int stage = stage_v;
         compute::gemm_scheduled(rA[0], rB[0], acc, [&](auto n_c) {
             constexpr int n = decltype(n_c)::value;
             if constexpr (n % 2 == 0 && n / 2 < 16) read_fragment(stage, 1, 1, n / 2);
@@ -483,12 +484,16 @@ __global__ void __launch_bounds__(Traits::kThreads) gemm_tile_w128(const InType*
     };
     {
         int k1 = 0;
-        for (; k1 + 2 < kTiles; ++k1) tile(k1, std::true_type{}, std::true_type{});
+        for (; k1 + 3 < kTiles; k1 += 2) {
+            tile(k1, std::true_type{}, std::true_type{}, std::integral_constant<int, 0>{});
+            tile(k1 + 1, std::true_type{}, std::true_type{}, std::integral_constant<int, 1>{});
+        }
+        for (; k1 + 2 < kTiles; ++k1) tile(k1, std::true_type{}, std::true_type{}, k1 & 1);
         if (k1 + 1 < kTiles) {
-            tile(k1, std::true_type{}, std::false_type{});
+            tile(k1, std::true_type{}, std::false_type{}, k1 & 1);
             ++k1;
         }
-        tile(k1, std::false_type{}, std::false_type{});
+        tile(k1, std::false_type{}, std::false_type{}, k1 & 1);
     }
     compute::settle_accumulators(acc);
 
