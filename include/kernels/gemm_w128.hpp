@@ -163,9 +163,20 @@ __global__ void __launch_bounds__(T::kThreads)
     const __half* b_base = Bt + size_t(n0) * ldb + z * K;
     C += z * size_t(M) * ldc;
     const unsigned int lds_base = static_cast<unsigned int>(reinterpret_cast<uintptr_t>(lds));
-    auto load_dst = [&](int stage, int q) -> unsigned int {
-        return __builtin_amdgcn_readfirstlane(lds_base + stage * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +
-                                              (q < 8 ? wave * T::kLoads + q : wave * T::kLoadsB + (q - 8)) * 1024);
+    // the LDS destination of load q per stage: scalar registers of their own, so that the load's m0 is one s_mov away
+    // (an addition per load, recomputed in the loop, was a third instruction behind the MFMA the load rides on)
+    unsigned int dst_of[T::kStages][kNumLoads];
+#pragma unroll
+    for (int st = 0; st < T::kStages; ++st)
+#pragma unroll
+        for (int q = 0; q < kNumLoads; ++q) {
+            dst_of[st][q] = __builtin_amdgcn_readfirstlane(lds_base + st * T::kStageBytes + (q < 8 ? 0 : T::kABytes) +
+                                                           (q < 8 ? wave * T::kLoads + q : wave * T::kLoadsB + (q - 8)) * 1024);
+            asm volatile("" : "+s"(dst_of[st][q]));
+        }
+    auto load_dst = [&](int stage, int q) __attribute__((always_inline)) -> unsigned int {
+        if constexpr (T::kStages == 2) return stage ? dst_of[1][q] : dst_of[0][q];
+        else return stage == 0 ? dst_of[0][q] : stage == 1 ? dst_of[1][q] : dst_of[2][q];
     };
     // Rows a multiple of 32 KiB apart put the same k-tile of every row of every panel into the same few memory
     // channels, and all workgroups walk K in step. Each XCD then starts at a different eighth of K and wraps around
