@@ -159,7 +159,7 @@ int tcu_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K, int
  * ranges multiplied by different workgroups (the WAVE128_KSPLIT kernel with 128 x 128 tiles, or the WAVE128 kernel where
  * those tiles fill the chip by themselves; f32 partial products into `workspace`, [splits, M, N]) and a second kernel
  * adds the partial products. tcu_gemm_workspace_bytes(M, N, K) is the workspace
- * this takes, or 0 when the product is not split (more than 128 tiles of 256 x 256, M or N not multiples of 256,
+ * this takes, or 0 when the product is not split (more than 128 tiles of 256 x 256, M or N not multiples of 16,
  * less than 512 of K per range, or the unsplit kernel expected to be as fast): then, and when `workspace` is NULL,
  * the call is tcu_gemm_f16 with TCU_GEMM_AUTO. The workspace (16-byte aligned device
  * memory) is the caller's and free to reuse once the work enqueued here has run. Results differ from the unsplit

@@ -124,12 +124,14 @@ def test_gemm_ragged_shapes(tcu, oracle, device, M, N, K, out_dtype):
                                           (1024, 2048, 16384, 2), (2048, 2048, 32768, 4), (2048, 2048, 8192, 1),
                                           (2048, 4096, 2048, 1),
                                           (1536, 1536, 4096, 1), (1024, 1024, 8192, 4), (1024, 1024, 4096, 1), (256, 512, 512, 1),
+                                          (752, 1808, 8192, 2), (528, 512, 8192, 8), (272, 400, 8192, 16),
                                           (2048, 2048, 2048, 1)])
 @pytest.mark.parametrize("out_dtype", ["f32", "f16"])
 def test_gemm_split_k_with_workspace(tcu, oracle, device, M, N, K, splits, out_dtype):
     """tcu_gemm_f16_ws: few output tiles and a long K are split over K (f32 partial products in the caller's workspace,
     then a reduction) where that is expected to beat the unsplit launch - the partial products from the kernel with
-    128 x 128 tiles whose wavefronts split K once more (first four cases and 1024 x 1024 x 8192) or, where those tiles alone fill the chip, from
+    128 x 128 tiles whose wavefronts split K once more (first four cases, 1024 x 1024 x 8192, and - with edge tiles - the
+    three shapes that are not whole tiles) or, where those tiles alone fill the chip, from
     the one with 256 x 256 tiles (2048 x 2048 x 32768); against the oracle and against the unsplit kernel; the workspace size is splits * M * N * 4, bytes past it stay untouched; shapes that are not split (last six
     cases: among them 2048 x 2048 x 8192 and 1536 x 1536 x 4096, where the kernel whose wavefronts split K inside the
     workgroup is the faster plan) take the ordinary path and need no workspace."""

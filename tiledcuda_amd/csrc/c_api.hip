@@ -379,7 +379,8 @@ bool gemm_w128k_is_the_choice(int M, int N, int K) {
     const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
     // the fewer tiles, the longer K has to be (1408 x 1280 x 4096, 110 tiles: 24.7 against 26.1 us; 1536 x 1280 x 2048, 120:
     // 15.6 against 14.2; 1792^2 x 1024, 196: 11.8 against 13.2; 1536^2 x 1024, 144: 10.3 against 10.0)
-    return tiles >= (K >= 4096 ? 100 : K >= 1536 ? 128 : 150) && tiles <= 256;
+    // (512 x 2304 x 8192, 72 tiles: 40.3 against 42.7; 2304 x 640 x 8192, 90: 41.3 against 46.8)
+    return tiles >= (K >= 8192 ? 72 : K >= 4096 ? 100 : K >= 1536 ? 128 : 150) && tiles <= 256;
 }
 
 /// Whether AUTO sends an unsplit product to the 256 x 128 tile: at most 128 tiles of 256 x 256 (half of the chip or
@@ -484,8 +485,10 @@ struct GemmSplitPlan {
 GemmSplitPlan gemm_split_plan(int M, int N, int K) {
     using T = GemmW128Traits;
     GemmSplitPlan plan{1, false};
-    if (M % T::kBM != 0 || N % T::kBN != 0 || K % T::kBK != 0) return plan;
-    const long tiles = (long)(M / T::kBM) * (N / T::kBN);
+    if (M % 16 != 0 || N % 16 != 0 || K % T::kBK != 0) return plan;
+    const bool whole256 = M % T::kBM == 0 && N % T::kBN == 0;  // the 256 x 256 form splits whole tiles only
+    const long tiles = (long)((M + T::kBM - 1) / T::kBM) * ((N + T::kBN - 1) / T::kBN);
+    const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);  // (the 128 x 128 form has edge tiles)
     if (tiles > 128) return plan;
     double unsplit_us = pipelined_plan(M, N, K).us;
     // the kernels AUTO would run instead of the pipelined one
@@ -493,7 +496,7 @@ GemmSplitPlan gemm_split_plan(int M, int N, int K) {
     if (gemm_narrow_is_the_choice(M, N, K)) unsplit_us = std::min(unsplit_us, gemm_narrow_us(M, N, K));
     double best_us = 0.95 * unsplit_us;
     const double plane_us = 2.0 * double(M) * N * 4 / 5.3e6;  // a plane of partial products written and read once
-    for (int s = 2; s * tiles <= 256 && K % (s * T::kBK) == 0 && K / s >= 512; s *= 2) {
+    for (int s = 2; whole256 && s * tiles <= 256 && K % (s * T::kBK) == 0 && K / s >= 512; s *= 2) {
         const double us = 10.0 + 1.4 * (K / s / T::kBK) + s * plane_us;
         if (us < best_us) {
             plan = {s, false};
@@ -504,8 +507,8 @@ GemmSplitPlan gemm_split_plan(int M, int N, int K) {
     // reduction through LDS and the epilogues + per 128 of a range 0.62 us with up to 128 workgroups, rising to 0.95 us
     // with 256 (their loads share the L2s) - measured on 256^2 x 8192 ... 1024 x 2048 x 16384 with 2 to 16 ranges
     if ((long)K * 256 < (1l << 32)) {
-        for (int s = 2; s * tiles * 4 <= 256 && K % (s * 128) == 0 && K / s >= 512; s *= 2) {
-            const long groups = s * tiles * 4;
+        for (int s = 2; s * tiles128 <= 256 && K % (s * 128) == 0 && K / s >= 512; s *= 2) {
+            const long groups = s * tiles128;
             const double per_tile = 0.62 + 0.33 * (groups > 128 ? double(groups - 128) / 128.0 : 0.0);
             const double us = 8.0 + per_tile * (K / s / 128) + s * plane_us;
             if (us < best_us) {
@@ -528,9 +531,13 @@ int gemm_splitk(const __half* A, const __half* B, OutType* C, int M, int N, int 
     int rc;
     if (plan.tiles128) {
         using Tk = GemmW128kTraits;
-        const int tiles = (M / Tk::kBM) * (N / Tk::kBN);
-        rc = launch(&gemm_w128k<float, false, Tk>, dim3(tiles, plan.splits), dim3(Tk::kThreads), Tk::kLdsBytes, stream, A, B,
-                    partial, M, N, K / plan.splits, K, K, N);
+        const int tiles = ((M + Tk::kBM - 1) / Tk::kBM) * ((N + Tk::kBN - 1) / Tk::kBN);
+        if (M % Tk::kBM == 0 && N % Tk::kBN == 0)
+            rc = launch(&gemm_w128k<float, false, Tk>, dim3(tiles, plan.splits), dim3(Tk::kThreads), Tk::kLdsBytes, stream, A,
+                        B, partial, M, N, K / plan.splits, K, K, N);
+        else  // edge tiles: rows beyond M or N loaded from the last valid row, stores guarded
+            rc = launch(&gemm_w128k<float, true, Tk>, dim3(tiles, plan.splits), dim3(Tk::kThreads), Tk::kLdsBytes, stream, A,
+                        B, partial, M, N, K / plan.splits, K, K, N);
     } else {
         const int tiles = (M / T::kBM) * (N / T::kBN);
         rc = launch(&gemm_w128<float>, dim3(tiles, plan.splits), dim3(T::kThreads), T::kLdsBytes, stream, A, B, partial, M, N,
